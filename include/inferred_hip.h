@@ -1,0 +1,257 @@
+/* inferred_hip.h — C ABI of the MI355X (gfx950) backend for the per-token model loop.
+ *
+ * Every `it_hip_*` op below replaces one method of the reference's backend seam,
+ * `trait Ops` (/root/reference src/ops/mod.rs:489-1426), with the same argument
+ * order and meaning: Rust slices become (pointer, length) pairs, the argument
+ * structs become the plain-old-data structs declared here, and `&self` becomes the
+ * opaque `it_hip*`.  All pointers are HOST pointers, exactly as at the seam: the
+ * backend keeps device copies keyed on the host address (activation mirrors,
+ * resident weights, device-owned KV and recurrent-state slabs) and moves data only
+ * at `host_wrote` / `host_needs` / first touch.
+ *
+ * Conventions carried over from the reference:
+ *  - batch size is derived from buffer lengths, never passed (mod.rs:462-488);
+ *  - ops return nothing; the first error is kept and later calls keep going; poll
+ *    it_hip_take_error() after the run (src/ops/cuda/ops/mod.rs:91-110);
+ *  - one host thread drives one backend; all device work is issued in call order;
+ *  - never pass a sub-slice of an activation (a prefix is fine).
+ */
+#ifndef INFERRED_HIP_H
+#define INFERRED_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type codes (src/gguf/types.rs:62-100) */
+enum { IT_F32 = 0, IT_F16 = 1, IT_Q8_0 = 8, IT_BF16 = 30, IT_NVFP4 = 40 };
+
+/* struct Weights, src/ops/mod.rs:62-92 */
+typedef struct {
+    const uint8_t* data;
+    uint64_t len; /* bytes */
+    uint32_t ty;
+    uint32_t pooled;
+    uint64_t n_in, n_out;
+} it_weights;
+
+/* struct Experts, src/ops/mod.rs:107-152 */
+typedef struct {
+    const uint8_t* data;
+    uint64_t len;
+    uint32_t ty;
+    uint32_t _pad;
+    uint64_t n_in, n_out, n_expert;
+    const uint8_t* scale; /* n_expert little-endian f32, NULL when the file has none */
+    uint64_t scale_len;   /* bytes */
+} it_experts;
+
+/* struct Attn, src/ops/mod.rs:228-276; n_q is derived from q_len */
+typedef struct {
+    const float* q;
+    uint64_t q_len;
+    const uint16_t* k;
+    const uint16_t* v;
+    uint64_t kv_len; /* elements in each slab */
+    uint64_t kv_dim, n_pos, head_dim, n_head, n_head_kv;
+    float scale;
+} it_attn;
+
+/* struct Delta, src/ops/mod.rs:337-358; n_tokens = v_len / (n_v_heads * head_v_dim) */
+typedef struct {
+    const float *q, *k, *v, *alpha, *beta, *ssm_a, *dt_bias;
+    uint64_t n_tokens;
+    uint64_t head_k_dim, head_v_dim, n_k_heads, n_v_heads;
+} it_delta;
+
+/* enum Route, src/ops/mod.rs:176-218 */
+enum { IT_ROUTE_HOST = 0, IT_ROUTE_DEVICE = 1 };
+typedef struct {
+    uint32_t kind;
+    uint32_t _pad;
+    const uint64_t* ids;  /* Host: n_tok * n_used expert ids, token-major */
+    const float* weights; /* Host: normalized weights, same order */
+    uint64_t n_used, n_tok;
+} it_route;
+
+/* struct TierCounters, src/ops/mod.rs:364-401 */
+typedef struct {
+    uint64_t fetched, fetch_bytes, read_us, upload_us, writes_us, picks_wait_us, picks_copy_us;
+    uint64_t prefetch_reads, prefetch_used, lookups, host_reads, slot_bytes;
+    uint64_t vram_free, vram_total, mirrors, mirror_bytes;
+    uint32_t oversubscribed, _pad;
+    uint64_t slots, resident_bytes, weight_bytes, kv_bytes, quant_bytes, pool_bytes;
+} it_tier_counters;
+
+/* struct ExpertStats, src/ops/cuda/experts.rs:210-315 (the all-resident subset) */
+typedef struct {
+    uint64_t slots, slot_bytes, resident, pool, host_slots, evictions, fetched, lookups, hits;
+    uint32_t oversubscribed, _pad;
+} it_expert_stats;
+
+typedef struct it_hip it_hip;
+
+/* flags for it_hip_create */
+enum {
+    IT_HIP_EXACT = 1,    /* every reduction in the CPU path's order (bit-identical results) */
+    IT_HIP_NO_GRAPH = 2, /* never capture decode passes into a HIP graph */
+};
+
+/* Cuda::new, src/ops/cuda/mod.rs:757-935.  NULL on failure with a message in err. */
+it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len);
+void it_hip_destroy(it_hip* be);
+/* Cuda::take_error: 1 and the message when an error is pending (and clears it), else 0 */
+int it_hip_take_error(it_hip* be, char* msg, size_t msg_len);
+/* check_expert_types, src/ops/mod.rs:29-55, for this backend: 0 = supported */
+int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* msg, size_t msg_len);
+
+/* ---- required trait methods ---- */
+void it_hip_rms_norm(it_hip*, const float* x, uint64_t x_len, const float* weight, uint64_t w_len, float eps,
+                     float* out, uint64_t out_len); /* mod.rs:497 */
+void it_hip_rms_norm_heads(it_hip*, float* x, uint64_t x_len, const float* weight, uint64_t w_len,
+                           uint64_t head_dim, float eps); /* mod.rs:502 */
+void it_hip_matmul(it_hip*, const it_weights* w, const float* x, uint64_t x_len, float* out,
+                   uint64_t out_len); /* mod.rs:520 */
+void it_hip_rope_neox(it_hip*, float* x, uint64_t x_len, uint64_t pos, uint64_t head_dim, uint64_t n_rot,
+                      uint64_t n_heads, float theta_base); /* mod.rs:545 */
+void it_hip_softmax(it_hip*, float* x, uint64_t x_len, uint64_t row);   /* mod.rs:567 */
+void it_hip_attend(it_hip*, const it_attn* a, float* out, uint64_t out_len); /* mod.rs:589 */
+void it_hip_silu_mul(it_hip*, float* gate, uint64_t gate_len, const float* up, uint64_t up_len); /* :592 */
+void it_hip_l2_norm_heads(it_hip*, float* x, uint64_t x_len, uint64_t head_dim, float eps); /* :613 */
+void it_hip_ssm_conv(it_hip*, float* state, uint64_t state_len, const float* x, uint64_t x_len,
+                     const float* weight, uint64_t w_len, uint64_t kernel, float* out,
+                     uint64_t out_len); /* mod.rs:647 */
+void it_hip_gather_chunks(it_hip*, const float* src, uint64_t src_len, uint64_t chunk, uint64_t stride,
+                          uint64_t offset, float* out, uint64_t out_len); /* mod.rs:664 */
+void it_hip_sigmoid_mul(it_hip*, float* x, uint64_t x_len, const float* g, uint64_t g_len); /* :746 */
+void it_hip_delta_rule(it_hip*, const it_delta* d, float* state, uint64_t state_len, float* out,
+                       uint64_t out_len); /* mod.rs:785 */
+void it_hip_add_assign(it_hip*, float* a, uint64_t a_len, const float* b, uint64_t b_len); /* :788 */
+
+/* ---- methods whose defaults touch host memory, overridden for the device ---- */
+void it_hip_scale(it_hip*, float* buf, uint64_t len, float s); /* mod.rs:600 */
+void it_hip_scatter_chunks(it_hip*, const float* src, uint64_t src_len, uint64_t chunk, uint64_t stride,
+                           uint64_t offset, float* dst, uint64_t dst_len); /* mod.rs:730 */
+void it_hip_matmul_pair(it_hip*, const it_weights* a, const it_weights* b, const float* x, uint64_t x_len,
+                        float* out_a, uint64_t out_a_len, float* out_b, uint64_t out_b_len); /* :1012 */
+void it_hip_matmul_experts(it_hip*, const it_experts* w, const it_route* route, const float* x,
+                           uint64_t x_len, float* out, uint64_t out_len); /* mod.rs:1049 */
+void it_hip_moe_glu(it_hip*, const it_experts* gate, const it_experts* up, const it_route* route,
+                    const float* x, uint64_t x_len, float* out, uint64_t out_len, float* scratch,
+                    uint64_t scratch_len); /* mod.rs:1105 */
+void it_hip_moe_finish(it_hip*, float* out, uint64_t out_len, uint64_t at, uint64_t n, const float* rows,
+                       uint64_t rows_len, const it_route* route, const float* shared, uint64_t shared_len,
+                       const float* logit, uint64_t logit_len, uint64_t logit_at); /* mod.rs:1134 */
+/* Ops::route (mod.rs:1191): the choice stays on the device; *out is a Device route */
+void it_hip_route(it_hip*, float* probs, uint64_t probs_len, uint64_t n_expert, uint64_t n_used,
+                  it_route* out);
+void it_hip_add_scaled_rows(it_hip*, float* acc, uint64_t acc_len, const float* rows, uint64_t rows_len,
+                            const float* scales, uint64_t scales_len); /* mod.rs:1228 */
+void it_hip_add_scaled_sigmoid(it_hip*, float* acc, uint64_t acc_len, const float* b, uint64_t b_len,
+                               const float* logit, uint64_t logit_len); /* mod.rs:1250 */
+void it_hip_add_scaled(it_hip*, float* a, uint64_t a_len, const float* b, uint64_t b_len,
+                       float scale); /* mod.rs:1265 */
+void it_hip_kv_write(it_hip*, uint16_t* slab, uint64_t slab_len, uint64_t offset, const float* src,
+                     uint64_t src_len); /* mod.rs:1421 */
+
+/* ---- residency protocol (mod.rs:1360-1419) ---- */
+void it_hip_host_wrote(it_hip*, const float* buf, uint64_t len);
+void it_hip_host_needs(it_hip*, float* buf, uint64_t len);
+void it_hip_begin_pass(it_hip*, uint64_t n_tokens);
+void it_hip_end_pass(it_hip*);
+void it_hip_forget_state(it_hip*);
+void it_hip_read_state(it_hip*, float* host, uint64_t len);
+/* the KV analogue of read_state, for checkpoints: bring a slab's device copy home */
+void it_hip_read_kv(it_hip*, uint16_t* slab, uint64_t len);
+
+/* ---- reporting hooks (mod.rs:1300-1358) ---- */
+void it_hip_device_report(it_hip*);
+void it_hip_reserve_activations(it_hip*, uint64_t bytes);
+int it_hip_tier_counters(it_hip*, it_tier_counters* out);
+/* "label=value\n" lines into buf; returns bytes written */
+size_t it_hip_config_report(it_hip*, char* buf, size_t buf_len);
+/* one-time cost charged to the first passes (weight upload + repack), microseconds */
+uint64_t it_hip_setup_cost(it_hip*, char* label, size_t label_len);
+void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x, uint64_t x_len, uint64_t k);
+
+/* ---- expert cache API, all-resident tier (src/ops/cuda/ops/placement.rs:15-363) ---- */
+void it_hip_set_expert_budget(it_hip*, uint64_t bytes);
+void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes);
+void it_hip_set_expert_slots(it_hip*, uint64_t n);
+void it_hip_set_expert_pool(it_hip*, uint64_t n);
+void it_hip_expert_stats(it_hip*, it_expert_stats* out);
+/* GCLOCK victim choice (src/ops/cuda/experts.rs:2215-2233) as a pure function over a
+ * ring of heat counters and lease flags; returns the victim index or -1 when every
+ * slot is leased.  Never selects a victim in the all-resident tier; kept for tests. */
+int64_t it_hip_clock_pick(uint8_t* heat, const uint8_t* leased, uint64_t n, uint64_t* hand);
+
+/* ---- extensions (no counterpart in the reference's trait) ---- */
+/* first strict maximum of a device-current activation, computed on the device
+ * (the rule of Profile::record_token, src/profile.rs:192-213) */
+uint32_t it_hip_argmax(it_hip*, const float* buf, uint64_t len);
+void it_hip_sync(it_hip*);
+/* forget every mirror and resident weight (tests reuse host addresses) */
+void it_hip_drop_mirrors(it_hip*);
+uint64_t it_hip_launch_count(it_hip*);
+
+/* ---- model + engine: the host side of the loop over this backend ----------
+ * Qwen35::load / forward (src/model/qwen35.rs:755-858, 956-1127) and
+ * Engine::{new, prefill, decode, generate, reset} (src/engine/mod.rs:147-437). */
+typedef struct it_model it_model;
+typedef struct it_engine it_engine;
+typedef void (*it_trace_fn)(void* user, const char* name, uint32_t layer, const float* data, uint64_t n);
+
+it_model* it_model_open(const char* gguf_path, char* err, size_t err_len);
+void it_model_close(it_model*);
+/* n_layer n_embd n_vocab n_head n_head_kv head_dim n_expert n_expert_used expert_ff n_rot */
+void it_model_dims(const it_model*, uint64_t out[10]);
+/* weight bytes one decode token reads (src/model/qwen35.rs:875-939) */
+uint64_t it_model_decode_weight_bytes(const it_model*);
+it_engine* it_engine_new(it_model*, it_hip*, uint64_t n_ctx, uint64_t max_batch);
+void it_engine_free(it_engine*);
+void it_engine_reset(it_engine*);
+void it_engine_set_trace(it_engine*, it_trace_fn fn, void* user);
+uint64_t it_engine_pos(const it_engine*);
+/* one forward pass at the current position; logits (n_vocab) may be NULL. 0 = ok */
+int it_engine_forward(it_engine*, const uint32_t* tokens, uint64_t n, float* logits);
+/* chunked prefill; logits of the last token (may be NULL) */
+int it_engine_prefill(it_engine*, const uint32_t* tokens, uint64_t n, float* logits);
+/* greedy generation; returns tokens produced or a negative error */
+int64_t it_engine_generate(it_engine*, const uint32_t* prompt, uint64_t n_prompt, uint64_t max_new,
+                           uint32_t* out_ids, float* last_logits);
+/* greedy decode of `n` more tokens from the last logits, argmax on the device; for
+ * throughput runs.  Returns tokens produced. */
+int64_t it_engine_decode_greedy(it_engine*, uint64_t n, uint32_t* out_ids);
+const char* it_engine_last_error(it_engine*);
+/* bring device-owned state home and return host pointers (parity tests, checkpoints) */
+const float* it_engine_ssm_state(it_engine*, uint64_t layer, uint64_t* len);
+const float* it_engine_conv_state(it_engine*, uint64_t layer, uint64_t* len);
+const uint16_t* it_engine_k_slab(it_engine*, uint64_t slot, uint64_t* len);
+const uint16_t* it_engine_v_slab(it_engine*, uint64_t slot, uint64_t* len);
+
+/* ---- synthetic GGUF writer (the reference ships none; its model tests need real
+ * files, tests/common/mod.rs:10-44) ---- */
+typedef struct {
+    uint64_t n_layer, n_embd, n_vocab;
+    uint64_t n_head, n_head_kv, head_dim, n_rot;
+    uint64_t n_expert, n_expert_used, expert_ff, shared_ff;
+    uint64_t ssm_d_conv, ssm_d_state, ssm_n_group, ssm_dt_rank; /* d_inner = d_state * dt_rank */
+    uint64_t full_attention_interval;
+    float rope_theta, rms_eps;
+    uint32_t dense_type;  /* IT_Q8_0 */
+    uint32_t expert_type; /* IT_Q8_0 or IT_NVFP4 */
+    uint32_t router_type; /* IT_Q8_0 or IT_F32 */
+    uint32_t _pad;
+    uint64_t seed;
+    float weight_std; /* N(0, std) for Q8_0 matrices */
+    uint32_t n_threads;
+} it_synth_config;
+/* 0 = ok */
+int it_synth_write_gguf(const char* path, const it_synth_config* cfg, char* err, size_t err_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

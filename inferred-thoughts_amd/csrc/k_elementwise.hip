@@ -1,0 +1,427 @@
+// Norms, RoPE, softmax, elementwise ops, KV write, conv, activation quantization.
+//
+// Each kernel keeps the accumulation order of the reference's scalar CPU path
+// (/root/reference src/ops/naive.rs) wherever the `exact` flag is set; the fast
+// variants reorder only the long f64 sums (tree instead of serial).
+#include "it_device.h"
+#include "kernels.h"
+
+namespace itk {
+
+static inline int blocks_for(int64_t n, int threads) {
+    int64_t b = (n + threads - 1) / threads;
+    if (b > 65535LL * 16) b = 65535LL * 16;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+// ------------------------------------------------------------------ sum of squares
+// Serial f64 accumulation of f32 squares (naive.rs:633-640) by one lane, or a tree.
+// `buf` holds the row in LDS.  Returns the sum to every thread of the block.
+template <int THREADS>
+__device__ double block_sumsq(const float* buf, int n, int exact, double* red) {
+    if (exact) {
+        if (threadIdx.x == 0) {
+            double sum = 0.0;
+            for (int i = 0; i < n; i++) sum += (double)(buf[i] * buf[i]);
+            red[0] = sum;
+        }
+        __syncthreads();
+        return red[0];
+    }
+    double part = 0.0;
+    for (int i = threadIdx.x; i < n; i += THREADS) part += (double)(buf[i] * buf[i]);
+    for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double sum = 0.0;
+        for (int w = 0; w < THREADS / 64; w++) sum += red[w];
+        red[0] = sum;
+    }
+    __syncthreads();
+    return red[0];
+}
+
+// naive.rs:139-152: out = x * scale * w, two f32 multiplies left to right.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void rms_norm_k(const float* __restrict__ x, const float* __restrict__ w,
+                                                      float eps, float* __restrict__ out, int nd, int exact) {
+    extern __shared__ float lds[];
+    __shared__ double red[THREADS / 64 + 1];
+    const float* row = x + (int64_t)blockIdx.x * nd;
+    float* o = out + (int64_t)blockIdx.x * nd;
+    for (int i = threadIdx.x; i < nd; i += THREADS) lds[i] = row[i];
+    __syncthreads();
+    double sum = block_sumsq<THREADS>(lds, nd, exact, red);
+    float mean = (float)(sum / (double)nd);
+    float scale = 1.0f / sqrtf(mean + eps);
+    for (int i = threadIdx.x; i < nd; i += THREADS) o[i] = lds[i] * scale * w[i];
+}
+
+void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
+              hipStream_t s) {
+    if (n_rows <= 0) return;
+    hipLaunchKernelGGL(rms_norm_k<256>, dim3((unsigned)n_rows), dim3(256), nd * sizeof(float), s, x, w, eps, out,
+                       nd, exact);
+}
+
+// naive.rs:154-164 (mode 0) and naive.rs:254-273 (mode 1: l2, eps clamps the norm).
+__global__ __launch_bounds__(64) void head_norm_k(float* __restrict__ x, const float* __restrict__ w, int hd,
+                                                  float eps, int mode, int exact) {
+    extern __shared__ float lds[];
+    __shared__ double red[2];
+    float* head = x + (int64_t)blockIdx.x * hd;
+    for (int i = threadIdx.x; i < hd; i += 64) lds[i] = head[i];
+    __syncthreads();
+    double sum = block_sumsq<64>(lds, hd, exact, red);
+    float scale;
+    if (mode == 0) {
+        float mean = (float)(sum / (double)hd);
+        scale = 1.0f / sqrtf(mean + eps);
+        for (int i = threadIdx.x; i < hd; i += 64) head[i] = lds[i] * scale * w[i];
+    } else {
+        float nrm = sqrtf((float)sum);
+        scale = 1.0f / fmaxf(nrm, eps);
+        for (int i = threadIdx.x; i < hd; i += 64) head[i] = lds[i] * scale;
+    }
+}
+
+void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int exact,
+                    hipStream_t s) {
+    if (n_heads <= 0) return;
+    hipLaunchKernelGGL(head_norm_k, dim3((unsigned)n_heads), dim3(64), head_dim * sizeof(float), s, x, w,
+                       head_dim, eps, 0, exact);
+}
+void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s) {
+    if (n_heads <= 0) return;
+    hipLaunchKernelGGL(head_norm_k, dim3((unsigned)n_heads), dim3(64), head_dim * sizeof(float), s, x,
+                       (const float*)nullptr, head_dim, eps, 1, exact);
+}
+
+// naive.rs:180-218.  The (cos, sin) table is built on the host in f64 and narrowed,
+// exactly as the reference builds it; entry [pos][i] = (cos, sin)(pos * theta^(-2i/n_rot)).
+__global__ void rope_k(float* __restrict__ x, const float2* __restrict__ table, int half, int64_t total,
+                       int pos, const int* __restrict__ pos_dyn, int head_dim, int n_heads) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int p0 = pos_dyn ? *pos_dyn : pos;
+    int i = (int)(idx % half);
+    int64_t th = idx / half;  // token * n_heads + head
+    int64_t t = th / n_heads;
+    float2 cs = table[(int64_t)(p0 + t) * half + i];
+    float* head = x + th * head_dim;
+    float x0 = head[i], x1 = head[i + half];
+    head[i] = x0 * cs.x - x1 * cs.y;
+    head[i + half] = x0 * cs.y + x1 * cs.x;
+}
+
+void rope_neox(float* x, const float2* table, int table_half, int64_t n_tok, int pos, const int* pos_dyn,
+               int head_dim, int n_rot, int n_heads, hipStream_t s) {
+    int half = n_rot / 2;
+    int64_t total = n_tok * n_heads * half;
+    if (total <= 0) return;
+    (void)table_half;
+    hipLaunchKernelGGL(rope_k, dim3(blocks_for(total, 256)), dim3(256), 0, s, x, table, half, total, pos,
+                       pos_dyn, head_dim, n_heads);
+}
+
+// naive.rs:362-376: max, exp(v - max) with a serial sum, divide.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void softmax_k(float* __restrict__ x, int row, int exact) {
+    extern __shared__ float lds[];
+    __shared__ float red[THREADS / 64 + 1];
+    float* r = x + (int64_t)blockIdx.x * row;
+    float m = -INFINITY;
+    for (int i = threadIdx.x; i < row; i += THREADS) {
+        float v = r[i];
+        lds[i] = v;
+        m = fmaxf(m, v);
+    }
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_down(m, off, 64));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float mm = red[0];
+        for (int w = 1; w < THREADS / 64; w++) mm = fmaxf(mm, red[w]);
+        red[THREADS / 64] = mm;
+    }
+    __syncthreads();
+    m = red[THREADS / 64];
+    float part = 0.0f;
+    for (int i = threadIdx.x; i < row; i += THREADS) {
+        float e = it_expf(lds[i] - m);
+        lds[i] = e;
+        part += e;
+    }
+    __syncthreads();
+    float sum;
+    if (exact) {
+        if (threadIdx.x == 0) {
+            float acc = 0.0f;
+            for (int i = 0; i < row; i++) acc += lds[i];
+            red[0] = acc;
+        }
+        __syncthreads();
+        sum = red[0];
+    } else {
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_down(part, off, 64);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = part;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float acc = 0.0f;
+            for (int w = 0; w < THREADS / 64; w++) acc += red[w];
+            red[0] = acc;
+        }
+        __syncthreads();
+        sum = red[0];
+    }
+    for (int i = threadIdx.x; i < row; i += THREADS) r[i] = lds[i] / sum;
+}
+
+void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s) {
+    if (n_rows <= 0 || row <= 0) return;
+    hipLaunchKernelGGL(softmax_k<256>, dim3((unsigned)n_rows), dim3(256), row * sizeof(float), s, x, row, exact);
+}
+
+// ------------------------------------------------------------------ elementwise
+__global__ void silu_mul_k(float* __restrict__ g, const float* __restrict__ u, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        float v = g[i];
+        g[i] = it_silu(v) * u[i];
+    }
+}
+__global__ void sigmoid_mul_k(float* __restrict__ x, const float* __restrict__ g, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        x[i] *= it_sigmoid(g[i]);
+}
+__global__ void add_assign_k(float* __restrict__ a, const float* __restrict__ b, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        a[i] += b[i];
+}
+__global__ void scale_k(float* __restrict__ a, float v, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        a[i] *= v;
+}
+__global__ void add_scaled_k(float* __restrict__ a, const float* __restrict__ b, float v, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        a[i] += b[i] * v;
+}
+__global__ void add_scaled_sigmoid_k(float* __restrict__ a, const float* __restrict__ b,
+                                     const float* __restrict__ logit, int64_t n) {
+    float sg = it_sigmoid(logit[0]);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        a[i] += b[i] * sg;
+}
+__global__ void add_scaled_rows_k(float* __restrict__ acc, int64_t n, const float* __restrict__ rows,
+                                  const float* __restrict__ scales, int n_scales) {
+    for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+        float v = 0.0f;
+        for (int e = 0; e < n_scales; e++) v += scales[e] * rows[(int64_t)e * n + j];
+        acc[j] = v;
+    }
+}
+__global__ void gather_chunks_k(const float* __restrict__ src, int64_t chunk, int64_t stride, int64_t offset,
+                                float* __restrict__ out, int64_t out_len) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < out_len;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        int64_t c = i / chunk, j = i % chunk;
+        out[i] = src[c * stride + offset + j];
+    }
+}
+__global__ void scatter_chunks_k(const float* __restrict__ src, int64_t src_len, int64_t chunk, int64_t stride,
+                                 int64_t offset, float* __restrict__ dst) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < src_len;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        int64_t c = i / chunk, j = i % chunk;
+        dst[offset + c * stride + j] = src[i];
+    }
+}
+// ops/mod.rs:1421-1425: f32 -> f16 round to nearest even.
+__global__ void kv_write_k(uint16_t* __restrict__ slab, int64_t offset, const int* __restrict__ offset_dyn,
+                           int64_t offset_mul, const float* __restrict__ src, int64_t n) {
+    int64_t off = offset_dyn ? (int64_t)(*offset_dyn) * offset_mul : offset;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        slab[off + i] = it_f32_to_f16(src[i]);
+}
+__global__ void fill_zero_k(uint32_t* p, int64_t n_words) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words;
+         i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = 0u;
+}
+
+#define EW_LAUNCH(kern, n, ...)                                                              \
+    do {                                                                                     \
+        if ((n) > 0) hipLaunchKernelGGL(kern, dim3(blocks_for((n), 256)), dim3(256), 0, s, __VA_ARGS__); \
+    } while (0)
+
+void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s) { EW_LAUNCH(silu_mul_k, n, gate, up, n); }
+void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s) { EW_LAUNCH(sigmoid_mul_k, n, x, g, n); }
+void add_assign(float* a, const float* b, int64_t n, hipStream_t s) { EW_LAUNCH(add_assign_k, n, a, b, n); }
+void scale(float* a, float v, int64_t n, hipStream_t s) { EW_LAUNCH(scale_k, n, a, v, n); }
+void add_scaled(float* a, const float* b, float v, int64_t n, hipStream_t s) {
+    EW_LAUNCH(add_scaled_k, n, a, b, v, n);
+}
+void add_scaled_rows(float* acc, int64_t n, const float* rows, const float* scales, int n_scales,
+                     hipStream_t s) {
+    EW_LAUNCH(add_scaled_rows_k, n, acc, n, rows, scales, n_scales);
+}
+void add_scaled_sigmoid(float* acc, const float* b, int64_t n, const float* logit, hipStream_t s) {
+    EW_LAUNCH(add_scaled_sigmoid_k, n, acc, b, logit, n);
+}
+void gather_chunks(const float* src, int64_t chunk, int64_t stride, int64_t offset, float* out,
+                   int64_t out_len, hipStream_t s) {
+    EW_LAUNCH(gather_chunks_k, out_len, src, chunk, stride, offset, out, out_len);
+}
+void scatter_chunks(const float* src, int64_t src_len, int64_t chunk, int64_t stride, int64_t offset,
+                    float* dst, hipStream_t s) {
+    EW_LAUNCH(scatter_chunks_k, src_len, src, src_len, chunk, stride, offset, dst);
+}
+void kv_write(uint16_t* slab, int64_t offset, const int* offset_dyn, int64_t offset_mul, const float* src,
+              int64_t n, hipStream_t s) {
+    EW_LAUNCH(kv_write_k, n, slab, offset, offset_dyn, offset_mul, src, n);
+}
+void fill_zero(void* p, int64_t bytes, hipStream_t s) {
+    int64_t words = bytes / 4;
+    EW_LAUNCH(fill_zero_k, words, (uint32_t*)p, words);
+}
+
+// ------------------------------------------------------------------ Q8_0 activations
+// naive.rs:652-675: per 32: amax, d = amax/127, id = d ? 1/d : 0, q = round-half-away(x*id)
+// saturated to i8, scale stored through f16.  Eight lanes share a block.
+__global__ void quantize_q8_0_k(const float* __restrict__ x, float* __restrict__ scales,
+                                int8_t* __restrict__ quants, int64_t n_blocks) {
+    int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = gid >> 3;
+    int sub = (int)(gid & 7);
+    bool live = b < n_blocks;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) v = *(const float4*)(x + b * 32 + sub * 4);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    if (!live) return;
+    float d = amax / 127.0f;
+    float id = d != 0.0f ? 1.0f / d : 0.0f;
+    float r[4] = {roundf(v.x * id), roundf(v.y * id), roundf(v.z * id), roundf(v.w * id)};
+    uint32_t packed = 0;
+    for (int i = 0; i < 4; i++) {
+        float c = fminf(fmaxf(r[i], -128.0f), 127.0f);
+        int q = (r[i] != r[i]) ? 0 : (int)c;
+        packed |= ((uint32_t)(q & 0xff)) << (8 * i);
+    }
+    *(uint32_t*)(quants + b * 32 + sub * 4) = packed;
+    if (sub == 0) scales[b] = it_f16_to_f32(it_f32_to_f16(d));
+}
+
+void quantize_q8_0(const float* x, float* scales, int8_t* quants, int64_t n, hipStream_t s) {
+    int64_t n_blocks = n / 32;
+    if (n_blocks <= 0) return;
+    int64_t threads = n_blocks * 8;
+    hipLaunchKernelGGL(quantize_q8_0_k, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, x, scales,
+                       quants, n_blocks);
+}
+
+// ------------------------------------------------------------------ causal conv + silu
+// naive.rs:275-315.  One thread per channel walks the batch in order with the
+// window in registers; state is [channel][kernel-1], oldest first.
+template <int KEEP>
+__global__ void ssm_conv_k(float* __restrict__ state, const float* __restrict__ x, const float* __restrict__ w,
+                           int nc, int n_tok, float* __restrict__ out) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= nc) return;
+    float past[KEEP], wt[KEEP + 1];
+    for (int k = 0; k < KEEP; k++) past[k] = state[(int64_t)c * KEEP + k];
+    for (int k = 0; k <= KEEP; k++) wt[k] = w[(int64_t)c * (KEEP + 1) + k];
+    for (int t = 0; t < n_tok; t++) {
+        float xv = x[(int64_t)t * nc + c];
+        float sum = 0.0f;
+        for (int k = 0; k < KEEP; k++) sum += past[k] * wt[k];
+        sum += xv * wt[KEEP];
+        out[(int64_t)t * nc + c] = it_silu(sum);
+        for (int k = 0; k + 1 < KEEP; k++) past[k] = past[k + 1];
+        past[KEEP - 1] = xv;
+    }
+    for (int k = 0; k < KEEP; k++) state[(int64_t)c * KEEP + k] = past[k];
+}
+
+void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
+              hipStream_t s) {
+    if (nc <= 0 || n_tok <= 0) return;
+    dim3 grid((nc + 127) / 128), block(128);
+    switch (kernel) {
+        case 2: hipLaunchKernelGGL(ssm_conv_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+        case 3: hipLaunchKernelGGL(ssm_conv_k<2>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+        case 4: hipLaunchKernelGGL(ssm_conv_k<3>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+        case 5: hipLaunchKernelGGL(ssm_conv_k<4>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+        default: break;  // the caller validates `kernel`
+    }
+}
+
+// ------------------------------------------------------------------ argmax
+// First strict maximum (ties to the lower index), /root/reference src/profile.rs:192-213.
+__global__ __launch_bounds__(256) void argmax_part_k(const float* __restrict__ x, int64_t n,
+                                                     int32_t* __restrict__ pidx, float* __restrict__ pval) {
+    __shared__ float sv[256];
+    __shared__ int si[256];
+    int64_t per = (n + gridDim.x - 1) / gridDim.x;
+    int64_t lo = per * blockIdx.x, hi = lo + per < n ? lo + per : n;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+        float v = x[i];
+        if (v > bv || bi == 0x7fffffff) {
+            // strided scan visits ascending indices per thread, so strict > keeps the lowest
+            if (bi == 0x7fffffff || v > bv) {
+                bv = v;
+                bi = (int)i;
+            }
+        }
+    }
+    sv[threadIdx.x] = bv;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            float ov = sv[threadIdx.x + off];
+            int oi = si[threadIdx.x + off];
+            float mv = sv[threadIdx.x];
+            int mi = si[threadIdx.x];
+            bool take = (oi != 0x7fffffff) && (mi == 0x7fffffff || ov > mv || (ov == mv && oi < mi));
+            if (take) {
+                sv[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        pidx[blockIdx.x] = si[0];
+        pval[blockIdx.x] = sv[0];
+    }
+}
+__global__ void argmax_final_k(const int32_t* __restrict__ pidx, const float* __restrict__ pval, int n_part,
+                               int32_t* __restrict__ out) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float bv = 0.f;
+    int bi = 0x7fffffff;
+    for (int p = 0; p < n_part; p++) {
+        int oi = pidx[p];
+        float ov = pval[p];
+        if (oi == 0x7fffffff) continue;
+        if (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    out[0] = bi == 0x7fffffff ? 0 : bi;
+}
+
+void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s) {
+    int parts = 64;
+    hipLaunchKernelGGL(argmax_part_k, dim3(parts), dim3(256), 0, s, x, n, scratch_idx, scratch_val);
+    hipLaunchKernelGGL(argmax_final_k, dim3(1), dim3(64), 0, s, scratch_idx, scratch_val, parts, out);
+}
+
+}  // namespace itk

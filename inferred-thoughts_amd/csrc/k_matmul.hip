@@ -1,0 +1,318 @@
+// Quantized matmuls: weight repack, the decode GEMV (dense, per-expert, fused
+// gate/up), and the tiled batch kernel.
+//
+// Arithmetic is the reference CPU path's (/root/reference src/ops/naive.rs):
+//   Q8_0  (naive.rs:691-704): per 32-block  sumf += (float)isum * (dw * dx)
+//   NVFP4 (naive.rs:714-734): per 16-sub-block sumf += (dy * d) * (float)(lo + hi)
+// with the f32 chain walked serially in ascending block order.  Every per-block
+// term is computed by its own lane (integer dot via v_dot4_i32_i8, exact), written
+// to LDS, and one lane per output row folds the terms in order — so the result is
+// the CPU result bit for bit while the HBM stream stays 128-bit coalesced.
+#include "it_device.h"
+#include "kernels.h"
+
+namespace itk {
+
+// ------------------------------------------------------------------ repack
+// file Q8_0 block = [f16 d][32 x i8]  ->  quants[row][n_in] + scales[row][n_in/32]
+__global__ void repack_q8_0_k(const uint8_t* __restrict__ raw, int8_t* __restrict__ q,
+                              uint16_t* __restrict__ scales, int64_t n_blocks) {
+    // 8 lanes per block, 4 bytes each
+    int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = gid >> 3;
+    int sub = (int)(gid & 7);
+    if (b >= n_blocks) return;
+    const uint8_t* blk = raw + b * 34;
+    // 34-byte blocks are only 2-byte aligned: assemble from u16 loads
+    const uint16_t* p = (const uint16_t*)(blk + 2 + sub * 4);
+    uint32_t v = (uint32_t)p[0] | ((uint32_t)p[1] << 16);
+    *(uint32_t*)(q + b * 32 + sub * 4) = v;
+    if (sub == 0) scales[b] = *(const uint16_t*)blk;
+}
+void repack_q8_0(const uint8_t* raw, int8_t* q, uint16_t* scales, int64_t n_rows, int n_in, hipStream_t s) {
+    int64_t n_blocks = n_rows * (n_in / 32);
+    if (n_blocks <= 0) return;
+    int64_t threads = n_blocks * 8;
+    hipLaunchKernelGGL(repack_q8_0_k, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw, q, scales,
+                       n_blocks);
+}
+
+// file NVFP4 block = [4 x ue4m3][32 nibble bytes] -> nibbles[row][n_in/2] + scales[row][n_in/16]
+__global__ void repack_nvfp4_k(const uint8_t* __restrict__ raw, uint8_t* __restrict__ nib,
+                               uint8_t* __restrict__ scales, int64_t n_blocks) {
+    // 9 dwords per block; 8 lanes move nibbles, lane 0 also moves the scales
+    int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t b = gid >> 3;
+    int sub = (int)(gid & 7);
+    if (b >= n_blocks) return;
+    const uint32_t* blk = (const uint32_t*)(raw + b * 36);
+    ((uint32_t*)nib)[b * 8 + sub] = blk[1 + sub];
+    if (sub == 0) ((uint32_t*)scales)[b] = blk[0];
+}
+void repack_nvfp4(const uint8_t* raw, uint8_t* nib, uint8_t* scales, int64_t n_rows, int n_in, hipStream_t s) {
+    int64_t n_blocks = n_rows * (n_in / 64);
+    if (n_blocks <= 0) return;
+    int64_t threads = n_blocks * 8;
+    hipLaunchKernelGGL(repack_nvfp4_k, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw, nib,
+                       scales, n_blocks);
+}
+
+// ------------------------------------------------------------------ E2M1 nibbles -> int8
+// kvalues (doubled E2M1, /root/reference src/quant/mod.rs:265) through two byte
+// permutes: magnitude by the low 3 bits, then the sign bit picks +mag or -mag.
+IT_DEV uint32_t fp4x4_to_i8x4(uint32_t v) {  // v: four nibbles, one per byte
+    const uint32_t TPlo = 0x03020100u, TPhi = 0x0c080604u;
+    const uint32_t TNlo = 0xfdfeff00u, TNhi = 0xf4f8fafcu;
+    uint32_t idx = v & 0x07070707u;
+    uint32_t mag = __builtin_amdgcn_perm(TPhi, TPlo, idx);
+    uint32_t neg = __builtin_amdgcn_perm(TNhi, TNlo, idx);
+    uint32_t sel = ((v >> 1) & 0x04040404u) | 0x03020100u;
+    return __builtin_amdgcn_perm(neg, mag, sel);
+}
+
+IT_DEV int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+
+// One 32-element unit of a Q8_0 row against activation block `a` (8 dwords).
+IT_DEV float unit_q8_0(const uint4 w0, const uint4 w1, uint16_t dw_bits, const uint4 a0, const uint4 a1,
+                       float dx) {
+    int s = 0;
+    s = dot4(w0.x, a0.x, s); s = dot4(w0.y, a0.y, s); s = dot4(w0.z, a0.z, s); s = dot4(w0.w, a0.w, s);
+    s = dot4(w1.x, a1.x, s); s = dot4(w1.y, a1.y, s); s = dot4(w1.z, a1.z, s); s = dot4(w1.w, a1.w, s);
+    float dw = it_f16_to_f32(dw_bits);
+    return (float)s * (dw * dx);
+}
+
+// One 32-element unit (two 16-element sub-blocks) of an NVFP4 row.
+IT_DEV void unit_nvfp4(const uint4 w, uint32_t sc2, const uint4 a0, const uint4 a1, float dy, float* tA,
+                       float* tB) {
+    int sa = 0, sb = 0;
+    sa = dot4(fp4x4_to_i8x4(w.x & 0x0f0f0f0fu), a0.x, sa);
+    sa = dot4(fp4x4_to_i8x4(w.y & 0x0f0f0f0fu), a0.y, sa);
+    sa = dot4(fp4x4_to_i8x4((w.x >> 4) & 0x0f0f0f0fu), a0.z, sa);
+    sa = dot4(fp4x4_to_i8x4((w.y >> 4) & 0x0f0f0f0fu), a0.w, sa);
+    sb = dot4(fp4x4_to_i8x4(w.z & 0x0f0f0f0fu), a1.x, sb);
+    sb = dot4(fp4x4_to_i8x4(w.w & 0x0f0f0f0fu), a1.y, sb);
+    sb = dot4(fp4x4_to_i8x4((w.z >> 4) & 0x0f0f0f0fu), a1.z, sb);
+    sb = dot4(fp4x4_to_i8x4((w.w >> 4) & 0x0f0f0f0fu), a1.w, sb);
+    float dA = it_ue4m3_to_f32(sc2 & 0xffu), dB = it_ue4m3_to_f32((sc2 >> 8) & 0xffu);
+    *tA = (dy * dA) * (float)sa;
+    *tB = (dy * dB) * (float)sb;
+}
+
+// ------------------------------------------------------------------ GEMV
+struct GemvP {
+    const uint8_t *q, *s;     // weights (gate when GLU)
+    const uint8_t *q2, *s2;   // up weights when GLU
+    int64_t q_stride, s_stride;  // bytes per expert (0 for a dense matrix)
+    const int32_t* ids;       // expert id per y, or null
+    const float *scale2, *scale2_up;  // per-expert second scales or null
+    const float* act_scales;  // [x_rows][n_in/32]
+    const int8_t* act_quants; // [x_rows][n_in]
+    float* out;               // [n_y][n_out]
+    int n_in, n_out, rows_per_wave;
+    int x_mode, n_used;       // 0: row per y, 1: row y / n_used, 2: row 0
+    float out_scale;
+};
+
+constexpr int GEMV_WAVES = 4;
+
+template <int FMT, bool GLU>
+__global__ __launch_bounds__(64 * GEMV_WAVES) void gemv_k(GemvP p) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int U = p.n_in >> 5;                     // 32-element units per row
+    const int TPU = (FMT == W_NVFP4) ? 2 : 1;      // terms per unit
+    const int T = U * TPU;                         // terms per row
+    const int R = p.rows_per_wave;
+    const int tstride = T + 1;
+    float* terms = lds + (size_t)wave * R * tstride * (GLU ? 2 : 1);
+    float* terms2 = terms + (size_t)R * tstride;
+
+    const int y = blockIdx.y;
+    const int row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
+    if (row0 >= p.n_out) return;
+    const int nrows = min(R, p.n_out - row0);
+
+    int64_t e = p.ids ? (int64_t)p.ids[y] : 0;
+    const uint8_t* wq = p.q + e * p.q_stride;
+    const uint8_t* ws = p.s + e * p.s_stride;
+    const uint8_t* wq2 = GLU ? p.q2 + e * p.q_stride : nullptr;
+    const uint8_t* ws2 = GLU ? p.s2 + e * p.s_stride : nullptr;
+    int xr = p.x_mode == 0 ? y : (p.x_mode == 1 ? y / p.n_used : 0);
+    const int8_t* aq = p.act_quants + (int64_t)xr * p.n_in;
+    const float* as = p.act_scales + (int64_t)xr * U;
+
+    const int items = nrows * U;
+    for (int base = 0; base < items; base += 64) {
+        int it = base + lane;
+        if (it < items) {
+            int r = it / U, u = it - r * U;
+            int64_t row = row0 + r;
+            const uint4* ap = (const uint4*)(aq + u * 32);
+            uint4 a0 = ap[0], a1 = ap[1];
+            float dx = as[u];
+            if (FMT == W_Q8_0) {
+                const uint4* wp = (const uint4*)(wq + row * p.n_in + u * 32);
+                uint16_t dw = ((const uint16_t*)ws)[row * U + u];
+                terms[r * tstride + u] = unit_q8_0(wp[0], wp[1], dw, a0, a1, dx);
+                if (GLU) {
+                    const uint4* wp2 = (const uint4*)(wq2 + row * p.n_in + u * 32);
+                    uint16_t dw2 = ((const uint16_t*)ws2)[row * U + u];
+                    terms2[r * tstride + u] = unit_q8_0(wp2[0], wp2[1], dw2, a0, a1, dx);
+                }
+            } else {
+                uint4 w = *(const uint4*)(wq + row * (p.n_in >> 1) + u * 16);
+                uint32_t sc = ((const uint16_t*)ws)[row * U + u];
+                float tA, tB;
+                unit_nvfp4(w, sc, a0, a1, dx, &tA, &tB);
+                terms[r * tstride + 2 * u] = tA;
+                terms[r * tstride + 2 * u + 1] = tB;
+                if (GLU) {
+                    uint4 w2 = *(const uint4*)(wq2 + row * (p.n_in >> 1) + u * 16);
+                    uint32_t sc2 = ((const uint16_t*)ws2)[row * U + u];
+                    unit_nvfp4(w2, sc2, a0, a1, dx, &tA, &tB);
+                    terms2[r * tstride + 2 * u] = tA;
+                    terms2[r * tstride + 2 * u + 1] = tB;
+                }
+            }
+        }
+    }
+    // the wave's own LDS region: a wave-level barrier is enough
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (lane < nrows) {
+        const float* tr = terms + lane * tstride;
+        float acc = 0.0f;
+        for (int k = 0; k < T; k++) acc += tr[k];
+        float* o = p.out + (int64_t)y * p.n_out + row0 + lane;
+        if (GLU) {
+            const float* tr2 = terms2 + lane * tstride;
+            float acc2 = 0.0f;
+            for (int k = 0; k < T; k++) acc2 += tr2[k];
+            if (p.scale2) acc *= p.scale2[e];
+            if (p.scale2_up) acc2 *= p.scale2_up[e];
+            *o = it_silu(acc) * acc2;
+        } else {
+            if (p.scale2) acc *= p.scale2[e];
+            if (p.out_scale != 1.0f) acc *= p.out_scale;
+            *o = acc;
+        }
+    }
+}
+
+static int pick_rows_per_wave(int n_out, int n_y) {
+    // aim for >= ~2048 waves in flight, cap the fold's idle lanes at 16 rows per wave
+    int64_t want_waves = 2048;
+    int64_t r = ((int64_t)n_out * n_y) / want_waves;
+    int R = 1;
+    while (R < 16 && R * 2 <= r) R *= 2;
+    return R;
+}
+
+template <int FMT, bool GLU>
+static void launch_gemv(GemvP p, int n_y, hipStream_t s) {
+    int R = pick_rows_per_wave(p.n_out, n_y);
+    int T = (p.n_in / 32) * (FMT == W_NVFP4 ? 2 : 1);
+    auto lds_for = [&](int r) { return (size_t)GEMV_WAVES * r * (T + 1) * sizeof(float) * (GLU ? 2 : 1); };
+    while (R > 1 && lds_for(R) > 48 * 1024) R /= 2;
+    p.rows_per_wave = R;
+    size_t lds = lds_for(R);
+    int gx = (p.n_out + R * GEMV_WAVES - 1) / (R * GEMV_WAVES);
+    hipLaunchKernelGGL((gemv_k<FMT, GLU>), dim3(gx, n_y), dim3(64 * GEMV_WAVES), lds, s, p);
+}
+
+// ------------------------------------------------------------------ unquantized weights
+// naive.rs:843-861: serial f32 fold over the row, one thread per output.
+template <int FMT>
+__global__ void dense_float_k(const uint8_t* __restrict__ w, const float* __restrict__ x, float* __restrict__ out,
+                              int n_in, int n_out, int n_tok, float out_scale) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)n_out * n_tok) return;
+    int j = (int)(idx % n_out);
+    int64_t t = idx / n_out;
+    const float* xt = x + t * n_in;
+    float sum = 0.0f;
+    if (FMT == W_F32) {
+        const float* row = (const float*)w + (int64_t)j * n_in;
+        for (int i = 0; i < n_in; i++) sum += row[i] * xt[i];
+    } else {
+        const uint16_t* row = (const uint16_t*)w + (int64_t)j * n_in;
+        for (int i = 0; i < n_in; i++)
+            sum += (FMT == W_F16 ? it_f16_to_f32(row[i]) : it_bf16_to_f32(row[i])) * xt[i];
+    }
+    if (out_scale != 1.0f) sum *= out_scale;
+    out[t * n_out + j] = sum;
+}
+
+void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
+            float* out, float out_scale, hipStream_t s) {
+    if (n_tok <= 0 || w.n_out <= 0) return;
+    if (w.fmt == W_Q8_0 || w.fmt == W_NVFP4) {
+        GemvP p{};
+        p.q = (const uint8_t*)w.q;
+        p.s = (const uint8_t*)w.scales;
+        p.act_scales = act_scales;
+        p.act_quants = act_quants;
+        p.out = out;
+        p.n_in = w.n_in;
+        p.n_out = w.n_out;
+        p.x_mode = 0;
+        p.n_used = 1;
+        p.out_scale = out_scale;
+        if (w.fmt == W_Q8_0) launch_gemv<W_Q8_0, false>(p, n_tok, s);
+        else launch_gemv<W_NVFP4, false>(p, n_tok, s);
+        return;
+    }
+    int64_t total = (int64_t)w.n_out * n_tok;
+    dim3 grid((unsigned)((total + 127) / 128)), block(128);
+    const uint8_t* wp = (const uint8_t*)w.q;
+    if (w.fmt == W_F32)
+        hipLaunchKernelGGL(dense_float_k<W_F32>, grid, block, 0, s, wp, x, out, w.n_in, w.n_out, n_tok, out_scale);
+    else if (w.fmt == W_F16)
+        hipLaunchKernelGGL(dense_float_k<W_F16>, grid, block, 0, s, wp, x, out, w.n_in, w.n_out, n_tok, out_scale);
+    else
+        hipLaunchKernelGGL(dense_float_k<W_BF16>, grid, block, 0, s, wp, x, out, w.n_in, w.n_out, n_tok,
+                           out_scale);
+}
+
+static GemvP experts_params(const ExpertsView& w, const int32_t* ids, int n_used, int x_mode,
+                            const float* act_scales, const int8_t* act_quants, float* out) {
+    GemvP p{};
+    p.q = (const uint8_t*)w.q;
+    p.s = (const uint8_t*)w.scales;
+    p.q_stride = w.q_stride;
+    p.s_stride = w.s_stride;
+    p.ids = ids;
+    p.scale2 = w.scale2;
+    p.act_scales = act_scales;
+    p.act_quants = act_quants;
+    p.out = out;
+    p.n_in = w.n_in;
+    p.n_out = w.n_out;
+    p.x_mode = x_mode;
+    p.n_used = n_used < 1 ? 1 : n_used;
+    p.out_scale = 1.0f;
+    return p;
+}
+
+void matmul_experts(const ExpertsView& w, const int32_t* ids, int n_picks, int n_used, int x_mode,
+                    const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s) {
+    if (n_picks <= 0) return;
+    GemvP p = experts_params(w, ids, n_used, x_mode, act_scales, act_quants, out);
+    if (w.fmt == W_Q8_0) launch_gemv<W_Q8_0, false>(p, n_picks, s);
+    else launch_gemv<W_NVFP4, false>(p, n_picks, s);
+}
+
+void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids, int n_picks, int n_used,
+             int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s) {
+    if (n_picks <= 0) return;
+    GemvP p = experts_params(gate, ids, n_used, x_mode, act_scales, act_quants, out);
+    p.q2 = (const uint8_t*)up.q;
+    p.s2 = (const uint8_t*)up.scales;
+    p.scale2_up = up.scale2;
+    if (gate.fmt == W_Q8_0) launch_gemv<W_Q8_0, true>(p, n_picks, s);
+    else launch_gemv<W_NVFP4, true>(p, n_picks, s);
+}
+
+}  // namespace itk

@@ -1,0 +1,94 @@
+// Device-side router and the routed FFN's tail.
+//
+// route_topk follows /root/reference src/ops/mod.rs:1191-1216: n_used rounds, each an
+// ascending scan that takes a new best only on a strict '>' (ties to the lower id),
+// then the picked probabilities summed in pick order and divided by
+// max(sum, 6.103515625e-5).  moe_finish follows src/ops/mod.rs:1134-1171.
+#include "it_device.h"
+#include "kernels.h"
+
+namespace itk {
+
+__global__ __launch_bounds__(256) void route_topk_k(const float* __restrict__ probs, int n_expert, int n_used,
+                                                    int32_t* __restrict__ ids, float* __restrict__ weights) {
+    extern __shared__ float p[];            // n_expert probabilities
+    __shared__ float rv[256];
+    __shared__ int ri[256];
+    __shared__ int picked[64];
+    const int t = blockIdx.x;
+    const float* row = probs + (int64_t)t * n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += 256) p[e] = row[e];
+    __syncthreads();
+    for (int r = 0; r < n_used; r++) {
+        float bv = 0.0f;
+        int bi = -1;
+        for (int e = threadIdx.x; e < n_expert; e += 256) {
+            bool taken = false;
+            for (int k = 0; k < r; k++) taken |= (picked[k] == e);
+            if (taken) continue;
+            if (bi < 0 || p[e] > bv) {
+                bv = p[e];
+                bi = e;
+            }
+        }
+        rv[threadIdx.x] = bv;
+        ri[threadIdx.x] = bi;
+        __syncthreads();
+        for (int off = 128; off > 0; off >>= 1) {
+            if ((int)threadIdx.x < off) {
+                int oi = ri[threadIdx.x + off], mi = ri[threadIdx.x];
+                float ov = rv[threadIdx.x + off], mv = rv[threadIdx.x];
+                bool take = oi >= 0 && (mi < 0 || ov > mv || (ov == mv && oi < mi));
+                if (take) {
+                    rv[threadIdx.x] = ov;
+                    ri[threadIdx.x] = oi;
+                }
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) picked[r] = ri[0];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        float sum = 0.0f;
+        for (int r = 0; r < n_used; r++) sum += p[picked[r]];
+        float denom = fmaxf(sum, 6.103515625e-5f);
+        for (int r = 0; r < n_used; r++) {
+            ids[(int64_t)t * n_used + r] = picked[r];
+            weights[(int64_t)t * n_used + r] = p[picked[r]] / denom;
+        }
+    }
+}
+
+void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,
+                hipStream_t s) {
+    if (n_tok <= 0) return;
+    hipLaunchKernelGGL(route_topk_k, dim3(n_tok), dim3(256), n_expert * sizeof(float), s, probs, n_expert, n_used,
+                       ids, weights);
+}
+
+__global__ void moe_finish_k(float* __restrict__ out, int64_t at, int n, const float* __restrict__ rows,
+                             const float* __restrict__ weights, int n_tok, int n_used,
+                             const float* __restrict__ shared, const float* __restrict__ logit,
+                             int64_t logit_at) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)n_tok * n) return;
+    int64_t t = idx / n;
+    int j = (int)(idx - t * n);
+    float g = it_sigmoid(logit[logit_at + t]);
+    const float* w = weights + t * n_used;
+    float v = 0.0f;
+    for (int e = 0; e < n_used; e++) v += w[e] * rows[(t * n_used + e) * n + j];
+    v += shared[t * n + j] * g;
+    out[at + t * n + j] = v;
+}
+
+void moe_finish(float* out, int64_t at, int n, const float* rows, const float* weights, int n_tok, int n_used,
+                const float* shared, const float* logit, int64_t logit_at, hipStream_t s) {
+    int64_t total = (int64_t)n_tok * n;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(moe_finish_k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, out, at, n, rows,
+                       weights, n_tok, n_used, shared, logit, logit_at);
+}
+
+}  // namespace itk

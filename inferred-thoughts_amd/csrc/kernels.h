@@ -1,0 +1,108 @@
+// Launch wrappers for every HIP kernel in the library.  Plain pointers and sizes
+// only; every pointer is a device pointer.  `dyn` pointers, when non-null, name a
+// device int that overrides the by-value scalar beside them — that is what lets a
+// captured decode graph stay valid while the position advances.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace itk {
+
+// ---- weight formats on the device (repacked at upload) ----------------------
+// Q8_0:  quants int8 [n_rows][n_in], scales f16 [n_rows][n_in/32]
+// NVFP4: nibbles u8 [n_rows][n_in/2] (byte j of sub-block s = elements j, j+8 of
+//        that sub-block, as in the file), scales u8 [n_rows][n_in/16]
+// F32/F16/BF16: file layout (row-major), read as is.
+enum WFmt : int { W_F32 = 0, W_F16 = 1, W_Q8_0 = 8, W_BF16 = 30, W_NVFP4 = 40 };
+
+struct WView {
+    const void* q;       // quants / nibbles / raw rows
+    const void* scales;  // per-block scales (null for F32/F16/BF16)
+    int fmt;
+    int n_in, n_out;
+};
+
+// repack kernels: file layout -> device layout
+void repack_q8_0(const uint8_t* raw, int8_t* q, uint16_t* scales, int64_t n_rows, int n_in, hipStream_t s);
+void repack_nvfp4(const uint8_t* raw, uint8_t* nib, uint8_t* scales, int64_t n_rows, int n_in, hipStream_t s);
+
+// ---- activation quantization --------------------------------------------------
+void quantize_q8_0(const float* x, float* scales, int8_t* quants, int64_t n, hipStream_t s);
+
+// ---- matmul family -------------------------------------------------------------
+// out[t][j] = dot(w.row(j), x[t]); act is the Q8_0 form of x for quantized formats.
+void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
+            float* out, float out_scale, hipStream_t s);
+
+struct ExpertsView {
+    const void* q;       // expert e at q + e*q_stride
+    const void* scales;  // expert e at scales + e*s_stride
+    int64_t q_stride, s_stride;
+    int fmt, n_in, n_out, n_expert;
+    const float* scale2;  // per-expert second scale or null
+};
+// One matmul per pick.  x rows: mode 0 = one row per pick, 1 = one row per token
+// (pick i reads row i / n_used), 2 = a single shared row.
+void matmul_experts(const ExpertsView& w, const int32_t* ids, int n_picks, int n_used, int x_mode,
+                    const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);
+// out[i] = silu(gate_e . x * sg_e) * (up_e . x * su_e)
+void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids, int n_picks, int n_used,
+             int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);
+
+// ---- router ----------------------------------------------------------------------
+void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);
+void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,
+                hipStream_t s);
+void moe_finish(float* out, int64_t at, int n, const float* rows, const float* weights, int n_tok, int n_used,
+                const float* shared, const float* logit, int64_t logit_at, hipStream_t s);
+
+// ---- norms and elementwise ------------------------------------------------------
+void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
+              hipStream_t s);
+void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int exact,
+                    hipStream_t s);
+void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s);
+void rope_neox(float* x, const float2* table, int table_half, int64_t n_tok, int pos, const int* pos_dyn,
+               int head_dim, int n_rot, int n_heads, hipStream_t s);
+void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s);
+void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s);
+void add_assign(float* a, const float* b, int64_t n, hipStream_t s);
+void scale(float* a, float v, int64_t n, hipStream_t s);
+void add_scaled(float* a, const float* b, float v, int64_t n, hipStream_t s);
+void add_scaled_rows(float* acc, int64_t n, const float* rows, const float* scales, int n_scales,
+                     hipStream_t s);
+void add_scaled_sigmoid(float* acc, const float* b, int64_t n, const float* logit, hipStream_t s);
+void gather_chunks(const float* src, int64_t chunk, int64_t stride, int64_t offset, float* out,
+                   int64_t out_len, hipStream_t s);
+void scatter_chunks(const float* src, int64_t src_len, int64_t chunk, int64_t stride, int64_t offset,
+                    float* dst, hipStream_t s);
+void kv_write(uint16_t* slab, int64_t offset, const int* offset_dyn, int64_t offset_mul, const float* src,
+              int64_t n, hipStream_t s);
+void fill_zero(void* p, int64_t bytes, hipStream_t s);
+void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s);
+
+// ---- gated delta net ---------------------------------------------------------------
+void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
+              hipStream_t s);
+struct DeltaArgs {
+    const float *q, *k, *v, *alpha, *beta, *ssm_a, *dt_bias;
+    int n_tokens, head_k_dim, head_v_dim, n_k_heads, n_v_heads;
+};
+void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, hipStream_t s);
+
+// ---- attention -------------------------------------------------------------------------
+struct AttnArgs {
+    const float* q;
+    const uint16_t *k, *v;
+    int n_q, kv_dim, n_pos, head_dim, n_head, n_head_kv;
+    float scale;
+    const int* n_pos_dyn;  // overrides n_pos when non-null (decode graphs)
+};
+// exact: the oracle's order (scores, serial softmax sum, positions outermost).
+// scratch: n_q * n_head * n_pos floats.
+void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s);
+// split-K flash decoding; scratch: n_q*n_head*n_split*(head_dim+2) floats.
+int attend_split_count(int n_pos_max);
+void attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);
+
+}  // namespace itk

@@ -1,0 +1,35 @@
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+sys.path.insert(0, str(ROOT / "inferred-thoughts_amd"))
+sys.path.insert(0, str(ROOT))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def golden_dir():
+    return ROOT / "tests" / "golden"
+
+
+@pytest.fixture(scope="session")
+def tiny_gguf(tmp_path_factory):
+    """Config 1 of the baseline: tiny hybrid MoE, all Q8_0, seed 0."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "tiny_q8_0.gguf"
+    ih.synth_write_gguf(str(p), ih.tiny_config(seed=0))
+    return p
+
+
+@pytest.fixture(scope="session")
+def tiny_nvfp4_gguf(tmp_path_factory):
+    """The tiny shape with NVFP4 experts and per-expert scales (exercises config 5's formats)."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "tiny_nvfp4.gguf"
+    ih.synth_write_gguf(str(p), ih.tiny_config(seed=1, expert_type=ih.NVFP4))
+    return p
