@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Decode throughput of the 35B-A3B-shaped NVFP4 synthetic model on one MI355X.
+
+A step is one decode token through the whole per-token loop (48 layers in a 3:1
+GDN:attention pattern, 512 experts top-10 + shared, NVFP4 experts, Q8_0 dense) after a
+layer-at-a-time prefill of a 5,700-token random-id prompt at ctx 8192.  Weights are
+synthetic (seed 0), generated on this machine into a GGUF and uploaded once, so every
+input is resident in HBM before the timed region starts.
+
+Prints ONE JSON line: decode tok/s, the HBM roofline of the dominant kernel (algorithmic
+bytes / HIP-event time on the launch stream) and of the whole token, and the CPU oracle
+timed on this box's host cores on a bounded sample of the same model.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "inferred-thoughts_amd"))
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def model_path(args):
+    base = Path("/dev/shm") if Path("/dev/shm").is_dir() and os.access("/dev/shm", os.W_OK) else Path("/tmp")
+    return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}.gguf"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=48, help="48 is the baseline config; fewer only for quick checks")
+    ap.add_argument("--prompt", type=int, default=5700)
+    ap.add_argument("--ctx", type=int, default=8192)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
+    ap.add_argument("--exact", action="store_true", help="CPU-order reductions (bit-exact mode)")
+    ap.add_argument("--keep", action="store_true", help="keep the generated GGUF")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no collective; see DESIGN.md "
+              "for how it would shard); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import inferred_hip as ih
+    import torch
+
+    t0 = time.time()
+    path = model_path(args)
+    cfg = ih.big_config(seed=args.seed, n_layer=args.layers, n_threads=min(16, os.cpu_count() or 8))
+    if not path.exists():
+        ih.synth_write_gguf(path, cfg)
+    t_synth = time.time() - t0
+    print(f"[bench] model {path} ({path.stat().st_size / 2**30:.1f} GiB) ready in {t_synth:.1f}s", file=sys.stderr, flush=True)
+
+    be = ih.Hip(exact=args.exact)
+    model = ih.Model(path)
+    eng = ih.Engine(model, be, args.ctx)
+    rng = np.random.default_rng(args.seed)
+    prompt = rng.integers(0, model.n_vocab, args.prompt).astype(np.uint32)
+
+    # first pass uploads and repacks every weight: charge it to setup, not to prefill
+    t1 = time.time()
+    eng.forward(prompt[:1], want_logits=False)
+    be.sync()
+    t_upload = time.time() - t1
+    eng.reset()
+    print(f"[bench] weights resident in {t_upload:.1f}s", file=sys.stderr, flush=True)
+
+    t2 = time.time()
+    eng.prefill(prompt, want_logits=False)
+    be.sync(); torch.cuda.synchronize()
+    t_prefill = time.time() - t2
+    print(f"[bench] prefill {args.prompt} tok in {t_prefill:.2f}s", file=sys.stderr, flush=True)
+
+    eng.decode_greedy(args.warmup)
+    be.sync(); torch.cuda.synchronize()
+    pos0 = eng.pos
+    t3 = time.perf_counter()
+    ids = eng.decode_greedy(args.steps)
+    be.sync(); torch.cuda.synchronize()
+    dt = time.perf_counter() - t3
+    assert len(ids) == args.steps
+    tok_s = args.steps / dt
+    graph_stats = be.graph_stats()
+    l0 = be.launch_count(); eng.decode_greedy(1); launches_per_token = be.launch_count() - l0
+
+    # per-kernel device time over a second identical stretch, HIP events on the launch stream
+    be.profile_begin()
+    n_prof = min(args.steps, 16)
+    eng.decode_greedy(n_prof)
+    rows = be.profile_end()
+    err = be.take_error()
+    if err:
+        raise SystemExit(f"device error: {err}")
+
+    # algorithmic bytes of one decode token (weights once + GDN state r+w + KV read)
+    n_attn = sum(1 for il in range(args.layers) if (il + 1) % 4 == 0)
+    n_gdn = args.layers - n_attn
+    w_bytes = model.decode_weight_bytes()
+    state_bytes = n_gdn * 2 * (32 * 128 * 128 * 4) + n_gdn * 2 * (3 * 8192 * 4)
+    kv_bytes = n_attn * (pos0 + args.steps // 2) * 512 * 2 * 2
+    tok_bytes = w_bytes + state_bytes + kv_bytes
+    whole = tok_bytes * tok_s / 1e9
+
+    rows.sort(key=lambda r: -r["ms"])
+    dom = rows[0] if rows else None
+    kernels = {r["name"]: {"launches": r["launches"], "ms_per_token": r["ms"] / n_prof,
+                           "gb_s": (r["bytes"] / 1e9) / (r["ms"] / 1e3) if r["ms"] > 0 and r["bytes"] else None}
+               for r in rows}
+    roofline = None
+    if dom:
+        ach = (dom["bytes"] / 1e9) / (dom["ms"] / 1e3)
+        roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                    "avg_launch_us": round(1e3 * dom["ms"] / dom["launches"], 2),
+                    "bytes_per_launch": dom["bytes"] // dom["launches"]}
+
+    cpu = None
+    if not args.no_cpu:
+        from oracle import binding as ob
+        cores = min(16, os.cpu_count() or 1)
+        ob.lib().orc_set_threads(cores)
+        om = ob.Model(path)
+        oe = ob.Engine(om, 64)
+        n_pre, n_dec = 8, 6
+        oe.forward(prompt[:n_pre])
+        tc = time.perf_counter()
+        out, _ = oe.generate(prompt[n_pre:n_pre + 1], n_dec + 1)   # one more pass primes the loop, n_dec decode passes
+        dtc = time.perf_counter() - tc
+        cpu = {"value": round((n_dec + 1) / dtc, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+               "sample": f"{n_dec + 1} single-token passes of the same {args.layers}-layer model at positions "
+                         f"{n_pre}..{n_pre + n_dec} (context {n_pre + n_dec}, not 5,700), spin-split rows over {cores} threads"}
+        oe.close(); om.close()
+        ob.lib().orc_set_threads(1)
+
+    line = {
+        "metric": "decode tok/s & % HBM roofline, 35B-A3B-shape NVFP4 synthetic; prefill tok/s",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(1e3 * dt / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 dot / f32 accumulate (NVFP4 + Q8_0 weights, Q8_0 activations)",
+        "data": "synthetic",
+        "config": {"workload": "config 5: full 35B-A3B-shaped model, greedy decode after a 5,700-token prefill at ctx 8192"
+                               if args.layers == 48 and args.prompt == 5700 else
+                               f"REDUCED check run: {args.layers} layers, prompt {args.prompt}",
+                   "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "decode_pos": int(pos0),
+                   "experts": "512 top-10 + shared, NVFP4", "dense": "Q8_0 (router and ssm_alpha/beta Q8_0)",
+                   "mode": "exact" if args.exact else "fast", "batch": 1},
+        "prefill_tok_s": round(args.prompt / t_prefill, 1),
+        "bytes_per_token": int(tok_bytes),
+        "token_roofline": {"bound": "hbm", "achieved": round(whole, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(whole / HBM_PEAK_GBS, 4)},
+        "roofline": roofline,
+        "kernels": kernels,
+        "cpu_baseline": cpu,
+        "setup_s": {"synth": round(t_synth, 1), "upload_repack": round(t_upload, 1)},
+        "graph": graph_stats, "launches_per_token": launches_per_token,
+    }
+    print(json.dumps(line), flush=True)
+    eng.close(); model.close(); be.close()
+    if not args.keep:
+        try:
+            path.unlink()
+        except OSError:
+            pass
+
+
+if __name__ == "__main__":
+    main()

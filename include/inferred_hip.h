@@ -192,9 +192,24 @@ int64_t it_hip_clock_pick(uint8_t* heat, const uint8_t* leased, uint64_t n, uint
  * (the rule of Profile::record_token, src/profile.rs:192-213) */
 uint32_t it_hip_argmax(it_hip*, const float* buf, uint64_t len);
 void it_hip_sync(it_hip*);
-/* forget every mirror and resident weight (tests reuse host addresses) */
+/* per-kernel-family device time, measured with HIP events recorded on the launch
+ * stream around every launch between begin and end (at most 16384 launches) */
+typedef struct {
+    char name[48];
+    uint64_t launches;
+    double ms_total;
+    uint64_t bytes_total; /* algorithmic bytes: weights read once + activations in and out */
+} it_profile_row;
+void it_hip_profile_begin(it_hip*);
+int it_hip_profile_end(it_hip*, it_profile_row* rows, int max_rows);
+/* forget the device copy keyed on one host address: call before freeing a buffer
+ * the backend has seen, or a later allocation at the same address reads stale data */
+void it_hip_release(it_hip*, const void* host);
+/* forget every mirror and resident weight (call when the model file is unmapped) */
 void it_hip_drop_mirrors(it_hip*);
 uint64_t it_hip_launch_count(it_hip*);
+/* decode graphs: captures, replays, fallbacks to eager */
+void it_hip_graph_stats(it_hip*, uint64_t out[3]);
 
 /* ---- model + engine: the host side of the loop over this backend ----------
  * Qwen35::load / forward (src/model/qwen35.rs:755-858, 956-1127) and

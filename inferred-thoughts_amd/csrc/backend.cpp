@@ -30,6 +30,124 @@ uint64_t now_us() {
 }
 }  // namespace
 
+// FNV-1a over the raw bytes of each argument
+template <class... A>
+static uint64_t sig_of(const A&... a) {
+    uint64_t h = 0xcbf29ce484222325ull;
+    auto mix = [&](const void* p, size_t n) {
+        const uint8_t* b = (const uint8_t*)p;
+        for (size_t i = 0; i < n; i++) h = (h ^ b[i]) * 0x100000001b3ull;
+    };
+    (mix(&a, sizeof(a)), ...);
+    return h;
+}
+
+const int* it_hip::dyn_slot(int value) {
+    if (mode == Mode::Eager) return nullptr;
+    if (dyn_count >= DYN_CAP) {
+        need_eager("too many position-dependent launches in one pass");
+        return nullptr;
+    }
+    dyn_host[dyn_count] = value;
+    return dyn_dev + dyn_count++;
+}
+
+void it_hip::dyn_rotate() {
+    dyn_cur ^= 1;
+    if (dyn_evt_used[dyn_cur]) check(hipEventSynchronize(dyn_evt[dyn_cur]), "wait for the position staging buffer");
+    dyn_evt_used[dyn_cur] = false;
+    dyn_host = dyn_hosts[dyn_cur];
+    dyn_count = 0;
+}
+void it_hip::dyn_upload() {
+    if (!dyn_count) return;
+    check(hipMemcpyAsync(dyn_dev, dyn_host, dyn_count * sizeof(int), hipMemcpyHostToDevice, stream), "upload positions");
+    if (hipEventRecord(dyn_evt[dyn_cur], stream) == hipSuccess) dyn_evt_used[dyn_cur] = true;
+}
+
+void it_hip::drop_graph() {
+    if (graph.exec) (void)hipGraphExecDestroy(graph.exec);
+    if (graph.graph) (void)hipGraphDestroy(graph.graph);
+    graph.exec = nullptr;
+    graph.graph = nullptr;
+    graph.valid = false;
+    graph.signature.clear();
+    stable_passes = 0;
+}
+
+void it_hip::need_eager(const char* why) {
+    if (mode == Mode::Eager) return;
+    (void)why;
+    if (mode == Mode::Capture) {
+        hipGraph_t g = nullptr;
+        (void)hipStreamEndCapture(stream, &g);
+        if (g) (void)hipGraphDestroy(g);
+        (void)hipGetLastError();
+    }
+    drop_graph();
+    graph_aborts++;
+    mode = Mode::Eager;
+    for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
+    precopies.clear();
+    dyn_upload();
+    auto todo = std::move(pending);
+    pending.clear();
+    for (auto& f : todo) f(stream);
+    check(hipGetLastError(), "kernel launch");
+}
+
+void it_hip::finish_pass() {
+    if (mode == Mode::Eager) {
+        if (pass_tokens == 1 && allow_graph && !mid_pass_read && !prof_on) {
+            stable_passes = (pass_signature == prev_signature && !pass_signature.empty()) ? stable_passes + 1 : 0;
+            prev_signature = pass_signature;
+        } else {
+            stable_passes = 0;
+        }
+        return;
+    }
+    if (mode == Mode::Capture) {
+        hipGraph_t g = nullptr;
+        hipError_t e = hipStreamEndCapture(stream, &g);
+        mode = Mode::Eager;
+        if (e == hipSuccess && g) {
+            hipGraphExec_t ex = nullptr;
+            e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+            if (e == hipSuccess && ex) {
+                drop_graph();
+                graph.graph = g;
+                graph.exec = ex;
+                graph.signature = pass_signature;
+                graph.valid = true;
+                graph_captures++;
+                stable_passes = 1;
+            } else if (g) {
+                (void)hipGraphDestroy(g);
+            }
+        }
+        (void)hipGetLastError();
+        if (!graph.valid) {  // could not build a graph: run the pass eagerly
+            mode = Mode::Replay;  // reuse the fallback path
+            need_eager("graph instantiation failed");
+            allow_graph = false;
+            return;
+        }
+    } else {  // Replay
+        mode = Mode::Eager;
+        if (replay_cursor != graph.signature.size()) {
+            mode = Mode::Replay;
+            need_eager("the pass ended early");
+            return;
+        }
+    }
+    for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
+    precopies.clear();
+    dyn_upload();
+    check(hipGraphLaunch(graph.exec, stream), "hipGraphLaunch");
+    graph_launches++;
+    pending.clear();
+}
+
 void it_hip::fail(const std::string& what) {
     if (!has_error) {
         has_error = true;
@@ -46,6 +164,7 @@ bool it_hip::check(hipError_t e, const char* what) {
 it_hip::Act* it_hip::act_slot(const float* host, size_t len) {
     Act& a = acts[host];
     if (a.cap < len) {
+        need_eager("an activation mirror has to grow");
         float* fresh = nullptr;
         size_t cap = len;
         if (!check(hipMalloc((void**)&fresh, cap * sizeof(float)), "hipMalloc(activation mirror)")) return nullptr;
@@ -67,9 +186,12 @@ float* it_hip::act_in(const float* host, size_t len) {
     Act* a = act_slot(host, len);
     if (!a) return nullptr;
     if (!a->dev_current) {
-        if (!check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream),
-                   "upload activation"))
+        if (mode != Mode::Eager) {
+            precopies.push_back(PreCopy{a->dev, host, len * sizeof(float)});
+        } else if (!check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream),
+                          "upload activation")) {
             return nullptr;
+        }
         h2d++;
         h2d_bytes += len * sizeof(float);
         a->dev_current = true;
@@ -96,6 +218,7 @@ bool it_hip::act_quantized(const float* host, size_t len, const float** scales, 
     if (!x) return false;
     Act& a = acts[host];
     if (a.q_cap < len) {
+        need_eager("a quantized-activation buffer has to grow");
         if (a.q_scales) {
             check(hipStreamSynchronize(stream), "sync before quant free");
             quant_bytes -= a.q_cap / 32 * 4 + a.q_cap;
@@ -112,8 +235,10 @@ bool it_hip::act_quantized(const float* host, size_t len, const float** scales, 
         a.q_valid = false;
     }
     if (!a.q_valid || a.q_len != len) {
-        quantize_q8_0(x, a.q_scales, a.q_quants, (int64_t)len, stream);
-        launches++;
+        float* qs = a.q_scales;
+        int8_t* qq = a.q_quants;
+        submit(FAM_OTHER, len * 5, sig_of(101, x, qs, qq, len),
+               [=](hipStream_t s) { quantize_q8_0(x, qs, qq, (int64_t)len, s); });
         a.q_valid = true;
         a.q_len = len;
     }
@@ -126,6 +251,7 @@ bool it_hip::act_quantized(const float* host, size_t len, const float** scales, 
 const float* it_hip::const_in(const float* host, size_t len) {
     auto it = consts.find(host);
     if (it != consts.end() && it->second.len >= len) return it->second.dev;
+    need_eager("a constant is uploaded for the first time");
     Const c;
     if (!check(hipMalloc((void**)&c.dev, len * sizeof(float)), "hipMalloc(constant)")) return nullptr;
     if (!check(hipMemcpyAsync(c.dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream), "upload constant"))
@@ -158,6 +284,7 @@ const it_hip::Resident* it_hip::resident(const uint8_t* data, uint64_t len, uint
         fail(std::string(who) + ": weight byte length does not match its shape");
         return nullptr;
     }
+    need_eager("a weight is uploaded for the first time");
     uint64_t t0 = now_us();
     Resident r;
     r.fmt = (int)ty;
@@ -175,7 +302,6 @@ const it_hip::Resident* it_hip::resident(const uint8_t* data, uint64_t len, uint
             !check(hipMalloc(&r.scales, r.s_bytes), "hipMalloc(q8_0 scales)"))
             return nullptr;
         repack_q8_0((const uint8_t*)raw, (int8_t*)r.q, (uint16_t*)r.scales, (int64_t)rows, (int)n_in, stream);
-        launches++;
         check(hipStreamSynchronize(stream), "repack q8_0");
         (void)hipFree(raw);
     } else if (ty == IT_NVFP4) {
@@ -185,7 +311,6 @@ const it_hip::Resident* it_hip::resident(const uint8_t* data, uint64_t len, uint
             !check(hipMalloc(&r.scales, r.s_bytes), "hipMalloc(nvfp4 scales)"))
             return nullptr;
         repack_nvfp4((const uint8_t*)raw, (uint8_t*)r.q, (uint8_t*)r.scales, (int64_t)rows, (int)n_in, stream);
-        launches++;
         check(hipStreamSynchronize(stream), "repack nvfp4");
         (void)hipFree(raw);
     } else {
@@ -246,6 +371,7 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
     }
     Resident* rw = &weights[w->data];
     if (w->scale && w->scale_len && !rw->scale2) {
+        need_eager("expert scales are uploaded for the first time");
         if (!check(hipMalloc((void**)&rw->scale2, w->scale_len), "hipMalloc(expert scales)")) return false;
         if (!check(hipMemcpyAsync(rw->scale2, w->scale, w->scale_len, hipMemcpyHostToDevice, stream),
                    "upload expert scales"))
@@ -272,6 +398,7 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
 // ------------------------------------------------------------------ slabs
 void* it_hip::slab_in(const void* host, size_t bytes, bool is_state) {
     Slab& s = slabs[host];
+    if (!s.dev || s.bytes < bytes || !s.dev_owned) need_eager("a slab is uploaded");
     if (s.dev && s.bytes < bytes) {
         check(hipStreamSynchronize(stream), "sync before slab free");
         (void)hipFree(s.dev);
@@ -297,6 +424,7 @@ void* it_hip::slab_in(const void* host, size_t bytes, bool is_state) {
 // ------------------------------------------------------------------ route storage
 bool it_hip::route_reserve(size_t picks) {
     if (route_cap >= picks) return true;
+    need_eager("route storage has to grow");
     if (route_ids) {
         check(hipStreamSynchronize(stream), "sync before route free");
         (void)hipFree(route_ids);
@@ -327,6 +455,7 @@ bool it_hip::route_stage(const it_route* r, const int32_t** ids, const float** w
             fail("route: empty host route");
             return false;
         }
+        need_eager("a host route is staged");
         if (!route_reserve(picks)) return false;
         std::vector<int32_t> tmp(picks);
         for (size_t i = 0; i < picks; i++) tmp[i] = (int32_t)r->ids[i];
@@ -354,7 +483,8 @@ const float2* it_hip::rope_table(float theta, uint64_t n_rot, uint64_t need_pos)
     uint64_t key = ((uint64_t)tb << 32) | n_rot;
     Rope& r = ropes[key];
     if (r.cap_pos >= need_pos) return r.dev;
-    size_t cap = r.cap_pos ? r.cap_pos : 1024;
+    need_eager("the rope table has to grow");
+    size_t cap = r.cap_pos ? r.cap_pos : 8192;
     while (cap < need_pos) cap *= 2;
     size_t half = n_rot / 2;
     std::vector<float2> tab(cap * half);
@@ -379,6 +509,7 @@ const float2* it_hip::rope_table(float theta, uint64_t n_rot, uint64_t need_pos)
 
 float* it_hip::scratch_f32(size_t floats) {
     if (attn_scratch_cap >= floats) return attn_scratch;
+    need_eager("attention scratch has to grow");
     if (attn_scratch) {
         check(hipStreamSynchronize(stream), "sync before scratch free");
         (void)hipFree(attn_scratch);
@@ -391,7 +522,33 @@ float* it_hip::scratch_f32(size_t floats) {
     return attn_scratch;
 }
 
+// ------------------------------------------------------------------ event timing
+hipEvent_t it_hip::prof_event() {
+    if (prof_pool_next < prof_pool.size()) return prof_pool[prof_pool_next++];
+    hipEvent_t e = nullptr;
+    if (prof_pool.size() >= 32768 || hipEventCreate(&e) != hipSuccess) return nullptr;
+    prof_pool.push_back(e);
+    prof_pool_next++;
+    return e;
+}
+it_hip::Span::Span(it_hip* b, int fam, uint64_t bytes) : be(b), live(false) {
+    if (!b->prof_on) return;
+    s.a = b->prof_event();
+    s.b = b->prof_event();
+    if (!s.a || !s.b) return;
+    s.fam = fam;
+    s.bytes = bytes;
+    live = hipEventRecord(s.a, b->stream) == hipSuccess;
+}
+it_hip::Span::~Span() {
+    if (!live) return;
+    if (hipEventRecord(s.b, be->stream) == hipSuccess) be->prof_spans.push_back(s);
+}
+
 void it_hip::drop_all() {
+    need_eager("mirrors are dropped");
+    drop_graph();
+    prev_signature.clear();
     if (stream) (void)hipStreamSynchronize(stream);
     for (auto& kv : acts) {
         if (kv.second.dev) (void)hipFree(kv.second.dev);
@@ -426,10 +583,13 @@ it_hip::~it_hip() {
     if (argmax_val) (void)hipFree(argmax_val);
     if (argmax_out) (void)hipFree(argmax_out);
     if (argmax_host) (void)hipHostFree(argmax_host);
+    for (auto e : prof_pool) (void)hipEventDestroy(e);
     if (dyn_dev) (void)hipFree(dyn_dev);
-    if (dyn_host) (void)hipHostFree(dyn_host);
-    if (graph.exec) (void)hipGraphExecDestroy(graph.exec);
-    if (graph.graph) (void)hipGraphDestroy(graph.graph);
+    for (int i = 0; i < 2; i++) {
+        if (dyn_hosts[i]) (void)hipHostFree(dyn_hosts[i]);
+        if (dyn_evt[i]) (void)hipEventDestroy(dyn_evt[i]);
+    }
+    drop_graph();
     if (stream) (void)hipStreamDestroy(stream);
 }
 
@@ -459,6 +619,15 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
         delete be;
         return bad(std::string("hipStreamCreate: ") + hipGetErrorString(e));
     }
+    if (hipMalloc((void**)&be->dyn_dev, it_hip::DYN_CAP * sizeof(int)) != hipSuccess ||
+        hipHostMalloc((void**)&be->dyn_hosts[0], it_hip::DYN_CAP * sizeof(int), hipHostMallocDefault) != hipSuccess ||
+        hipHostMalloc((void**)&be->dyn_hosts[1], it_hip::DYN_CAP * sizeof(int), hipHostMallocDefault) != hipSuccess ||
+        hipEventCreateWithFlags(&be->dyn_evt[0], hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&be->dyn_evt[1], hipEventDisableTiming) != hipSuccess) {
+        delete be;
+        return bad("cannot allocate the position staging buffers");
+    }
+    be->dyn_host = be->dyn_hosts[0];
     return be;
 }
 
@@ -488,7 +657,6 @@ int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* m
     return 1;
 }
 
-#define BE_STREAM be->stream
 #define REQUIRE(cond, msg)   \
     do {                     \
         if (!(cond)) {       \
@@ -496,6 +664,11 @@ int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* m
             return;          \
         }                    \
     } while (0)
+
+enum OpId : int {
+    OP_RMS = 1, OP_RMS_HEADS, OP_L2, OP_MATMUL, OP_ROPE, OP_SOFTMAX, OP_ATTEND, OP_EW, OP_SCALE, OP_CONV, OP_GATHER,
+    OP_SCATTER, OP_DELTA, OP_ROUTE, OP_EXPERTS, OP_GLU, OP_FINISH, OP_ROWS, OP_SIGADD, OP_KVWRITE
+};
 
 void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w, uint64_t w_len, float eps,
                      float* out, uint64_t out_len) {
@@ -507,8 +680,10 @@ void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w,
     float* dout = (out == x) ? dx : be->act_out(out, out_len);
     if (!dw || !dx || !dout) return;
     if (out == x) be->acts[x].q_valid = false;
-    rms_norm(dx, dw, eps, dout, (int64_t)(x_len / w_len), (int)w_len, be->exact, BE_STREAM);
-    be->launches++;
+    int64_t rows = (int64_t)(x_len / w_len);
+    int nd = (int)w_len, exact = be->exact;
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS, dx, dw, eps, dout, rows, nd),
+               [=](hipStream_t s) { rms_norm(dx, dw, eps, dout, rows, nd, exact, s); });
 }
 
 void it_hip_rms_norm_heads(it_hip* be, float* x, uint64_t x_len, const float* w, uint64_t w_len,
@@ -519,8 +694,22 @@ void it_hip_rms_norm_heads(it_hip* be, float* x, uint64_t x_len, const float* w,
     const float* dw = be->const_in(w, w_len);
     float* dx = be->act_inout(x, x_len);
     if (!dw || !dx) return;
-    rms_norm_heads(dx, dw, (int)head_dim, eps, (int64_t)(x_len / head_dim), be->exact, BE_STREAM);
-    be->launches++;
+    int hd = (int)head_dim, exact = be->exact;
+    int64_t heads = (int64_t)(x_len / head_dim);
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS_HEADS, dx, dw, hd, eps, heads),
+               [=](hipStream_t s) { rms_norm_heads(dx, dw, hd, eps, heads, exact, s); });
+}
+
+void it_hip_l2_norm_heads(it_hip* be, float* x, uint64_t x_len, uint64_t head_dim, float eps) {
+    REQUIRE(head_dim > 0 && x_len % head_dim == 0, "l2_norm_heads: head_dim must divide x.len()");
+    REQUIRE(head_dim <= 12288, "l2_norm_heads: head longer than the kernel's LDS tile");
+    if (x_len == 0) return;
+    float* dx = be->act_inout(x, x_len);
+    if (!dx) return;
+    int hd = (int)head_dim, exact = be->exact;
+    int64_t heads = (int64_t)(x_len / head_dim);
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_L2, dx, hd, eps, heads),
+               [=](hipStream_t s) { l2_norm_heads(dx, hd, eps, heads, exact, s); });
 }
 
 static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, float* out,
@@ -548,8 +737,10 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     }
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
-    matmul(v, dx, as, aq, (int)n, dout, 1.0f, BE_STREAM);
-    be->launches++;
+    int nt = (int)n;
+    be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
+               sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout),
+               [=](hipStream_t s) { matmul(v, dx, as, aq, nt, dout, 1.0f, s); });
 }
 
 void it_hip_matmul(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, float* out,
@@ -574,9 +765,11 @@ void it_hip_rope_neox(it_hip* be, float* x, uint64_t x_len, uint64_t pos, uint64
     const float2* tab = be->rope_table(theta, n_rot, pos + n);
     float* dx = be->act_inout(x, x_len);
     if (!tab || !dx) return;
-    rope_neox(dx, tab, (int)(n_rot / 2), (int64_t)n, (int)pos, nullptr, (int)head_dim, (int)n_rot, (int)n_heads,
-              BE_STREAM);
-    be->launches++;
+    const int* dyn = be->dyn_slot((int)pos);
+    int pv = dyn ? 0 : (int)pos, half = (int)(n_rot / 2), hd = (int)head_dim, nr = (int)n_rot, nh = (int)n_heads;
+    int64_t nt = (int64_t)n;
+    be->submit(it_hip::FAM_OTHER, x_len * 8, sig_of(OP_ROPE, dx, tab, half, nt, dyn, hd, nr, nh),
+               [=](hipStream_t s) { rope_neox(dx, tab, half, nt, pv, dyn, hd, nr, nh, s); });
 }
 
 void it_hip_softmax(it_hip* be, float* x, uint64_t x_len, uint64_t row) {
@@ -585,8 +778,10 @@ void it_hip_softmax(it_hip* be, float* x, uint64_t x_len, uint64_t row) {
     REQUIRE(row <= 12288, "softmax: row longer than the kernel's LDS tile");
     float* dx = be->act_inout(x, x_len);
     if (!dx) return;
-    softmax_rows(dx, (int64_t)(x_len / row), (int)row, be->exact, BE_STREAM);
-    be->launches++;
+    int64_t rows = (int64_t)(x_len / row);
+    int r = (int)row, exact = be->exact;
+    be->submit(it_hip::FAM_ROUTER, x_len * 8, sig_of(OP_SOFTMAX, dx, rows, r),
+               [=](hipStream_t s) { softmax_rows(dx, rows, r, exact, s); });
 }
 
 void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
@@ -606,21 +801,34 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
     uint16_t* dv = (uint16_t*)be->slab_in(a->v, a->kv_len * 2, false);
     float* dout = be->act_out(out, out_len);
     if (!dq || !dk || !dv || !dout) return;
-    AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, (int)a->n_pos, (int)a->head_dim,
-                  (int)a->n_head, (int)a->n_head_kv, a->scale, nullptr};
     uint64_t group = a->n_head / a->n_head_kv;
     bool split_ok = (group == 1 || group == 2 || group == 4 || group == 8) && a->head_dim <= 256;
+    bool graphed = be->mode != it_hip::Mode::Eager;
+    // a graphed pass keeps one launch shape while the context grows: size for the whole slab
+    uint64_t n_pos_cap = graphed ? a->kv_len / a->kv_dim : a->n_pos;
+    uint64_t bytes = a->n_pos * a->n_head_kv * a->head_dim * 4 + a->q_len * 8;
     if (be->exact || !split_ok) {
-        float* sc = be->scratch_f32((size_t)(n_q * a->n_head * a->n_pos));
+        float* sc = be->scratch_f32((size_t)(n_q * a->n_head * n_pos_cap));
         if (!sc) return;
-        attend_exact(args, sc, dout, BE_STREAM);
-        be->launches++;
+        const int* dyn = be->dyn_slot((int)a->n_pos);
+        AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? (int)n_pos_cap : (int)a->n_pos, (int)a->head_dim,
+                      (int)a->n_head, (int)a->n_head_kv, a->scale, dyn};
+        AttnArgs sg = args;
+        be->submit(it_hip::FAM_ATTEND, bytes,
+                   sig_of(OP_ATTEND, 0, sg.q, sg.k, sg.v, sg.n_q, sg.kv_dim, dyn ? sg.n_pos : 0, sg.head_dim, sg.n_head,
+                          sg.n_head_kv, sg.scale, dyn, sc, dout),
+                   [=](hipStream_t s) { attend_exact(args, sc, dout, s); });
     } else {
-        int n_split = attend_split_count((int)a->n_pos);
+        int n_split = attend_split_count((int)n_pos_cap);
         float* sc = be->scratch_f32((size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2));
         if (!sc) return;
-        attend_split(args, n_split, sc, dout, BE_STREAM);
-        be->launches += 2;
+        const int* dyn = be->dyn_slot((int)a->n_pos);
+        AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? 0 : (int)a->n_pos, (int)a->head_dim,
+                      (int)a->n_head, (int)a->n_head_kv, a->scale, dyn};
+        be->submit(it_hip::FAM_ATTEND, bytes,
+                   sig_of(OP_ATTEND, 1, dq, dk, dv, args.n_q, args.kv_dim, args.head_dim, args.n_head, args.n_head_kv,
+                          args.scale, dyn, dyn ? n_split : 0, sc, dout),
+                   [=](hipStream_t s) { attend_split(args, n_split, sc, dout, s); });
     }
 }
 
@@ -634,13 +842,15 @@ static void ew2(it_hip* be, float* a, uint64_t a_len, const float* b, uint64_t b
     float* da = be->act_inout(a, a_len);
     float* db = be->act_in(b, b_len);
     if (!da || !db) return;
-    switch (op) {
-        case 0: silu_mul(da, db, (int64_t)a_len, be->stream); break;
-        case 1: sigmoid_mul(da, db, (int64_t)a_len, be->stream); break;
-        case 2: add_assign(da, db, (int64_t)a_len, be->stream); break;
-        case 3: add_scaled(da, db, v, (int64_t)a_len, be->stream); break;
-    }
-    be->launches++;
+    int64_t n = (int64_t)a_len;
+    be->submit(it_hip::FAM_OTHER, a_len * 12, sig_of(OP_EW, op, da, db, n, v), [=](hipStream_t s) {
+        switch (op) {
+            case 0: silu_mul(da, db, n, s); break;
+            case 1: sigmoid_mul(da, db, n, s); break;
+            case 2: add_assign(da, db, n, s); break;
+            case 3: add_scaled(da, db, v, n, s); break;
+        }
+    });
 }
 
 void it_hip_silu_mul(it_hip* be, float* gate, uint64_t gate_len, const float* up, uint64_t up_len) {
@@ -656,22 +866,12 @@ void it_hip_add_scaled(it_hip* be, float* a, uint64_t a_len, const float* b, uin
     ew2(be, a, a_len, b, b_len, "add_scaled", 3, scale_v);
 }
 
-void it_hip_scale(it_hip* be, float* buf, uint64_t len, float s) {
+void it_hip_scale(it_hip* be, float* buf, uint64_t len, float sv) {
     if (len == 0) return;
     float* d = be->act_inout(buf, len);
     if (!d) return;
-    scale(d, s, (int64_t)len, BE_STREAM);
-    be->launches++;
-}
-
-void it_hip_l2_norm_heads(it_hip* be, float* x, uint64_t x_len, uint64_t head_dim, float eps) {
-    REQUIRE(head_dim > 0 && x_len % head_dim == 0, "l2_norm_heads: head_dim must divide x.len()");
-    REQUIRE(head_dim <= 12288, "l2_norm_heads: head longer than the kernel's LDS tile");
-    if (x_len == 0) return;
-    float* dx = be->act_inout(x, x_len);
-    if (!dx) return;
-    l2_norm_heads(dx, (int)head_dim, eps, (int64_t)(x_len / head_dim), be->exact, BE_STREAM);
-    be->launches++;
+    int64_t n = (int64_t)len;
+    be->submit(it_hip::FAM_OTHER, len * 8, sig_of(OP_SCALE, d, sv, n), [=](hipStream_t s) { scale(d, sv, n, s); });
 }
 
 void it_hip_ssm_conv(it_hip* be, float* state, uint64_t state_len, const float* x, uint64_t x_len,
@@ -688,8 +888,9 @@ void it_hip_ssm_conv(it_hip* be, float* state, uint64_t state_len, const float* 
     float* dx = be->act_in(x, x_len);
     float* dout = be->act_out(out, out_len);
     if (!dw || !dstate || !dx || !dout) return;
-    ssm_conv(dstate, dx, dw, (int)kernel, (int)nc, (int)(x_len / nc), dout, BE_STREAM);
-    be->launches++;
+    int k = (int)kernel, c = (int)nc, nt = (int)(x_len / nc);
+    be->submit(it_hip::FAM_OTHER, x_len * 8 + state_len * 8, sig_of(OP_CONV, dstate, dx, dw, k, c, nt, dout),
+               [=](hipStream_t s) { ssm_conv(dstate, dx, dw, k, c, nt, dout, s); });
 }
 
 void it_hip_gather_chunks(it_hip* be, const float* src, uint64_t src_len, uint64_t chunk, uint64_t stride,
@@ -701,8 +902,9 @@ void it_hip_gather_chunks(it_hip* be, const float* src, uint64_t src_len, uint64
     float* ds = be->act_in(src, src_len);
     float* dout = be->act_out(out, out_len);
     if (!ds || !dout) return;
-    gather_chunks(ds, (int64_t)chunk, (int64_t)stride, (int64_t)offset, dout, (int64_t)out_len, BE_STREAM);
-    be->launches++;
+    int64_t c = (int64_t)chunk, st = (int64_t)stride, off = (int64_t)offset, ol = (int64_t)out_len;
+    be->submit(it_hip::FAM_OTHER, out_len * 8, sig_of(OP_GATHER, ds, c, st, off, dout, ol),
+               [=](hipStream_t s) { gather_chunks(ds, c, st, off, dout, ol, s); });
 }
 
 void it_hip_scatter_chunks(it_hip* be, const float* src, uint64_t src_len, uint64_t chunk, uint64_t stride,
@@ -714,8 +916,9 @@ void it_hip_scatter_chunks(it_hip* be, const float* src, uint64_t src_len, uint6
     float* ds = be->act_in(src, src_len);
     float* dd = be->act_inout(dst, dst_len);
     if (!ds || !dd) return;
-    scatter_chunks(ds, (int64_t)src_len, (int64_t)chunk, (int64_t)stride, (int64_t)offset, dd, BE_STREAM);
-    be->launches++;
+    int64_t sl = (int64_t)src_len, c = (int64_t)chunk, st = (int64_t)stride, off = (int64_t)offset;
+    be->submit(it_hip::FAM_OTHER, src_len * 8, sig_of(OP_SCATTER, ds, sl, c, st, off, dd),
+               [=](hipStream_t s) { scatter_chunks(ds, sl, c, st, off, dd, s); });
 }
 
 void it_hip_delta_rule(it_hip* be, const it_delta* d, float* state, uint64_t state_len, float* out,
@@ -741,8 +944,11 @@ void it_hip_delta_rule(it_hip* be, const it_delta* d, float* state, uint64_t sta
     if (!dq || !dk || !dv || !da || !db || !dssm || !ddt || !dstate || !dout) return;
     DeltaArgs args{dq, dk, dv, da, db, dssm, ddt, (int)n, (int)d->head_k_dim, (int)d->head_v_dim,
                    (int)d->n_k_heads, (int)d->n_v_heads};
-    delta_rule(args, dstate, dout, be->exact, BE_STREAM);
-    be->launches++;
+    int exact = be->exact;
+    be->submit(it_hip::FAM_DELTA, state_len * 8 + n * (2 * kper + 2 * vper) * 4,
+               sig_of(OP_DELTA, dq, dk, dv, da, db, dssm, ddt, args.n_tokens, args.head_k_dim, args.head_v_dim,
+                      args.n_k_heads, args.n_v_heads, dstate, dout),
+               [=](hipStream_t s) { delta_rule(args, dstate, dout, exact, s); });
 }
 
 void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_expert, uint64_t n_used,
@@ -758,8 +964,11 @@ void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_exper
     REQUIRE(n_tok < (1ull << 24), "route: too many tokens");
     float* dp = be->act_in(probs, probs_len);
     if (!dp || !be->route_reserve((size_t)(n_tok * n_used))) return;
-    route_topk(dp, (int)n_tok, (int)n_expert, (int)n_used, be->route_ids, be->route_w, BE_STREAM);
-    be->launches++;
+    int32_t* ids = be->route_ids;
+    float* rw = be->route_w;
+    int nt = (int)n_tok, ne = (int)n_expert, nu = (int)n_used;
+    be->submit(it_hip::FAM_ROUTER, probs_len * 4, sig_of(OP_ROUTE, dp, nt, ne, nu, ids, rw),
+               [=](hipStream_t s) { route_topk(dp, nt, ne, nu, ids, rw, s); });
     be->route_n_used = n_used;
     be->route_n_tok = n_tok;
 }
@@ -798,8 +1007,10 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     if (!be->act_quantized(x, x_len, &as, &aq, nullptr)) return;
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
-    matmul_experts(v, ids, (int)picks, (int)n_used, x_mode_of(rows, picks), as, aq, dout, BE_STREAM);
-    be->launches++;
+    int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
+               sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout),
+               [=](hipStream_t s) { matmul_experts(v, ids, np, nu, xm, as, aq, dout, s); });
     be->expert_lookups += picks;
 }
 
@@ -830,8 +1041,11 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     if (!be->act_quantized(x, x_len, &as, &aq, nullptr)) return;
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
-    moe_glu(g, u, ids, (int)picks, (int)n_used, x_mode_of(rows, picks), as, aq, dout, BE_STREAM);
-    be->launches++;
+    int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    be->submit(it_hip::FAM_MOE_GLU, 2 * picks * (gate->len / gate->n_expert) + x_len + out_len * 4,
+               sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
+                      as, aq, dout),
+               [=](hipStream_t s) { moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s); });
     be->expert_lookups += 2 * picks;
 }
 
@@ -846,6 +1060,7 @@ void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, ui
         // weights only: stage them without needing ids
         uint64_t picks = route->n_used * route->n_tok;
         REQUIRE(picks > 0, "moe_finish: empty route");
+        be->need_eager("a host route is staged");
         if (!be->route_reserve((size_t)picks)) return;
         if (!be->check(hipMemcpyAsync(be->route_w, route->weights, picks * 4, hipMemcpyHostToDevice, be->stream), "upload weights")) return;
         be->check(hipStreamSynchronize(be->stream), "upload weights");
@@ -869,8 +1084,10 @@ void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, ui
     bool covers_all = (at == 0 && n_tok * n == out_len);
     float* dout = covers_all ? be->act_out(out, out_len) : be->act_inout(out, out_len);
     if (!dr || !ds || !dl || !dout) return;
-    moe_finish(dout, (int64_t)at, (int)n, dr, rw, (int)n_tok, (int)n_used, ds, dl, (int64_t)logit_at, BE_STREAM);
-    be->launches++;
+    int64_t a64 = (int64_t)at, la = (int64_t)logit_at;
+    int ni = (int)n, nt = (int)n_tok, nu = (int)n_used;
+    be->submit(it_hip::FAM_OTHER, rows_len * 4 + n_tok * n * 8, sig_of(OP_FINISH, dout, a64, ni, dr, rw, nt, nu, ds, dl, la),
+               [=](hipStream_t s) { moe_finish(dout, a64, ni, dr, rw, nt, nu, ds, dl, la, s); });
 }
 
 void it_hip_add_scaled_rows(it_hip* be, float* acc, uint64_t acc_len, const float* rows, uint64_t rows_len,
@@ -882,8 +1099,10 @@ void it_hip_add_scaled_rows(it_hip* be, float* acc, uint64_t acc_len, const floa
     float* dsc = be->act_in(scales, scales_len);
     float* da = be->act_out(acc, acc_len);
     if (!dr || !dsc || !da) return;
-    add_scaled_rows(da, (int64_t)acc_len, dr, dsc, (int)scales_len, BE_STREAM);
-    be->launches++;
+    int64_t n = (int64_t)acc_len;
+    int ns = (int)scales_len;
+    be->submit(it_hip::FAM_OTHER, rows_len * 4, sig_of(OP_ROWS, da, n, dr, dsc, ns),
+               [=](hipStream_t s) { add_scaled_rows(da, n, dr, dsc, ns, s); });
 }
 
 void it_hip_add_scaled_sigmoid(it_hip* be, float* acc, uint64_t acc_len, const float* b, uint64_t b_len,
@@ -894,8 +1113,9 @@ void it_hip_add_scaled_sigmoid(it_hip* be, float* acc, uint64_t acc_len, const f
     float* db = be->act_in(b, b_len);
     float* dl = be->act_in(logit, logit_len);
     if (!da || !db || !dl) return;
-    add_scaled_sigmoid(da, db, (int64_t)acc_len, dl, BE_STREAM);
-    be->launches++;
+    int64_t n = (int64_t)acc_len;
+    be->submit(it_hip::FAM_OTHER, acc_len * 12, sig_of(OP_SIGADD, da, db, n, dl),
+               [=](hipStream_t s) { add_scaled_sigmoid(da, db, n, dl, s); });
 }
 
 void it_hip_kv_write(it_hip* be, uint16_t* slab, uint64_t slab_len, uint64_t offset, const float* src,
@@ -905,9 +1125,22 @@ void it_hip_kv_write(it_hip* be, uint16_t* slab, uint64_t slab_len, uint64_t off
     float* ds = be->act_in(src, src_len);
     uint16_t* dslab = (uint16_t*)be->slab_in(slab, slab_len * 2, false);
     if (!ds || !dslab) return;
-    kv_write(dslab, (int64_t)offset, nullptr, 0, ds, (int64_t)src_len, BE_STREAM);
-    be->launches++;
+    // a graphed decode pass writes row `pos` of the slab: offset = pos * src_len
+    const int* dyn = nullptr;
+    int64_t mul = 0, off = (int64_t)offset, n = (int64_t)src_len;
+    if (be->mode != it_hip::Mode::Eager && offset % src_len == 0 && offset / src_len < (1ull << 31)) {
+        dyn = be->dyn_slot((int)(offset / src_len));
+        if (dyn) {
+            mul = n;
+            off = 0;
+        }
+    } else {
+        be->need_eager("a kv_write offset is not a whole row");
+    }
+    be->submit(it_hip::FAM_OTHER, src_len * 6, sig_of(OP_KVWRITE, dslab, dyn, mul, dyn ? (int64_t)0 : (int64_t)0, ds, n),
+               [=](hipStream_t s) { kv_write(dslab, off, dyn, mul, ds, n, s); });
 }
+
 
 // ------------------------------------------------------------------ residency
 void it_hip_host_wrote(it_hip* be, const float* buf, uint64_t len) {
@@ -922,7 +1155,12 @@ void it_hip_host_wrote(it_hip* be, const float* buf, uint64_t len) {
 void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
     auto it = be->acts.find(buf);
     if (it == be->acts.end() || !it->second.dev_current) return;
-    if (be->in_pass) be->mid_pass_read = true;
+    if (be->in_pass) {
+        // a read inside a pass cannot be served from a graph that has not run yet:
+        // graphs are latched off for this backend (src/ops/cuda/ops/mod.rs:565-582)
+        be->mid_pass_read = true;
+        be->need_eager("the host read a device buffer inside a pass");
+    }
     size_t n = len < it->second.cap ? len : it->second.cap;
     if (!be->check(hipMemcpyAsync(buf, it->second.dev, n * sizeof(float), hipMemcpyDeviceToHost, be->stream), "download activation")) return;
     be->check(hipStreamSynchronize(be->stream), "download activation");
@@ -931,15 +1169,36 @@ void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
 }
 
 void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
+    if (be->in_pass) be->finish_pass();
     be->in_pass = true;
     be->pass_tokens = n_tokens;
+    be->pass_signature.clear();
+    be->pending.clear();
+    be->precopies.clear();
+    be->dyn_rotate();
+    be->replay_cursor = 0;
+    be->mode = it_hip::Mode::Eager;
+    if (n_tokens == 1 && be->allow_graph && !be->mid_pass_read && !be->prof_on && !be->has_error) {
+        if (be->graph.valid) {
+            be->mode = it_hip::Mode::Replay;
+        } else if (be->stable_passes >= 1) {
+            if (hipStreamBeginCapture(be->stream, hipStreamCaptureModeRelaxed) == hipSuccess)
+                be->mode = it_hip::Mode::Capture;
+            else
+                (void)hipGetLastError();
+        }
+    }
     for (auto& kv : be->acts) {
         kv.second.dev_current = false;
         kv.second.q_valid = false;
     }
 }
 
-void it_hip_end_pass(it_hip* be) { be->in_pass = false; }
+void it_hip_end_pass(it_hip* be) {
+    if (!be->in_pass) return;
+    be->finish_pass();
+    be->in_pass = false;
+}
 
 void it_hip_forget_state(it_hip* be) {
     for (auto& kv : be->slabs)
@@ -947,6 +1206,7 @@ void it_hip_forget_state(it_hip* be) {
 }
 
 void it_hip_read_state(it_hip* be, float* host, uint64_t len) {
+    be->need_eager("a state slab is read");
     auto it = be->slabs.find(host);
     if (it == be->slabs.end() || !it->second.dev_owned) return;
     size_t bytes = len * 4 < it->second.bytes ? len * 4 : it->second.bytes;
@@ -957,6 +1217,7 @@ void it_hip_read_state(it_hip* be, float* host, uint64_t len) {
 }
 
 void it_hip_read_kv(it_hip* be, uint16_t* slab, uint64_t len) {
+    be->need_eager("a kv slab is read");
     auto it = be->slabs.find(slab);
     if (it == be->slabs.end() || !it->second.dev_owned) return;
     size_t bytes = len * 2 < it->second.bytes ? len * 2 : it->second.bytes;
@@ -1059,6 +1320,7 @@ uint32_t it_hip_argmax(it_hip* be, const float* buf, uint64_t len) {
             !be->check(hipHostMalloc((void**)&be->argmax_host, 4, hipHostMallocDefault), "hipHostMalloc(argmax)"))
             return 0;
     }
+    be->need_eager("argmax");
     argmax(d, (int64_t)len, be->argmax_out, be->argmax_idx, be->argmax_val, be->stream);
     be->launches += 2;
     if (!be->check(hipMemcpyAsync(be->argmax_host, be->argmax_out, 4, hipMemcpyDeviceToHost, be->stream), "download argmax")) return 0;
@@ -1066,6 +1328,73 @@ uint32_t it_hip_argmax(it_hip* be, const float* buf, uint64_t len) {
     be->d2h++;
     be->d2h_bytes += 4;
     return (uint32_t)*be->argmax_host;
+}
+
+void it_hip_release(it_hip* be, const void* host) {
+    be->need_eager("a buffer is released");
+    be->drop_graph();  // a captured graph may hold the pointers being freed
+    auto a = be->acts.find(host);
+    auto s = be->slabs.find(host);
+    auto c = be->consts.find(host);
+    if (a == be->acts.end() && s == be->slabs.end() && c == be->consts.end()) return;
+    be->check(hipStreamSynchronize(be->stream), "sync before release");
+    if (a != be->acts.end()) {
+        be->mirror_bytes -= a->second.cap * sizeof(float);
+        if (a->second.q_scales) be->quant_bytes -= a->second.q_cap / 32 * 4 + a->second.q_cap;
+        if (a->second.dev) (void)hipFree(a->second.dev);
+        if (a->second.q_scales) (void)hipFree(a->second.q_scales);
+        if (a->second.q_quants) (void)hipFree(a->second.q_quants);
+        be->acts.erase(a);
+    }
+    if (s != be->slabs.end()) {
+        be->kv_bytes -= s->second.bytes;
+        if (s->second.dev) (void)hipFree(s->second.dev);
+        be->slabs.erase(s);
+    }
+    if (c != be->consts.end()) {
+        be->const_bytes -= c->second.len * 4;
+        if (c->second.dev) (void)hipFree(c->second.dev);
+        be->consts.erase(c);
+    }
+}
+
+void it_hip_graph_stats(it_hip* be, uint64_t out[3]) {
+    out[0] = be->graph_captures;
+    out[1] = be->graph_launches;
+    out[2] = be->graph_aborts;
+}
+
+void it_hip_profile_begin(it_hip* be) {
+    be->need_eager("profiling");
+    be->check(hipStreamSynchronize(be->stream), "sync");
+    be->prof_spans.clear();
+    be->prof_pool_next = 0;
+    be->prof_on = true;
+}
+
+int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
+    static const char* names[it_hip::FAM_COUNT] = {"matmul (dense GEMV/GEMM)", "moe_glu (expert gate+up)",
+                                                   "matmul_experts (expert down)", "delta_rule", "attend",
+                                                   "norms", "router (softmax + top-k)", "other"};
+    be->prof_on = false;
+    be->check(hipStreamSynchronize(be->stream), "sync");
+    it_profile_row acc[it_hip::FAM_COUNT];
+    memset(acc, 0, sizeof acc);
+    for (auto& sp : be->prof_spans) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, sp.a, sp.b) != hipSuccess) continue;
+        acc[sp.fam].launches++;
+        acc[sp.fam].ms_total += ms;
+        acc[sp.fam].bytes_total += sp.bytes;
+    }
+    int n = 0;
+    for (int f = 0; f < it_hip::FAM_COUNT && n < max_rows; f++) {
+        if (!acc[f].launches) continue;
+        snprintf(acc[f].name, sizeof acc[f].name, "%s", names[f]);
+        rows[n++] = acc[f];
+    }
+    be->prof_spans.clear();
+    return n;
 }
 
 void it_hip_sync(it_hip* be) { be->check(hipStreamSynchronize(be->stream), "sync"); }

@@ -10,6 +10,8 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <cstring>
+#include <functional>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -120,16 +122,79 @@ struct it_hip {
     };
     Graph graph;
     enum class Mode { Eager, Capture, Replay } mode = Mode::Eager;
-    uint64_t decode_passes = 0;
-    std::vector<uint64_t> pass_signature;
+    std::vector<uint64_t> pass_signature, prev_signature;
+    int stable_passes = 0;      // consecutive eager decode passes with the same op sequence
     size_t replay_cursor = 0;
-    bool replay_broken = false;
+    uint64_t graph_launches = 0, graph_captures = 0, graph_aborts = 0;
+    // work of the pass being captured or replayed, kept so it can run eagerly if the graph path breaks
+    std::vector<std::function<void(hipStream_t)>> pending;
+    struct PreCopy {
+        void* dev;
+        const void* host;
+        size_t bytes;
+    };
+    std::vector<PreCopy> precopies;  // host -> device inputs of a graphed pass, issued before the graph
     int* dyn_dev = nullptr;    // device ints read by position-dependent kernels
-    int* dyn_host = nullptr;   // pinned staging
-    size_t dyn_count = 0, dyn_cap = 0;
-    bool graph_note(uint64_t sig);  // returns true when the kernel must actually be launched
-    const int* dyn_slot(int value);
+    // pinned staging, double-buffered: a pass may fill one while the previous pass's async
+    // copy of the other has not run yet
+    int* dyn_hosts[2] = {nullptr, nullptr};
+    hipEvent_t dyn_evt[2] = {nullptr, nullptr};
+    bool dyn_evt_used[2] = {false, false};
+    int dyn_cur = 0;
+    int* dyn_host = nullptr;   // = dyn_hosts[dyn_cur]
+    void dyn_rotate();
+    void dyn_upload();
+    size_t dyn_count = 0;
+    static constexpr size_t DYN_CAP = 4096;
+    const int* dyn_slot(int value);   // null in eager mode: the kernel takes the scalar by value
+    void need_eager(const char* why); // leave capture/replay: run what the pass queued so far eagerly
+    void finish_pass();
     bool mid_pass_read = false;
+
+    // Every kernel launch goes through here.  `sig` hashes the launch's static arguments
+    // (pointers, shapes); position-dependent scalars never enter it.
+    template <class F>
+    void submit(int fam, uint64_t bytes, uint64_t sig, F&& f) {
+        launches++;
+        if (mode == Mode::Eager) {
+            if (in_pass && pass_tokens == 1) pass_signature.push_back(sig);
+            Span sp(this, fam, bytes);
+            f(stream);
+            check(hipGetLastError(), "kernel launch");
+            return;
+        }
+        pending.emplace_back(f);
+        pass_signature.push_back(sig);
+        if (mode == Mode::Capture) {
+            f(stream);
+            if (hipGetLastError() != hipSuccess) need_eager("a launch failed during capture");
+        } else if (replay_cursor >= graph.signature.size() || graph.signature[replay_cursor] != sig) {
+            need_eager("the op sequence changed");
+        } else {
+            replay_cursor++;
+        }
+    }
+
+    // ---- per-kernel-family timing with HIP events on the launch stream
+    enum Family { FAM_MATMUL = 0, FAM_MOE_GLU, FAM_MOE_DOWN, FAM_DELTA, FAM_ATTEND, FAM_NORM, FAM_ROUTER, FAM_OTHER, FAM_COUNT };
+    struct ProfSpan {
+        hipEvent_t a, b;
+        int fam;
+        uint64_t bytes;
+    };
+    bool prof_on = false;
+    std::vector<ProfSpan> prof_spans;
+    std::vector<hipEvent_t> prof_pool;
+    size_t prof_pool_next = 0;
+    hipEvent_t prof_event();
+    // RAII span: records an event before and after the launches issued inside its scope
+    struct Span {
+        it_hip* be;
+        ProfSpan s;
+        bool live;
+        Span(it_hip* b, int fam, uint64_t bytes);
+        ~Span();
+    };
 
     // ---- counters
     uint64_t launches = 0, h2d = 0, d2h = 0, h2d_bytes = 0, d2h_bytes = 0;
@@ -139,5 +204,6 @@ struct it_hip {
     uint64_t expert_budget = 0, expert_host_budget = 0, expert_slots_req = 0;
 
     void drop_all();
+    void drop_graph();
     ~it_hip();
 };

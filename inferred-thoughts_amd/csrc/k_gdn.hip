@@ -18,7 +18,7 @@ template <int DK>
 __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restrict__ state,
                                                    float* __restrict__ out, float q_scale) {
     __shared__ float tile[64 * (DK + 1)];
-    __shared__ float kq[2 * DK];
+    __shared__ __align__(16) float kq[2 * DK];
     const int lane = threadIdx.x;
     const int dv = d.head_v_dim;
     const int blocks_per_head = (dv + 63) / 64;
@@ -29,9 +29,23 @@ __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restric
     const int rows_here = min(64, dv - jb * 64);
     float* S = state + ((int64_t)h * dv + (int64_t)jb * 64) * DK;
 
-    for (int idx = lane; idx < rows_here * DK; idx += 64) {
-        int r = idx / DK, c = idx - r * DK;
-        tile[r * (DK + 1) + c] = S[idx];
+    // 64 rows x DK floats = 16*DK float4; every load is issued before the first LDS write
+    {
+        constexpr int V = DK / 4;  // float4 per row
+        const float4* S4 = (const float4*)S;
+        float4 stage[V];
+#pragma unroll
+        for (int it = 0; it < V; it++) {
+            int idx4 = it * 64 + lane;
+            stage[it] = (idx4 < rows_here * V) ? S4[idx4] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int it = 0; it < V; it++) {
+            int idx4 = it * 64 + lane;
+            int r = idx4 / V, c = (idx4 - r * V) * 4;
+            float* t = tile + r * (DK + 1) + c;
+            t[0] = stage[it].x; t[1] = stage[it].y; t[2] = stage[it].z; t[3] = stage[it].w;
+        }
     }
     __syncthreads();
     float row[DK];
@@ -52,17 +66,25 @@ __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restric
         float beta = 1.0f / (1.0f + it_expf(-d.beta[(int64_t)t * d.n_v_heads + h]));
         float v = live ? d.v[(int64_t)t * vper + h * dv + j] : 0.0f;
         float pred = 0.0f;
+        const float4* k4 = (const float4*)kq;
+        const float4* q4 = (const float4*)(kq + DK);
 #pragma unroll
-        for (int i = 0; i < DK; i++) {
-            row[i] *= g;
-            pred += row[i] * kq[i];
+        for (int i = 0; i < DK; i += 4) {
+            float4 kk = k4[i / 4];
+            row[i] *= g;     pred += row[i] * kk.x;
+            row[i + 1] *= g; pred += row[i + 1] * kk.y;
+            row[i + 2] *= g; pred += row[i + 2] * kk.z;
+            row[i + 3] *= g; pred += row[i + 3] * kk.w;
         }
         float delta = beta * (v - pred);
         float o = 0.0f;
 #pragma unroll
-        for (int i = 0; i < DK; i++) {
-            row[i] += kq[i] * delta;
-            o += row[i] * (kq[DK + i] * q_scale);
+        for (int i = 0; i < DK; i += 4) {
+            float4 kk = k4[i / 4], qq = q4[i / 4];
+            row[i] += kk.x * delta;     o += row[i] * (qq.x * q_scale);
+            row[i + 1] += kk.y * delta; o += row[i + 1] * (qq.y * q_scale);
+            row[i + 2] += kk.z * delta; o += row[i + 2] * (qq.z * q_scale);
+            row[i + 3] += kk.w * delta; o += row[i + 3] * (qq.w * q_scale);
         }
         if (live) out[(int64_t)t * vper + h * dv + j] = o;
     }
@@ -71,9 +93,16 @@ __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restric
     for (int i = 0; i < DK; i++)
         if (live) tile[lane * (DK + 1) + i] = row[i];
     __syncthreads();
-    for (int idx = lane; idx < rows_here * DK; idx += 64) {
-        int r = idx / DK, c = idx - r * DK;
-        S[idx] = tile[r * (DK + 1) + c];
+    {
+        constexpr int V = DK / 4;
+        float4* S4 = (float4*)S;
+#pragma unroll
+        for (int it = 0; it < V; it++) {
+            int idx4 = it * 64 + lane;
+            int r = idx4 / V, c = (idx4 - r * V) * 4;
+            const float* t = tile + r * (DK + 1) + c;
+            if (idx4 < rows_here * V) S4[idx4] = make_float4(t[0], t[1], t[2], t[3]);
+        }
     }
 }
 

@@ -482,7 +482,25 @@ it_engine* it_engine_new(it_model* m, it_hip* be, uint64_t n_ctx, uint64_t max_b
     e->ssm.assign(d.layers() * d.ssm_len(), 0.0f);
     return e;
 }
-void it_engine_free(it_engine* e) { delete e; }
+void it_engine_free(it_engine* e) {
+    if (!e) return;
+    // the host buffers are about to be freed: drop the device copies keyed on them
+    HostBuf* bufs[] = {&e->x, &e->normed, &e->mixed, &e->ffn_out, &e->qg, &e->q, &e->g, &e->k, &e->v, &e->attn,
+                       &e->qkv, &e->z, &e->alpha, &e->beta, &e->convo, &e->q_part, &e->k_part, &e->v_part, &e->core,
+                       &e->router, &e->e_gate, &e->e_up, &e->e_out, &e->e_in, &e->g_all, &e->u_all, &e->o_all,
+                       &e->shexp_logit, &e->last, &e->final_norm, &e->logits};
+    for (HostBuf* b : bufs)
+        if (!b->v.empty()) it_hip_release(e->be, b->p());
+    for (uint64_t s = 0; s < e->m->n_kv_layer; s++) {
+        it_hip_release(e->be, e->k_slab(s));
+        it_hip_release(e->be, e->v_slab(s));
+    }
+    for (uint64_t il = 0; il < e->m->d.layers(); il++) {
+        it_hip_release(e->be, e->conv_of(il));
+        it_hip_release(e->be, e->ssm_of(il));
+    }
+    delete e;
+}
 
 // Engine::reset, src/engine/mod.rs:296-306
 void it_engine_reset(it_engine* e) {

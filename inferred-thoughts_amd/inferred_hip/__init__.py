@@ -68,6 +68,10 @@ class ExpertStats(C.Structure):
                                       "fetched", "lookups", "hits")] + [("oversubscribed", c_u32), ("_pad", c_u32)]
 
 
+class ProfileRow(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("launches", c_u64), ("ms_total", C.c_double), ("bytes_total", c_u64)]
+
+
 class SynthConfig(C.Structure):
     _fields_ = [(n, c_u64) for n in ("n_layer", "n_embd", "n_vocab", "n_head", "n_head_kv", "head_dim", "n_rot",
                                       "n_expert", "n_expert_used", "expert_ff", "shared_ff", "ssm_d_conv",
@@ -87,7 +91,7 @@ it_hip_kv_write it_hip_host_wrote it_hip_host_needs it_hip_begin_pass it_hip_end
 it_hip_read_state it_hip_read_kv it_hip_device_report it_hip_reserve_activations it_hip_tier_counters
 it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_budget
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
-it_hip_clock_pick it_hip_argmax it_hip_sync it_hip_drop_mirrors it_hip_launch_count it_model_open
+it_hip_clock_pick it_hip_argmax it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_model_open
 it_model_close it_model_dims it_model_decode_weight_bytes it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
@@ -166,8 +170,12 @@ def lib() -> C.CDLL:
         "it_hip_clock_pick": (C.c_int64, [vp, vp, u64, vp]),
         "it_hip_argmax": (u32, [vp, vp, u64]),
         "it_hip_sync": (None, [vp]),
+        "it_hip_profile_begin": (None, [vp]),
+        "it_hip_profile_end": (C.c_int, [vp, vp, C.c_int]),
+        "it_hip_release": (None, [vp, vp]),
         "it_hip_drop_mirrors": (None, [vp]),
         "it_hip_launch_count": (u64, [vp]),
+        "it_hip_graph_stats": (None, [vp, vp]),
         "it_model_open": (vp, [C.c_char_p, C.c_char_p, C.c_size_t]),
         "it_model_close": (None, [vp]),
         "it_model_dims": (None, [vp, vp]),
@@ -366,11 +374,25 @@ class Hip:
     def sync(self):
         self.L.it_hip_sync(self.h)
 
+    def profile_begin(self):
+        self.L.it_hip_profile_begin(self.h)
+
+    def profile_end(self):
+        rows = (ProfileRow * 16)()
+        n = self.L.it_hip_profile_end(self.h, rows, 16)
+        return [dict(name=rows[i].name.decode(), launches=int(rows[i].launches), ms=float(rows[i].ms_total),
+                     bytes=int(rows[i].bytes_total)) for i in range(n)]
+
     def drop_mirrors(self):
         self.L.it_hip_drop_mirrors(self.h)
 
     def launch_count(self) -> int:
         return int(self.L.it_hip_launch_count(self.h))
+
+    def graph_stats(self):
+        v = (c_u64 * 3)()
+        self.L.it_hip_graph_stats(self.h, v)
+        return {"captures": int(v[0]), "replays": int(v[1]), "aborts": int(v[2])}
 
     def tier_counters(self) -> TierCounters:
         t = TierCounters()
