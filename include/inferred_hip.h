@@ -97,6 +97,7 @@ typedef struct it_hip it_hip;
 enum {
     IT_HIP_EXACT = 1,    /* every reduction in the CPU path's order (bit-identical results) */
     IT_HIP_NO_GRAPH = 2, /* never capture decode passes into a HIP graph */
+    IT_HIP_NO_FUSE = 4,  /* capture decode passes op by op, without the fused kernels */
 };
 
 /* Cuda::new, src/ops/cuda/mod.rs:757-935.  NULL on failure with a message in err. */
@@ -208,8 +209,8 @@ void it_hip_release(it_hip*, const void* host);
 /* forget every mirror and resident weight (call when the model file is unmapped) */
 void it_hip_drop_mirrors(it_hip*);
 uint64_t it_hip_launch_count(it_hip*);
-/* decode graphs: captures, replays, fallbacks to eager */
-void it_hip_graph_stats(it_hip*, uint64_t out[3]);
+/* decode graphs: captures, replays, fallbacks to eager, kernel launches in the captured graph */
+void it_hip_graph_stats(it_hip*, uint64_t out[4]);
 
 /* ---- model + engine: the host side of the loop over this backend ----------
  * Qwen35::load / forward (src/model/qwen35.rs:755-858, 956-1127) and

@@ -9,6 +9,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 using namespace itk;
@@ -78,12 +79,6 @@ void it_hip::drop_graph() {
 void it_hip::need_eager(const char* why) {
     if (mode == Mode::Eager) return;
     (void)why;
-    if (mode == Mode::Capture) {
-        hipGraph_t g = nullptr;
-        (void)hipStreamEndCapture(stream, &g);
-        if (g) (void)hipGraphDestroy(g);
-        (void)hipGetLastError();
-    }
     drop_graph();
     graph_aborts++;
     mode = Mode::Eager;
@@ -92,7 +87,7 @@ void it_hip::need_eager(const char* why) {
     dyn_upload();
     auto todo = std::move(pending);
     pending.clear();
-    for (auto& f : todo) f(stream);
+    for (auto& op : todo) op.run(stream);
     check(hipGetLastError(), "kernel launch");
 }
 
@@ -107,8 +102,17 @@ void it_hip::finish_pass() {
         return;
     }
     if (mode == Mode::Capture) {
+        // inputs first (they are not part of the graph), then record the fused pass
+        for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
+        precopies.clear();
         hipGraph_t g = nullptr;
-        hipError_t e = hipStreamEndCapture(stream, &g);
+        hipError_t e = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed);
+        if (e == hipSuccess) {
+            run_fused(pending);
+            hipError_t le = hipGetLastError();
+            e = hipStreamEndCapture(stream, &g);
+            if (le != hipSuccess) e = le;
+        }
         mode = Mode::Eager;
         if (e == hipSuccess && g) {
             hipGraphExec_t ex = nullptr;
@@ -237,7 +241,10 @@ bool it_hip::act_quantized(const float* host, size_t len, const float** scales, 
     if (!a.q_valid || a.q_len != len) {
         float* qs = a.q_scales;
         int8_t* qq = a.q_quants;
-        submit(FAM_OTHER, len * 5, sig_of(101, x, qs, qq, len),
+        OpRec rec;
+        rec.id = 101;  // OP_QUANT
+        rec.p[0] = x; rec.p[1] = qs; rec.p[2] = qq; rec.i[0] = (int64_t)len;
+        submit(FAM_OTHER, len * 5, sig_of(101, x, qs, qq, len), rec,
                [=](hipStream_t s) { quantize_q8_0(x, qs, qq, (int64_t)len, s); });
         a.q_valid = true;
         a.q_len = len;
@@ -615,6 +622,7 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->device = device;
     be->exact = (flags & IT_HIP_EXACT) != 0;
     be->allow_graph = (flags & IT_HIP_NO_GRAPH) == 0;
+    be->fuse_enabled = (flags & IT_HIP_NO_FUSE) == 0 && getenv("INFERRED_HIP_NO_FUSE") == nullptr;
     if ((e = hipStreamCreate(&be->stream)) != hipSuccess) {
         delete be;
         return bad(std::string("hipStreamCreate: ") + hipGetErrorString(e));
@@ -665,10 +673,6 @@ int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* m
         }                    \
     } while (0)
 
-enum OpId : int {
-    OP_RMS = 1, OP_RMS_HEADS, OP_L2, OP_MATMUL, OP_ROPE, OP_SOFTMAX, OP_ATTEND, OP_EW, OP_SCALE, OP_CONV, OP_GATHER,
-    OP_SCATTER, OP_DELTA, OP_ROUTE, OP_EXPERTS, OP_GLU, OP_FINISH, OP_ROWS, OP_SIGADD, OP_KVWRITE
-};
 
 void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w, uint64_t w_len, float eps,
                      float* out, uint64_t out_len) {
@@ -682,7 +686,9 @@ void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w,
     if (out == x) be->acts[x].q_valid = false;
     int64_t rows = (int64_t)(x_len / w_len);
     int nd = (int)w_len, exact = be->exact;
-    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS, dx, dw, eps, dout, rows, nd),
+    it_hip::OpRec rec;
+    rec.id = OP_RMS; rec.p[0] = dx; rec.p[1] = dw; rec.p[2] = dout; rec.i[0] = rows; rec.i[1] = nd; rec.f[0] = eps;
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS, dx, dw, eps, dout, rows, nd), rec,
                [=](hipStream_t s) { rms_norm(dx, dw, eps, dout, rows, nd, exact, s); });
 }
 
@@ -696,7 +702,9 @@ void it_hip_rms_norm_heads(it_hip* be, float* x, uint64_t x_len, const float* w,
     if (!dw || !dx) return;
     int hd = (int)head_dim, exact = be->exact;
     int64_t heads = (int64_t)(x_len / head_dim);
-    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS_HEADS, dx, dw, hd, eps, heads),
+    it_hip::OpRec rec;
+    rec.id = OP_RMS_HEADS; rec.p[0] = dx; rec.p[1] = dw; rec.i[0] = hd; rec.i[1] = heads; rec.f[0] = eps;
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS_HEADS, dx, dw, hd, eps, heads), rec,
                [=](hipStream_t s) { rms_norm_heads(dx, dw, hd, eps, heads, exact, s); });
 }
 
@@ -708,7 +716,9 @@ void it_hip_l2_norm_heads(it_hip* be, float* x, uint64_t x_len, uint64_t head_di
     if (!dx) return;
     int hd = (int)head_dim, exact = be->exact;
     int64_t heads = (int64_t)(x_len / head_dim);
-    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_L2, dx, hd, eps, heads),
+    it_hip::OpRec rec;
+    rec.id = OP_L2; rec.p[0] = dx; rec.i[0] = hd; rec.i[1] = heads; rec.f[0] = eps;
+    be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_L2, dx, hd, eps, heads), rec,
                [=](hipStream_t s) { l2_norm_heads(dx, hd, eps, heads, exact, s); });
 }
 
@@ -738,8 +748,11 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int nt = (int)n;
+    it_hip::OpRec rec;
+    rec.id = OP_MATMUL; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = dx; rec.p[3] = as; rec.p[4] = aq; rec.p[5] = dout;
+    rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = nt;
     be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
-               sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout),
+               sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout), rec,
                [=](hipStream_t s) { matmul(v, dx, as, aq, nt, dout, 1.0f, s); });
 }
 
@@ -768,7 +781,10 @@ void it_hip_rope_neox(it_hip* be, float* x, uint64_t x_len, uint64_t pos, uint64
     const int* dyn = be->dyn_slot((int)pos);
     int pv = dyn ? 0 : (int)pos, half = (int)(n_rot / 2), hd = (int)head_dim, nr = (int)n_rot, nh = (int)n_heads;
     int64_t nt = (int64_t)n;
-    be->submit(it_hip::FAM_OTHER, x_len * 8, sig_of(OP_ROPE, dx, tab, half, nt, dyn, hd, nr, nh),
+    it_hip::OpRec rec;
+    rec.id = OP_ROPE; rec.p[0] = dx; rec.p[1] = tab; rec.p[2] = dyn;
+    rec.i[0] = half; rec.i[1] = nt; rec.i[2] = hd; rec.i[3] = nr; rec.i[4] = nh; rec.i[5] = pv;
+    be->submit(it_hip::FAM_OTHER, x_len * 8, sig_of(OP_ROPE, dx, tab, half, nt, dyn, hd, nr, nh), rec,
                [=](hipStream_t s) { rope_neox(dx, tab, half, nt, pv, dyn, hd, nr, nh, s); });
 }
 
@@ -780,7 +796,9 @@ void it_hip_softmax(it_hip* be, float* x, uint64_t x_len, uint64_t row) {
     if (!dx) return;
     int64_t rows = (int64_t)(x_len / row);
     int r = (int)row, exact = be->exact;
-    be->submit(it_hip::FAM_ROUTER, x_len * 8, sig_of(OP_SOFTMAX, dx, rows, r),
+    it_hip::OpRec rec;
+    rec.id = OP_SOFTMAX; rec.p[0] = dx; rec.i[0] = rows; rec.i[1] = r;
+    be->submit(it_hip::FAM_ROUTER, x_len * 8, sig_of(OP_SOFTMAX, dx, rows, r), rec,
                [=](hipStream_t s) { softmax_rows(dx, rows, r, exact, s); });
 }
 
@@ -814,9 +832,13 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? (int)n_pos_cap : (int)a->n_pos, (int)a->head_dim,
                       (int)a->n_head, (int)a->n_head_kv, a->scale, dyn};
         AttnArgs sg = args;
+        it_hip::OpRec rec;
+        rec.id = OP_ATTEND; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = dyn; rec.p[4] = sc; rec.p[5] = dout;
+        rec.i[0] = args.n_q; rec.i[1] = args.kv_dim; rec.i[2] = args.head_dim; rec.i[3] = args.n_head;
+        rec.i[4] = args.n_head_kv; rec.i[6] = 1; rec.f[0] = args.scale;  // exact form: launched as is
         be->submit(it_hip::FAM_ATTEND, bytes,
                    sig_of(OP_ATTEND, 0, sg.q, sg.k, sg.v, sg.n_q, sg.kv_dim, dyn ? sg.n_pos : 0, sg.head_dim, sg.n_head,
-                          sg.n_head_kv, sg.scale, dyn, sc, dout),
+                          sg.n_head_kv, sg.scale, dyn, sc, dout), rec,
                    [=](hipStream_t s) { attend_exact(args, sc, dout, s); });
     } else {
         int n_split = attend_split_count((int)n_pos_cap);
@@ -825,9 +847,13 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         const int* dyn = be->dyn_slot((int)a->n_pos);
         AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? 0 : (int)a->n_pos, (int)a->head_dim,
                       (int)a->n_head, (int)a->n_head_kv, a->scale, dyn};
+        it_hip::OpRec rec;
+        rec.id = OP_ATTEND; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = dyn; rec.p[4] = sc; rec.p[5] = dout;
+        rec.i[0] = args.n_q; rec.i[1] = args.kv_dim; rec.i[2] = args.head_dim; rec.i[3] = args.n_head;
+        rec.i[4] = args.n_head_kv; rec.i[5] = n_split; rec.i[6] = 0; rec.i[7] = args.n_pos; rec.f[0] = args.scale;
         be->submit(it_hip::FAM_ATTEND, bytes,
                    sig_of(OP_ATTEND, 1, dq, dk, dv, args.n_q, args.kv_dim, args.head_dim, args.n_head, args.n_head_kv,
-                          args.scale, dyn, dyn ? n_split : 0, sc, dout),
+                          args.scale, dyn, dyn ? n_split : 0, sc, dout), rec,
                    [=](hipStream_t s) { attend_split(args, n_split, sc, dout, s); });
     }
 }
@@ -843,7 +869,9 @@ static void ew2(it_hip* be, float* a, uint64_t a_len, const float* b, uint64_t b
     float* db = be->act_in(b, b_len);
     if (!da || !db) return;
     int64_t n = (int64_t)a_len;
-    be->submit(it_hip::FAM_OTHER, a_len * 12, sig_of(OP_EW, op, da, db, n, v), [=](hipStream_t s) {
+    it_hip::OpRec rec;
+    rec.id = OP_EW; rec.p[0] = da; rec.p[1] = db; rec.i[0] = op; rec.i[1] = n; rec.f[0] = v;
+    be->submit(it_hip::FAM_OTHER, a_len * 12, sig_of(OP_EW, op, da, db, n, v), rec, [=](hipStream_t s) {
         switch (op) {
             case 0: silu_mul(da, db, n, s); break;
             case 1: sigmoid_mul(da, db, n, s); break;
@@ -871,7 +899,9 @@ void it_hip_scale(it_hip* be, float* buf, uint64_t len, float sv) {
     float* d = be->act_inout(buf, len);
     if (!d) return;
     int64_t n = (int64_t)len;
-    be->submit(it_hip::FAM_OTHER, len * 8, sig_of(OP_SCALE, d, sv, n), [=](hipStream_t s) { scale(d, sv, n, s); });
+    it_hip::OpRec rec;
+    rec.id = OP_SCALE;
+    be->submit(it_hip::FAM_OTHER, len * 8, sig_of(OP_SCALE, d, sv, n), rec, [=](hipStream_t s) { scale(d, sv, n, s); });
 }
 
 void it_hip_ssm_conv(it_hip* be, float* state, uint64_t state_len, const float* x, uint64_t x_len,
@@ -889,7 +919,9 @@ void it_hip_ssm_conv(it_hip* be, float* state, uint64_t state_len, const float* 
     float* dout = be->act_out(out, out_len);
     if (!dw || !dstate || !dx || !dout) return;
     int k = (int)kernel, c = (int)nc, nt = (int)(x_len / nc);
-    be->submit(it_hip::FAM_OTHER, x_len * 8 + state_len * 8, sig_of(OP_CONV, dstate, dx, dw, k, c, nt, dout),
+    it_hip::OpRec rec;
+    rec.id = OP_CONV; rec.p[0] = dstate; rec.p[1] = dx; rec.p[2] = dw; rec.p[3] = dout; rec.i[0] = k; rec.i[1] = c; rec.i[2] = nt;
+    be->submit(it_hip::FAM_OTHER, x_len * 8 + state_len * 8, sig_of(OP_CONV, dstate, dx, dw, k, c, nt, dout), rec,
                [=](hipStream_t s) { ssm_conv(dstate, dx, dw, k, c, nt, dout, s); });
 }
 
@@ -903,7 +935,9 @@ void it_hip_gather_chunks(it_hip* be, const float* src, uint64_t src_len, uint64
     float* dout = be->act_out(out, out_len);
     if (!ds || !dout) return;
     int64_t c = (int64_t)chunk, st = (int64_t)stride, off = (int64_t)offset, ol = (int64_t)out_len;
-    be->submit(it_hip::FAM_OTHER, out_len * 8, sig_of(OP_GATHER, ds, c, st, off, dout, ol),
+    it_hip::OpRec rec;
+    rec.id = OP_GATHER; rec.p[0] = ds; rec.p[1] = dout; rec.i[0] = c; rec.i[1] = st; rec.i[2] = off; rec.i[3] = ol;
+    be->submit(it_hip::FAM_OTHER, out_len * 8, sig_of(OP_GATHER, ds, c, st, off, dout, ol), rec,
                [=](hipStream_t s) { gather_chunks(ds, c, st, off, dout, ol, s); });
 }
 
@@ -917,7 +951,9 @@ void it_hip_scatter_chunks(it_hip* be, const float* src, uint64_t src_len, uint6
     float* dd = be->act_inout(dst, dst_len);
     if (!ds || !dd) return;
     int64_t sl = (int64_t)src_len, c = (int64_t)chunk, st = (int64_t)stride, off = (int64_t)offset;
-    be->submit(it_hip::FAM_OTHER, src_len * 8, sig_of(OP_SCATTER, ds, sl, c, st, off, dd),
+    it_hip::OpRec rec;
+    rec.id = OP_SCATTER;
+    be->submit(it_hip::FAM_OTHER, src_len * 8, sig_of(OP_SCATTER, ds, sl, c, st, off, dd), rec,
                [=](hipStream_t s) { scatter_chunks(ds, sl, c, st, off, dd, s); });
 }
 
@@ -945,9 +981,13 @@ void it_hip_delta_rule(it_hip* be, const it_delta* d, float* state, uint64_t sta
     DeltaArgs args{dq, dk, dv, da, db, dssm, ddt, (int)n, (int)d->head_k_dim, (int)d->head_v_dim,
                    (int)d->n_k_heads, (int)d->n_v_heads};
     int exact = be->exact;
+    it_hip::OpRec rec;
+    rec.id = OP_DELTA; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = da; rec.p[4] = db; rec.p[5] = dssm;
+    rec.p[6] = ddt; rec.p[7] = dstate; rec.p[8] = dout;
+    rec.i[0] = args.n_tokens; rec.i[1] = args.head_k_dim; rec.i[2] = args.head_v_dim; rec.i[3] = args.n_k_heads; rec.i[4] = args.n_v_heads;
     be->submit(it_hip::FAM_DELTA, state_len * 8 + n * (2 * kper + 2 * vper) * 4,
                sig_of(OP_DELTA, dq, dk, dv, da, db, dssm, ddt, args.n_tokens, args.head_k_dim, args.head_v_dim,
-                      args.n_k_heads, args.n_v_heads, dstate, dout),
+                      args.n_k_heads, args.n_v_heads, dstate, dout), rec,
                [=](hipStream_t s) { delta_rule(args, dstate, dout, exact, s); });
 }
 
@@ -967,7 +1007,9 @@ void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_exper
     int32_t* ids = be->route_ids;
     float* rw = be->route_w;
     int nt = (int)n_tok, ne = (int)n_expert, nu = (int)n_used;
-    be->submit(it_hip::FAM_ROUTER, probs_len * 4, sig_of(OP_ROUTE, dp, nt, ne, nu, ids, rw),
+    it_hip::OpRec rec;
+    rec.id = OP_ROUTE; rec.p[0] = dp; rec.p[1] = ids; rec.p[2] = rw; rec.i[0] = nt; rec.i[1] = ne; rec.i[2] = nu;
+    be->submit(it_hip::FAM_ROUTER, probs_len * 4, sig_of(OP_ROUTE, dp, nt, ne, nu, ids, rw), rec,
                [=](hipStream_t s) { route_topk(dp, nt, ne, nu, ids, rw, s); });
     be->route_n_used = n_used;
     be->route_n_tok = n_tok;
@@ -1008,8 +1050,12 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    it_hip::OpRec rec;
+    rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
+    rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
+    rec.i[6] = v.q_stride; rec.i[7] = v.s_stride;
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
-               sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout),
+               sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) { matmul_experts(v, ids, np, nu, xm, as, aq, dout, s); });
     be->expert_lookups += picks;
 }
@@ -1042,9 +1088,14 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    it_hip::OpRec rec;
+    rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
+    rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
+    rec.i[0] = g.fmt; rec.i[1] = g.n_in; rec.i[2] = g.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
+    rec.i[6] = g.q_stride; rec.i[7] = g.s_stride;
     be->submit(it_hip::FAM_MOE_GLU, 2 * picks * (gate->len / gate->n_expert) + x_len + out_len * 4,
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
-                      as, aq, dout),
+                      as, aq, dout), rec,
                [=](hipStream_t s) { moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s); });
     be->expert_lookups += 2 * picks;
 }
@@ -1086,7 +1137,10 @@ void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, ui
     if (!dr || !ds || !dl || !dout) return;
     int64_t a64 = (int64_t)at, la = (int64_t)logit_at;
     int ni = (int)n, nt = (int)n_tok, nu = (int)n_used;
-    be->submit(it_hip::FAM_OTHER, rows_len * 4 + n_tok * n * 8, sig_of(OP_FINISH, dout, a64, ni, dr, rw, nt, nu, ds, dl, la),
+    it_hip::OpRec rec;
+    rec.id = OP_FINISH; rec.p[0] = dout; rec.p[1] = dr; rec.p[2] = rw; rec.p[3] = ds; rec.p[4] = dl;
+    rec.i[0] = a64; rec.i[1] = ni; rec.i[2] = nt; rec.i[3] = nu; rec.i[4] = la;
+    be->submit(it_hip::FAM_OTHER, rows_len * 4 + n_tok * n * 8, sig_of(OP_FINISH, dout, a64, ni, dr, rw, nt, nu, ds, dl, la), rec,
                [=](hipStream_t s) { moe_finish(dout, a64, ni, dr, rw, nt, nu, ds, dl, la, s); });
 }
 
@@ -1101,7 +1155,9 @@ void it_hip_add_scaled_rows(it_hip* be, float* acc, uint64_t acc_len, const floa
     if (!dr || !dsc || !da) return;
     int64_t n = (int64_t)acc_len;
     int ns = (int)scales_len;
-    be->submit(it_hip::FAM_OTHER, rows_len * 4, sig_of(OP_ROWS, da, n, dr, dsc, ns),
+    it_hip::OpRec rec;
+    rec.id = OP_ROWS;
+    be->submit(it_hip::FAM_OTHER, rows_len * 4, sig_of(OP_ROWS, da, n, dr, dsc, ns), rec,
                [=](hipStream_t s) { add_scaled_rows(da, n, dr, dsc, ns, s); });
 }
 
@@ -1114,7 +1170,9 @@ void it_hip_add_scaled_sigmoid(it_hip* be, float* acc, uint64_t acc_len, const f
     float* dl = be->act_in(logit, logit_len);
     if (!da || !db || !dl) return;
     int64_t n = (int64_t)acc_len;
-    be->submit(it_hip::FAM_OTHER, acc_len * 12, sig_of(OP_SIGADD, da, db, n, dl),
+    it_hip::OpRec rec;
+    rec.id = OP_SIGADD;
+    be->submit(it_hip::FAM_OTHER, acc_len * 12, sig_of(OP_SIGADD, da, db, n, dl), rec,
                [=](hipStream_t s) { add_scaled_sigmoid(da, db, n, dl, s); });
 }
 
@@ -1137,7 +1195,9 @@ void it_hip_kv_write(it_hip* be, uint16_t* slab, uint64_t slab_len, uint64_t off
     } else {
         be->need_eager("a kv_write offset is not a whole row");
     }
-    be->submit(it_hip::FAM_OTHER, src_len * 6, sig_of(OP_KVWRITE, dslab, dyn, mul, dyn ? (int64_t)0 : (int64_t)0, ds, n),
+    it_hip::OpRec rec;
+    rec.id = OP_KVWRITE; rec.p[0] = dslab; rec.p[1] = dyn; rec.p[2] = ds; rec.i[0] = mul; rec.i[1] = off; rec.i[2] = n;
+    be->submit(it_hip::FAM_OTHER, src_len * 6, sig_of(OP_KVWRITE, dslab, dyn, mul, ds, n), rec,
                [=](hipStream_t s) { kv_write(dslab, off, dyn, mul, ds, n, s); });
 }
 
@@ -1182,10 +1242,7 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
         if (be->graph.valid) {
             be->mode = it_hip::Mode::Replay;
         } else if (be->stable_passes >= 1) {
-            if (hipStreamBeginCapture(be->stream, hipStreamCaptureModeRelaxed) == hipSuccess)
-                be->mode = it_hip::Mode::Capture;
-            else
-                (void)hipGetLastError();
+            be->mode = it_hip::Mode::Capture;
         }
     }
     for (auto& kv : be->acts) {
@@ -1358,10 +1415,11 @@ void it_hip_release(it_hip* be, const void* host) {
     }
 }
 
-void it_hip_graph_stats(it_hip* be, uint64_t out[3]) {
+void it_hip_graph_stats(it_hip* be, uint64_t out[4]) {
     out[0] = be->graph_captures;
     out[1] = be->graph_launches;
     out[2] = be->graph_aborts;
+    out[3] = be->fused_launches;
 }
 
 void it_hip_profile_begin(it_hip* be) {

@@ -18,6 +18,32 @@
 
 #include "../../include/inferred_hip.h"
 #include "kernels.h"
+#include "kernels_fused.h"
+
+// Seam ops as recorded for the fuser.  Pointer/int slots per op:
+//   RMS        p: x, w, out                 i: rows, nd                       f: eps
+//   RMS_HEADS  p: x, w                      i: head_dim, heads                f: eps
+//   L2         p: x                         i: head_dim, heads                f: eps
+//   QUANT      p: x, scales, quants         i: len
+//   MATMUL     p: wq, ws, x, act_scales, act_quants, out   i: fmt, n_in, n_out, n_tok
+//   CONV       p: state, x, w, out          i: kernel, channels, n_tok
+//   GATHER     p: src, out                  i: chunk, stride, offset, out_len
+//   DELTA      p: q, k, v, alpha, beta, ssm_a, dt_bias, state, out   i: n_tok, dk, dv, n_k, n_v
+//   EW         p: a, b                      i: op (0 silu_mul, 1 sigmoid_mul, 2 add_assign, 3 add_scaled), n
+//   SOFTMAX    p: x                         i: rows, row
+//   ROUTE      p: probs, ids, weights       i: n_tok, n_expert, n_used
+//   GLU        p: gq, gs, uq, us, gscale2, uscale2, ids, act_scales, act_quants, out
+//              i: fmt, n_in, n_out, picks, n_used, x_mode, q_stride, s_stride
+//   EXPERTS    p: q, s, scale2, ids, act_scales, act_quants, out     i: as GLU
+//   FINISH     p: out, rows, weights, shared, logit   i: at, n, n_tok, n_used, logit_at
+//   ROPE       p: x, table, dyn             i: half, n_tok, head_dim, n_rot, n_heads, pos
+//   KVWRITE    p: slab, dyn, src            i: mul, offset, n
+//   ATTEND     p: q, k, v, dyn, scratch, out   i: n_q, kv_dim, head_dim, n_head, n_head_kv, n_split, exact, n_pos  f: scale
+enum OpId : int {
+    OP_RMS = 1, OP_RMS_HEADS, OP_L2, OP_MATMUL, OP_ROPE, OP_SOFTMAX, OP_ATTEND, OP_EW, OP_SCALE, OP_CONV, OP_GATHER,
+    OP_SCATTER, OP_DELTA, OP_ROUTE, OP_EXPERTS, OP_GLU, OP_FINISH, OP_ROWS, OP_SIGADD, OP_KVWRITE,
+    OP_QUANT = 101
+};
 
 struct it_hip {
     // ---- configuration
@@ -127,7 +153,19 @@ struct it_hip {
     size_t replay_cursor = 0;
     uint64_t graph_launches = 0, graph_captures = 0, graph_aborts = 0;
     // work of the pass being captured or replayed, kept so it can run eagerly if the graph path breaks
-    std::vector<std::function<void(hipStream_t)>> pending;
+    // One seam op as the fuser sees it: an id, its device pointers and integer
+    // arguments (meaning per op, see the OpId table in backend.cpp), and the launch.
+    struct OpRec {
+        int id = 0;
+        const void* p[12] = {};
+        int64_t i[10] = {};
+        float f[2] = {};
+        std::function<void(hipStream_t)> run;
+    };
+    std::vector<OpRec> pending;
+    bool fuse_enabled = true;
+    uint64_t fused_launches = 0;  // launches in the captured graph after fusion
+    void run_fused(std::vector<OpRec>& ops);
     struct PreCopy {
         void* dev;
         const void* host;
@@ -154,7 +192,7 @@ struct it_hip {
     // Every kernel launch goes through here.  `sig` hashes the launch's static arguments
     // (pointers, shapes); position-dependent scalars never enter it.
     template <class F>
-    void submit(int fam, uint64_t bytes, uint64_t sig, F&& f) {
+    void submit(int fam, uint64_t bytes, uint64_t sig, OpRec rec, F&& f) {
         launches++;
         if (mode == Mode::Eager) {
             if (in_pass && pass_tokens == 1) pass_signature.push_back(sig);
@@ -163,11 +201,11 @@ struct it_hip {
             check(hipGetLastError(), "kernel launch");
             return;
         }
-        pending.emplace_back(f);
+        rec.run = f;
+        pending.push_back(std::move(rec));
         pass_signature.push_back(sig);
         if (mode == Mode::Capture) {
-            f(stream);
-            if (hipGetLastError() != hipSuccess) need_eager("a launch failed during capture");
+            // queued: the whole pass is fused and captured at end_pass
         } else if (replay_cursor >= graph.signature.size() || graph.signature[replay_cursor] != sig) {
             need_eager("the op sequence changed");
         } else {

@@ -1,0 +1,467 @@
+// Rewrites the seam ops of one single-token pass into fused launches.
+//
+// The op sequence a qwen35moe forward issues per layer is fixed
+// (/root/reference src/model/qwen35.rs:1006-1093, 1138-1328, 1587-1700), so each block
+// is matched as a whole: op ids in order plus the pointer links between them
+// (an op's output must be the next one's input).  A block that does not match
+// exactly — a different model, a traced pass, an NVFP4 shared expert with second
+// scales — is simply issued op by op.  A fused launch sits at the position of its
+// block's first op; everything it replaces is dropped, except an activation
+// quantization that some unfused op still reads.
+#include "backend.h"
+
+using namespace itk;
+using Op = it_hip::OpRec;
+
+namespace {
+
+struct Plan {
+    std::vector<Op>& ops;
+    std::vector<char> consumed;
+    std::vector<std::vector<std::function<void(hipStream_t)>>> at;  // fused launches keyed by position
+    explicit Plan(std::vector<Op>& o) : ops(o), consumed(o.size(), 0), at(o.size()) {}
+    bool ids(size_t i, std::initializer_list<int> want) const {
+        if (i + want.size() > ops.size()) return false;
+        size_t k = i;
+        for (int w : want)
+            if (ops[k++].id != w) return false;
+        return true;
+    }
+    void take(size_t i, size_t n) {
+        for (size_t k = i; k < i + n; k++) consumed[k] = 1;
+    }
+};
+
+bool quantized_fmt(int64_t f) { return f == W_Q8_0 || f == W_NVFP4; }
+
+// MATMUL `m` reads activation `x` (f32) whose Q8_0 form was produced by QUANT `q`, one token.
+bool mm_reads(const Op& m, const void* x, const Op& q) {
+    return m.id == OP_MATMUL && m.p[2] == x && m.p[3] == q.p[1] && m.p[4] == q.p[2] && m.i[3] == 1 &&
+           quantized_fmt(m.i[0]) && m.i[1] == q.i[0];
+}
+
+FusedMat mat_of(const Op& m, int epi, float* out_override = nullptr) {
+    FusedMat f{};
+    f.q = (const uint8_t*)m.p[0];
+    f.s = (const uint8_t*)m.p[1];
+    f.out = out_override ? out_override : (float*)m.p[5];
+    f.n_out = (int)m.i[2];
+    f.fmt = (int)m.i[0];
+    f.epi = epi;
+    return f;
+}
+
+// GDN mixer: 18 ops -> fused_gemv (norm + qkv/z/alpha/beta + conv) + gdn_core + fused_gemv (ssm_out += x)
+bool match_gdn(Plan& pl, size_t i, int exact) {
+    if (!pl.ids(i, {OP_RMS, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_MATMUL, OP_MATMUL, OP_CONV, OP_GATHER, OP_GATHER,
+                    OP_GATHER, OP_L2, OP_L2, OP_DELTA, OP_RMS_HEADS, OP_EW, OP_QUANT, OP_MATMUL, OP_EW}))
+        return false;
+    auto& o = pl.ops;
+    const Op &rms = o[i], &q1 = o[i + 1], &mqkv = o[i + 2], &mz = o[i + 3], &ma = o[i + 4], &mb = o[i + 5];
+    const Op &conv = o[i + 6], &g0 = o[i + 7], &g1 = o[i + 8], &g2 = o[i + 9], &l0 = o[i + 10], &l1 = o[i + 11];
+    const Op &dl = o[i + 12], &rh = o[i + 13], &sm = o[i + 14], &q2 = o[i + 15], &mo = o[i + 16], &add = o[i + 17];
+    const void* normed = rms.p[2];
+    if (rms.i[0] != 1 || q1.p[0] != normed || q1.i[0] != rms.i[1]) return false;
+    if (!mm_reads(mqkv, normed, q1) || !mm_reads(mz, normed, q1) || !mm_reads(ma, normed, q1) ||
+        !mm_reads(mb, normed, q1))
+        return false;
+    int64_t dk = dl.i[1], dv = dl.i[2], nk = dl.i[3], nv = dl.i[4];
+    int64_t kdim = nk * dk, vdim = nv * dv, cdim = 2 * kdim + vdim;
+    if (dl.i[0] != 1 || dk != dv || (dk != 64 && dk != 128)) return false;
+    if (conv.i[0] != 4 || conv.i[2] != 1 || conv.i[1] != cdim || conv.p[1] != mqkv.p[5] || mqkv.i[2] != cdim) return false;
+    const void* cv = conv.p[3];
+    auto gather_is = [&](const Op& g, int64_t chunk, int64_t off) {
+        return g.p[0] == cv && g.i[0] == chunk && g.i[1] == cdim && g.i[2] == off && g.i[3] == chunk;
+    };
+    if (!gather_is(g0, kdim, 0) || !gather_is(g1, kdim, kdim) || !gather_is(g2, vdim, 2 * kdim)) return false;
+    if (l0.p[0] != g0.p[1] || l1.p[0] != g1.p[1] || l0.i[0] != dk || l1.i[0] != dk || l0.f[0] != l1.f[0]) return false;
+    if (dl.p[0] != g0.p[1] || dl.p[1] != g1.p[1] || dl.p[2] != g2.p[1] || dl.p[3] != ma.p[5] || dl.p[4] != mb.p[5])
+        return false;
+    if (ma.i[2] != nv || mb.i[2] != nv || mz.i[2] != vdim) return false;
+    if (rh.p[0] != dl.p[8] || rh.i[0] != dv || rh.i[1] != nv) return false;
+    if (sm.i[0] != 0 || sm.p[0] != mz.p[5] || sm.p[1] != dl.p[8] || sm.i[1] != vdim) return false;
+    const void* z = mz.p[5];
+    if (q2.p[0] != z || q2.i[0] != vdim || !mm_reads(mo, z, q2)) return false;
+    if (add.i[0] != 2 || add.p[1] != mo.p[5] || add.p[0] != rms.p[0] || add.i[1] != mo.i[2]) return false;
+
+    FusedGemvP a{};
+    a.x = (const float*)rms.p[0];
+    a.norm_w = (const float*)rms.p[1];
+    a.x_copy = (float*)normed;
+    a.eps = rms.f[0];
+    a.n_in = (int)rms.i[1];
+    a.mode = 1;
+    a.exact = exact;
+    a.n_mats = 4;
+    a.m[0] = mat_of(mqkv, 1, (float*)cv);
+    a.m[1] = mat_of(mz, 0);
+    a.m[2] = mat_of(ma, 0);
+    a.m[3] = mat_of(mb, 0);
+    a.conv_state = (float*)conv.p[0];
+    a.conv_w = (const float*)conv.p[2];
+
+    GdnCoreP c{};
+    c.conv = (const float*)cv;
+    c.alpha = (const float*)dl.p[3];
+    c.beta = (const float*)dl.p[4];
+    c.ssm_a = (const float*)dl.p[5];
+    c.dt_bias = (const float*)dl.p[6];
+    c.state = (float*)dl.p[7];
+    c.core = (float*)dl.p[8];
+    c.n_k_heads = (int)nk;
+    c.n_v_heads = (int)nv;
+    c.exact = exact;
+    c.eps = l0.f[0];
+    c.q_scale = 1.0f / sqrtf((float)dk);
+    int dki = (int)dk;
+    if (nv > 64) return false;
+
+    // ssm_out reads silu(z) * rms_norm_heads(core): formed in the GEMV's prologue
+    FusedGemvP b{};
+    b.x = (const float*)dl.p[8];
+    b.norm_w = (const float*)rh.p[1];
+    b.gate = (const float*)z;
+    b.eps = rh.f[0];
+    b.n_in = (int)vdim;
+    b.mode = 2;
+    b.head_dim = (int)dv;
+    b.exact = exact;
+    b.n_mats = 1;
+    b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
+
+    pl.take(i, 18);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    pl.at[i].push_back([=](hipStream_t s) { gdn_core(c, dki, s); });
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    return true;
+}
+
+// rms_norm [+ whole-row gather copy] + quantize + 1..4 matmuls on the same activation
+bool match_norm_matmuls(Plan& pl, size_t i, int exact) {
+    auto& o = pl.ops;
+    if (i + 2 >= o.size() || o[i].id != OP_RMS || o[i].i[0] != 1) return false;
+    size_t k = i + 1;
+    const void* act = o[i].p[2];
+    float* copy2 = nullptr;
+    if (o[k].id == OP_GATHER && o[k].p[0] == act && o[k].i[0] == o[i].i[1] && o[k].i[2] == 0 &&
+        o[k].i[3] == o[i].i[1]) {
+        copy2 = (float*)o[k].p[1];
+        act = o[k].p[1];
+        k++;
+    }
+    if (k >= o.size() || o[k].id != OP_QUANT || o[k].p[0] != act || o[k].i[0] != o[i].i[1]) return false;
+    const Op& q = o[k];
+    size_t m0 = k + 1, n = 0;
+    while (n < 4 && m0 + n < o.size() && mm_reads(o[m0 + n], act, q)) n++;
+    if (n == 0) return false;
+    FusedGemvP a{};
+    a.x = (const float*)o[i].p[0];
+    a.norm_w = (const float*)o[i].p[1];
+    a.x_copy = (float*)o[i].p[2];
+    a.x_copy2 = copy2;
+    a.eps = o[i].f[0];
+    a.n_in = (int)o[i].i[1];
+    a.mode = 1;
+    a.exact = exact;
+    a.n_mats = (int)n;
+    for (size_t j = 0; j < n; j++) a.m[j] = mat_of(o[m0 + j], 0);
+    pl.take(i, m0 + n - i);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    return true;
+}
+
+// quantize + matmul + add_assign of the result into another buffer
+bool match_matmul_residual(Plan& pl, size_t i, int exact) {
+    auto& o = pl.ops;
+    if (!pl.ids(i, {OP_QUANT, OP_MATMUL, OP_EW})) return false;
+    const Op &q = o[i], &m = o[i + 1], &add = o[i + 2];
+    if (!mm_reads(m, q.p[0], q) || add.i[0] != 2 || add.p[1] != m.p[5] || add.i[1] != m.i[2] || add.p[0] == q.p[0])
+        return false;
+    FusedGemvP b{};
+    b.x = (const float*)q.p[0];
+    b.n_in = (int)q.i[0];
+    b.exact = exact;
+    b.n_mats = 1;
+    b.m[0] = mat_of(m, 2, (float*)add.p[0]);
+    pl.take(i, 3);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    return true;
+}
+
+// last-row gather + final norm + LM head
+bool match_final(Plan& pl, size_t i, int exact) {
+    auto& o = pl.ops;
+    if (!pl.ids(i, {OP_GATHER, OP_RMS, OP_QUANT, OP_MATMUL})) return false;
+    const Op &g = o[i], &rms = o[i + 1], &q = o[i + 2], &m = o[i + 3];
+    if (g.i[3] != g.i[0] || rms.p[0] != g.p[1] || rms.i[0] != 1 || rms.i[1] != g.i[0]) return false;
+    if (q.p[0] != rms.p[2] || q.i[0] != rms.i[1] || !mm_reads(m, rms.p[2], q)) return false;
+    FusedGemvP a{};
+    a.x = (const float*)g.p[0] + g.i[2];
+    a.norm_w = (const float*)rms.p[1];
+    a.x_copy = (float*)rms.p[2];
+    a.eps = rms.f[0];
+    a.n_in = (int)rms.i[1];
+    a.mode = 1;
+    a.exact = exact;
+    a.n_mats = 1;
+    a.m[0] = mat_of(m, 0);
+    pl.take(i, 4);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    return true;
+}
+
+
+// attention mixer: 18 ops -> fused_gemv (norm + wq/wk/wv) + attn_prep + split-K attend with the
+// gate folded into its merge + fused_gemv (wo += x)
+bool match_attn(Plan& pl, size_t i, int exact) {
+    if (!pl.ids(i, {OP_RMS, OP_QUANT, OP_MATMUL, OP_GATHER, OP_GATHER, OP_MATMUL, OP_MATMUL, OP_RMS_HEADS, OP_RMS_HEADS,
+                    OP_ROPE, OP_ROPE, OP_KVWRITE, OP_KVWRITE, OP_ATTEND, OP_EW, OP_QUANT, OP_MATMUL, OP_EW}))
+        return false;
+    auto& o = pl.ops;
+    const Op &rms = o[i], &q1 = o[i + 1], &mq = o[i + 2], &gq = o[i + 3], &gg = o[i + 4], &mk = o[i + 5], &mv = o[i + 6];
+    const Op &nq = o[i + 7], &nk = o[i + 8], &rq = o[i + 9], &rk = o[i + 10], &wk = o[i + 11], &wv = o[i + 12];
+    const Op &at = o[i + 13], &sg = o[i + 14], &q2 = o[i + 15], &mo = o[i + 16], &add = o[i + 17];
+    const void* normed = rms.p[2];
+    if (rms.i[0] != 1 || q1.p[0] != normed || q1.i[0] != rms.i[1]) return false;
+    if (!mm_reads(mq, normed, q1) || !mm_reads(mk, normed, q1) || !mm_reads(mv, normed, q1)) return false;
+    if (at.i[0] != 1 || !at.p[3]) return false;  // one query row, graphed position
+    int64_t hd = at.i[2], nh = at.i[3], nkv = at.i[4], kvd = at.i[1];
+    const void* qg = mq.p[5];
+    if (mq.i[2] != 2 * hd * nh || mk.i[2] != nkv * hd || mv.i[2] != nkv * hd || kvd != nkv * hd) return false;
+    auto gather_is = [&](const Op& g, int64_t off) {
+        return g.p[0] == qg && g.i[0] == hd && g.i[1] == 2 * hd && g.i[2] == off && g.i[3] == hd * nh;
+    };
+    if (!gather_is(gq, 0) || !gather_is(gg, hd)) return false;
+    const void *qb = gq.p[1], *gb = gg.p[1], *kb = mk.p[5], *vb = mv.p[5];
+    if (nq.p[0] != qb || nq.i[0] != hd || nq.i[1] != nh || nk.p[0] != kb || nk.i[0] != hd || nk.i[1] != nkv ||
+        nq.f[0] != nk.f[0])
+        return false;
+    if (rq.p[0] != qb || rk.p[0] != kb || rq.p[1] != rk.p[1] || !rq.p[2] || !rk.p[2] || rq.i[1] != 1 || rk.i[1] != 1 ||
+        rq.i[2] != hd || rk.i[2] != hd || rq.i[3] != rk.i[3] || rq.i[4] != nh || rk.i[4] != nkv)
+        return false;
+    if (wk.p[2] != kb || wv.p[2] != vb || !wk.p[1] || !wv.p[1] || wk.i[0] != kvd || wv.i[0] != kvd || wk.i[2] != kvd ||
+        wv.i[2] != kvd || wk.p[0] != at.p[1] || wv.p[0] != at.p[2])
+        return false;
+    if (at.p[0] != qb) return false;
+    const void* attn = at.p[5];
+    if (sg.i[0] != 1 || sg.p[0] != attn || sg.p[1] != gb || sg.i[1] != hd * nh) return false;
+    if (q2.p[0] != attn || q2.i[0] != hd * nh || !mm_reads(mo, attn, q2)) return false;
+    if (add.i[0] != 2 || add.p[1] != mo.p[5] || add.p[0] != rms.p[0] || add.i[1] != mo.i[2]) return false;
+
+    FusedGemvP a{};
+    a.x = (const float*)rms.p[0];
+    a.norm_w = (const float*)rms.p[1];
+    a.x_copy = (float*)normed;
+    a.eps = rms.f[0];
+    a.n_in = (int)rms.i[1];
+    a.mode = 1;
+    a.exact = exact;
+    a.n_mats = 3;
+    a.m[0] = mat_of(mq, 0);
+    a.m[1] = mat_of(mk, 0);
+    a.m[2] = mat_of(mv, 0);
+
+    AttnPrepP pp{};
+    pp.qg = (const float*)qg;
+    pp.k = (const float*)kb;
+    pp.v = (const float*)vb;
+    pp.q_norm = (const float*)nq.p[1];
+    pp.k_norm = (const float*)nk.p[1];
+    pp.rope = (const float2*)rq.p[1];
+    pp.pos_dyn = (const int*)rq.p[2];
+    pp.q = (float*)qb;
+    pp.k_slab = (uint16_t*)wk.p[0];
+    pp.v_slab = (uint16_t*)wv.p[0];
+    pp.n_head = (int)nh;
+    pp.n_head_kv = (int)nkv;
+    pp.head_dim = (int)hd;
+    pp.n_rot = (int)rq.i[3];
+    pp.kv_dim = (int)kvd;
+    pp.exact = exact;
+    pp.eps = nq.f[0];
+
+    AttnArgs aa{(const float*)qb, (const uint16_t*)at.p[1], (const uint16_t*)at.p[2], 1, (int)kvd, 0, (int)hd, (int)nh,
+                (int)nkv, at.f[0], (const int*)at.p[3]};
+    int n_split = (int)at.i[5];
+    float* scratch = (float*)at.p[4];
+    float* attn_out = (float*)attn;
+    const float* gate = (const float*)qg + hd;
+    int gate_stride = (int)(2 * hd);
+
+    FusedGemvP b{};
+    b.x = (const float*)attn;
+    b.n_in = (int)(hd * nh);
+    b.exact = exact;
+    b.n_mats = 1;
+    b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
+
+    pl.take(i, 18);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    pl.at[i].push_back([=](hipStream_t s) { attn_prep(pp, s); });
+    if (at.i[6] == 0) {
+        pl.at[i].push_back([=](hipStream_t s) { attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s); });
+    } else {
+        // the exact attention kernel and its gate stay as they are
+        auto run_attend = at.run, run_gate = sg.run, run_gather_gate = gg.run;
+        pl.at[i].push_back(run_gather_gate);
+        pl.at[i].push_back(run_attend);
+        pl.at[i].push_back(run_gate);
+    }
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    return true;
+}
+
+// routed FFN: 17 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
+bool match_ffn(Plan& pl, size_t i, int exact) {
+    if (!pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT, OP_EXPERTS,
+                    OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW}))
+        return false;
+    auto& o = pl.ops;
+    const Op &rms = o[i], &ga = o[i + 1], &q1 = o[i + 2], &mr = o[i + 3], &ml = o[i + 4], &sm = o[i + 5], &rt = o[i + 6];
+    const Op &glu = o[i + 7], &q2 = o[i + 8], &ex = o[i + 9], &sgm = o[i + 10], &sum_ = o[i + 11], &sil = o[i + 12];
+    const Op &q3 = o[i + 13], &sdm = o[i + 14], &fin = o[i + 15], &add = o[i + 16];
+    int64_t nd = rms.i[1];
+    if (rms.i[0] != 1) return false;
+    if (ga.p[0] != rms.p[2] || ga.i[0] != nd || ga.i[2] != 0 || ga.i[3] != nd) return false;
+    const void* x = ga.p[1];
+    if (q1.p[0] != x || q1.i[0] != nd || !mm_reads(mr, x, q1) || !mm_reads(ml, x, q1) || ml.i[2] != 1) return false;
+    int64_t ne = mr.i[2];
+    const void* router = mr.p[5];
+    if (sm.p[0] != router || sm.i[0] != 1 || sm.i[1] != ne) return false;
+    if (rt.p[0] != router || rt.i[0] != 1 || rt.i[1] != ne) return false;
+    int64_t nu = rt.i[2];
+    if (nu > 63 || ne > 4096) return false;
+    if (glu.p[6] != rt.p[1] || glu.p[7] != q1.p[1] || glu.p[8] != q1.p[2] || glu.i[1] != nd || glu.i[3] != nu ||
+        glu.i[4] != nu || !quantized_fmt(glu.i[0]))
+        return false;
+    int64_t ff = glu.i[2];
+    const void* g_all = glu.p[9];
+    if (q2.p[0] != g_all || q2.i[0] != nu * ff) return false;
+    if (ex.p[3] != rt.p[1] || ex.p[4] != q2.p[1] || ex.p[5] != q2.p[2] || ex.i[1] != ff || ex.i[2] != nd ||
+        ex.i[3] != nu || ex.i[5] != 0 || !quantized_fmt(ex.i[0]))
+        return false;
+    if (!mm_reads(sgm, x, q1) || !mm_reads(sum_, x, q1) || sgm.i[2] != sum_.i[2] || sgm.i[0] != sum_.i[0]) return false;
+    int64_t sff = sgm.i[2];
+    const void* e_gate = sgm.p[5];
+    if (sil.i[0] != 0 || sil.p[0] != e_gate || sil.p[1] != sum_.p[5] || sil.i[1] != sff) return false;
+    if (q3.p[0] != e_gate || q3.i[0] != sff || !mm_reads(sdm, e_gate, q3) || sdm.i[2] != nd) return false;
+    if (fin.p[1] != ex.p[6] || fin.p[2] != rt.p[2] || fin.p[3] != sdm.p[5] || fin.p[4] != ml.p[5] || fin.i[0] != 0 ||
+        fin.i[1] != nd || fin.i[2] != 1 || fin.i[3] != nu || fin.i[4] != 0)
+        return false;
+    if (add.i[0] != 2 || add.p[1] != fin.p[0] || add.p[0] != rms.p[0] || add.i[1] != nd) return false;
+
+    FusedGemvP a{};
+    a.x = (const float*)rms.p[0];
+    a.norm_w = (const float*)rms.p[1];
+    a.x_copy = (float*)rms.p[2];
+    a.x_copy2 = (float*)x;
+    a.eps = rms.f[0];
+    a.n_in = (int)nd;
+    a.mode = 1;
+    a.exact = exact;
+    a.n_mats = 2;
+    a.m[0] = mat_of(mr, 0);
+    a.m[1] = mat_of(ml, 0);
+
+    MoeGluP g{};
+    g.x = (const float*)x;
+    g.logits = (const float*)router;
+    g.gq = (const uint8_t*)glu.p[0];
+    g.gs = (const uint8_t*)glu.p[1];
+    g.uq = (const uint8_t*)glu.p[2];
+    g.us = (const uint8_t*)glu.p[3];
+    g.gscale2 = (const float*)glu.p[4];
+    g.uscale2 = (const float*)glu.p[5];
+    g.q_stride = glu.i[6];
+    g.s_stride = glu.i[7];
+    g.fmt = (int)glu.i[0];
+    g.n_in = (int)nd;
+    g.n_out = (int)ff;
+    g.n_expert = (int)ne;
+    g.n_used = (int)nu;
+    g.exact = exact;
+    g.sh_gq = (const uint8_t*)sgm.p[0];
+    g.sh_gs = (const uint8_t*)sgm.p[1];
+    g.sh_uq = (const uint8_t*)sum_.p[0];
+    g.sh_us = (const uint8_t*)sum_.p[1];
+    g.sh_fmt = (int)sgm.i[0];
+    g.sh_n_out = (int)sff;
+    g.out = (float*)g_all;
+    g.sh_out = (float*)e_gate;
+    g.route_ids = (int32_t*)rt.p[1];
+    g.route_w = (float*)rt.p[2];
+
+    MoeDownP d{};
+    d.g_all = (const float*)g_all;
+    d.g_shared = (const float*)e_gate;
+    d.q = (const uint8_t*)ex.p[0];
+    d.s = (const uint8_t*)ex.p[1];
+    d.scale2 = (const float*)ex.p[2];
+    d.q_stride = ex.i[6];
+    d.s_stride = ex.i[7];
+    d.fmt = (int)ex.i[0];
+    d.n_in = (int)ff;
+    d.n_out = (int)nd;
+    d.n_used = (int)nu;
+    d.sh_q = (const uint8_t*)sdm.p[0];
+    d.sh_s = (const uint8_t*)sdm.p[1];
+    d.sh_fmt = (int)sdm.i[0];
+    d.sh_n_in = (int)sff;
+    d.route_ids = (const int32_t*)rt.p[1];
+    d.route_w = (const float*)rt.p[2];
+    d.logit = (const float*)ml.p[5];
+    d.x = (float*)rms.p[0];
+
+    pl.take(i, 17);
+    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    pl.at[i].push_back([=](hipStream_t s) { moe_glu_fused(g, s); });
+    pl.at[i].push_back([=](hipStream_t s) { moe_down_fused(d, s); });
+    return true;
+}
+
+bool references(const Op& op, const void* a, const void* b) {
+    for (const void* p : op.p)
+        if (p && (p == a || p == b)) return true;
+    return false;
+}
+
+}  // namespace
+
+void it_hip::run_fused(std::vector<OpRec>& ops) {
+    Plan pl(ops);
+    if (fuse_enabled) {
+        for (size_t i = 0; i < ops.size(); i++) {
+            if (pl.consumed[i]) continue;
+            if (match_gdn(pl, i, exact)) continue;
+            if (match_attn(pl, i, exact)) continue;
+            if (match_ffn(pl, i, exact)) continue;
+            if (match_final(pl, i, exact)) continue;
+            if (match_norm_matmuls(pl, i, exact)) continue;
+            if (match_matmul_residual(pl, i, exact)) continue;
+        }
+        // a dropped quantization whose output an unfused op still reads is put back
+        for (size_t i = 0; i < ops.size(); i++) {
+            if (!pl.consumed[i] || ops[i].id != OP_QUANT) continue;
+            for (size_t k = i + 1; k < ops.size(); k++) {
+                if (pl.consumed[k]) continue;
+                if (ops[k].id == OP_QUANT && ops[k].p[1] == ops[i].p[1]) break;  // re-quantized later
+                if (references(ops[k], ops[i].p[1], ops[i].p[2])) {
+                    pl.consumed[i] = 0;
+                    break;
+                }
+            }
+        }
+    }
+    uint64_t n = 0;
+    for (size_t i = 0; i < ops.size(); i++) {
+        for (auto& f : pl.at[i]) {
+            f(stream);
+            n++;
+        }
+        if (!pl.consumed[i]) {
+            ops[i].run(stream);
+            n++;
+        }
+    }
+    fused_launches = n;
+}

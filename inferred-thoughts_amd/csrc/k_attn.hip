@@ -78,7 +78,6 @@ void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s) 
 
 // ------------------------------------------------------------------ split-K
 constexpr int CHUNK = 128;
-constexpr int MAXG = 8;  // query heads per kv head handled by one block
 
 int attend_split_count(int n_pos_max) { return (n_pos_max + CHUNK - 1) / CHUNK; }
 
@@ -186,7 +185,9 @@ __global__ __launch_bounds__(256) void attend_split_k(AttnArgs a, int n_split, f
     }
 }
 
-__global__ void attend_merge_k(const float* __restrict__ part, int n_split, int hd, float* __restrict__ out) {
+// gate (optional): out *= sigmoid(gate[head * gate_stride + i]) — the attention block's output gate
+__global__ void attend_merge_k(const float* __restrict__ part, int n_split, int hd, float* __restrict__ out,
+                               const float* __restrict__ gate, int gate_stride) {
     const float* p = part + (int64_t)blockIdx.x * n_split * (hd + 2);
     float m = -INFINITY;
     for (int s = 0; s < n_split; s++) m = fmaxf(m, p[(int64_t)s * (hd + 2) + hd]);
@@ -201,11 +202,18 @@ __global__ void attend_merge_k(const float* __restrict__ part, int n_split, int 
             float ms = p[(int64_t)s * (hd + 2) + hd];
             if (ms != -INFINITY) acc += p[(int64_t)s * (hd + 2) + i] * __expf(ms - m);
         }
-        out[(int64_t)blockIdx.x * hd + i] = acc / l;
+        float r = acc / l;
+        if (gate) r *= it_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + i]);
+        out[(int64_t)blockIdx.x * hd + i] = r;
     }
 }
 
 void attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hipStream_t s) {
+    attend_split_gated(a, n_split, scratch, out, nullptr, 0, s);
+}
+
+void attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* out, const float* gate,
+                        int gate_stride, hipStream_t s) {
     if (a.n_q <= 0) return;
     const int G = a.n_head / a.n_head_kv;
     dim3 grid(a.n_q * a.n_head_kv, n_split), block(256);
@@ -218,7 +226,7 @@ void attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hi
         default: return;  // the caller falls back to the exact kernel for other group sizes
     }
     hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(a.head_dim < 256 ? 64 : 256), 0, s, scratch,
-                       n_split, a.head_dim, out);
+                       n_split, a.head_dim, out, gate, gate_stride);
 }
 
 }  // namespace itk

@@ -1,0 +1,84 @@
+// Argument structs and launchers of the fused single-token kernels (k_fused.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace itk {
+
+struct FusedMat {
+    const uint8_t* q;
+    const uint8_t* s;
+    float* out;
+    int n_out, fmt;
+    int epi;     // 0 store, 1 causal conv (kernel 4) + silu, 2 accumulate into out
+    int group0;  // filled by the launcher
+};
+struct FusedGemvP {
+    const float* x;       // [n_in] f32
+    const float* norm_w;  // rms_norm weight (mode 1: [n_in]; mode 2: [head_dim])
+    const float* gate;    // mode 2: silu gate, [n_in]
+    float* x_copy;        // optional: the activation after the prologue, f32, written by block 0
+    float* x_copy2;       // optional second copy (a whole-row gather of it)
+    float eps;
+    int n_in, mode, head_dim, exact, n_mats, rows_per_wave, total_groups;
+    FusedMat m[4];
+    float* conv_state;    // epi 1
+    const float* conv_w;
+};
+void fused_gemv(FusedGemvP p, hipStream_t s);
+
+struct GdnCoreP {
+    const float* conv;  // [q | k | v] after conv + silu
+    const float *alpha, *beta, *ssm_a, *dt_bias;
+    float* state;       // [n_v_heads][dv][dk]
+    float* core;        // out: delta-rule read-out, [n_v_heads * dv]
+    int n_k_heads, n_v_heads, exact;
+    float eps, q_scale;
+};
+void gdn_core(const GdnCoreP& p, int dk, hipStream_t s);
+
+struct MoeGluP {
+    const float* x;        // normed activation, f32 [n_in]
+    const float* logits;   // router logits [n_expert] (before softmax)
+    const uint8_t *gq, *gs, *uq, *us;
+    const float *gscale2, *uscale2;
+    int64_t q_stride, s_stride;
+    int fmt, n_in, n_out, n_expert, n_used, exact, rows_per_wave;
+    const uint8_t *sh_gq, *sh_gs, *sh_uq, *sh_us;
+    int sh_fmt, sh_n_out;
+    float* out;            // [n_used][n_out]
+    float* sh_out;         // [sh_n_out]
+    int32_t* route_ids;    // [n_used] written for the down stage
+    float* route_w;
+};
+void moe_glu_fused(MoeGluP p, hipStream_t s);
+
+struct MoeDownP {
+    const float* g_all;     // [n_used][n_in]
+    const float* g_shared;  // [sh_n_in]
+    const uint8_t *q, *s;
+    const float* scale2;
+    int64_t q_stride, s_stride;
+    int fmt, n_in, n_out, n_used, rows_per_wave;
+    const uint8_t *sh_q, *sh_s;
+    int sh_fmt, sh_n_in;
+    const int32_t* route_ids;
+    const float* route_w;
+    const float* logit;     // shared expert gate logit
+    float* x;               // residual stream, accumulated into
+};
+void moe_down_fused(MoeDownP p, hipStream_t s);
+
+struct AttnPrepP {
+    const float *qg, *k, *v;     // wq output [n_head][2*head_dim], k and v projections
+    const float *q_norm, *k_norm;
+    const float2* rope;
+    const int* pos_dyn;
+    float* q;                     // out [n_head*head_dim]
+    uint16_t *k_slab, *v_slab;
+    int n_head, n_head_kv, head_dim, n_rot, kv_dim, exact;
+    float eps;
+};
+void attn_prep(const AttnPrepP& p, hipStream_t s);
+
+}  // namespace itk

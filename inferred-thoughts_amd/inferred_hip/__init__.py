@@ -14,7 +14,7 @@ from pathlib import Path
 import numpy as np
 
 F32, F16, Q8_0, BF16, NVFP4 = 0, 1, 8, 30, 40
-EXACT, NO_GRAPH = 1, 2
+EXACT, NO_GRAPH, NO_FUSE = 1, 2, 4
 
 _HERE = Path(__file__).resolve().parent
 LIB_PATH = _HERE / "libinferred_hip.so"
@@ -228,10 +228,10 @@ class HipError(RuntimeError):
 class Hip:
     """One backend instance: `Cuda::new` of the reference, for gfx950."""
 
-    def __init__(self, exact: bool = False, graph: bool = True, device: int = 0):
+    def __init__(self, exact: bool = False, graph: bool = True, device: int = 0, fuse: bool = True):
         self.L = lib()
         err = C.create_string_buffer(512)
-        flags = (EXACT if exact else 0) | (0 if graph else NO_GRAPH)
+        flags = (EXACT if exact else 0) | (0 if graph else NO_GRAPH) | (0 if fuse else NO_FUSE)
         self.h = self.L.it_hip_create(flags, device, err, 512)
         if not self.h:
             raise HipError(err.value.decode())
@@ -390,9 +390,9 @@ class Hip:
         return int(self.L.it_hip_launch_count(self.h))
 
     def graph_stats(self):
-        v = (c_u64 * 3)()
+        v = (c_u64 * 4)()
         self.L.it_hip_graph_stats(self.h, v)
-        return {"captures": int(v[0]), "replays": int(v[1]), "aborts": int(v[2])}
+        return {"captures": int(v[0]), "replays": int(v[1]), "aborts": int(v[2]), "graph_kernels": int(v[3])}
 
     def tier_counters(self) -> TierCounters:
         t = TierCounters()

@@ -77,3 +77,62 @@ def test_context_overflow_is_refused_before_any_write(hip, tiny_gguf):
         e.forward(prompt_ids(9))
     assert e.pos == 0
     e.close(); hm.close()
+
+
+def test_decode_graph_is_fused_and_replayed(hip, tiny_gguf):
+    """The greedy run above goes through the captured, fused decode graph: check that it really did."""
+    import inferred_hip as ih
+    hip.drop_mirrors()
+    hm = ih.Model(tiny_gguf); e = ih.Engine(hm, hip, 64)
+    before = hip.graph_stats()
+    ids, _ = e.generate(prompt_ids(8), 12)
+    after = hip.graph_stats()
+    assert after["captures"] > before["captures"] and after["replays"] >= before["replays"] + 6
+    assert after["aborts"] == before["aborts"]
+    l0 = hip.launch_count(); e.forward([int(ids[-1])]); per_token = hip.launch_count() - l0
+    assert after["graph_kernels"] * 3 < per_token, (after, per_token)   # ~35 seam ops per layer -> <= 8 kernels
+    e.close(); hm.close()
+
+
+@pytest.mark.parametrize("which", ["tiny_gguf", "tiny_nvfp4_gguf"])
+def test_unfused_and_ungraphed_paths_agree(request, which):
+    """Fusion and graph capture change the launches, never the arithmetic."""
+    import inferred_hip as ih
+    path = request.getfixturevalue(which)
+    prompt = prompt_ids(16, seed=5)
+    outs = []
+    for kw in (dict(graph=False), dict(graph=True, fuse=False), dict(graph=True, fuse=True)):
+        be = ih.Hip(exact=True, **kw)
+        hm = ih.Model(path); e = ih.Engine(hm, be, 64)
+        ids, logits = e.generate(prompt, 24)
+        assert be.take_error() is None
+        outs.append((ids, logits, e.ssm_state(2)))
+        e.close(); hm.close(); be.close()
+    for ids, logits, st in outs[1:]:
+        assert np.array_equal(ids, outs[0][0])
+        assert_bits_equal(logits, outs[0][1], "logits")
+        assert_bits_equal(st, outs[0][2], "ssm state")
+
+
+@pytest.mark.parametrize("which", ["tiny_gguf", "tiny_nvfp4_gguf"])
+def test_fast_mode_stays_within_tolerance(request, which):
+    """Tree sums, split-K attention and the lane-split delta rule: activations within 1e-3 of the oracle."""
+    import inferred_hip as ih
+    from oracle import binding as ob
+    path = request.getfixturevalue(which)
+    prompt = prompt_ids(48, seed=7)
+    om = ob.Model(path); oe = ob.Engine(om, 128)
+    lo = oe.forward(prompt)
+    be = ih.Hip(exact=False)
+    hm = ih.Model(path); he = ih.Engine(hm, be, 128)
+    lh = he.forward(prompt)
+    nxt = [int(np.argmax(lo))]
+    for _ in range(8):                      # decode steps: eager, then captured, then replayed
+        lo = oe.forward(nxt); lh = he.forward(nxt)
+        tol = 1e-3 * max(1.0, float(np.abs(lo).max()))
+        assert np.abs(lh - lo).max() <= tol, np.abs(lh - lo).max()
+        nxt = [int(np.argmax(lo))]
+    s_h, s_o = he.ssm_state(0), oe.ssm_state(0)
+    assert np.abs(s_h - s_o).max() <= 1e-3 * max(1.0, float(np.abs(s_o).max()))
+    assert be.take_error() is None
+    he.close(); hm.close(); be.close(); oe.close(); om.close()
