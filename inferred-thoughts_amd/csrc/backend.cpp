@@ -592,6 +592,7 @@ it_hip::~it_hip() {
     if (argmax_host) (void)hipHostFree(argmax_host);
     for (auto e : prof_pool) (void)hipEventDestroy(e);
     if (dyn_dev) (void)hipFree(dyn_dev);
+    if (route_counter) (void)hipFree(route_counter);
     for (int i = 0; i < 2; i++) {
         if (dyn_hosts[i]) (void)hipHostFree(dyn_hosts[i]);
         if (dyn_evt[i]) (void)hipEventDestroy(dyn_evt[i]);
@@ -636,6 +637,11 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
         return bad("cannot allocate the position staging buffers");
     }
     be->dyn_host = be->dyn_hosts[0];
+    if (hipMalloc((void**)&be->route_counter, sizeof(unsigned)) != hipSuccess ||
+        hipMemset(be->route_counter, 0, sizeof(unsigned)) != hipSuccess) {
+        delete be;
+        return bad("cannot allocate the router counter");
+    }
     return be;
 }
 

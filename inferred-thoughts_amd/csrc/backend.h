@@ -164,6 +164,7 @@ struct it_hip {
     };
     std::vector<OpRec> pending;
     bool fuse_enabled = true;
+    unsigned* route_counter = nullptr;  // device word used by the fused router (zero between launches)
     uint64_t fused_launches = 0;  // launches in the captured graph after fusion
     void run_fused(std::vector<OpRec>& ops);
     struct PreCopy {

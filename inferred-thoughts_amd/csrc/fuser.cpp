@@ -312,7 +312,7 @@ bool match_attn(Plan& pl, size_t i, int exact) {
 }
 
 // routed FFN: 17 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
-bool match_ffn(Plan& pl, size_t i, int exact) {
+bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     if (!pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT, OP_EXPERTS,
                     OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW}))
         return false;
@@ -330,7 +330,7 @@ bool match_ffn(Plan& pl, size_t i, int exact) {
     if (sm.p[0] != router || sm.i[0] != 1 || sm.i[1] != ne) return false;
     if (rt.p[0] != router || rt.i[0] != 1 || rt.i[1] != ne) return false;
     int64_t nu = rt.i[2];
-    if (nu > 63 || ne > 4096) return false;
+    if (nu > 16 || ne > nd || !counter) return false;
     if (glu.p[6] != rt.p[1] || glu.p[7] != q1.p[1] || glu.p[8] != q1.p[2] || glu.i[1] != nd || glu.i[3] != nu ||
         glu.i[4] != nu || !quantized_fmt(glu.i[0]))
         return false;
@@ -362,10 +362,14 @@ bool match_ffn(Plan& pl, size_t i, int exact) {
     a.n_mats = 2;
     a.m[0] = mat_of(mr, 0);
     a.m[1] = mat_of(ml, 0);
+    a.route_counter = counter;
+    a.n_expert = (int)ne;
+    a.n_used = (int)nu;
+    a.route_ids = (int32_t*)rt.p[1];
+    a.route_w = (float*)rt.p[2];
 
     MoeGluP g{};
     g.x = (const float*)x;
-    g.logits = (const float*)router;
     g.gq = (const uint8_t*)glu.p[0];
     g.gs = (const uint8_t*)glu.p[1];
     g.uq = (const uint8_t*)glu.p[2];
@@ -388,8 +392,7 @@ bool match_ffn(Plan& pl, size_t i, int exact) {
     g.sh_n_out = (int)sff;
     g.out = (float*)g_all;
     g.sh_out = (float*)e_gate;
-    g.route_ids = (int32_t*)rt.p[1];
-    g.route_w = (float*)rt.p[2];
+    g.route_ids = (const int32_t*)rt.p[1];
 
     MoeDownP d{};
     d.g_all = (const float*)g_all;
@@ -434,7 +437,7 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
             if (pl.consumed[i]) continue;
             if (match_gdn(pl, i, exact)) continue;
             if (match_attn(pl, i, exact)) continue;
-            if (match_ffn(pl, i, exact)) continue;
+            if (match_ffn(pl, i, exact, route_counter)) continue;
             if (match_final(pl, i, exact)) continue;
             if (match_norm_matmuls(pl, i, exact)) continue;
             if (match_matmul_residual(pl, i, exact)) continue;

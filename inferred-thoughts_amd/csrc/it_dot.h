@@ -46,4 +46,21 @@ IT_DEV void unit_nvfp4(const uint4 w, uint32_t sc2, const uint4 a0, const uint4 
     *tB = (dy * dB) * (float)sb;
 }
 
+// Serial ascending fold of T per-block terms from a 16-byte aligned LDS row: the loads are
+// issued four float4 at a time so the chain of adds never waits on LDS latency.
+IT_DEV float fold_terms(const float* tr, int T) {
+    float acc = 0.0f;
+    int k = 0;
+    const float4* t4 = (const float4*)tr;
+    for (; k + 16 <= T; k += 16) {
+        float4 a = t4[k / 4], b = t4[k / 4 + 1], c = t4[k / 4 + 2], d = t4[k / 4 + 3];
+        acc += a.x; acc += a.y; acc += a.z; acc += a.w;
+        acc += b.x; acc += b.y; acc += b.z; acc += b.w;
+        acc += c.x; acc += c.y; acc += c.z; acc += c.w;
+        acc += d.x; acc += d.y; acc += d.z; acc += d.w;
+    }
+    for (; k < T; k++) acc += tr[k];
+    return acc;
+}
+
 }  // namespace itk

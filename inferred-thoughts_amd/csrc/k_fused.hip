@@ -57,28 +57,55 @@ IT_DEV void wave_lds_sync() {
 }
 
 // Terms of `nrows` rows starting at `row0` of one matrix against the LDS activation.
-template <int FMT>
-__device__ void wave_row_terms(const uint8_t* wq, const uint8_t* ws, int n_in, int row0, int nrows,
-                               const int8_t* xq, const float* xs, float* terms, int tstride, int lane) {
+// Two phases so every HBM load of the group is in flight before the first dot: a lane
+// owns IPL (row, 32-element unit) items, loads them all, then computes.
+template <int IPL>
+struct RowRegs {
+    uint4 wa[IPL], wb[IPL];
+    uint32_t sc[IPL];
+};
+
+template <int FMT, int IPL>
+__device__ __forceinline__ void load_items(RowRegs<IPL>& rr, const uint8_t* wq, const uint8_t* ws, int n_in, int row0,
+                                           int nrows, int lane) {
     const int U = n_in >> 5;
     const int items = nrows * U;
-    for (int base = 0; base < items; base += 64) {
-        int it = base + lane;
+#pragma unroll
+    for (int k = 0; k < IPL; k++) {
+        int it = k * 64 + lane;
         if (it < items) {
             int r = it / U, u = it - r * U;
             int64_t row = row0 + r;
+            if (FMT == W_Q8_0) {
+                const uint4* wp = (const uint4*)(wq + row * n_in + u * 32);
+                rr.wa[k] = wp[0];
+                rr.wb[k] = wp[1];
+            } else {
+                rr.wa[k] = *(const uint4*)(wq + row * (n_in >> 1) + u * 16);
+            }
+            rr.sc[k] = ((const uint16_t*)ws)[row * U + u];
+        }
+    }
+}
+
+template <int FMT, int IPL>
+__device__ __forceinline__ void compute_items(const RowRegs<IPL>& rr, int n_in, int nrows, const int8_t* xq,
+                                              const float* xs, float* terms, int tstride, int lane) {
+    const int U = n_in >> 5;
+    const int items = nrows * U;
+#pragma unroll
+    for (int k = 0; k < IPL; k++) {
+        int it = k * 64 + lane;
+        if (it < items) {
+            int r = it / U, u = it - r * U;
             const uint4* ap = (const uint4*)(xq + u * 32);
             uint4 a0 = ap[0], a1 = ap[1];
             float dx = xs[u];
             if (FMT == W_Q8_0) {
-                const uint4* wp = (const uint4*)(wq + row * n_in + u * 32);
-                uint16_t dw = ((const uint16_t*)ws)[row * U + u];
-                terms[r * tstride + u] = unit_q8_0(wp[0], wp[1], dw, a0, a1, dx);
+                terms[r * tstride + u] = unit_q8_0(rr.wa[k], rr.wb[k], (uint16_t)rr.sc[k], a0, a1, dx);
             } else {
-                uint4 w = *(const uint4*)(wq + row * (n_in >> 1) + u * 16);
-                uint32_t sc = ((const uint16_t*)ws)[row * U + u];
                 float tA, tB;
-                unit_nvfp4(w, sc, a0, a1, dx, &tA, &tB);
+                unit_nvfp4(rr.wa[k], rr.sc[k], a0, a1, dx, &tA, &tB);
                 terms[r * tstride + 2 * u] = tA;
                 terms[r * tstride + 2 * u + 1] = tB;
             }
@@ -86,18 +113,137 @@ __device__ void wave_row_terms(const uint8_t* wq, const uint8_t* ws, int n_in, i
     }
 }
 
-IT_DEV float fold_terms(const float* tr, int T) {
-    float acc = 0.0f;
-    for (int k = 0; k < T; k++) acc += tr[k];
-    return acc;
+template <int FMT, int IPL>
+__device__ __forceinline__ void wave_row_terms_n(const uint8_t* wq, const uint8_t* ws, int n_in, int row0, int nrows,
+                                                 const int8_t* xq, const float* xs, float* terms, int tstride,
+                                                 int lane) {
+    RowRegs<IPL> rr;
+    load_items<FMT, IPL>(rr, wq, ws, n_in, row0, nrows, lane);
+    compute_items<FMT, IPL>(rr, n_in, nrows, xq, xs, terms, tstride, lane);
+}
+
+// nrows * (n_in / 32) must not exceed 512 (the launchers size rows_per_wave for that)
+template <int FMT>
+__device__ void wave_row_terms(const uint8_t* wq, const uint8_t* ws, int n_in, int row0, int nrows,
+                               const int8_t* xq, const float* xs, float* terms, int tstride, int lane) {
+    const int items = nrows * (n_in >> 5);
+    if (items <= 64) wave_row_terms_n<FMT, 1>(wq, ws, n_in, row0, nrows, xq, xs, terms, tstride, lane);
+    else if (items <= 128) wave_row_terms_n<FMT, 2>(wq, ws, n_in, row0, nrows, xq, xs, terms, tstride, lane);
+    else if (items <= 256) wave_row_terms_n<FMT, 4>(wq, ws, n_in, row0, nrows, xq, xs, terms, tstride, lane);
+    else wave_row_terms_n<FMT, 8>(wq, ws, n_in, row0, nrows, xq, xs, terms, tstride, lane);
 }
 
 // ------------------------------------------------------------------ fused_gemv
 // prologue modes: 0 = the activation as is; 1 = rms_norm(x, norm_w); 2 = per-head
 // rms_norm of x (weight norm_w[head_dim]) gated by silu(gate): silu(g) * ((x*scale)*w)
-__global__ __launch_bounds__(256) void fused_gemv_k(FusedGemvP p) {
+// ------------------------------------------------------------------ router in one wave
+// softmax over all experts, then n_used rounds of arg-max with ties to the lower id, the
+// picked probabilities summed in pick order (src/ops/mod.rs:1191-1216, naive.rs:362-376).
+// Called by one wave; probs (LDS, n_expert floats) holds the logits on entry.
+__device__ void wave_route(float* probs, int n_expert, int n_used, int exact, int* ids, float* weights, int lane) {
+    float m = -INFINITY;
+    for (int e = lane; e < n_expert; e += 64) m = fmaxf(m, probs[e]);
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    float part = 0.0f;
+    for (int e = lane; e < n_expert; e += 64) {
+        float v = it_expf(probs[e] - m);
+        probs[e] = v;
+        part += v;
+    }
+    wave_lds_sync();
+    float sum;
+    if (exact) {
+        float acc = 0.0f;
+        if (lane == 0)
+            for (int e = 0; e < n_expert; e++) acc += probs[e];
+        sum = __shfl(acc, 0, 64);
+    } else {
+        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+        sum = part;
+    }
+    for (int e = lane; e < n_expert; e += 64) probs[e] = probs[e] / sum;
+    wave_lds_sync();
+    float picked_p = 0.0f;  // lane r keeps pick r's probability
+    int picked_id = -1;
+    for (int r = 0; r < n_used; r++) {
+        float bv = 0.0f;
+        int bi = -1;
+        for (int e = lane; e < n_expert; e += 64) {
+            float v = probs[e];
+            if (v < 0.0f) continue;  // taken (probabilities are never negative)
+            if (bi < 0 || v > bv) {
+                bv = v;
+                bi = e;
+            }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            float ov = __shfl_xor(bv, o, 64);
+            int oi = __shfl_xor(bi, o, 64);
+            bool take = oi >= 0 && (bi < 0 || ov > bv || (ov == bv && oi < bi));
+            if (take) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (lane == r) {
+            picked_p = bv;
+            picked_id = bi;
+        }
+        if (lane == 0 && bi >= 0) probs[bi] = -1.0f;
+        wave_lds_sync();
+    }
+    // sum in pick order, serial f32
+    float s = 0.0f;
+    for (int r = 0; r < n_used; r++) s += __shfl(picked_p, r, 64);
+    float denom = fmaxf(s, 6.103515625e-5f);
+    if (lane < n_used) {
+        ids[lane] = picked_id;
+        weights[lane] = picked_p / denom;
+    }
+    wave_lds_sync();
+}
+
+constexpr int FG_THREADS = 512;
+
+IT_DEV int mat_index(const FusedGemvP& p, int g) {
+    int mi = 0;
+#pragma unroll
+    for (int k = 1; k < 4; k++)
+        if (k < p.n_mats && g >= p.m[k].group0) mi = k;
+    return mi;
+}
+
+// fold each row's terms in order and apply the matrix's epilogue
+IT_DEV void finish_rows(const FusedGemvP& p, const FusedMat& m, int row0, int nrows, const float* terms, int tstride,
+                        int nb, int lane) {
+    if (lane >= nrows) return;
+    const int T = m.fmt == W_NVFP4 ? nb * 2 : nb;
+    float acc = fold_terms(terms + lane * tstride, T);
+    const int j = row0 + lane;
+    if (m.epi == 0) {
+        m.out[j] = acc;
+    } else if (m.epi == 2) {
+        m.out[j] += acc;
+    } else {
+        // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
+        float* past = p.conv_state + (int64_t)j * 3;
+        const float* w = p.conv_w + (int64_t)j * 4;
+        float p0 = past[0], p1 = past[1], p2 = past[2];
+        float sum = 0.0f;
+        sum += p0 * w[0];
+        sum += p1 * w[1];
+        sum += p2 * w[2];
+        sum += acc * w[3];
+        m.out[j] = it_silu(sum);
+        past[0] = p1;
+        past[1] = p2;
+        past[2] = acc;
+    }
+}
+
+__global__ __launch_bounds__(FG_THREADS) void fused_gemv_k(FusedGemvP p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ double red[5];
+    __shared__ double red[FG_THREADS / 64 + 1];
     __shared__ float hscale[64];
     const int n_in = p.n_in, nb = n_in >> 5;
     float* xf = (float*)smem;
@@ -106,13 +252,29 @@ __global__ __launch_bounds__(256) void fused_gemv_k(FusedGemvP p) {
     float* terms_all = (float*)(xq + n_in);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    for (int i = tid; i < n_in; i += 256) xf[i] = p.x[i];
+    // the first row group's weights start moving before the activation prologue runs
+    constexpr int W = FG_THREADS / 64;
+    const int R = p.rows_per_wave;
+    const int tstride = nb * 2 + 4;
+    float* terms = terms_all + (size_t)wave * R * tstride;
+    const int g0 = blockIdx.x * W + wave;
+    const bool has0 = g0 < p.total_groups;
+    const FusedMat& m0 = p.m[has0 ? mat_index(p, g0) : 0];
+    const int row00 = has0 ? (g0 - m0.group0) * R : 0;
+    const int nrows0 = has0 ? min(R, m0.n_out - row00) : 0;
+    RowRegs<8> rr;
+    if (has0) {
+        if (m0.fmt == W_NVFP4) load_items<W_NVFP4, 8>(rr, m0.q, m0.s, n_in, row00, nrows0, lane);
+        else load_items<W_Q8_0, 8>(rr, m0.q, m0.s, n_in, row00, nrows0, lane);
+    }
+
+    for (int i = tid; i < n_in; i += FG_THREADS) xf[i] = p.x[i];
     __syncthreads();
     if (p.mode == 1) {
-        double sum = block_sumsq<256>(xf, n_in, p.exact, red);
+        double sum = block_sumsq<FG_THREADS>(xf, n_in, p.exact, red);
         float mean = (float)(sum / (double)n_in);
         float scale = 1.0f / sqrtf(mean + p.eps);
-        for (int i = tid; i < n_in; i += 256) xf[i] = xf[i] * scale * p.norm_w[i];
+        for (int i = tid; i < n_in; i += FG_THREADS) xf[i] = xf[i] * scale * p.norm_w[i];
         __syncthreads();
     } else if (p.mode == 2) {
         const int hd = p.head_dim, nh = n_in / hd;  // nh <= 64 (checked on the host)
@@ -125,7 +287,7 @@ __global__ __launch_bounds__(256) void fused_gemv_k(FusedGemvP p) {
             }
         } else {
             // 4 lanes per head
-            for (int h0 = 0; h0 < nh; h0 += 64) {
+            for (int h0 = 0; h0 < nh; h0 += FG_THREADS / 4) {
                 int h = h0 + (tid >> 2), sub = tid & 3;
                 double part = 0.0;
                 if (h < nh)
@@ -136,7 +298,7 @@ __global__ __launch_bounds__(256) void fused_gemv_k(FusedGemvP p) {
             }
         }
         __syncthreads();
-        for (int i = tid; i < n_in; i += 256) {
+        for (int i = tid; i < n_in; i += FG_THREADS) {
             float core = xf[i] * hscale[i / hd] * p.norm_w[i % hd];
             xf[i] = it_silu(p.gate[i]) * core;
         }
@@ -144,64 +306,72 @@ __global__ __launch_bounds__(256) void fused_gemv_k(FusedGemvP p) {
     }
     if (blockIdx.x == 0) {
         if (p.x_copy)
-            for (int i = tid; i < n_in; i += 256) p.x_copy[i] = xf[i];
+            for (int i = tid; i < n_in; i += FG_THREADS) p.x_copy[i] = xf[i];
         if (p.x_copy2)
-            for (int i = tid; i < n_in; i += 256) p.x_copy2[i] = xf[i];
+            for (int i = tid; i < n_in; i += FG_THREADS) p.x_copy2[i] = xf[i];
     }
     lds_quantize_q8_0(xf, n_in, xs, xq);
     __syncthreads();
 
-    const int R = p.rows_per_wave;
-    const int tstride = nb * 2 + 1;
-    float* terms = terms_all + (size_t)wave * R * tstride;
-    for (int g = blockIdx.x * 4 + wave; g < p.total_groups; g += gridDim.x * 4) {
-        int mi = 0;
-#pragma unroll
-        for (int k = 1; k < 4; k++)
-            if (k < p.n_mats && g >= p.m[k].group0) mi = k;
-        const FusedMat& m = p.m[mi];
+    if (has0) {
+        if (m0.fmt == W_NVFP4) compute_items<W_NVFP4, 8>(rr, n_in, nrows0, xq, xs, terms, tstride, lane);
+        else compute_items<W_Q8_0, 8>(rr, n_in, nrows0, xq, xs, terms, tstride, lane);
+        wave_lds_sync();
+        finish_rows(p, m0, row00, nrows0, terms, tstride, nb, lane);
+        wave_lds_sync();
+    }
+    for (int g = g0 + gridDim.x * W; g < p.total_groups; g += gridDim.x * W) {
+        const FusedMat& m = p.m[mat_index(p, g)];
         const int row0 = (g - m.group0) * R;
         const int nrows = min(R, m.n_out - row0);
-        const int T = m.fmt == W_NVFP4 ? nb * 2 : nb;
         if (m.fmt == W_NVFP4) wave_row_terms<W_NVFP4>(m.q, m.s, n_in, row0, nrows, xq, xs, terms, tstride, lane);
         else wave_row_terms<W_Q8_0>(m.q, m.s, n_in, row0, nrows, xq, xs, terms, tstride, lane);
         wave_lds_sync();
-        if (lane < nrows) {
-            float acc = fold_terms(terms + lane * tstride, T);
-            const int j = row0 + lane;
-            if (m.epi == 0) {
-                m.out[j] = acc;
-            } else if (m.epi == 2) {
-                m.out[j] += acc;
-            } else {
-                // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
-                float* past = p.conv_state + (int64_t)j * 3;
-                const float* w = p.conv_w + (int64_t)j * 4;
-                float p0 = past[0], p1 = past[1], p2 = past[2];
-                float sum = 0.0f;
-                sum += p0 * w[0];
-                sum += p1 * w[1];
-                sum += p2 * w[2];
-                sum += acc * w[3];
-                m.out[j] = it_silu(sum);
-                past[0] = p1;
-                past[1] = p2;
-                past[2] = acc;
+        finish_rows(p, m, row0, nrows, terms, tstride, nb, lane);
+        wave_lds_sync();
+    }
+    if (p.route_counter) {
+        // The block that finishes last turns the router logits (matrix 0's output) into the
+        // token's expert choice, so the next kernel starts with the ids in hand.
+        __shared__ int is_last;
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            unsigned prev = atomicAdd(p.route_counter, 1u);
+            is_last = prev == gridDim.x - 1;
+        }
+        __syncthreads();
+        if (is_last) {
+            __threadfence();
+            float* probs = xf;  // n_expert <= n_in (checked on the host)
+            for (int i = tid; i < p.n_expert; i += FG_THREADS)
+                probs[i] = __hip_atomic_load(p.m[0].out + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            if (wave == 0) {
+                __shared__ int rids[64];
+                __shared__ float rwts[64];
+                wave_route(probs, p.n_expert, p.n_used, p.exact, rids, rwts, lane);
+                if (lane < p.n_used) {
+                    p.route_ids[lane] = rids[lane];
+                    p.route_w[lane] = rwts[lane];
+                }
+                if (lane == 0) *p.route_counter = 0u;
             }
         }
-        wave_lds_sync();
     }
 }
 
 void fused_gemv(FusedGemvP p, hipStream_t s) {
+    constexpr int W = FG_THREADS / 64;
     int total_rows = 0;
     for (int i = 0; i < p.n_mats; i++) total_rows += p.m[i].n_out;
     const int nb = p.n_in / 32;
-    // one block per CU (two when there is plenty of work), each wave striding over row groups
+    // enough waves to cover HBM latency: aim for ~4096 row groups, at most 512 items per wave pass
     int R = 1;
-    while (R < 8 && total_rows / (R * 2) >= 1024) R *= 2;
+    while (R < 16 && total_rows / (R * 2) >= 4096) R *= 2;
+    while (R > 1 && R * nb > 512) R /= 2;
     auto lds_for = [&](int r) {
-        return (size_t)p.n_in * 4 + (size_t)((nb + 3) & ~3) * 4 + p.n_in + (size_t)4 * r * (nb * 2 + 1) * 4;
+        return (size_t)p.n_in * 4 + (size_t)((nb + 3) & ~3) * 4 + p.n_in + (size_t)W * r * (nb * 2 + 4) * 4;
     };
     while (R > 1 && lds_for(R) > 60 * 1024) R /= 2;
     p.rows_per_wave = R;
@@ -211,10 +381,11 @@ void fused_gemv(FusedGemvP p, hipStream_t s) {
         g += (p.m[i].n_out + R - 1) / R;
     }
     p.total_groups = g;
-    int blocks = (g + 3) / 4;
-    int cap = total_rows >= 32768 ? 512 : 256;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(fused_gemv_k, dim3(blocks), dim3(256), lds_for(R), s, p);
+    int blocks = (g + W - 1) / W;
+    // one block per CU: every block pays the activation prologue, so more blocks than CUs
+    // only repeats it (measured: 256 blocks 12 us, 772 blocks 22 us for norm + 12k rows of 2048)
+    if (blocks > 256) blocks = 256;
+    hipLaunchKernelGGL(fused_gemv_k, dim3(blocks), dim3(FG_THREADS), lds_for(R), s, p);
 }
 
 // ------------------------------------------------------------------ gdn rows
@@ -358,101 +529,20 @@ void gdn_core(const GdnCoreP& p, int dk, hipStream_t s) {
     }
 }
 
-// ------------------------------------------------------------------ router in one wave
-// softmax over all experts, then n_used rounds of arg-max with ties to the lower id, the
-// picked probabilities summed in pick order (src/ops/mod.rs:1191-1216, naive.rs:362-376).
-// Called by one wave; probs (LDS, n_expert floats) holds the logits on entry.
-__device__ void wave_route(float* probs, int n_expert, int n_used, int exact, int* ids, float* weights, int lane) {
-    float m = -INFINITY;
-    for (int e = lane; e < n_expert; e += 64) m = fmaxf(m, probs[e]);
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    float part = 0.0f;
-    for (int e = lane; e < n_expert; e += 64) {
-        float v = it_expf(probs[e] - m);
-        probs[e] = v;
-        part += v;
-    }
-    wave_lds_sync();
-    float sum;
-    if (exact) {
-        float acc = 0.0f;
-        if (lane == 0)
-            for (int e = 0; e < n_expert; e++) acc += probs[e];
-        sum = __shfl(acc, 0, 64);
-    } else {
-        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-        sum = part;
-    }
-    for (int e = lane; e < n_expert; e += 64) probs[e] = probs[e] / sum;
-    wave_lds_sync();
-    float picked_p = 0.0f;  // lane r keeps pick r's probability
-    int picked_id = -1;
-    for (int r = 0; r < n_used; r++) {
-        float bv = 0.0f;
-        int bi = -1;
-        for (int e = lane; e < n_expert; e += 64) {
-            float v = probs[e];
-            if (v < 0.0f) continue;  // taken (probabilities are never negative)
-            if (bi < 0 || v > bv) {
-                bv = v;
-                bi = e;
-            }
-        }
-        for (int o = 32; o > 0; o >>= 1) {
-            float ov = __shfl_xor(bv, o, 64);
-            int oi = __shfl_xor(bi, o, 64);
-            bool take = oi >= 0 && (bi < 0 || ov > bv || (ov == bv && oi < bi));
-            if (take) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        if (lane == r) {
-            picked_p = bv;
-            picked_id = bi;
-        }
-        if (lane == 0 && bi >= 0) probs[bi] = -1.0f;
-        wave_lds_sync();
-    }
-    // sum in pick order, serial f32
-    float s = 0.0f;
-    for (int r = 0; r < n_used; r++) s += __shfl(picked_p, r, 64);
-    float denom = fmaxf(s, 6.103515625e-5f);
-    if (lane < n_used) {
-        ids[lane] = picked_id;
-        weights[lane] = picked_p / denom;
-    }
-    wave_lds_sync();
-}
-
 // ------------------------------------------------------------------ moe_glu_fused
 // grid (row blocks, n_used + 1): y < n_used is routed pick y, y == n_used the shared expert.
 __global__ __launch_bounds__(256) void moe_glu_fused_k(MoeGluP p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int ids[64];
-    __shared__ float wts[64];
     const int n_in = p.n_in, nb = n_in >> 5;
-    float* xf = (float*)smem;                       // n_in floats, then reused
+    float* xf = (float*)smem;
     float* xs = xf + n_in;
     int8_t* xq = (int8_t*)(xs + ((nb + 3) & ~3));
-    float* probs = (float*)(xq + n_in);             // n_expert floats
-    float* terms_all = probs + ((p.n_expert + 3) & ~3);
+    float* terms_all = (float*)(xq + n_in);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    for (int i = tid; i < n_in; i += 256) xf[i] = p.x[i];
-    for (int i = tid; i < p.n_expert; i += 256) probs[i] = p.logits[i];
-    __syncthreads();
-    if (wave == 0) wave_route(probs, p.n_expert, p.n_used, p.exact, ids, wts, lane);
-    lds_quantize_q8_0(xf, n_in, xs, xq);
-    __syncthreads();
     const int y = blockIdx.y;
-    if (blockIdx.x == 0 && y == 0 && tid < p.n_used) {
-        p.route_ids[tid] = ids[tid];
-        p.route_w[tid] = wts[tid];
-    }
     const bool shared = y == p.n_used;
     const int fmt = shared ? p.sh_fmt : p.fmt;
-    const int64_t e = shared ? 0 : ids[y];
+    const int64_t e = shared ? 0 : p.route_ids[y];
     const uint8_t* gq = shared ? p.sh_gq : p.gq + e * p.q_stride;
     const uint8_t* gs = shared ? p.sh_gs : p.gs + e * p.s_stride;
     const uint8_t* uq = shared ? p.sh_uq : p.uq + e * p.q_stride;
@@ -461,19 +551,46 @@ __global__ __launch_bounds__(256) void moe_glu_fused_k(MoeGluP p) {
     float* out = shared ? p.sh_out : p.out + (int64_t)y * p.n_out;
 
     const int R = p.rows_per_wave;
-    const int tstride = nb * 2 + 1;
+    const int tstride = nb * 2 + 4;
     float* tg = terms_all + (size_t)wave * 2 * R * tstride;
     float* tu = tg + (size_t)R * tstride;
     const int T = fmt == W_NVFP4 ? nb * 2 : nb;
     const int groups = (n_out + R - 1) / R;
-    for (int g = blockIdx.x * 4 + wave; g < groups; g += gridDim.x * 4) {
-        const int row0 = g * R, nrows = min(R, n_out - row0);
+    // first group's gate and up rows start moving before the activation is quantized
+    const int g0 = blockIdx.x * 4 + wave;
+    const bool has0 = g0 < groups;
+    const int row00 = g0 * R, nrows0 = has0 ? min(R, n_out - row00) : 0;
+    RowRegs<4> rg, ru;
+    if (has0) {
         if (fmt == W_NVFP4) {
-            wave_row_terms<W_NVFP4>(gq, gs, n_in, row0, nrows, xq, xs, tg, tstride, lane);
-            wave_row_terms<W_NVFP4>(uq, us, n_in, row0, nrows, xq, xs, tu, tstride, lane);
+            load_items<W_NVFP4, 4>(rg, gq, gs, n_in, row00, nrows0, lane);
+            load_items<W_NVFP4, 4>(ru, uq, us, n_in, row00, nrows0, lane);
         } else {
-            wave_row_terms<W_Q8_0>(gq, gs, n_in, row0, nrows, xq, xs, tg, tstride, lane);
-            wave_row_terms<W_Q8_0>(uq, us, n_in, row0, nrows, xq, xs, tu, tstride, lane);
+            load_items<W_Q8_0, 4>(rg, gq, gs, n_in, row00, nrows0, lane);
+            load_items<W_Q8_0, 4>(ru, uq, us, n_in, row00, nrows0, lane);
+        }
+    }
+    for (int i = tid; i < n_in; i += 256) xf[i] = p.x[i];
+    __syncthreads();
+    lds_quantize_q8_0(xf, n_in, xs, xq);
+    __syncthreads();
+    for (int g = g0; g < groups; g += gridDim.x * 4) {
+        const int row0 = g * R, nrows = min(R, n_out - row0);
+        if (g != g0) {
+            if (fmt == W_NVFP4) {
+                load_items<W_NVFP4, 4>(rg, gq, gs, n_in, row0, nrows, lane);
+                load_items<W_NVFP4, 4>(ru, uq, us, n_in, row0, nrows, lane);
+            } else {
+                load_items<W_Q8_0, 4>(rg, gq, gs, n_in, row0, nrows, lane);
+                load_items<W_Q8_0, 4>(ru, uq, us, n_in, row0, nrows, lane);
+            }
+        }
+        if (fmt == W_NVFP4) {
+            compute_items<W_NVFP4, 4>(rg, n_in, nrows, xq, xs, tg, tstride, lane);
+            compute_items<W_NVFP4, 4>(ru, n_in, nrows, xq, xs, tu, tstride, lane);
+        } else {
+            compute_items<W_Q8_0, 4>(rg, n_in, nrows, xq, xs, tg, tstride, lane);
+            compute_items<W_Q8_0, 4>(ru, n_in, nrows, xq, xs, tu, tstride, lane);
         }
         wave_lds_sync();
         if (lane < nrows) {
@@ -492,14 +609,14 @@ __global__ __launch_bounds__(256) void moe_glu_fused_k(MoeGluP p) {
 void moe_glu_fused(MoeGluP p, hipStream_t s) {
     const int nb = p.n_in / 32;
     int R = 4;
+    while (R > 1 && R * nb > 256) R /= 2;
     auto lds_for = [&](int r) {
-        return (size_t)p.n_in * 4 + (size_t)((nb + 3) & ~3) * 4 + p.n_in + (size_t)((p.n_expert + 3) & ~3) * 4 +
-               (size_t)4 * 2 * r * (nb * 2 + 1) * 4;
+        return (size_t)p.n_in * 4 + (size_t)((nb + 3) & ~3) * 4 + p.n_in + (size_t)4 * 2 * r * (nb * 2 + 4) * 4;
     };
     while (R > 1 && lds_for(R) > 60 * 1024) R /= 2;
     p.rows_per_wave = R;
     int n_out = p.n_out > p.sh_n_out ? p.n_out : p.sh_n_out;
-    int gx = (n_out + 32 - 1) / 32;  // about 32 rows per block
+    int gx = (n_out + 4 * R - 1) / (4 * R);  // one row group per wave
     if (gx < 1) gx = 1;
     hipLaunchKernelGGL(moe_glu_fused_k, dim3(gx, p.n_used + 1), dim3(256), lds_for(R), s, p);
 }
@@ -513,43 +630,60 @@ __global__ __launch_bounds__(256) void moe_down_fused_k(MoeDownP p) {
     const int sh_in = p.sh_n_in, sh_nb = sh_in >> 5;
     const int NU = p.n_used;
     // LDS: per pick quantized activation, then the shared one
-    float* stage = (float*)smem;                                 // max(n_in, sh_in) floats
-    const int stage_n = n_in > sh_in ? n_in : sh_in;
-    float* xs = stage + stage_n;                                  // NU*nb + sh_nb scales
+    float* xs = (float*)smem;                                     // NU*nb + sh_nb scales
     int8_t* xq = (int8_t*)(xs + ((NU * nb + sh_nb + 3) & ~3));    // NU*n_in + sh_in quants
     float* terms_all = (float*)(xq + ((NU * n_in + sh_in + 15) & ~15));
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int y = 0; y <= NU; y++) {
-        const int len = y < NU ? n_in : sh_in;
-        const float* src = y < NU ? p.g_all + (int64_t)y * n_in : p.g_shared;
-        for (int i = tid; i < len; i += 256) stage[i] = src[i];
-        __syncthreads();
-        lds_quantize_q8_0(stage, len, xs + y * nb, xq + y * n_in);
-        __syncthreads();
-    }
-    const int R = p.rows_per_wave;
+    constexpr int MAXU = 16;  // n_used <= 16 (checked on the host)
+    const int R = p.rows_per_wave;  // R * (n_in / 32) <= 64: one item per lane per expert
     const int T = p.fmt == W_NVFP4 ? nb * 2 : nb;
     const int shT = p.sh_fmt == W_NVFP4 ? sh_nb * 2 : sh_nb;
     const int Tmax = (T > shT ? T : shT);
-    const int tstride = Tmax + 1;
+    const int tstride = Tmax + 4;
     // terms[(y * R + r) * tstride + k]
     float* terms = terms_all + (size_t)wave * (NU + 1) * R * tstride;
-    const float gate = it_sigmoid(p.logit[0]);
     const int groups = (p.n_out + R - 1) / R;
-    for (int g = blockIdx.x * 4 + wave; g < groups; g += gridDim.x * 4) {
+    RowRegs<1> rr[MAXU], rsh;
+    auto load_all = [&](int row0, int nrows) {
+#pragma unroll
+        for (int y = 0; y < MAXU; y++) {
+            if (y < NU) {
+                const int64_t e = p.route_ids[y];
+                if (p.fmt == W_NVFP4) load_items<W_NVFP4, 1>(rr[y], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row0, nrows, lane);
+                else load_items<W_Q8_0, 1>(rr[y], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row0, nrows, lane);
+            }
+        }
+        if (p.sh_fmt == W_NVFP4) load_items<W_NVFP4, 1>(rsh, p.sh_q, p.sh_s, sh_in, row0, nrows, lane);
+        else load_items<W_Q8_0, 1>(rsh, p.sh_q, p.sh_s, sh_in, row0, nrows, lane);
+    };
+    const int g0 = blockIdx.x * 4 + wave;
+    if (g0 < groups) load_all(g0 * R, min(R, p.n_out - g0 * R));
+    const float gate = it_sigmoid(p.logit[0]);
+    // stage all NU + 1 intermediates as f32 (the term region is free until the main loop)
+    {
+        float* all = terms_all;
+        const int total = NU * n_in + sh_in;
+        for (int i = tid; i < total; i += 256) all[i] = i < NU * n_in ? p.g_all[i] : p.g_shared[i - NU * n_in];
+        __syncthreads();
+        // one Q8_0 block per 8 lanes; picks and the shared vector are back to back and 32-aligned
+        lds_quantize_q8_0(all, total, xs, xq);
+        __syncthreads();
+    }
+    for (int g = g0; g < groups; g += gridDim.x * 4) {
         const int row0 = g * R, nrows = min(R, p.n_out - row0);
-        for (int y = 0; y < NU; y++) {
-            const int64_t e = p.route_ids[y];
-            const uint8_t* wq = p.q + e * p.q_stride;
-            const uint8_t* ws = p.s + e * p.s_stride;
-            float* t = terms + (size_t)y * R * tstride;
-            if (p.fmt == W_NVFP4) wave_row_terms<W_NVFP4>(wq, ws, n_in, row0, nrows, xq + y * n_in, xs + y * nb, t, tstride, lane);
-            else wave_row_terms<W_Q8_0>(wq, ws, n_in, row0, nrows, xq + y * n_in, xs + y * nb, t, tstride, lane);
+        if (g != g0) load_all(row0, nrows);
+#pragma unroll
+        for (int y = 0; y < MAXU; y++) {
+            if (y < NU) {
+                float* t = terms + (size_t)y * R * tstride;
+                if (p.fmt == W_NVFP4) compute_items<W_NVFP4, 1>(rr[y], n_in, nrows, xq + y * n_in, xs + y * nb, t, tstride, lane);
+                else compute_items<W_Q8_0, 1>(rr[y], n_in, nrows, xq + y * n_in, xs + y * nb, t, tstride, lane);
+            }
         }
         {
             float* t = terms + (size_t)NU * R * tstride;
-            if (p.sh_fmt == W_NVFP4) wave_row_terms<W_NVFP4>(p.sh_q, p.sh_s, sh_in, row0, nrows, xq + NU * n_in, xs + NU * nb, t, tstride, lane);
-            else wave_row_terms<W_Q8_0>(p.sh_q, p.sh_s, sh_in, row0, nrows, xq + NU * n_in, xs + NU * nb, t, tstride, lane);
+            if (p.sh_fmt == W_NVFP4) compute_items<W_NVFP4, 1>(rsh, sh_in, nrows, xq + NU * n_in, xs + NU * nb, t, tstride, lane);
+            else compute_items<W_Q8_0, 1>(rsh, sh_in, nrows, xq + NU * n_in, xs + NU * nb, t, tstride, lane);
         }
         wave_lds_sync();
         // lane = (y, r): fold its dot, park it in slot 0 of its own term row
@@ -580,18 +714,20 @@ void moe_down_fused(MoeDownP p, hipStream_t s) {
     const int nb = p.n_in / 32, sh_nb = p.sh_n_in / 32;
     const int T = (p.fmt == W_NVFP4 ? nb * 2 : nb), shT = (p.sh_fmt == W_NVFP4 ? sh_nb * 2 : sh_nb);
     const int Tmax = T > shT ? T : shT;
-    const int stage_n = p.n_in > p.sh_n_in ? p.n_in : p.sh_n_in;
     int R = 4;
     while (R > 1 && (p.n_used + 1) * R > 64) R /= 2;
+    while (R > 1 && (R * nb > 64 || R * sh_nb > 64)) R /= 2;
     auto lds_for = [&](int r) {
-        return (size_t)stage_n * 4 + (size_t)((p.n_used * nb + sh_nb + 3) & ~3) * 4 +
-               (size_t)((p.n_used * p.n_in + p.sh_n_in + 15) & ~15) + (size_t)4 * (p.n_used + 1) * r * (Tmax + 1) * 4;
+        size_t terms = (size_t)4 * (p.n_used + 1) * r * (Tmax + 4) * 4;
+        size_t stage = (size_t)(p.n_used * p.n_in + p.sh_n_in) * 4;  // f32 staging shares the term region
+        return (size_t)((p.n_used * nb + sh_nb + 3) & ~3) * 4 + (size_t)((p.n_used * p.n_in + p.sh_n_in + 15) & ~15) +
+               (terms > stage ? terms : stage);
     };
     while (R > 1 && lds_for(R) > 60 * 1024) R /= 2;
     p.rows_per_wave = R;
     int groups = (p.n_out + R - 1) / R;
     int blocks = (groups + 3) / 4;
-    if (blocks > 256) blocks = 256;
+    if (blocks > 512) blocks = 512;
     hipLaunchKernelGGL(moe_down_fused_k, dim3(blocks), dim3(256), lds_for(R), s, p);
 }
 

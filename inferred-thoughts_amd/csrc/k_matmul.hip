@@ -77,13 +77,13 @@ constexpr int GEMV_WAVES = 4;
 
 template <int FMT, bool GLU>
 __global__ __launch_bounds__(64 * GEMV_WAVES) void gemv_k(GemvP p) {
-    extern __shared__ float lds[];
+    extern __shared__ __align__(16) float lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int U = p.n_in >> 5;                     // 32-element units per row
     const int TPU = (FMT == W_NVFP4) ? 2 : 1;      // terms per unit
     const int T = U * TPU;                         // terms per row
     const int R = p.rows_per_wave;
-    const int tstride = T + 1;
+    const int tstride = T + 4;
     float* terms = lds + (size_t)wave * R * tstride * (GLU ? 2 : 1);
     float* terms2 = terms + (size_t)R * tstride;
 
@@ -141,14 +141,10 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void gemv_k(GemvP p) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (lane < nrows) {
-        const float* tr = terms + lane * tstride;
-        float acc = 0.0f;
-        for (int k = 0; k < T; k++) acc += tr[k];
+        float acc = fold_terms(terms + lane * tstride, T);
         float* o = p.out + (int64_t)y * p.n_out + row0 + lane;
         if (GLU) {
-            const float* tr2 = terms2 + lane * tstride;
-            float acc2 = 0.0f;
-            for (int k = 0; k < T; k++) acc2 += tr2[k];
+            float acc2 = fold_terms(terms2 + lane * tstride, T);
             if (p.scale2) acc *= p.scale2[e];
             if (p.scale2_up) acc2 *= p.scale2_up[e];
             *o = it_silu(acc) * acc2;
@@ -173,7 +169,7 @@ template <int FMT, bool GLU>
 static void launch_gemv(GemvP p, int n_y, hipStream_t s) {
     int R = pick_rows_per_wave(p.n_out, n_y);
     int T = (p.n_in / 32) * (FMT == W_NVFP4 ? 2 : 1);
-    auto lds_for = [&](int r) { return (size_t)GEMV_WAVES * r * (T + 1) * sizeof(float) * (GLU ? 2 : 1); };
+    auto lds_for = [&](int r) { return (size_t)GEMV_WAVES * r * (T + 4) * sizeof(float) * (GLU ? 2 : 1); };
     while (R > 1 && lds_for(R) > 48 * 1024) R /= 2;
     p.rows_per_wave = R;
     size_t lds = lds_for(R);

@@ -24,6 +24,11 @@ struct FusedGemvP {
     FusedMat m[4];
     float* conv_state;    // epi 1
     const float* conv_w;
+    // optional: matrix 0 is the router; the last block to finish picks the experts
+    unsigned* route_counter;  // zero between launches
+    int n_expert, n_used;
+    int32_t* route_ids;
+    float* route_w;
 };
 void fused_gemv(FusedGemvP p, hipStream_t s);
 
@@ -39,7 +44,6 @@ void gdn_core(const GdnCoreP& p, int dk, hipStream_t s);
 
 struct MoeGluP {
     const float* x;        // normed activation, f32 [n_in]
-    const float* logits;   // router logits [n_expert] (before softmax)
     const uint8_t *gq, *gs, *uq, *us;
     const float *gscale2, *uscale2;
     int64_t q_stride, s_stride;
@@ -48,8 +52,7 @@ struct MoeGluP {
     int sh_fmt, sh_n_out;
     float* out;            // [n_used][n_out]
     float* sh_out;         // [sh_n_out]
-    int32_t* route_ids;    // [n_used] written for the down stage
-    float* route_w;
+    const int32_t* route_ids;  // [n_used], chosen by the router kernel
 };
 void moe_glu_fused(MoeGluP p, hipStream_t s);
 
