@@ -847,7 +847,7 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
                           sg.n_head_kv, sg.scale, dyn, sc, dout), rec,
                    [=](hipStream_t s) { attend_exact(args, sc, dout, s); });
     } else {
-        int n_split = attend_split_count((int)n_pos_cap);
+        int n_split = attend_split_count((int)n_pos_cap, (int)n_q, (int)a->head_dim, (int)group);
         float* sc = be->scratch_f32((size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2));
         if (!sc) return;
         const int* dyn = be->dyn_slot((int)a->n_pos);

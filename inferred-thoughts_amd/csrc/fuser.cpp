@@ -8,6 +8,7 @@
 // scales — is simply issued op by op.  A fused launch sits at the position of its
 // block's first op; everything it replaces is dropped, except an activation
 // quantization that some unfused op still reads.
+#include <cstdlib>
 #include "backend.h"
 
 using namespace itk;
@@ -362,7 +363,8 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     a.n_mats = 2;
     a.m[0] = mat_of(mr, 0);
     a.m[1] = mat_of(ml, 0);
-    a.route_counter = counter;
+    // fast mode ranks the logits inside the expert kernel instead (no cross-block hand-off)
+    a.route_counter = exact ? counter : nullptr;
     a.n_expert = (int)ne;
     a.n_used = (int)nu;
     a.route_ids = (int32_t*)rt.p[1];
@@ -393,6 +395,11 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     g.out = (float*)g_all;
     g.sh_out = (float*)e_gate;
     g.route_ids = (const int32_t*)rt.p[1];
+    if (!exact) {
+        g.logits = (const float*)router;
+        g.route_ids_out = (int32_t*)rt.p[1];
+        g.route_w_out = (float*)rt.p[2];
+    }
 
     MoeDownP d{};
     d.g_all = (const float*)g_all;
@@ -406,6 +413,7 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     d.n_in = (int)ff;
     d.n_out = (int)nd;
     d.n_used = (int)nu;
+    d.exact = exact;
     d.sh_q = (const uint8_t*)sdm.p[0];
     d.sh_s = (const uint8_t*)sdm.p[1];
     d.sh_fmt = (int)sdm.i[0];

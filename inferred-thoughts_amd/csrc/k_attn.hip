@@ -79,7 +79,6 @@ void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s) 
 // ------------------------------------------------------------------ split-K
 constexpr int CHUNK = 128;
 
-int attend_split_count(int n_pos_max) { return (n_pos_max + CHUNK - 1) / CHUNK; }
 
 // partial layout per (t, head, split): [hd acc][m][l]
 template <int G>
@@ -185,24 +184,197 @@ __global__ __launch_bounds__(256) void attend_split_k(AttnArgs a, int n_split, f
     }
 }
 
-// gate (optional): out *= sigmoid(gate[head * gate_stride + i]) — the attention block's output gate
-__global__ void attend_merge_k(const float* __restrict__ part, int n_split, int hd, float* __restrict__ out,
-                               const float* __restrict__ gate, int gate_stride) {
+// ------------------------------------------------------------------ split-K for a few queries (decode)
+// One block per (query, kv head, 64-position tile).  The K and V tiles are staged into LDS
+// with coalesced 16-byte loads (every thread has its 2 * HD / 32 loads in flight at once),
+// scores are computed with lane = position (wave w takes query heads w, w+4, ...), the
+// tile's softmax statistics come from wave reductions, and the weighted values with
+// lane = output dimensions (wave w takes positions 16w..16w+15; the four partial sums meet
+// in LDS).  Partial layout as above: [hd acc][m][l] per (t, head, split).
+constexpr int TILE = 64;
+
+template <int HD, int G>
+__global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, float* __restrict__ part) {
+    constexpr int CPR = HD / 8;            // 16-byte chunks per K or V row
+    constexpr int KSTR = HD * 2 + 16;      // K row stride in LDS: padded so lanes reading rows do not collide
+    constexpr int DPL = HD / 64;           // output dimensions per lane
+    constexpr int NLD = TILE * CPR / 256;  // 16-byte loads per thread per tile
+    __shared__ __align__(16) unsigned char tiles[TILE * KSTR + TILE * HD * 2];
+    unsigned char* ktile = tiles;
+    unsigned char* vtile = tiles + TILE * KSTR;
+    __shared__ __align__(16) float qs[G * HD];
+    __shared__ __align__(16) float sc[TILE * G];
+    __shared__ float mrow[G], lrow[G];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_pos_last = a.n_pos_dyn ? *a.n_pos_dyn : a.n_pos;
+    const int t = blockIdx.x / a.n_head_kv, h_kv = blockIdx.x % a.n_head_kv;
+    const int split = blockIdx.y;
+    const int n_pos = n_pos_last - a.n_q + 1 + t;
+    const int s0 = split * TILE;
+    const int len = min(TILE, n_pos - s0);
+    const int off = h_kv * HD;
+    const int h0 = h_kv * G;
+    float* my_part = part + (((int64_t)t * a.n_head + h0) * n_split + split) * (HD + 2);
+    const int64_t part_head_stride = (int64_t)n_split * (HD + 2);
+    if (len <= 0) {
+        if (tid < G) {
+            float* p = my_part + tid * part_head_stride;
+            p[HD] = -INFINITY;
+            p[HD + 1] = 0.0f;
+        }
+        return;
+    }
+    // stage K and V (rows past the context are zero)
+    {
+        uint4 kr[NLD], vr[NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            const int idx = tid + i * 256, pos = idx / CPR, c = idx % CPR;
+            if (pos < len) {
+                const int64_t g = (int64_t)(s0 + pos) * a.kv_dim + off + c * 8;
+                kr[i] = *(const uint4*)(a.k + g);
+                vr[i] = *(const uint4*)(a.v + g);
+            } else {
+                kr[i] = make_uint4(0, 0, 0, 0);
+                vr[i] = make_uint4(0, 0, 0, 0);
+            }
+        }
+        for (int i = tid; i < G * HD / 4; i += 256)
+            ((float4*)qs)[i] = ((const float4*)(a.q + ((int64_t)t * a.n_head + h0) * HD))[i];
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            const int idx = tid + i * 256, pos = idx / CPR, c = idx % CPR;
+            *(uint4*)(ktile + pos * KSTR + c * 16) = kr[i];
+            *(uint4*)(vtile + pos * HD * 2 + c * 16) = vr[i];
+        }
+    }
+    __syncthreads();
+    // scores and the tile's softmax statistics: lane = position
+    for (int g = wave; g < G; g += 4) {
+        const unsigned char* krow = ktile + lane * KSTR;
+        const float* q = qs + g * HD;
+        float acc = 0.0f;
+#pragma unroll 4
+        for (int i = 0; i < HD; i += 8) {
+            const uint4 kk = *(const uint4*)(krow + i * 2);
+            const float4 q0 = *(const float4*)(q + i), q1 = *(const float4*)(q + i + 4);
+            acc += q0.x * it_f16_to_f32((uint16_t)(kk.x & 0xffff)) + q0.y * it_f16_to_f32((uint16_t)(kk.x >> 16)) +
+                   q0.z * it_f16_to_f32((uint16_t)(kk.y & 0xffff)) + q0.w * it_f16_to_f32((uint16_t)(kk.y >> 16)) +
+                   q1.x * it_f16_to_f32((uint16_t)(kk.z & 0xffff)) + q1.y * it_f16_to_f32((uint16_t)(kk.z >> 16)) +
+                   q1.z * it_f16_to_f32((uint16_t)(kk.w & 0xffff)) + q1.w * it_f16_to_f32((uint16_t)(kk.w >> 16));
+        }
+        const float sco = lane < len ? acc * a.scale : -INFINITY;
+        float m = sco;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        const float p = lane < len ? __expf(sco - m) : 0.0f;
+        float l = p;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+        sc[lane * G + g] = p;
+        if (lane == 0) {
+            mrow[g] = m;
+            lrow[g] = l;
+        }
+    }
+    __syncthreads();
+    // weighted values: lane = DPL output dimensions, this wave's quarter of the positions
+    float acc[G][DPL];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int d = 0; d < DPL; d++) acc[g][d] = 0.0f;
+#pragma unroll 4
+    for (int s = wave * (TILE / 4); s < (wave + 1) * (TILE / 4); s++) {
+        float v[DPL];
+        const unsigned char* vrow = vtile + s * HD * 2 + lane * DPL * 2;
+        if (DPL == 4) {
+            const uint2 r = *(const uint2*)vrow;
+            v[0] = it_f16_to_f32((uint16_t)(r.x & 0xffff));
+            v[1 % DPL] = it_f16_to_f32((uint16_t)(r.x >> 16));
+            v[2 % DPL] = it_f16_to_f32((uint16_t)(r.y & 0xffff));
+            v[3 % DPL] = it_f16_to_f32((uint16_t)(r.y >> 16));
+        } else if (DPL == 2) {
+            const uint32_t r = *(const uint32_t*)vrow;
+            v[0] = it_f16_to_f32((uint16_t)(r & 0xffff));
+            v[1 % DPL] = it_f16_to_f32((uint16_t)(r >> 16));
+        } else {
+            v[0] = it_f16_to_f32(*(const uint16_t*)vrow);
+        }
+        float p[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) p[g] = sc[s * G + g];
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int d = 0; d < DPL; d++) acc[g][d] += p[g] * v[d];
+    }
+    __syncthreads();  // the tiles are dead: their space takes the four waves' partial sums
+    static_assert(4 * G * HD * 4 <= TILE * KSTR + TILE * HD * 2, "partial sums must fit in the tile space");
+    float* red = (float*)tiles;  // [4][G][HD]
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int d = 0; d < DPL; d++) red[(wave * G + g) * HD + lane * DPL + d] = acc[g][d];
+    __syncthreads();
+    for (int i = tid; i < G * HD; i += 256) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) sum += red[w * G * HD + i];
+        my_part[(i / HD) * part_head_stride + (i % HD)] = sum;
+    }
+    if (tid < G) {
+        float* p = my_part + tid * part_head_stride;
+        p[HD] = mrow[tid];
+        p[HD + 1] = lrow[tid];
+    }
+}
+
+// gate (optional): out *= sigmoid(gate[head * gate_stride + i]) — the attention block's output gate.
+// One block per (query, head).  Only the splits that hold positions are visited (n_live of them);
+// their weights exp(m_s - m) are formed once, in LDS.
+__global__ __launch_bounds__(256) void attend_merge_k(const float* __restrict__ part, int n_split, int hd,
+                                                      float* __restrict__ out, const float* __restrict__ gate,
+                                                      int gate_stride, int n_q, int n_head, int chunk, int n_pos_arg,
+                                                      const int* n_pos_dyn) {
+    extern __shared__ float wsplit[];  // [n_split]
+    __shared__ float redm[4], redl[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+    const int t = blockIdx.x / n_head;
+    const int n_pos = (n_pos_dyn ? *n_pos_dyn : n_pos_arg) - n_q + 1 + t;
+    int n_live = (n_pos + chunk - 1) / chunk;
+    if (n_live > n_split) n_live = n_split;
     const float* p = part + (int64_t)blockIdx.x * n_split * (hd + 2);
     float m = -INFINITY;
-    for (int s = 0; s < n_split; s++) m = fmaxf(m, p[(int64_t)s * (hd + 2) + hd]);
+    for (int s = tid; s < n_live; s += blockDim.x) m = fmaxf(m, p[(int64_t)s * (hd + 2) + hd]);
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (lane == 0) redm[wave] = m;
+    __syncthreads();
+    m = redm[0];
+    for (int w = 1; w < nw; w++) m = fmaxf(m, redm[w]);
     float l = 0.0f;
-    for (int s = 0; s < n_split; s++) {
-        float ms = p[(int64_t)s * (hd + 2) + hd];
-        if (ms != -INFINITY) l += p[(int64_t)s * (hd + 2) + hd + 1] * __expf(ms - m);
+    for (int s = tid; s < n_live; s += blockDim.x) {
+        const float ms = p[(int64_t)s * (hd + 2) + hd];
+        const float w = ms != -INFINITY ? __expf(ms - m) : 0.0f;
+        wsplit[s] = w;
+        l += p[(int64_t)s * (hd + 2) + hd + 1] * w;
     }
-    for (int i = threadIdx.x; i < hd; i += blockDim.x) {
-        float acc = 0.0f;
-        for (int s = 0; s < n_split; s++) {
-            float ms = p[(int64_t)s * (hd + 2) + hd];
-            if (ms != -INFINITY) acc += p[(int64_t)s * (hd + 2) + i] * __expf(ms - m);
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+    if (lane == 0) redl[wave] = l;
+    __syncthreads();
+    l = 0.0f;
+    for (int w = 0; w < nw; w++) l += redl[w];
+    for (int i = tid; i < hd; i += blockDim.x) {
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+        int s = 0;
+        for (; s + 4 <= n_live; s += 4) {
+            a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
+            a1 += p[(int64_t)(s + 1) * (hd + 2) + i] * wsplit[s + 1];
+            a2 += p[(int64_t)(s + 2) * (hd + 2) + i] * wsplit[s + 2];
+            a3 += p[(int64_t)(s + 3) * (hd + 2) + i] * wsplit[s + 3];
         }
-        float r = acc / l;
+        for (; s < n_live; s++) a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
+        float r = ((a0 + a1) + (a2 + a3)) / l;
         if (gate) r *= it_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + i]);
         out[(int64_t)blockIdx.x * hd + i] = r;
     }
@@ -212,21 +384,52 @@ void attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hi
     attend_split_gated(a, n_split, scratch, out, nullptr, 0, s);
 }
 
+// queries at or below this count take the tile kernel (chunk TILE); larger batches the
+// position-per-thread kernel (chunk CHUNK)
+constexpr int TILE_MAX_Q = 16;
+static bool tile_path(int n_q, int head_dim, int G) {
+    return n_q <= TILE_MAX_Q && (head_dim == 64 || head_dim == 128 || head_dim == 256) && G <= 8;
+}
+
+int attend_split_count(int n_pos_max, int n_q, int head_dim, int group) {
+    const int chunk = tile_path(n_q, head_dim, group) ? TILE : CHUNK;
+    return (n_pos_max + chunk - 1) / chunk;
+}
+
 void attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* out, const float* gate,
                         int gate_stride, hipStream_t s) {
     if (a.n_q <= 0) return;
     const int G = a.n_head / a.n_head_kv;
     dim3 grid(a.n_q * a.n_head_kv, n_split), block(256);
-    size_t lds = ((size_t)G * a.head_dim + (size_t)CHUNK * G) * sizeof(float);
-    switch (G) {
-        case 1: hipLaunchKernelGGL(attend_split_k<1>, grid, block, lds, s, a, n_split, scratch); break;
-        case 2: hipLaunchKernelGGL(attend_split_k<2>, grid, block, lds, s, a, n_split, scratch); break;
-        case 4: hipLaunchKernelGGL(attend_split_k<4>, grid, block, lds, s, a, n_split, scratch); break;
-        case 8: hipLaunchKernelGGL(attend_split_k<8>, grid, block, lds, s, a, n_split, scratch); break;
-        default: return;  // the caller falls back to the exact kernel for other group sizes
+    const bool tile = tile_path(a.n_q, a.head_dim, G);
+    if (tile) {
+#define IT_TILE(HD, GG) hipLaunchKernelGGL((attend_tile_k<HD, GG>), grid, block, 0, s, a, n_split, scratch)
+#define IT_TILE_G(HD)                  \
+    switch (G) {                       \
+        case 1: IT_TILE(HD, 1); break; \
+        case 2: IT_TILE(HD, 2); break; \
+        case 4: IT_TILE(HD, 4); break; \
+        case 8: IT_TILE(HD, 8); break; \
+        default: return;               \
     }
-    hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(a.head_dim < 256 ? 64 : 256), 0, s, scratch,
-                       n_split, a.head_dim, out, gate, gate_stride);
+        if (a.head_dim == 64) { IT_TILE_G(64) }
+        else if (a.head_dim == 128) { IT_TILE_G(128) }
+        else { IT_TILE_G(256) }
+#undef IT_TILE_G
+#undef IT_TILE
+    } else {
+        size_t lds = ((size_t)G * a.head_dim + (size_t)CHUNK * G) * sizeof(float);
+        switch (G) {
+            case 1: hipLaunchKernelGGL(attend_split_k<1>, grid, block, lds, s, a, n_split, scratch); break;
+            case 2: hipLaunchKernelGGL(attend_split_k<2>, grid, block, lds, s, a, n_split, scratch); break;
+            case 4: hipLaunchKernelGGL(attend_split_k<4>, grid, block, lds, s, a, n_split, scratch); break;
+            case 8: hipLaunchKernelGGL(attend_split_k<8>, grid, block, lds, s, a, n_split, scratch); break;
+            default: return;  // the caller falls back to the exact kernel for other group sizes
+        }
+    }
+    hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(a.head_dim < 256 ? 64 : 256),
+                       (size_t)n_split * sizeof(float), s, scratch, n_split, a.head_dim, out, gate, gate_stride, a.n_q,
+                       a.n_head, tile ? TILE : CHUNK, a.n_pos, a.n_pos_dyn);
 }
 
 }  // namespace itk

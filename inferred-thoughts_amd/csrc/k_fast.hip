@@ -1,0 +1,735 @@
+// Single-token kernels of the fast mode (reductions in wave order, not the CPU path's).
+//
+// The order-preserving kernels spend most of their time getting per-block terms into one
+// lane's hands.  Here every lane owns a fixed set of 16-byte weight chunks of a row, keeps
+// the matching activation chunks in registers for the whole kernel, and rows are reduced
+// with cross-lane shuffles; a wave has four chunk loads per lane in flight and fetches its
+// next row group while it reduces the current one.  The integer dots and the per-block
+// scale products are the ones the reference forms (src/quant/dot.rs); only the order in
+// which the per-block terms are added differs, so results agree to rounding, not by bit.
+//
+// A "chunk" is 16 bytes of a repacked weight row: 16 Q8_0 quants (half a block) or 32
+// NVFP4 nibbles (two sub-blocks).  A row of `cpr` chunks is spread over L = min(64, cpr)
+// lanes, CPL = cpr / L chunks each, so a wave covers P = 64 / L rows per step.
+#include "it_device.h"
+#include "it_dot.h"
+#include "kernels.h"
+#include "kernels_fused.h"
+
+namespace itk {
+namespace {
+
+constexpr int FT = 512, FW = FT / 64;  // threads and waves of the GEMV blocks
+
+// ------------------------------------------------------------------ chunk geometry
+struct Geo {
+    int cpl = 0, l = 0;
+    bool ok = false;
+};
+inline Geo geo_of(int fmt, int n_in) {
+    Geo g;
+    const int per = fmt == W_Q8_0 ? 16 : fmt == W_NVFP4 ? 32 : 0;
+    if (!per || n_in <= 0 || n_in % 32) return g;
+    const int cpr = n_in / per;
+    if (cpr & (cpr - 1)) return g;
+    if (cpr >= 64) {
+        g.l = 64;
+        g.cpl = cpr / 64;
+        g.ok = g.cpl <= 4;
+    } else {
+        g.l = cpr;
+        g.cpl = 1;
+        g.ok = cpr >= 8;
+    }
+    return g;
+}
+
+template <int FMT, int CPL> struct XChunks {
+    uint4 a[CPL], b[CPL];  // b: second half of an NVFP4 chunk's 32 activations
+    float d[CPL];
+};
+template <int CPL> struct WChunks {
+    uint4 w[CPL];
+    uint32_t sc[CPL];
+};
+
+// activation chunks of lane `sub` from the quantized activation in LDS
+template <int FMT, int CPL, int L>
+IT_DEV void load_x(XChunks<FMT, CPL>& x, const int8_t* xq, const float* xs, int sub) {
+#pragma unroll
+    for (int k = 0; k < CPL; k++) {
+        const int c = k * L + sub;
+        if (FMT == W_Q8_0) {
+            x.a[k] = *(const uint4*)(xq + c * 16);
+            x.d[k] = xs[c >> 1];
+        } else {
+            x.a[k] = *(const uint4*)(xq + c * 32);
+            x.b[k] = *(const uint4*)(xq + c * 32 + 16);
+            x.d[k] = xs[c];
+        }
+    }
+}
+
+template <int FMT, int CPL, int L>
+IT_DEV void load_w(WChunks<CPL>& t, const uint8_t* q, const uint8_t* s, int n_in, int64_t row, int sub, bool live) {
+    if (!live) {
+#pragma unroll
+        for (int k = 0; k < CPL; k++) {
+            t.w[k] = make_uint4(0, 0, 0, 0);
+            t.sc[k] = 0;
+        }
+        return;
+    }
+    const uint8_t* rp = q + row * (FMT == W_Q8_0 ? n_in : n_in >> 1);
+    const uint16_t* sp = (const uint16_t*)s + row * (n_in >> 5);
+#pragma unroll
+    for (int k = 0; k < CPL; k++) {
+        const int c = k * L + sub;
+        t.w[k] = *(const uint4*)(rp + c * 16);
+        t.sc[k] = FMT == W_Q8_0 ? sp[c >> 1] : sp[c];
+    }
+}
+
+template <int FMT, int CPL>
+IT_DEV float dot_chunks(const WChunks<CPL>& t, const XChunks<FMT, CPL>& x) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < CPL; k++) {
+        if (FMT == W_Q8_0) {
+            int s = 0;
+            s = dot4(t.w[k].x, x.a[k].x, s);
+            s = dot4(t.w[k].y, x.a[k].y, s);
+            s = dot4(t.w[k].z, x.a[k].z, s);
+            s = dot4(t.w[k].w, x.a[k].w, s);
+            acc += (float)s * (it_f16_to_f32((uint16_t)t.sc[k]) * x.d[k]);
+        } else {
+            float tA, tB;
+            unit_nvfp4(t.w[k], t.sc[k], x.a[k], x.b[k], x.d[k], &tA, &tB);
+            acc += tA;
+            acc += tB;
+        }
+    }
+    return acc;
+}
+
+template <int L> IT_DEV float reduce_lanes(float v) {
+#pragma unroll
+    for (int o = L / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ------------------------------------------------------------------ activation prologue
+// Q8_0 block quantization (naive.rs:652-675) of the quad a thread holds; the 8 threads of a
+// 32-block are neighbours in a wave.  Dead threads pass zeros and write nothing.
+IT_DEV void quant_quad(float4 v, bool live, int qi, int8_t* xq, float* xs) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    if (!live) return;
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float r[4] = {roundf(v.x * id), roundf(v.y * id), roundf(v.z * id), roundf(v.w * id)};
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float c = fminf(fmaxf(r[i], -128.0f), 127.0f);
+        const int q = (r[i] != r[i]) ? 0 : (int)c;
+        packed |= ((uint32_t)(q & 0xff)) << (8 * i);
+    }
+    *(uint32_t*)(xq + qi * 4) = packed;
+    if ((qi & 7) == 0) xs[qi >> 3] = it_f16_to_f32(it_f32_to_f16(d));
+}
+
+IT_DEV double quad_sumsq(float4 v) {
+    double s = (double)(v.x * v.x);
+    s += (double)(v.y * v.y);
+    s += (double)(v.z * v.z);
+    s += (double)(v.w * v.w);
+    return s;
+}
+
+// The activation of a fused GEMV, from global f32 to quantized LDS, held in registers in
+// between: thread t owns floats [4t, 4t+4) and [4(t+THREADS), ...).  n_in <= 8 * THREADS.
+//   mode 0: as is; 1: rms_norm(x, norm_w) (naive.rs:633-650); 2: per-head rms_norm gated by
+//   silu(gate) (head_dim / 4 a power of two <= 64, so a head sits inside one wave).
+// Ends with a block barrier; xq / xs are then complete.
+template <int THREADS>
+__device__ void stage_activation(const float* x, int n_in, int mode, const float* norm_w, const float* gate, int head_dim,
+                                 float eps, float* copy1, float* copy2, int8_t* xq, float* xs, double* red) {
+    const int tid = threadIdx.x;
+    const int nq = n_in >> 2;
+    float4 v[2];
+    bool live[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int qi = tid + k * THREADS;
+        live[k] = qi < nq;
+        v[k] = live[k] ? ((const float4*)x)[qi] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (mode == 1) {
+        float4 w[2];
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+            w[k] = live[k] ? ((const float4*)norm_w)[tid + k * THREADS] : make_float4(0.f, 0.f, 0.f, 0.f);
+        double part = quad_sumsq(v[0]) + quad_sumsq(v[1]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+        if ((tid & 63) == 0) red[tid >> 6] = part;
+        __syncthreads();
+        double sum = 0.0;
+#pragma unroll
+        for (int i = 0; i < THREADS / 64; i++) sum += red[i];
+        const float mean = (float)(sum / (double)n_in);
+        const float scale = 1.0f / sqrtf(mean + eps);
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            v[k].x = v[k].x * scale * w[k].x;
+            v[k].y = v[k].y * scale * w[k].y;
+            v[k].z = v[k].z * scale * w[k].z;
+            v[k].w = v[k].w * scale * w[k].w;
+        }
+    } else if (mode == 2) {
+        const int lh = head_dim >> 2;  // lanes per head
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int qi = tid + k * THREADS;
+            double part = quad_sumsq(v[k]);
+            for (int o = lh >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+            if (live[k]) {
+                const float hs = 1.0f / sqrtf((float)(part / (double)head_dim) + eps);
+                const float4 w = ((const float4*)norm_w)[qi & (lh - 1)];
+                const float4 g = ((const float4*)gate)[qi];
+                v[k].x = it_silu(g.x) * (v[k].x * hs * w.x);
+                v[k].y = it_silu(g.y) * (v[k].y * hs * w.y);
+                v[k].z = it_silu(g.z) * (v[k].z * hs * w.z);
+                v[k].w = it_silu(g.w) * (v[k].w * hs * w.w);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int qi = tid + k * THREADS;
+        if (live[k]) {
+            if (copy1) ((float4*)copy1)[qi] = v[k];
+            if (copy2) ((float4*)copy2)[qi] = v[k];
+        }
+        quant_quad(v[k], live[k], qi, xq, xs);
+    }
+    __syncthreads();
+}
+
+// ------------------------------------------------------------------ fused_gemv, fast
+IT_DEV int fast_mat_index(const FusedGemvP& p, int g) {
+    int mi = 0;
+#pragma unroll
+    for (int k = 1; k < 4; k++)
+        if (k < p.n_mats && g >= p.m[k].group0) mi = k;
+    return mi;
+}
+
+template <int FMT, int CPL, int L>
+__global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
+    constexpr int P = 64 / L;
+    constexpr int RB = CPL >= 4 ? 1 : 4 / CPL;  // steps per group: four chunk loads per lane in flight
+    constexpr int RG = RB * P;
+    __shared__ __align__(16) int8_t xq[FT * 8];
+    __shared__ float xs[FT * 8 / 32];
+    __shared__ double red[FW];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int sub = lane % L, rsub = lane / L;
+    const int n_in = p.n_in;
+    const int gstride = gridDim.x * FW;
+    int g = blockIdx.x * FW + wave;
+
+    WChunks<CPL> t[RB];
+    int mi = 0, row0 = 0;
+    auto fetch = [&](int gg) {
+        mi = fast_mat_index(p, gg);
+        const FusedMat& m = p.m[mi];
+        row0 = (gg - m.group0) * RG;
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const int row = row0 + r * P + rsub;
+            load_w<FMT, CPL, L>(t[r], m.q, m.s, n_in, row, sub, row < m.n_out);
+        }
+    };
+    // the first group's weights start moving before the activation prologue runs
+    if (g < p.total_groups) fetch(g);
+
+    const bool first = blockIdx.x == 0;
+    stage_activation<FT>(p.x, n_in, p.mode, p.norm_w, p.gate, p.head_dim, p.eps, first ? p.x_copy : nullptr,
+                         first ? p.x_copy2 : nullptr, xq, xs, red);
+    XChunks<FMT, CPL> x;
+    load_x<FMT, CPL, L>(x, xq, xs, sub);
+
+    while (g < p.total_groups) {
+        float acc[RB];
+#pragma unroll
+        for (int r = 0; r < RB; r++) acc[r] = dot_chunks<FMT, CPL>(t[r], x);
+        const int cmi = mi, crow0 = row0;
+        g += gstride;
+        if (g < p.total_groups) fetch(g);
+#pragma unroll
+        for (int r = 0; r < RB; r++) acc[r] = reduce_lanes<L>(acc[r]);
+        if (sub == 0) {
+            const FusedMat& m = p.m[cmi];
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                const int j = crow0 + r * P + rsub;
+                if (j >= m.n_out) continue;
+                const float a = acc[r];
+                if (m.epi == 0) {
+                    m.out[j] = a;
+                } else if (m.epi == 2) {
+                    m.out[j] += a;
+                } else {
+                    // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
+                    float* past = p.conv_state + (int64_t)j * 3;
+                    const float4 w = *(const float4*)(p.conv_w + (int64_t)j * 4);
+                    const float p0 = past[0], p1 = past[1], p2 = past[2];
+                    float sum = 0.0f;
+                    sum += p0 * w.x;
+                    sum += p1 * w.y;
+                    sum += p2 * w.z;
+                    sum += a * w.w;
+                    m.out[j] = it_silu(sum);
+                    past[0] = p1;
+                    past[1] = p2;
+                    past[2] = a;
+                }
+            }
+        }
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
+    if (p.exact || p.route_counter || p.n_mats < 1) return false;
+    const int fmt = p.m[0].fmt;
+    for (int i = 1; i < p.n_mats; i++)
+        if (p.m[i].fmt != fmt) return false;
+    const Geo g = geo_of(fmt, p.n_in);
+    if (!g.ok || p.n_in > FT * 8 || p.n_in % 32) return false;
+    if (!aligned16(p.x) || !aligned16(p.x_copy) || !aligned16(p.x_copy2)) return false;
+    if (p.mode == 1 && !aligned16(p.norm_w)) return false;
+    if (p.mode == 2) {
+        const int lh = p.head_dim / 4;
+        if (p.head_dim % 4 || lh < 1 || lh > 64 || (lh & (lh - 1)) || p.n_in % p.head_dim) return false;
+        if (!aligned16(p.norm_w) || !aligned16(p.gate)) return false;
+    }
+    for (int i = 0; i < p.n_mats; i++) {
+        if (!aligned16(p.m[i].q) || (reinterpret_cast<uintptr_t>(p.m[i].s) & 1)) return false;
+        if (p.m[i].epi == 1 && !aligned16(p.conv_w)) return false;
+    }
+    const int P = 64 / g.l, RB = g.cpl >= 4 ? 1 : 4 / g.cpl, RG = RB * P;
+    int groups = 0;
+    for (int i = 0; i < p.n_mats; i++) {
+        p.m[i].group0 = groups;
+        groups += (p.m[i].n_out + RG - 1) / RG;
+    }
+    p.total_groups = groups;
+    p.rows_per_wave = RG;
+    int blocks = (groups + FW - 1) / FW;
+    if (blocks > 1024) blocks = 1024;  // four resident blocks per CU; larger matrices loop
+    if (blocks < 1) blocks = 1;
+#define IT_LAUNCH(F, C, LL) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL>), dim3(blocks), dim3(FT), 0, s, p)
+    if (fmt == W_Q8_0) {
+        if (g.l == 64 && g.cpl == 1) IT_LAUNCH(W_Q8_0, 1, 64);
+        else if (g.l == 64 && g.cpl == 2) IT_LAUNCH(W_Q8_0, 2, 64);
+        else if (g.l == 64) IT_LAUNCH(W_Q8_0, 4, 64);
+        else if (g.l == 32) IT_LAUNCH(W_Q8_0, 1, 32);
+        else if (g.l == 16) IT_LAUNCH(W_Q8_0, 1, 16);
+        else IT_LAUNCH(W_Q8_0, 1, 8);
+    } else {
+        if (g.l == 64 && g.cpl == 1) IT_LAUNCH(W_NVFP4, 1, 64);
+        else if (g.l == 64 && g.cpl == 2) IT_LAUNCH(W_NVFP4, 2, 64);
+        else if (g.l == 64) IT_LAUNCH(W_NVFP4, 4, 64);
+        else if (g.l == 32) IT_LAUNCH(W_NVFP4, 1, 32);
+        else if (g.l == 16) IT_LAUNCH(W_NVFP4, 1, 16);
+        else IT_LAUNCH(W_NVFP4, 1, 8);
+    }
+#undef IT_LAUNCH
+    return true;
+}
+
+namespace {
+
+// ------------------------------------------------------------------ router in a block
+// softmax over n_expert logits, the n_used largest by (probability descending, id ascending),
+// weights = picked probabilities over their sum in pick order (src/ops/mod.rs:1191-1216,
+// naive.rs:362-376).  Every thread of the block calls this; ids / wts (LDS, n_used entries) are
+// complete after the final barrier.  n_expert <= 4 * THREADS, n_used <= 16.
+//
+// Selection is two-level.  (a) Every wave ranks its own 64 * K values against each other with
+// lane broadcasts: only values of wave rank < n_used can be in the global top n_used, and they
+// go to cand[wave][rank].  (b) The NW * n_used candidates are ranked against each other.
+template <int THREADS> struct RouteLds {
+    float redf[2 * (THREADS / 64)];
+    float cand_p[(THREADS / 64) * 16];
+    int cand_e[(THREADS / 64) * 16];
+};
+
+template <int THREADS>
+__device__ void block_route(const float* logits, int n_expert, int n_used, RouteLds<THREADS>& sh, int* ids, float* wts) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int NW = THREADS / 64;
+    const int K = (n_expert + THREADS - 1) / THREADS;  // experts per thread that can be live
+    float l[4];
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int e = tid + k * THREADS;
+        l[k] = e < n_expert ? logits[e] : -INFINITY;
+        m = fmaxf(m, l[k]);
+    }
+    if (tid < NW * 16) sh.cand_e[tid] = -1;  // a wave with fewer than n_used live experts leaves slots unset
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (lane == 0) sh.redf[wave] = m;
+    __syncthreads();
+    m = sh.redf[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) m = fmaxf(m, sh.redf[i]);
+    float v[4];
+    float part = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int e = tid + k * THREADS;
+        v[k] = e < n_expert ? it_expf(l[k] - m) : 0.0f;
+        part += v[k];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+    if (lane == 0) sh.redf[NW + wave] = part;
+    __syncthreads();
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NW; i++) sum += sh.redf[NW + i];
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = v[k] / sum;
+
+    // dead slots (id >= n_expert) hold 0 and the largest ids, so they never outrank a live one
+    int rank[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) {
+        if (k2 >= K) continue;
+        for (int j = 0; j < 64; j++) {
+            const float q = __shfl(v[k2], j, 64);
+            const int qe = (tid & ~63) + j + k2 * THREADS;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if (k >= K) continue;
+                const int e = tid + k * THREADS;
+                rank[k] += (q > v[k] || (q == v[k] && qe < e)) ? 1 : 0;
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int e = tid + k * THREADS;
+        if (k < K && e < n_expert && rank[k] < n_used) {
+            sh.cand_p[wave * 16 + rank[k]] = v[k];
+            sh.cand_e[wave * 16 + rank[k]] = e;
+        }
+    }
+    __syncthreads();
+    if (tid < NW * 16 && (tid & 15) < n_used) {
+        const int me = sh.cand_e[tid];
+        if (me >= 0) {
+            const float pv = sh.cand_p[tid];
+            int cnt = 0;
+            for (int w = 0; w < NW; w++)
+                for (int r = 0; r < n_used; r++) {
+                    const int qe = sh.cand_e[w * 16 + r];
+                    const float q = sh.cand_p[w * 16 + r];
+                    cnt += (qe >= 0 && (q > pv || (q == pv && qe < me))) ? 1 : 0;
+                }
+            if (cnt < n_used) {
+                ids[cnt] = me;
+                wts[cnt] = pv;
+            }
+        }
+    }
+    __syncthreads();
+    float s = 0.0f;
+    for (int r = 0; r < n_used; r++) s += wts[r];
+    const float denom = fmaxf(s, 6.103515625e-5f);
+    __syncthreads();
+    if (tid < n_used) wts[tid] = wts[tid] / denom;
+    __syncthreads();
+}
+
+// ------------------------------------------------------------------ moe_glu, fast
+// Jobs: n_used * ge routed groups (pick-major), then gs shared-expert groups.  A group is
+// RB steps of P (gate row, up row) pairs; out[row] = silu(gate.x * sg) * (up.x * su).
+struct GluGeo {
+    int e_cpl, e_l, e_groups, e_rg;
+    int s_cpl, s_l, s_groups, s_rg;
+};
+
+template <int FMT, int CPL, int L>
+IT_DEV void glu_job(const uint8_t* gq, const uint8_t* gs, const uint8_t* uq, const uint8_t* us, int n_in, int n_out,
+                    int row0, float sg, float su, const int8_t* xq, const float* xs, float* out, int lane,
+                    WChunks<CPL>* tg, WChunks<CPL>* tu, bool loaded) {
+    constexpr int P = 64 / L;
+    constexpr int RB = CPL >= 2 ? 1 : 2;
+    const int sub = lane % L, rsub = lane / L;
+    if (!loaded) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const int row = row0 + r * P + rsub;
+            load_w<FMT, CPL, L>(tg[r], gq, gs, n_in, row, sub, row < n_out);
+            load_w<FMT, CPL, L>(tu[r], uq, us, n_in, row, sub, row < n_out);
+        }
+    }
+    XChunks<FMT, CPL> x;
+    load_x<FMT, CPL, L>(x, xq, xs, sub);
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+        float ag = reduce_lanes<L>(dot_chunks<FMT, CPL>(tg[r], x));
+        float au = reduce_lanes<L>(dot_chunks<FMT, CPL>(tu[r], x));
+        const int row = row0 + r * P + rsub;
+        if (sub == 0 && row < n_out) {
+            ag *= sg;
+            au *= su;
+            out[row] = it_silu(ag) * au;
+        }
+    }
+}
+
+template <int EF, int ECPL, int EL, int SF, int SCPL, int SL>
+__global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
+    __shared__ __align__(16) int8_t xq[FT * 8];
+    __shared__ float xs[FT * 8 / 32];
+    __shared__ double red[FW];
+    __shared__ RouteLds<FT> route_sh;
+    __shared__ int ids[16];
+    __shared__ float wts[16];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_in = p.n_in;
+    const int routed_groups = p.n_used * gg.e_groups;
+    const int total = routed_groups + gg.s_groups;
+    const int gstride = gridDim.x * FW;
+    int g = blockIdx.x * FW + wave;
+
+    // a wave whose first job is a shared-expert group knows its rows before the router has run
+    WChunks<SCPL> sg[2], su[2];
+    const bool pre = g >= routed_groups && g < total;
+    if (pre) {
+        constexpr int P = 64 / SL, RB = SCPL >= 2 ? 1 : 2;
+        const int row0 = (g - routed_groups) * gg.s_rg;
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const int row = row0 + r * P + lane / SL;
+            load_w<SF, SCPL, SL>(sg[r], p.sh_gq, p.sh_gs, n_in, row, lane % SL, row < p.sh_n_out);
+            load_w<SF, SCPL, SL>(su[r], p.sh_uq, p.sh_us, n_in, row, lane % SL, row < p.sh_n_out);
+        }
+    }
+
+    stage_activation<FT>(p.x, n_in, 0, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, xq, xs, red);
+    if (p.logits) {
+        block_route<FT>(p.logits, p.n_expert, p.n_used, route_sh, ids, wts);
+        if (blockIdx.x == 0 && tid < p.n_used) {
+            p.route_ids_out[tid] = ids[tid];
+            p.route_w_out[tid] = wts[tid];
+        }
+    } else {
+        if (tid < p.n_used) ids[tid] = p.route_ids[tid];
+        __syncthreads();
+    }
+    bool loaded = pre;
+    for (; g < total; g += gstride) {
+        if (g < routed_groups) {
+            const int y = g / gg.e_groups, row0 = (g - y * gg.e_groups) * gg.e_rg;
+            const int64_t e = ids[y];
+            const float scg = p.gscale2 ? p.gscale2[e] : 1.0f, scu = p.uscale2 ? p.uscale2[e] : 1.0f;
+            WChunks<ECPL> tg[2], tu[2];
+            glu_job<EF, ECPL, EL>(p.gq + e * p.q_stride, p.gs + e * p.s_stride, p.uq + e * p.q_stride,
+                                  p.us + e * p.s_stride, n_in, p.n_out, row0, scg, scu, xq, xs,
+                                  p.out + (int64_t)y * p.n_out, lane, tg, tu, false);
+        } else {
+            const int row0 = (g - routed_groups) * gg.s_rg;
+            glu_job<SF, SCPL, SL>(p.sh_gq, p.sh_gs, p.sh_uq, p.sh_us, n_in, p.sh_n_out, row0, 1.0f, 1.0f, xq, xs,
+                                  p.sh_out, lane, sg, su, loaded);
+        }
+        loaded = false;
+    }
+}
+
+}  // namespace
+
+bool moe_glu_fast(MoeGluP p, hipStream_t s) {
+    if (p.exact) return false;
+    const Geo ge = geo_of(p.fmt, p.n_in), gs = geo_of(p.sh_fmt, p.n_in);
+    if (!ge.ok || !gs.ok || p.n_in > FT * 8 || p.n_used > 16 || p.n_used < 1) return false;
+    if (p.logits && (p.n_expert > FT * 4 || p.n_expert < p.n_used || !p.route_ids_out || !p.route_w_out)) return false;
+    if (!p.logits && !p.route_ids) return false;
+    if (!aligned16(p.x) || !aligned16(p.gq) || !aligned16(p.uq) || !aligned16(p.sh_gq) || !aligned16(p.sh_uq)) return false;
+    if (p.q_stride % 16 || p.s_stride % 2) return false;
+    GluGeo gg{};
+    gg.e_cpl = ge.cpl;
+    gg.e_l = ge.l;
+    gg.e_rg = (ge.cpl >= 2 ? 1 : 2) * (64 / ge.l);
+    gg.e_groups = (p.n_out + gg.e_rg - 1) / gg.e_rg;
+    gg.s_cpl = gs.cpl;
+    gg.s_l = gs.l;
+    gg.s_rg = (gs.cpl >= 2 ? 1 : 2) * (64 / gs.l);
+    gg.s_groups = (p.sh_n_out + gg.s_rg - 1) / gg.s_rg;
+    const int total = p.n_used * gg.e_groups + gg.s_groups;
+    int blocks = (total + FW - 1) / FW;
+    if (blocks > 1024) blocks = 1024;
+    if (blocks < 1) blocks = 1;
+    // the geometry of both formats follows from n_in: (CPL, L) for Q8_0 and for NVFP4
+#define IT_LAUNCH(EF, EC, EL, SF, SC, SL) \
+    hipLaunchKernelGGL((moe_glu_fast_k<EF, EC, EL, SF, SC, SL>), dim3(blocks), dim3(FT), 0, s, p, gg)
+#define IT_BY_FMT(QC, QL, NC, NL)                                                                       \
+    do {                                                                                                \
+        if (p.fmt == W_Q8_0 && p.sh_fmt == W_Q8_0) IT_LAUNCH(W_Q8_0, QC, QL, W_Q8_0, QC, QL);           \
+        else if (p.fmt == W_NVFP4 && p.sh_fmt == W_Q8_0) IT_LAUNCH(W_NVFP4, NC, NL, W_Q8_0, QC, QL);    \
+        else if (p.fmt == W_NVFP4 && p.sh_fmt == W_NVFP4) IT_LAUNCH(W_NVFP4, NC, NL, W_NVFP4, NC, NL);  \
+        else IT_LAUNCH(W_Q8_0, QC, QL, W_NVFP4, NC, NL);                                                \
+    } while (0)
+    switch (p.n_in) {
+        case 256: IT_BY_FMT(1, 16, 1, 8); break;
+        case 512: IT_BY_FMT(1, 32, 1, 16); break;
+        case 1024: IT_BY_FMT(1, 64, 1, 32); break;
+        case 2048: IT_BY_FMT(2, 64, 1, 64); break;
+        case 4096: IT_BY_FMT(4, 64, 2, 64); break;
+        default: return false;
+    }
+#undef IT_BY_FMT
+#undef IT_LAUNCH
+    return true;
+}
+
+namespace {
+
+// ------------------------------------------------------------------ moe_down, fast
+// x[j] += sum_y w_y * scale2_y * (down_y[j] . g_y) + sigmoid(logit) * (shared_down[j] . g_sh)
+// One wave step covers P = 64 / L output rows for every pick and the shared expert, so the
+// sum over experts never leaves the lane.
+constexpr int DT = 256, DW = DT / 64;
+constexpr int MAXU = 16;
+
+template <int EF, int ECPL, int L, int SF, int SCPL>
+__global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int P = 64 / L;
+    const int n_in = p.n_in, sh_in = p.sh_n_in, NU = p.n_used;
+    const int total = NU * n_in + sh_in;  // floats staged: picks back to back, then the shared vector
+    int8_t* xq = (int8_t*)smem;
+    float* xs = (float*)(smem + ((total + 15) & ~15));
+    __shared__ int ids[MAXU];
+    __shared__ float coef[MAXU];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int sub = lane % L, rsub = lane / L;
+    const int row = (blockIdx.x * DW + wave) * P + rsub;
+    const bool live = row < p.n_out;
+
+    // weights first: ids come from global, then every pick's chunk and the shared one
+    WChunks<ECPL> t[MAXU];
+    WChunks<SCPL> tsh;
+#pragma unroll
+    for (int y = 0; y < MAXU; y++) {
+        if (y < NU) {
+            const int64_t e = p.route_ids[y];
+            load_w<EF, ECPL, L>(t[y], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row, sub, live);
+        }
+    }
+    load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
+    if (tid < NU) {
+        const int e = p.route_ids[tid];
+        ids[tid] = e;
+        coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[e] : 1.0f);
+    }
+    const float gate = it_sigmoid(p.logit[0]);
+
+    // quantize all NU + 1 intermediates into LDS, four quads per thread per round
+    const int nq = total >> 2, nq_routed = (NU * n_in) >> 2;
+    for (int base = 0; base < nq; base += 4 * DT) {
+        float4 v[4];
+        bool lv[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int qi = base + k * DT + tid;
+            lv[k] = qi < nq;
+            v[k] = !lv[k] ? make_float4(0.f, 0.f, 0.f, 0.f)
+                          : qi < nq_routed ? ((const float4*)p.g_all)[qi] : ((const float4*)p.g_shared)[qi - nq_routed];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) quant_quad(v[k], lv[k], base + k * DT + tid, xq, xs);
+    }
+    __syncthreads();
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int y = 0; y < MAXU; y++) {
+        if (y < NU) {
+            XChunks<EF, ECPL> x;
+            load_x<EF, ECPL, L>(x, xq + y * n_in, xs + y * (n_in >> 5), sub);
+            acc += coef[y] * dot_chunks<EF, ECPL>(t[y], x);
+        }
+    }
+    {
+        XChunks<SF, SCPL> x;
+        load_x<SF, SCPL, L>(x, xq + NU * n_in, xs + NU * (n_in >> 5), sub);
+        acc += gate * dot_chunks<SF, SCPL>(tsh, x);
+    }
+    acc = reduce_lanes<L>(acc);
+    if (sub == 0 && live) p.x[row] += acc;
+}
+
+}  // namespace
+
+bool moe_down_fast(MoeDownP p, hipStream_t s) {
+    const Geo ge = geo_of(p.fmt, p.n_in);
+    if (!ge.ok || ge.cpl != 1 || p.n_used > MAXU || p.n_used < 1) return false;
+    const int L = ge.l;
+    // the shared expert's row is spread over the same L lanes
+    const int per_s = p.sh_fmt == W_Q8_0 ? 16 : p.sh_fmt == W_NVFP4 ? 32 : 0;
+    if (!per_s || p.sh_n_in % 32 || p.n_in % 32) return false;
+    const int cpr_s = p.sh_n_in / per_s;
+    if (cpr_s % L) return false;
+    const int scpl = cpr_s / L;
+    if (scpl != 1 && scpl != 2) return false;
+    if (!aligned16(p.g_all) || !aligned16(p.g_shared) || !aligned16(p.q) || !aligned16(p.sh_q) || p.q_stride % 16 ||
+        p.s_stride % 2)
+        return false;
+    const int total = p.n_used * p.n_in + p.sh_n_in;
+    const size_t lds = (size_t)((total + 15) & ~15) + (size_t)(total / 32) * 4;
+    if (lds > 60 * 1024) return false;
+    const int P = 64 / L;
+    const int blocks = (p.n_out + DW * P - 1) / (DW * P);
+#define IT_LAUNCH(EF, LL, SF, SC) hipLaunchKernelGGL((moe_down_fast_k<EF, 1, LL, SF, SC>), dim3(blocks), dim3(DT), lds, s, p)
+#define IT_BY_L(EF, SF, SC)                      \
+    do {                                         \
+        if (L == 64) IT_LAUNCH(EF, 64, SF, SC);  \
+        else if (L == 32) IT_LAUNCH(EF, 32, SF, SC); \
+        else if (L == 16) IT_LAUNCH(EF, 16, SF, SC); \
+        else IT_LAUNCH(EF, 8, SF, SC);           \
+    } while (0)
+    if (p.fmt == W_NVFP4 && p.sh_fmt == W_Q8_0) {
+        if (scpl == 1) IT_BY_L(W_NVFP4, W_Q8_0, 1);
+        else IT_BY_L(W_NVFP4, W_Q8_0, 2);
+    } else if (p.fmt == W_Q8_0 && p.sh_fmt == W_Q8_0) {
+        if (scpl == 1) IT_BY_L(W_Q8_0, W_Q8_0, 1);
+        else IT_BY_L(W_Q8_0, W_Q8_0, 2);
+    } else if (p.fmt == W_NVFP4 && p.sh_fmt == W_NVFP4) {
+        if (scpl == 1) IT_BY_L(W_NVFP4, W_NVFP4, 1);
+        else IT_BY_L(W_NVFP4, W_NVFP4, 2);
+    } else {
+        return false;
+    }
+#undef IT_BY_L
+#undef IT_LAUNCH
+    return true;
+}
+
+}  // namespace itk

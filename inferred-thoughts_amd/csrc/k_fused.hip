@@ -362,14 +362,24 @@ __global__ __launch_bounds__(FG_THREADS) void fused_gemv_k(FusedGemvP p) {
 }
 
 void fused_gemv(FusedGemvP p, hipStream_t s) {
+    if (fused_gemv_fast(p, s)) return;
     constexpr int W = FG_THREADS / 64;
     int total_rows = 0;
     for (int i = 0; i < p.n_mats; i++) total_rows += p.m[i].n_out;
     const int nb = p.n_in / 32;
     // enough waves to cover HBM latency: aim for ~4096 row groups, at most 512 items per wave pass
+    // fewest passes per wave over 256 blocks of W waves, then the fewest rows per pass
     int R = 1;
-    while (R < 16 && total_rows / (R * 2) >= 4096) R *= 2;
-    while (R > 1 && R * nb > 512) R /= 2;
+    {
+        int best = 1 << 30;
+        for (int r = 1; r <= 16 && r * nb <= 512; r *= 2) {
+            int passes = ((total_rows + r - 1) / r + 256 * W - 1) / (256 * W);
+            if (passes < best) {
+                best = passes;
+                R = r;
+            }
+        }
+    }
     auto lds_for = [&](int r) {
         return (size_t)p.n_in * 4 + (size_t)((nb + 3) & ~3) * 4 + p.n_in + (size_t)W * r * (nb * 2 + 4) * 4;
     };
@@ -607,6 +617,7 @@ __global__ __launch_bounds__(256) void moe_glu_fused_k(MoeGluP p) {
 }
 
 void moe_glu_fused(MoeGluP p, hipStream_t s) {
+    if (moe_glu_fast(p, s)) return;
     const int nb = p.n_in / 32;
     int R = 4;
     while (R > 1 && R * nb > 256) R /= 2;
@@ -711,6 +722,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_k(MoeDownP p) {
 }
 
 void moe_down_fused(MoeDownP p, hipStream_t s) {
+    if (!p.exact && moe_down_fast(p, s)) return;
     const int nb = p.n_in / 32, sh_nb = p.sh_n_in / 32;
     const int T = (p.fmt == W_NVFP4 ? nb * 2 : nb), shT = (p.sh_fmt == W_NVFP4 ? sh_nb * 2 : sh_nb);
     const int Tmax = T > shT ? T : shT;

@@ -102,7 +102,7 @@ struct AttnArgs {
 // scratch: n_q * n_head * n_pos floats.
 void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s);
 // split-K flash decoding; scratch: n_q*n_head*n_split*(head_dim+2) floats.
-int attend_split_count(int n_pos_max);
+int attend_split_count(int n_pos_max, int n_q, int head_dim, int group);
 void attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);
 // the same with the merge multiplying by sigmoid(gate[head * gate_stride + i]) (n_q == 1)
 void attend_split_gated(const AttnArgs& a, int n_split_max, float* scratch, float* out, const float* gate,

@@ -52,7 +52,12 @@ struct MoeGluP {
     int sh_fmt, sh_n_out;
     float* out;            // [n_used][n_out]
     float* sh_out;         // [sh_n_out]
-    const int32_t* route_ids;  // [n_used], chosen by the router kernel
+    const int32_t* route_ids;  // [n_used], chosen by the router kernel (when logits is null)
+    // fast mode: the router logits; every block ranks them itself and block 0 publishes the
+    // picks and their weights for the down kernel
+    const float* logits;
+    int32_t* route_ids_out;
+    float* route_w_out;
 };
 void moe_glu_fused(MoeGluP p, hipStream_t s);
 
@@ -62,7 +67,7 @@ struct MoeDownP {
     const uint8_t *q, *s;
     const float* scale2;
     int64_t q_stride, s_stride;
-    int fmt, n_in, n_out, n_used, rows_per_wave;
+    int fmt, n_in, n_out, n_used, rows_per_wave, exact;
     const uint8_t *sh_q, *sh_s;
     int sh_fmt, sh_n_in;
     const int32_t* route_ids;
@@ -83,5 +88,12 @@ struct AttnPrepP {
     float eps;
 };
 void attn_prep(const AttnPrepP& p, hipStream_t s);
+
+// Fast-mode forms (reductions in wave order).  Each returns false without launching when
+// the shapes, formats or alignments fall outside what it handles; the caller then uses the
+// order-preserving kernel.
+bool fused_gemv_fast(FusedGemvP p, hipStream_t s);
+bool moe_glu_fast(MoeGluP p, hipStream_t s);
+bool moe_down_fast(MoeDownP p, hipStream_t s);
 
 }  // namespace itk

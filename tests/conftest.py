@@ -27,6 +27,16 @@ def tiny_gguf(tmp_path_factory):
 
 
 @pytest.fixture(scope="session")
+def mid_gguf(tmp_path_factory):
+    """Config 5's layer shapes and formats (hidden 2048, NVFP4 experts of 512, head_dim 256, dk = dv = 128,
+    top-10 routing) cut down to 4 layers, 32 experts and a vocabulary of 8192: about 0.4 GB."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "mid_nvfp4.gguf"
+    ih.synth_write_gguf(str(p), ih.big_config(seed=2, n_layer=4, n_vocab=8192, n_expert=32, n_threads=8))
+    return p
+
+
+@pytest.fixture(scope="session")
 def tiny_nvfp4_gguf(tmp_path_factory):
     """The tiny shape with NVFP4 experts and per-expert scales (exercises config 5's formats)."""
     import inferred_hip as ih
