@@ -155,7 +155,7 @@ IT_DEV double quad_sumsq(float4 v) {
 //   silu(gate) (head_dim / 4 a power of two <= 64, so a head sits inside one wave).
 // Ends with a block barrier; xq / xs are then complete.
 template <int THREADS>
-__device__ void stage_activation(const float* x, int n_in, int mode, const float* norm_w, const float* gate, int head_dim,
+__device__ __forceinline__ void stage_activation(const float* x, int n_in, int mode, const float* norm_w, const float* gate, int head_dim,
                                  float eps, float* copy1, float* copy2, int8_t* xq, float* xs, double* red) {
     const int tid = threadIdx.x;
     const int nq = n_in >> 2;
@@ -362,20 +362,67 @@ namespace {
 // ------------------------------------------------------------------ router in a block
 // softmax over n_expert logits, the n_used largest by (probability descending, id ascending),
 // weights = picked probabilities over their sum in pick order (src/ops/mod.rs:1191-1216,
-// naive.rs:362-376).  Every thread of the block calls this; ids / wts (LDS, n_used entries) are
-// complete after the final barrier.  n_expert <= 4 * THREADS, n_used <= 16.
+// naive.rs:362-376).  Every thread of the block calls this.  After it returns, ids[r] and
+// wts[r] (LDS, 16 entries, zero past n_used) hold pick r and its probability; the return
+// value is the weights' denominator, the same in every thread.
+// n_expert <= 4 * THREADS, n_used <= 16.
 //
-// Selection is two-level.  (a) Every wave ranks its own 64 * K values against each other with
-// lane broadcasts: only values of wave rank < n_used can be in the global top n_used, and they
-// go to cand[wave][rank].  (b) The NW * n_used candidates are ranked against each other.
+// Selection is two-level, with every LDS loop of fixed length so its reads pipeline.  (a) Each
+// thread ranks its values among the 64 * K of its wave: only wave ranks < n_used can be in the
+// global top n_used, and they go to cand[wave][rank].  (b) The NW * 16 candidate slots are
+// ranked against each other.//
+// Probabilities are non-negative, so their bit patterns order like the values; a pick is
+// compared as the 64-bit key (probability bits, ~id): larger key = earlier pick, keys are
+// unique, and an empty slot is key 0.
 template <int THREADS> struct RouteLds {
     float redf[2 * (THREADS / 64)];
-    float cand_p[(THREADS / 64) * 16];
-    int cand_e[(THREADS / 64) * 16];
+    __attribute__((aligned(16))) unsigned long long keys[4 * THREADS];
+    __attribute__((aligned(16))) unsigned long long cand[(THREADS / 64) * 16];
 };
 
+IT_DEV unsigned long long route_key(float p, int e) {
+    return ((unsigned long long)__float_as_uint(p) << 32) | (unsigned long long)(~(unsigned)e);
+}
+
+// ranks this thread's key among the 64 keys of its wave and files the top n_used (n_expert <= THREADS)
+IT_DEV void wave_rank_one(const unsigned long long* wave_keys, unsigned long long key, int n_used,
+                          unsigned long long* cand) {
+    int rank = 0;
+    const ulonglong2* p2 = (const ulonglong2*)wave_keys;
+#pragma unroll
+    for (int j2 = 0; j2 < 32; j2++) {
+        const ulonglong2 q = p2[j2];
+        rank += q.x > key ? 1 : 0;
+        rank += q.y > key ? 1 : 0;
+    }
+    if (key != 0ull && rank < n_used) cand[rank] = key;
+}
+
+// the same with up to four keys per thread (n_expert > THREADS): kept out of line and rolled,
+// so the common kernel does not carry its registers
 template <int THREADS>
-__device__ void block_route(const float* logits, int n_expert, int n_used, RouteLds<THREADS>& sh, int* ids, float* wts) {
+__device__ __attribute__((noinline)) void wave_rank_many(const unsigned long long* keys, unsigned long long key0,
+                                                         unsigned long long key1, unsigned long long key2,
+                                                         unsigned long long key3, int K, int n_used,
+                                                         unsigned long long* cand) {
+    const unsigned long long key[4] = {key0, key1, key2, key3};
+    int rank[4] = {0, 0, 0, 0};
+    for (int k2 = 0; k2 < K; k2++) {
+        const unsigned long long* wk = keys + k2 * THREADS + (threadIdx.x & ~63);
+#pragma unroll 1
+        for (int j = 0; j < 64; j++) {
+            const unsigned long long q = wk[j];
+#pragma unroll
+            for (int k = 0; k < 4; k++) rank[k] += q > key[k] ? 1 : 0;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (k < K && key[k] != 0ull && rank[k] < n_used) cand[rank[k]] = key[k];
+}
+
+template <int THREADS>
+__device__ __forceinline__ float block_route(const float* logits, int n_expert, int n_used, RouteLds<THREADS>& sh, int* ids, float* wts) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int NW = THREADS / 64;
     const int K = (n_expert + THREADS - 1) / THREADS;  // experts per thread that can be live
@@ -384,10 +431,11 @@ __device__ void block_route(const float* logits, int n_expert, int n_used, Route
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int e = tid + k * THREADS;
-        l[k] = e < n_expert ? logits[e] : -INFINITY;
+        l[k] = (k < K && e < n_expert) ? logits[e] : -INFINITY;
         m = fmaxf(m, l[k]);
     }
-    if (tid < NW * 16) sh.cand_e[tid] = -1;  // a wave with fewer than n_used live experts leaves slots unset
+    if (tid < NW * 16) sh.cand[tid] = 0ull;  // slots a wave does not fill stay empty
+    if (tid < 16) wts[tid] = 0.0f;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
     if (lane == 0) sh.redf[wave] = m;
@@ -400,7 +448,7 @@ __device__ void block_route(const float* logits, int n_expert, int n_used, Route
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int e = tid + k * THREADS;
-        v[k] = e < n_expert ? it_expf(l[k] - m) : 0.0f;
+        v[k] = (k < K && e < n_expert) ? it_expf(l[k] - m) : 0.0f;
         part += v[k];
     }
 #pragma unroll
@@ -410,58 +458,47 @@ __device__ void block_route(const float* logits, int n_expert, int n_used, Route
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < NW; i++) sum += sh.redf[NW + i];
-#pragma unroll
-    for (int k = 0; k < 4; k++) v[k] = v[k] / sum;
-
-    // dead slots (id >= n_expert) hold 0 and the largest ids, so they never outrank a live one
-    int rank[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) {
-        if (k2 >= K) continue;
-        for (int j = 0; j < 64; j++) {
-            const float q = __shfl(v[k2], j, 64);
-            const int qe = (tid & ~63) + j + k2 * THREADS;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                if (k >= K) continue;
-                const int e = tid + k * THREADS;
-                rank[k] += (q > v[k] || (q == v[k] && qe < e)) ? 1 : 0;
-            }
-        }
-    }
+    unsigned long long key[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int e = tid + k * THREADS;
-        if (k < K && e < n_expert && rank[k] < n_used) {
-            sh.cand_p[wave * 16 + rank[k]] = v[k];
-            sh.cand_e[wave * 16 + rank[k]] = e;
-        }
+        v[k] = v[k] / sum;
+        key[k] = (k < K && e < n_expert) ? route_key(v[k], e) : 0ull;
+        if (k < K) sh.keys[e] = key[k];
     }
     __syncthreads();
-    if (tid < NW * 16 && (tid & 15) < n_used) {
-        const int me = sh.cand_e[tid];
-        if (me >= 0) {
-            const float pv = sh.cand_p[tid];
-            int cnt = 0;
-            for (int w = 0; w < NW; w++)
-                for (int r = 0; r < n_used; r++) {
-                    const int qe = sh.cand_e[w * 16 + r];
-                    const float q = sh.cand_p[w * 16 + r];
-                    cnt += (qe >= 0 && (q > pv || (q == pv && qe < me))) ? 1 : 0;
-                }
-            if (cnt < n_used) {
-                ids[cnt] = me;
-                wts[cnt] = pv;
-            }
+    if (K == 1) wave_rank_one(sh.keys + (tid & ~63), key[0], n_used, sh.cand + wave * 16);
+    else wave_rank_many<THREADS>(sh.keys, key[0], key[1], key[2], key[3], K, n_used, sh.cand + wave * 16);
+    __syncthreads();
+    {
+        // four threads per candidate slot, a quarter of the slots each
+        const int c = tid >> 2, part = tid & 3;
+        const unsigned long long me = sh.cand[c];
+        int cnt = 0;
+#pragma unroll
+        for (int c2 = 0; c2 < NW * 2; c2++) {
+            const ulonglong2 q = ((const ulonglong2*)sh.cand)[part * NW * 2 + c2];
+            cnt += q.x > me ? 1 : 0;
+            cnt += q.y > me ? 1 : 0;
+        }
+        cnt += __shfl_xor(cnt, 1, 64);
+        cnt += __shfl_xor(cnt, 2, 64);
+        if (part == 0 && me != 0ull && cnt < n_used) {
+            ids[cnt] = (int)~(unsigned)(me & 0xffffffffull);
+            wts[cnt] = __uint_as_float((unsigned)(me >> 32));
         }
     }
     __syncthreads();
     float s = 0.0f;
-    for (int r = 0; r < n_used; r++) s += wts[r];
-    const float denom = fmaxf(s, 6.103515625e-5f);
-    __syncthreads();
-    if (tid < n_used) wts[tid] = wts[tid] / denom;
-    __syncthreads();
+#pragma unroll
+    for (int r4 = 0; r4 < 4; r4++) {
+        const float4 w = ((const float4*)wts)[r4];
+        s += w.x;
+        s += w.y;
+        s += w.z;
+        s += w.w;
+    }
+    return fmaxf(s, 6.103515625e-5f);
 }
 
 // ------------------------------------------------------------------ moe_glu, fast
@@ -509,7 +546,7 @@ __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
     __shared__ double red[FW];
     __shared__ RouteLds<FT> route_sh;
     __shared__ int ids[16];
-    __shared__ float wts[16];
+    __shared__ __align__(16) float wts[16];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_in = p.n_in;
@@ -534,10 +571,10 @@ __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
 
     stage_activation<FT>(p.x, n_in, 0, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, xq, xs, red);
     if (p.logits) {
-        block_route<FT>(p.logits, p.n_expert, p.n_used, route_sh, ids, wts);
+        const float denom = block_route<FT>(p.logits, p.n_expert, p.n_used, route_sh, ids, wts);
         if (blockIdx.x == 0 && tid < p.n_used) {
             p.route_ids_out[tid] = ids[tid];
-            p.route_w_out[tid] = wts[tid];
+            p.route_w_out[tid] = wts[tid] / denom;
         }
     } else {
         if (tid < p.n_used) ids[tid] = p.route_ids[tid];
