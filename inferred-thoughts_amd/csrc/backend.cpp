@@ -147,8 +147,13 @@ void it_hip::finish_pass() {
     for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
     precopies.clear();
     dyn_upload();
-    check(hipGraphLaunch(graph.exec, stream), "hipGraphLaunch");
-    graph_launches++;
+    if (profile_pass) {
+        run_fused(pending);  // the launches the graph holds, each between two events
+        check(hipGetLastError(), "kernel launch");
+    } else {
+        check(hipGraphLaunch(graph.exec, stream), "hipGraphLaunch");
+        graph_launches++;
+    }
     pending.clear();
 }
 
@@ -841,7 +846,7 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         it_hip::OpRec rec;
         rec.id = OP_ATTEND; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = dyn; rec.p[4] = sc; rec.p[5] = dout;
         rec.i[0] = args.n_q; rec.i[1] = args.kv_dim; rec.i[2] = args.head_dim; rec.i[3] = args.n_head;
-        rec.i[4] = args.n_head_kv; rec.i[6] = 1; rec.f[0] = args.scale;  // exact form: launched as is
+        rec.i[4] = args.n_head_kv; rec.i[6] = 1; rec.i[8] = (int64_t)a->n_pos; rec.f[0] = args.scale;  // exact form: launched as is
         be->submit(it_hip::FAM_ATTEND, bytes,
                    sig_of(OP_ATTEND, 0, sg.q, sg.k, sg.v, sg.n_q, sg.kv_dim, dyn ? sg.n_pos : 0, sg.head_dim, sg.n_head,
                           sg.n_head_kv, sg.scale, dyn, sc, dout), rec,
@@ -856,7 +861,8 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         it_hip::OpRec rec;
         rec.id = OP_ATTEND; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = dyn; rec.p[4] = sc; rec.p[5] = dout;
         rec.i[0] = args.n_q; rec.i[1] = args.kv_dim; rec.i[2] = args.head_dim; rec.i[3] = args.n_head;
-        rec.i[4] = args.n_head_kv; rec.i[5] = n_split; rec.i[6] = 0; rec.i[7] = args.n_pos; rec.f[0] = args.scale;
+        rec.i[4] = args.n_head_kv; rec.i[5] = n_split; rec.i[6] = 0; rec.i[7] = args.n_pos; rec.i[8] = (int64_t)a->n_pos;
+        rec.f[0] = args.scale;
         be->submit(it_hip::FAM_ATTEND, bytes,
                    sig_of(OP_ATTEND, 1, dq, dk, dv, args.n_q, args.kv_dim, args.head_dim, args.n_head, args.n_head_kv,
                           args.scale, dyn, dyn ? n_split : 0, sc, dout), rec,
@@ -1244,10 +1250,14 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
     be->dyn_rotate();
     be->replay_cursor = 0;
     be->mode = it_hip::Mode::Eager;
-    if (n_tokens == 1 && be->allow_graph && !be->mid_pass_read && !be->prof_on && !be->has_error) {
+    be->profile_pass = false;
+    if (n_tokens == 1 && be->allow_graph && !be->mid_pass_read && !be->has_error) {
         if (be->graph.valid) {
+            // while profiling, the pass is recorded like a replay and its fused launches are
+            // then issued one by one between timing events instead of as the graph
             be->mode = it_hip::Mode::Replay;
-        } else if (be->stable_passes >= 1) {
+            be->profile_pass = be->prof_on;
+        } else if (be->stable_passes >= 1 && !be->prof_on) {
             be->mode = it_hip::Mode::Capture;
         }
     }
@@ -1439,7 +1449,9 @@ void it_hip_profile_begin(it_hip* be) {
 int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
     static const char* names[it_hip::FAM_COUNT] = {"matmul (dense GEMV/GEMM)", "moe_glu (expert gate+up)",
                                                    "matmul_experts (expert down)", "delta_rule", "attend",
-                                                   "norms", "router (softmax + top-k)", "other"};
+                                                   "norms", "router (softmax + top-k)", "other",
+                                                   "fused_gemv (norm + quantize + dense GEMVs)", "lm_head (norm + GEMV)",
+                                                   "gdn_rows (l2 norm + delta rule)", "attn_prep (norm + rope + kv write)"};
     be->prof_on = false;
     be->check(hipStreamSynchronize(be->stream), "sync");
     it_profile_row acc[it_hip::FAM_COUNT];

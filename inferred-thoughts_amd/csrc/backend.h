@@ -189,6 +189,7 @@ struct it_hip {
     void need_eager(const char* why); // leave capture/replay: run what the pass queued so far eagerly
     void finish_pass();
     bool mid_pass_read = false;
+    bool profile_pass = false;  // a replay-shaped pass whose fused launches run one by one between timing events
 
     // Every kernel launch goes through here.  `sig` hashes the launch's static arguments
     // (pointers, shapes); position-dependent scalars never enter it.
@@ -215,7 +216,8 @@ struct it_hip {
     }
 
     // ---- per-kernel-family timing with HIP events on the launch stream
-    enum Family { FAM_MATMUL = 0, FAM_MOE_GLU, FAM_MOE_DOWN, FAM_DELTA, FAM_ATTEND, FAM_NORM, FAM_ROUTER, FAM_OTHER, FAM_COUNT };
+    enum Family { FAM_MATMUL = 0, FAM_MOE_GLU, FAM_MOE_DOWN, FAM_DELTA, FAM_ATTEND, FAM_NORM, FAM_ROUTER, FAM_OTHER,
+                  FAM_FUSED_GEMV, FAM_LM_HEAD, FAM_GDN_ROWS, FAM_ATTN_PREP, FAM_COUNT };
     struct ProfSpan {
         hipEvent_t a, b;
         int fam;

@@ -19,7 +19,15 @@ namespace {
 struct Plan {
     std::vector<Op>& ops;
     std::vector<char> consumed;
-    std::vector<std::vector<std::function<void(hipStream_t)>>> at;  // fused launches keyed by position
+    struct Launch {
+        int fam;         // it_hip::Family, for the per-kernel timing
+        uint64_t bytes;  // algorithmic bytes of the launch (weights + state it must move once)
+        std::function<void(hipStream_t)> fn;
+    };
+    std::vector<std::vector<Launch>> at;  // fused launches keyed by position
+    void add(size_t i, int fam, uint64_t bytes, std::function<void(hipStream_t)> fn) {
+        at[i].push_back(Launch{fam, bytes, std::move(fn)});
+    }
     explicit Plan(std::vector<Op>& o) : ops(o), consumed(o.size(), 0), at(o.size()) {}
     bool ids(size_t i, std::initializer_list<int> want) const {
         if (i + want.size() > ops.size()) return false;
@@ -34,6 +42,16 @@ struct Plan {
 };
 
 bool quantized_fmt(int64_t f) { return f == W_Q8_0 || f == W_NVFP4; }
+
+// bytes of `rows` repacked rows of n_in weights (Q8_0: 34 per 32, NVFP4: 9 per 16)
+uint64_t rows_bytes(int fmt, uint64_t rows, uint64_t n_in) {
+    return fmt == W_NVFP4 ? rows * n_in * 9 / 16 : rows * n_in * 34 / 32;
+}
+uint64_t gemv_bytes(const FusedGemvP& p) {
+    uint64_t b = (uint64_t)p.n_in * 4;
+    for (int i = 0; i < p.n_mats; i++) b += rows_bytes(p.m[i].fmt, p.m[i].n_out, p.n_in) + (uint64_t)p.m[i].n_out * 4;
+    return b;
+}
 
 // MATMUL `m` reads activation `x` (f32) whose Q8_0 form was produced by QUANT `q`, one token.
 bool mm_reads(const Op& m, const void* x, const Op& q) {
@@ -131,9 +149,9 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
 
     pl.take(i, 18);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
-    pl.at[i].push_back([=](hipStream_t s) { gdn_core(c, dki, s); });
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a) + (uint64_t)cdim * 8 * 4, [=](hipStream_t s) { fused_gemv(a, s); });
+    pl.add(i, it_hip::FAM_GDN_ROWS, (uint64_t)nv * dv * dk * 8 + (uint64_t)(cdim + vdim) * 4, [=](hipStream_t s) { gdn_core(c, dki, s); });
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b) + (uint64_t)vdim * 4, [=](hipStream_t s) { fused_gemv(b, s); });
     return true;
 }
 
@@ -167,7 +185,7 @@ bool match_norm_matmuls(Plan& pl, size_t i, int exact) {
     a.n_mats = (int)n;
     for (size_t j = 0; j < n; j++) a.m[j] = mat_of(o[m0 + j], 0);
     pl.take(i, m0 + n - i);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
     return true;
 }
 
@@ -185,7 +203,7 @@ bool match_matmul_residual(Plan& pl, size_t i, int exact) {
     b.n_mats = 1;
     b.m[0] = mat_of(m, 2, (float*)add.p[0]);
     pl.take(i, 3);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b), [=](hipStream_t s) { fused_gemv(b, s); });
     return true;
 }
 
@@ -207,7 +225,7 @@ bool match_final(Plan& pl, size_t i, int exact) {
     a.n_mats = 1;
     a.m[0] = mat_of(m, 0);
     pl.take(i, 4);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
+    pl.add(i, it_hip::FAM_LM_HEAD, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
     return true;
 }
 
@@ -297,18 +315,20 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
 
     pl.take(i, 18);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
-    pl.at[i].push_back([=](hipStream_t s) { attn_prep(pp, s); });
+    // K and V rows of the live context, f16 (the position is the one this pass was recorded at)
+    const uint64_t kv_bytes = (uint64_t)at.i[8] * kvd * 2 * 2;
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
+    pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
     if (at.i[6] == 0) {
-        pl.at[i].push_back([=](hipStream_t s) { attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s); });
+        pl.add(i, it_hip::FAM_ATTEND, kv_bytes, [=](hipStream_t s) { attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s); });
     } else {
         // the exact attention kernel and its gate stay as they are
         auto run_attend = at.run, run_gate = sg.run, run_gather_gate = gg.run;
-        pl.at[i].push_back(run_gather_gate);
-        pl.at[i].push_back(run_attend);
-        pl.at[i].push_back(run_gate);
+        pl.add(i, it_hip::FAM_OTHER, 0, run_gather_gate);
+        pl.add(i, it_hip::FAM_ATTEND, kv_bytes, run_attend);
+        pl.add(i, it_hip::FAM_OTHER, 0, run_gate);
     }
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(b, s); });
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b), [=](hipStream_t s) { fused_gemv(b, s); });
     return true;
 }
 
@@ -424,9 +444,13 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     d.x = (float*)rms.p[0];
 
     pl.take(i, 17);
-    pl.at[i].push_back([=](hipStream_t s) { fused_gemv(a, s); });
-    pl.at[i].push_back([=](hipStream_t s) { moe_glu_fused(g, s); });
-    pl.at[i].push_back([=](hipStream_t s) { moe_down_fused(d, s); });
+    const uint64_t glu_b = 2 * rows_bytes(g.fmt, (uint64_t)nu * ff, nd) + 2 * rows_bytes(g.sh_fmt, sff, nd) + (uint64_t)nd * 4 +
+                           (uint64_t)(nu * ff + sff) * 4;
+    const uint64_t down_b = rows_bytes(d.fmt, (uint64_t)nu * nd, ff) + rows_bytes(d.sh_fmt, nd, sff) +
+                            (uint64_t)(nu * ff + sff) * 4 + (uint64_t)nd * 8;
+    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
+    pl.add(i, it_hip::FAM_MOE_GLU, glu_b, [=](hipStream_t s) { moe_glu_fused(g, s); });
+    pl.add(i, it_hip::FAM_MOE_DOWN, down_b, [=](hipStream_t s) { moe_down_fused(d, s); });
     return true;
 }
 
@@ -465,11 +489,13 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
     }
     uint64_t n = 0;
     for (size_t i = 0; i < ops.size(); i++) {
-        for (auto& f : pl.at[i]) {
-            f(stream);
+        for (auto& l : pl.at[i]) {
+            Span sp(this, l.fam, l.bytes);
+            l.fn(stream);
             n++;
         }
         if (!pl.consumed[i]) {
+            Span sp(this, FAM_OTHER, 0);
             ops[i].run(stream);
             n++;
         }
