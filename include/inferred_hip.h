@@ -192,6 +192,17 @@ int64_t it_hip_clock_pick(uint8_t* heat, const uint8_t* leased, uint64_t n, uint
 /* first strict maximum of a device-current activation, computed on the device
  * (the rule of Profile::record_token, src/profile.rs:192-213) */
 uint32_t it_hip_argmax(it_hip*, const float* buf, uint64_t len);
+/* Greedy feedback without a host round trip: picks the first strict maximum of `logits`
+ * (as it_hip_argmax), writes the dequantized row of `table` for that id into `x`
+ * (Model::embed, src/model/qwen35.rs:855-873: Q8_0, F16, BF16 or F32 tables) and files the
+ * id at ring_index in a device ring of 65536 ids.  Called inside a pass in place of the host
+ * embedding; `logits` names the device copy the previous pass left (the host copy is not
+ * consulted).  Returns 0 without doing anything when the table type is not handled or the
+ * logits have no device copy. */
+int it_hip_embed_argmax(it_hip*, const it_weights* table, const float* logits, uint64_t logits_len, float* x,
+                        uint64_t x_len, uint64_t ring_index);
+/* ids filed by it_hip_embed_argmax at ring indices first_index .. first_index + n (waits for the device) */
+void it_hip_read_tokens(it_hip*, uint64_t first_index, uint64_t n, uint32_t* out);
 void it_hip_sync(it_hip*);
 /* per-kernel-family device time, measured with HIP events recorded on the launch
  * stream around every launch between begin and end (at most 16384 launches) */

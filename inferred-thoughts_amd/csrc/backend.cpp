@@ -9,6 +9,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstdio>
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 
@@ -1382,17 +1383,25 @@ int64_t it_hip_clock_pick(uint8_t* heat, const uint8_t* leased, uint64_t n, uint
 }
 
 // ------------------------------------------------------------------ extensions
+}  // extern "C"
+
+bool it_hip::argmax_ready() {
+    if (argmax_idx) return true;
+    need_eager("argmax scratch is allocated");
+    return check(hipMalloc((void**)&argmax_idx, 64 * 4), "hipMalloc(argmax)") &&
+           check(hipMalloc((void**)&argmax_val, 64 * 4), "hipMalloc(argmax)") &&
+           check(hipMalloc((void**)&argmax_out, 4), "hipMalloc(argmax)") &&
+           check(hipMalloc((void**)&tok_ring, TOK_RING_CAP * 4), "hipMalloc(token ring)") &&
+           check(hipHostMalloc((void**)&argmax_host, 4, hipHostMallocDefault), "hipHostMalloc(argmax)");
+}
+
+extern "C" {
+
 uint32_t it_hip_argmax(it_hip* be, const float* buf, uint64_t len) {
     if (len == 0) return 0;
     float* d = be->act_in(buf, len);
     if (!d) return 0;
-    if (!be->argmax_idx) {
-        if (!be->check(hipMalloc((void**)&be->argmax_idx, 64 * 4), "hipMalloc(argmax)") ||
-            !be->check(hipMalloc((void**)&be->argmax_val, 64 * 4), "hipMalloc(argmax)") ||
-            !be->check(hipMalloc((void**)&be->argmax_out, 4), "hipMalloc(argmax)") ||
-            !be->check(hipHostMalloc((void**)&be->argmax_host, 4, hipHostMallocDefault), "hipHostMalloc(argmax)"))
-            return 0;
-    }
+    if (!be->argmax_ready()) return 0;
     be->need_eager("argmax");
     argmax(d, (int64_t)len, be->argmax_out, be->argmax_idx, be->argmax_val, be->stream);
     be->launches += 2;
@@ -1401,6 +1410,56 @@ uint32_t it_hip_argmax(it_hip* be, const float* buf, uint64_t len) {
     be->d2h++;
     be->d2h_bytes += 4;
     return (uint32_t)*be->argmax_host;
+}
+
+int it_hip_embed_argmax(it_hip* be, const it_weights* table, const float* logits, uint64_t logits_len, float* x,
+                        uint64_t x_len, uint64_t ring_index) {
+    if (!table || !logits || !x || table->n_out != logits_len || table->n_in != x_len || logits_len == 0 ||
+        logits_len >= (1ull << 31))
+        return 0;
+    if (table->ty != IT_Q8_0 && table->ty != IT_F16 && table->ty != IT_BF16 && table->ty != IT_F32) return 0;
+    if (be->has_error) return 0;
+    itk::WView w;
+    if (!be->weights_view(table, "embed_argmax", &w)) return 0;
+    // the logits are read where the previous pass left them: the device mirror, which begin_pass
+    // has already marked stale with respect to the host copy
+    auto lm = be->acts.find(logits);
+    if (lm == be->acts.end() || !lm->second.dev || lm->second.cap < logits_len) return 0;
+    float* dl = lm->second.dev;
+    float* dx = be->act_out(x, x_len);
+    if (!dx || !be->argmax_ready()) return 0;
+    const int slot = (int)(ring_index % it_hip::TOK_RING_CAP);
+    const int* dyn = be->dyn_slot(slot);
+    int32_t *out = be->argmax_out, *idx = be->argmax_idx, *ring = be->tok_ring;
+    float* val = be->argmax_val;
+    int64_t n = (int64_t)logits_len;
+    it_hip::OpRec rec;
+    rec.id = OP_EMBED; rec.p[0] = dl; rec.p[1] = dx; rec.p[2] = w.q; rec.i[0] = n; rec.i[1] = w.n_in;
+    be->launches += 2;
+    be->submit(it_hip::FAM_OTHER, logits_len * 4 + x_len * 6, sig_of(OP_EMBED, dl, dx, w.q, w.scales, w.fmt, n, w.n_in, dyn ? 1 : 0),
+               rec, [=](hipStream_t s) {
+                   argmax(dl, n, out, idx, val, s);
+                   embed_row(w, out, dx, ring, slot, dyn, s);
+               });
+    return 1;
+}
+
+void it_hip_read_tokens(it_hip* be, uint64_t first_index, uint64_t n, uint32_t* out) {
+    if (!n || !out) return;
+    if (be->in_pass) be->finish_pass();
+    if (!be->tok_ring || n > it_hip::TOK_RING_CAP) {
+        be->fail("read_tokens: no tokens were picked on the device, or more than the ring holds");
+        return;
+    }
+    be->check(hipStreamSynchronize(be->stream), "sync before reading token ids");
+    for (uint64_t i = 0; i < n;) {
+        const uint64_t at = (first_index + i) % it_hip::TOK_RING_CAP;
+        const uint64_t take = std::min<uint64_t>(n - i, it_hip::TOK_RING_CAP - at);
+        be->check(hipMemcpy(out + i, be->tok_ring + at, take * 4, hipMemcpyDeviceToHost), "download token ids");
+        i += take;
+    }
+    be->d2h++;
+    be->d2h_bytes += n * 4;
 }
 
 void it_hip_release(it_hip* be, const void* host) {

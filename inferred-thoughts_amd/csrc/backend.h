@@ -41,7 +41,7 @@
 //   ATTEND     p: q, k, v, dyn, scratch, out   i: n_q, kv_dim, head_dim, n_head, n_head_kv, n_split, exact, n_pos  f: scale
 enum OpId : int {
     OP_RMS = 1, OP_RMS_HEADS, OP_L2, OP_MATMUL, OP_ROPE, OP_SOFTMAX, OP_ATTEND, OP_EW, OP_SCALE, OP_CONV, OP_GATHER,
-    OP_SCATTER, OP_DELTA, OP_ROUTE, OP_EXPERTS, OP_GLU, OP_FINISH, OP_ROWS, OP_SIGADD, OP_KVWRITE,
+    OP_SCATTER, OP_DELTA, OP_ROUTE, OP_EXPERTS, OP_GLU, OP_FINISH, OP_ROWS, OP_SIGADD, OP_KVWRITE, OP_EMBED,
     OP_QUANT = 101
 };
 
@@ -135,6 +135,10 @@ struct it_hip {
     float* argmax_val = nullptr;
     int32_t* argmax_out = nullptr;
     int32_t* argmax_host = nullptr;  // pinned
+    bool argmax_ready();
+    // ids picked on the device by embed_argmax, in call order (a ring)
+    int32_t* tok_ring = nullptr;
+    static constexpr size_t TOK_RING_CAP = 1 << 16;
 
     // ---- pass / graph state
     bool in_pass = false;

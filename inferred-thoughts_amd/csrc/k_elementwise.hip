@@ -397,4 +397,37 @@ void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float
     hipLaunchKernelGGL(argmax_final_k, dim3(1), dim3(64), 0, s, scratch_idx, scratch_val, parts, out);
 }
 
+// ------------------------------------------------------------------ embedding row by device token id
+// x[i] = row `*token` of the table, dequantized exactly as the host does (Q8_0: f16 scale
+// times the int8 quant; F16/BF16 widened; F32 copied), and the id is filed in `ring`.
+__global__ __launch_bounds__(256) void embed_row_k(WView w, const int32_t* __restrict__ token, float* __restrict__ x,
+                                                   int32_t* __restrict__ ring, int ring_idx,
+                                                   const int* __restrict__ ring_dyn) {
+    const int64_t tok = *token;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && ring) ring[ring_dyn ? *ring_dyn : ring_idx] = (int32_t)tok;
+    const int n_in = w.n_in;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n_in; i += gridDim.x * 256) {
+        float v;
+        if (w.fmt == W_Q8_0) {
+            const int8_t q = ((const int8_t*)w.q)[tok * n_in + i];
+            const uint16_t d = ((const uint16_t*)w.scales)[tok * (n_in >> 5) + (i >> 5)];
+            v = it_f16_to_f32(d) * (float)q;
+        } else if (w.fmt == W_F16) {
+            v = it_f16_to_f32(((const uint16_t*)w.q)[tok * n_in + i]);
+        } else if (w.fmt == W_BF16) {
+            v = it_bf16_to_f32(((const uint16_t*)w.q)[tok * n_in + i]);
+        } else {
+            v = ((const float*)w.q)[tok * n_in + i];
+        }
+        x[i] = v;
+    }
+}
+
+void embed_row(const WView& w, const int32_t* token, float* x, int32_t* ring, int ring_idx, const int* ring_dyn,
+               hipStream_t s) {
+    int blocks = (w.n_in + 255) / 256;
+    if (blocks > 64) blocks = 64;
+    hipLaunchKernelGGL(embed_row_k, dim3(blocks), dim3(256), 0, s, w, token, x, ring, ring_idx, ring_dyn);
+}
+
 }  // namespace itk

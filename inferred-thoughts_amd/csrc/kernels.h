@@ -80,6 +80,10 @@ void kv_write(uint16_t* slab, int64_t offset, const int* offset_dyn, int64_t off
               int64_t n, hipStream_t s);
 void fill_zero(void* p, int64_t bytes, hipStream_t s);
 void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s);
+// x = dequantized row `*token` of an embedding table (Q8_0 repacked, F16, BF16 or F32); the id goes to
+// ring[ring_dyn ? *ring_dyn : ring_idx] when ring is non-null
+void embed_row(const WView& w, const int32_t* token, float* x, int32_t* ring, int ring_idx, const int* ring_dyn,
+               hipStream_t s);
 
 // ---- gated delta net ---------------------------------------------------------------
 void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,

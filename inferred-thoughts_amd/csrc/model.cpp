@@ -252,6 +252,7 @@ struct it_engine {
     it_hip* be;
     uint64_t n_ctx, max_batch;
     uint64_t len = 0;
+    uint64_t ring_next = 0;  // next slot of the backend's device token ring this engine files into
     std::vector<uint16_t> k_slabs, v_slabs;
     std::vector<float> conv, ssm;
     it_trace_fn trace = nullptr;
@@ -379,21 +380,32 @@ void gated_delta(it_engine* e, const Block& b, uint64_t il, uint64_t n) {
 }
 
 // Runs one pass; logits stay on the device unless `want_logits`.
-int forward(it_engine* e, const uint32_t* tokens, uint64_t n, uint64_t start, bool want_logits) {
+// `tokens == nullptr` is the greedy feedback pass: one token, chosen on the device as the arg-max
+// of the previous pass's logits and embedded there (its id lands at `ring_index` of the device ring).
+int forward(it_engine* e, const uint32_t* tokens, uint64_t n, uint64_t start, bool want_logits,
+            uint64_t ring_index = 0) {
     it_model* m = e->m;
     const Dims& d = m->d;
     it_hip* be = e->be;
     if (n == 0) { e->err = "forward: no tokens supplied"; return -1; }
     if (start + n > e->n_ctx) { e->err = "context overflow: position " + std::to_string(start + n - 1) + " with n_ctx " + std::to_string(e->n_ctx); return -2; }
-    for (uint64_t t = 0; t < n; t++)
+    for (uint64_t t = 0; tokens && t < n; t++)
         if (tokens[t] >= d.n_vocab) { e->err = "token id " + std::to_string(tokens[t]) + " outside the vocabulary"; return -3; }
     uint64_t nd = d.n_embd;
     it_hip_begin_pass(be, n);
     fit(e, n);
-    uint64_t row_bytes = itg::type_bytes(m->tok_embd.ty, nd);
-    for (uint64_t t = 0; t < n; t++)
-        ith::dequantize(m->tok_embd.ty, m->tok_embd.data + tokens[t] * row_bytes, nd, e->x.p() + t * nd);
-    it_hip_host_wrote(be, e->x.p(), n * nd);
+    if (tokens) {
+        uint64_t row_bytes = itg::type_bytes(m->tok_embd.ty, nd);
+        for (uint64_t t = 0; t < n; t++)
+            ith::dequantize(m->tok_embd.ty, m->tok_embd.data + tokens[t] * row_bytes, nd, e->x.p() + t * nd);
+        it_hip_host_wrote(be, e->x.p(), n * nd);
+    } else {
+        if (!it_hip_embed_argmax(be, &m->tok_embd, e->logits.p(), d.n_vocab, e->x.p(), nd, ring_index)) {
+            it_hip_end_pass(be);
+            e->err = "the embedding table's type has no device form";
+            return -4;
+        }
+    }
     e->tr("inp_embd", 0, e->x, n * nd);
     for (uint64_t il = 0; il < d.layers(); il++) {
         const Block& b = m->blocks[il];
@@ -555,9 +567,26 @@ int64_t it_engine_generate(it_engine* e, const uint32_t* prompt, uint64_t n_prom
     return (int64_t)produced;
 }
 
+// Greedy decoding with the token fed back on the device: passes are issued back to back and the
+// host waits once, at the end, to read the ids.  Falls back to a host round trip per token when
+// the embedding table has no device form.
 int64_t it_engine_decode_greedy(it_engine* e, uint64_t n, uint32_t* out_ids) {
     uint64_t nv = e->m->d.n_vocab;
     uint64_t produced = 0;
+    const uint32_t ty = e->m->tok_embd.ty;
+    const bool on_device = ty == IT_Q8_0 || ty == IT_F16 || ty == IT_BF16 || ty == IT_F32;
+    if (on_device) {
+        const uint64_t first = e->ring_next;
+        for (uint64_t i = 0; i < n && i < 65536; i++) {
+            if (e->len + 1 > e->n_ctx) break;
+            int rc = forward(e, nullptr, 1, e->len, false, e->ring_next);
+            if (rc) return rc;
+            e->ring_next++;
+            produced++;
+        }
+        if (produced && out_ids) it_hip_read_tokens(e->be, first, produced, out_ids);
+        return (int64_t)produced;
+    }
     for (uint64_t i = 0; i < n; i++) {
         if (e->len + 1 > e->n_ctx) break;
         uint32_t next = it_hip_argmax(e->be, e->logits.p(), nv);

@@ -91,7 +91,7 @@ it_hip_kv_write it_hip_host_wrote it_hip_host_needs it_hip_begin_pass it_hip_end
 it_hip_read_state it_hip_read_kv it_hip_device_report it_hip_reserve_activations it_hip_tier_counters
 it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_budget
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
-it_hip_clock_pick it_hip_argmax it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_model_open
+it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_model_open
 it_model_close it_model_dims it_model_decode_weight_bytes it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
@@ -122,6 +122,8 @@ def lib() -> C.CDLL:
     vp, u64, u32, f32 = C.c_void_p, c_u64, c_u32, c_f32
     sig = {
         "it_hip_create": (vp, [u32, C.c_int, C.c_char_p, C.c_size_t]),
+        "it_hip_embed_argmax": (C.c_int, [vp, vp, vp, u64, vp, u64, u64]),
+        "it_hip_read_tokens": (None, [vp, u64, u64, vp]),
         "it_hip_destroy": (None, [vp]),
         "it_hip_take_error": (C.c_int, [vp, C.c_char_p, C.c_size_t]),
         "it_hip_check_expert_types": (C.c_int, [u32, u32, u32, C.c_char_p, C.c_size_t]),

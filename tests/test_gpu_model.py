@@ -47,6 +47,26 @@ def test_greedy_tokens_bit_identical(hip, request, which):
     he.close(); hm.close(); oe.close(); om.close()
 
 
+@pytest.mark.parametrize("exact", [True, False])
+def test_device_fed_greedy_decode_equals_host_fed(tiny_gguf, exact):
+    """decode_greedy picks and embeds the next token on the device and never waits for the host between passes;
+    the ids must be the ones the host-fed loop (arg-max on the host, embedding row uploaded) produces."""
+    import inferred_hip as ih
+    prompt = prompt_ids(20, seed=11)
+    be = ih.Hip(exact=exact)
+    hm = ih.Model(tiny_gguf)
+    e1 = ih.Engine(hm, be, 128)
+    ids_host, _ = e1.generate(prompt, 40)
+    e1.close()
+    e2 = ih.Engine(hm, be, 128)
+    e2.prefill(prompt, want_logits=False)
+    ids_dev = np.concatenate([e2.decode_greedy(25), e2.decode_greedy(15)])   # two stretches share one ring
+    assert be.take_error() is None
+    assert np.array_equal(ids_dev, ids_host[:40]), (ids_dev[:10], ids_host[:10])
+    assert be.graph_stats()["replays"] >= 30
+    e2.close(); hm.close(); be.close()
+
+
 def test_batched_prefill_equals_token_by_token(hip, tiny_gguf):
     import inferred_hip as ih
     hip.drop_mirrors()
