@@ -105,6 +105,8 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len);
 void it_hip_destroy(it_hip* be);
 /* Cuda::take_error: 1 and the message when an error is pending (and clears it), else 0 */
 int it_hip_take_error(it_hip* be, char* msg, size_t msg_len);
+/* 1 when an error is already recorded; never waits for the device (extension) */
+int it_hip_has_error(it_hip* be);
 /* check_expert_types, src/ops/mod.rs:29-55, for this backend: 0 = supported */
 int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* msg, size_t msg_len);
 

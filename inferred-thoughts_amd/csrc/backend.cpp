@@ -666,6 +666,8 @@ int it_hip_take_error(it_hip* be, char* msg, size_t msg_len) {
     return 1;
 }
 
+int it_hip_has_error(it_hip* be) { return be->has_error ? 1 : 0; }
+
 int it_hip_check_expert_types(uint32_t gate, uint32_t up, uint32_t down, char* msg, size_t msg_len) {
     auto ok1 = [](uint32_t t) { return t == IT_Q8_0 || t == IT_NVFP4; };
     if (ok1(gate) && gate == up && ok1(down)) return 0;

@@ -434,6 +434,9 @@ int forward(it_engine* e, const uint32_t* tokens, uint64_t n, uint64_t start, bo
     it_hip_end_pass(be);
     if (want_logits) it_hip_host_needs(be, e->logits.p(), d.n_vocab);
     if (e->trace) e->tr("result_output", 0, e->logits, d.n_vocab);
+    // a device-fed pass does not wait for the device: only an error already recorded is looked at,
+    // and the caller polls once, with a wait, after its last pass
+    if (!tokens && !it_hip_has_error(be)) return 0;
     char msg[512];
     if (it_hip_take_error(be, msg, sizeof msg)) {
         e->err = msg;
@@ -584,7 +587,14 @@ int64_t it_engine_decode_greedy(it_engine* e, uint64_t n, uint32_t* out_ids) {
             e->ring_next++;
             produced++;
         }
-        if (produced && out_ids) it_hip_read_tokens(e->be, first, produced, out_ids);
+        if (produced && out_ids) {
+            it_hip_read_tokens(e->be, first, produced, out_ids);
+            char msg[512];
+            if (it_hip_take_error(e->be, msg, sizeof msg)) {
+                e->err = msg;
+                return -10;
+            }
+        }
         return (int64_t)produced;
     }
     for (uint64_t i = 0; i < n; i++) {

@@ -82,7 +82,7 @@ class SynthConfig(C.Structure):
 
 
 # every symbol include/inferred_hip.h declares
-EXPORTS = """it_hip_create it_hip_destroy it_hip_take_error it_hip_check_expert_types it_hip_rms_norm
+EXPORTS = """it_hip_create it_hip_destroy it_hip_take_error it_hip_has_error it_hip_check_expert_types it_hip_rms_norm
 it_hip_rms_norm_heads it_hip_matmul it_hip_rope_neox it_hip_softmax it_hip_attend it_hip_silu_mul
 it_hip_l2_norm_heads it_hip_ssm_conv it_hip_gather_chunks it_hip_sigmoid_mul it_hip_delta_rule
 it_hip_add_assign it_hip_scale it_hip_scatter_chunks it_hip_matmul_pair it_hip_matmul_experts it_hip_moe_glu
@@ -122,6 +122,7 @@ def lib() -> C.CDLL:
     vp, u64, u32, f32 = C.c_void_p, c_u64, c_u32, c_f32
     sig = {
         "it_hip_create": (vp, [u32, C.c_int, C.c_char_p, C.c_size_t]),
+        "it_hip_has_error": (C.c_int, [vp]),
         "it_hip_embed_argmax": (C.c_int, [vp, vp, vp, u64, vp, u64, u64]),
         "it_hip_read_tokens": (None, [vp, u64, u64, vp]),
         "it_hip_destroy": (None, [vp]),
