@@ -21,17 +21,14 @@ IT_DEV float it_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 
 // /root/reference src/quant/mod.rs:271-284: unsigned E4M3, bias 7, halved.
 IT_DEV float it_ue4m3_to_f32(uint32_t x) {
     x &= 0xffu;
-    if (x == 0 || x == 0x7f) return 0.0f;
-    int exp = (x >> 3) & 0xf;
-    float man = (float)(x & 7);
-    float raw;
-    if (exp == 0) {
-        raw = man * 0.001953125f;
-    } else {
-        float p = __uint_as_float((uint32_t)(exp - 7 + 127) << 23);
-        raw = (1.0f + man / 8.0f) * p;
-    }
-    return raw * 0.5f;
+    const uint32_t em = x & 0x7fu;
+    // normal: (1 + man/8) * 2^(exp-7) / 2 = exponent field exp + 119 with man in the top mantissa bits;
+    // subnormal (exp == 0): man * 2^-9 / 2.  Both are exact in f32, so this is the value the
+    // reference's arithmetic gives, without its branches.
+    const float normal = __uint_as_float((em << 20) + (119u << 23));
+    const float sub = (float)(em & 7u) * 0.0009765625f;
+    const float r = (em >> 3) ? normal : sub;
+    return x == 0x7fu ? 0.0f : r;
 }
 
 __device__ __constant__ const uint64_t IT_EXP2F_TAB[32] = {

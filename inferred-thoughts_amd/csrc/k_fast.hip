@@ -16,6 +16,21 @@
 #include "kernels.h"
 #include "kernels_fused.h"
 
+// Phase stamps for tuning: a build with -DIT_STAMPS records the 100 MHz wall clock of one block's
+// thread 0 at the marked points; the library build compiles them away.
+#ifdef IT_STAMPS
+__device__ long long it_stamps[32];
+__device__ int it_stamp_block;
+#define IT_STAMP(i)                                                                        \
+    do {                                                                                   \
+        if ((int)blockIdx.x == it_stamp_block && threadIdx.x == 0) it_stamps[i] = wall_clock64(); \
+    } while (0)
+#else
+#define IT_STAMP(i) \
+    do {            \
+    } while (0)
+#endif
+
 namespace itk {
 namespace {
 
@@ -244,6 +259,8 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     int g = blockIdx.x * FW + wave;
 
     WChunks<CPL> t[RB];
+    // the value an accumulating row adds to (epi 2) is fetched with the weights, not after the dot
+    float ep[RB];
     int mi = 0, row0 = 0;
     auto fetch = [&](int gg) {
         mi = fast_mat_index(p, gg);
@@ -253,6 +270,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
         for (int r = 0; r < RB; r++) {
             const int row = row0 + r * P + rsub;
             load_w<FMT, CPL, L>(t[r], m.q, m.s, n_in, row, sub, row < m.n_out);
+            if (sub == 0 && row < m.n_out && m.epi == 2) ep[r] = m.out[row];
         }
     };
     // the first group's weights start moving before the activation prologue runs
@@ -269,6 +287,9 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
 #pragma unroll
         for (int r = 0; r < RB; r++) acc[r] = dot_chunks<FMT, CPL>(t[r], x);
         const int cmi = mi, crow0 = row0;
+        float cp[RB];
+#pragma unroll
+        for (int r = 0; r < RB; r++) cp[r] = ep[r];
         g += gstride;
         if (g < p.total_groups) fetch(g);
 #pragma unroll
@@ -283,7 +304,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                 if (m.epi == 0) {
                     m.out[j] = a;
                 } else if (m.epi == 2) {
-                    m.out[j] += a;
+                    m.out[j] = cp[r] + a;
                 } else {
                     // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
                     float* past = p.conv_state + (int64_t)j * 3;
@@ -649,10 +670,13 @@ namespace {
 
 // ------------------------------------------------------------------ moe_down, fast
 // x[j] += sum_y w_y * scale2_y * (down_y[j] . g_y) + sigmoid(logit) * (shared_down[j] . g_sh)
-// One wave step covers P = 64 / L output rows for every pick and the shared expert, so the
-// sum over experts never leaves the lane.
+// A wave step covers P = 64 / L output rows.  Two waves share a row group: the even picks go
+// to one, the odd picks and the shared expert to the other, and the two partial sums meet in
+// LDS in a fixed order.  Loads are issued in the order they can be consumed: the small
+// intermediates first (they are quantized while the weights are still on their way), then
+// every weight chunk of the wave and the residual it will add to.
 constexpr int DT = 256, DW = DT / 64;
-constexpr int MAXU = 16;
+constexpr int MAXU = 16, HALFU = MAXU / 2;
 
 template <int EF, int ECPL, int L, int SF, int SCPL>
 __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
@@ -662,65 +686,71 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     const int total = NU * n_in + sh_in;  // floats staged: picks back to back, then the shared vector
     int8_t* xq = (int8_t*)smem;
     float* xs = (float*)(smem + ((total + 15) & ~15));
-    __shared__ int ids[MAXU];
     __shared__ float coef[MAXU];
+    __shared__ float partial[DW / 2][64];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = wave & 1, group = wave >> 1;
     const int sub = lane % L, rsub = lane / L;
-    const int row = (blockIdx.x * DW + wave) * P + rsub;
+    const int row = (blockIdx.x * (DW / 2) + group) * P + rsub;
     const bool live = row < p.n_out;
+    IT_STAMP(0);
 
-    // weights first: ids come from global, then every pick's chunk and the shared one
-    WChunks<ECPL> t[MAXU];
+    // the intermediates: up to six quads per thread (24 floats) cover 6144 floats per block
+    const int nq = total >> 2, nq_routed = (NU * n_in) >> 2;
+    constexpr int QR = 6;
+    float4 v[QR];
+#pragma unroll
+    for (int k = 0; k < QR; k++) {
+        const int qi = k * DT + tid;
+        v[k] = qi >= nq ? make_float4(0.f, 0.f, 0.f, 0.f)
+                        : qi < nq_routed ? ((const float4*)p.g_all)[qi] : ((const float4*)p.g_shared)[qi - nq_routed];
+    }
+    // this wave's picks: y = 2 * k + half
+    WChunks<ECPL> t[HALFU];
     WChunks<SCPL> tsh;
 #pragma unroll
-    for (int y = 0; y < MAXU; y++) {
+    for (int k = 0; k < HALFU; k++) {
+        const int y = 2 * k + half;
         if (y < NU) {
             const int64_t e = p.route_ids[y];
-            load_w<EF, ECPL, L>(t[y], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row, sub, live);
+            load_w<EF, ECPL, L>(t[k], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row, sub, live);
         }
     }
-    load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
-    if (tid < NU) {
-        const int e = p.route_ids[tid];
-        ids[tid] = e;
-        coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[e] : 1.0f);
-    }
+    if (half) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
+    const float x_old = (!half && sub == 0 && live) ? p.x[row] : 0.0f;
+    if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
     const float gate = it_sigmoid(p.logit[0]);
+    IT_STAMP(1);
 
-    // quantize all NU + 1 intermediates into LDS, four quads per thread per round
-    const int nq = total >> 2, nq_routed = (NU * n_in) >> 2;
-    for (int base = 0; base < nq; base += 4 * DT) {
-        float4 v[4];
-        bool lv[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int qi = base + k * DT + tid;
-            lv[k] = qi < nq;
-            v[k] = !lv[k] ? make_float4(0.f, 0.f, 0.f, 0.f)
-                          : qi < nq_routed ? ((const float4*)p.g_all)[qi] : ((const float4*)p.g_shared)[qi - nq_routed];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++) quant_quad(v[k], lv[k], base + k * DT + tid, xq, xs);
-    }
+    for (int k = 0; k < QR; k++) quant_quad(v[k], k * DT + tid < nq, k * DT + tid, xq, xs);
+    IT_STAMP(2);
     __syncthreads();
+    IT_STAMP(3);
 
     float acc = 0.0f;
 #pragma unroll
-    for (int y = 0; y < MAXU; y++) {
+    for (int k = 0; k < HALFU; k++) {
+        const int y = 2 * k + half;
         if (y < NU) {
             XChunks<EF, ECPL> x;
             load_x<EF, ECPL, L>(x, xq + y * n_in, xs + y * (n_in >> 5), sub);
-            acc += coef[y] * dot_chunks<EF, ECPL>(t[y], x);
+            acc += coef[y] * dot_chunks<EF, ECPL>(t[k], x);
         }
     }
-    {
+    if (half) {
         XChunks<SF, SCPL> x;
         load_x<SF, SCPL, L>(x, xq + NU * n_in, xs + NU * (n_in >> 5), sub);
         acc += gate * dot_chunks<SF, SCPL>(tsh, x);
     }
+    IT_STAMP(4);
     acc = reduce_lanes<L>(acc);
-    if (sub == 0 && live) p.x[row] += acc;
+    if (half) partial[group][lane] = acc;
+    __syncthreads();
+    IT_STAMP(5);
+    if (!half && sub == 0 && live) p.x[row] = x_old + (acc + partial[group][lane]);
+    IT_STAMP(6);
 }
 
 }  // namespace
@@ -741,9 +771,9 @@ bool moe_down_fast(MoeDownP p, hipStream_t s) {
         return false;
     const int total = p.n_used * p.n_in + p.sh_n_in;
     const size_t lds = (size_t)((total + 15) & ~15) + (size_t)(total / 32) * 4;
-    if (lds > 60 * 1024) return false;
+    if (lds > 60 * 1024 || total > 6 * DT * 4) return false;
     const int P = 64 / L;
-    const int blocks = (p.n_out + DW * P - 1) / (DW * P);
+    const int blocks = (p.n_out + (DW / 2) * P - 1) / ((DW / 2) * P);
 #define IT_LAUNCH(EF, LL, SF, SC) hipLaunchKernelGGL((moe_down_fast_k<EF, 1, LL, SF, SC>), dim3(blocks), dim3(DT), lds, s, p)
 #define IT_BY_L(EF, SF, SC)                      \
     do {                                         \
