@@ -333,13 +333,15 @@ __global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, fl
 // gate (optional): out *= sigmoid(gate[head * gate_stride + i]) — the attention block's output gate.
 // One block per (query, head).  Only the splits that hold positions are visited (n_live of them);
 // their weights exp(m_s - m) are formed once, in LDS.
-__global__ __launch_bounds__(256) void attend_merge_k(const float* __restrict__ part, int n_split, int hd,
-                                                      float* __restrict__ out, const float* __restrict__ gate,
-                                                      int gate_stride, int n_q, int n_head, int chunk, int n_pos_arg,
-                                                      const int* n_pos_dyn) {
-    extern __shared__ float wsplit[];  // [n_split]
-    __shared__ float redm[4], redl[4];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+__global__ __launch_bounds__(1024) void attend_merge_k(const float* __restrict__ part, int n_split, int hd,
+                                                       float* __restrict__ out, const float* __restrict__ gate,
+                                                       int gate_stride, int n_q, int n_head, int chunk, int n_pos_arg,
+                                                       const int* n_pos_dyn) {
+    // blockDim = 4 * hd: four groups of hd threads, group g sums the splits s = g (mod 4)
+    extern __shared__ float wsplit[];  // [n_split] then [4][hd]
+    __shared__ float redm[16], redl[16];
+    float* accs = wsplit + n_split;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = (blockDim.x + 63) >> 6;
     const int t = blockIdx.x / n_head;
     const int n_pos = (n_pos_dyn ? *n_pos_dyn : n_pos_arg) - n_q + 1 + t;
     int n_live = (n_pos + chunk - 1) / chunk;
@@ -364,17 +366,18 @@ __global__ __launch_bounds__(256) void attend_merge_k(const float* __restrict__ 
     __syncthreads();
     l = 0.0f;
     for (int w = 0; w < nw; w++) l += redl[w];
-    for (int i = tid; i < hd; i += blockDim.x) {
-        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-        int s = 0;
-        for (; s + 4 <= n_live; s += 4) {
-            a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
-            a1 += p[(int64_t)(s + 1) * (hd + 2) + i] * wsplit[s + 1];
-            a2 += p[(int64_t)(s + 2) * (hd + 2) + i] * wsplit[s + 2];
-            a3 += p[(int64_t)(s + 3) * (hd + 2) + i] * wsplit[s + 3];
-        }
-        for (; s < n_live; s++) a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
-        float r = ((a0 + a1) + (a2 + a3)) / l;
+    const int g = tid / hd, i = tid - g * hd;
+    float a0 = 0.0f, a1 = 0.0f;
+    int s = g;
+    for (; s + 4 < n_live; s += 8) {
+        a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
+        a1 += p[(int64_t)(s + 4) * (hd + 2) + i] * wsplit[s + 4];
+    }
+    if (s < n_live) a0 += p[(int64_t)s * (hd + 2) + i] * wsplit[s];
+    accs[g * hd + i] = a0 + a1;
+    __syncthreads();
+    if (g == 0) {
+        float r = ((accs[i] + accs[hd + i]) + (accs[2 * hd + i] + accs[3 * hd + i])) / l;
         if (gate) r *= it_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + i]);
         out[(int64_t)blockIdx.x * hd + i] = r;
     }
@@ -427,9 +430,9 @@ void attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* o
             default: return;  // the caller falls back to the exact kernel for other group sizes
         }
     }
-    hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(a.head_dim < 256 ? 64 : 256),
-                       (size_t)n_split * sizeof(float), s, scratch, n_split, a.head_dim, out, gate, gate_stride, a.n_q,
-                       a.n_head, tile ? TILE : CHUNK, a.n_pos, a.n_pos_dyn);
+    hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(4 * a.head_dim),
+                       (size_t)(n_split + 4 * a.head_dim) * sizeof(float), s, scratch, n_split, a.head_dim, out, gate,
+                       gate_stride, a.n_q, a.n_head, tile ? TILE : CHUNK, a.n_pos, a.n_pos_dyn);
 }
 
 }  // namespace itk
