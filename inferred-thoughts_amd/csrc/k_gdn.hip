@@ -106,10 +106,102 @@ __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restric
     }
 }
 
+// ------------------------------------------------------------------ fast form over a batch
+// 32 value rows per block, 8 lanes per row (DK / 8 keys each): the row's dots are reduced
+// with three lane exchanges, so the sums are not in the CPU path's order (fast mode only).
+// The gates of every token of the batch are formed once, up front, in LDS; each token's
+// k, q and v are fetched one token ahead of their use, straight from global memory, so a
+// step needs no block barrier.
+template <int DK>
+__global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __restrict__ state,
+                                                         float* __restrict__ out, float q_scale) {
+    constexpr int SEG = DK / 8;
+    constexpr int V4 = SEG / 4;
+    extern __shared__ float gates[];  // [n_tokens][2]: decay g, write strength beta
+    const int tid = threadIdx.x, seg = tid & 7;
+    const int dv = d.head_v_dim;
+    const int bph = dv / 32;
+    const int h = blockIdx.x / bph, jb = blockIdx.x % bph, kh = h % d.n_k_heads;
+    const int j = jb * 32 + (tid >> 3);
+    const int kper = d.n_k_heads * DK, vper = d.n_v_heads * dv;
+    for (int t = tid; t < d.n_tokens; t += 256) {
+        const float a = d.alpha[(int64_t)t * d.n_v_heads + h] + d.dt_bias[h];
+        const float softplus = a > 20.0f ? a : it_logf(1.0f + it_expf(a));
+        gates[2 * t] = it_expf(softplus * d.ssm_a[h]);
+        gates[2 * t + 1] = 1.0f / (1.0f + it_expf(-d.beta[(int64_t)t * d.n_v_heads + h]));
+    }
+    float* S = state + ((int64_t)h * dv + j) * DK + seg * SEG;
+    float row[SEG];
+#pragma unroll
+    for (int i = 0; i < V4; i++) {
+        const float4 t4 = ((const float4*)S)[i];
+        row[4 * i] = t4.x; row[4 * i + 1] = t4.y; row[4 * i + 2] = t4.z; row[4 * i + 3] = t4.w;
+    }
+    const float* kbase = d.k + kh * DK + seg * SEG;
+    const float* qbase = d.q + kh * DK + seg * SEG;
+    const float* vbase = d.v + h * dv + j;
+    float4 kn[V4], qn[V4];
+    float vn;
+#pragma unroll
+    for (int i = 0; i < V4; i++) {
+        kn[i] = ((const float4*)kbase)[i];
+        qn[i] = ((const float4*)qbase)[i];
+    }
+    vn = vbase[0];
+    __syncthreads();
+    for (int t = 0; t < d.n_tokens; t++) {
+        float kk[SEG], qq[SEG];
+#pragma unroll
+        for (int i = 0; i < V4; i++) {
+            kk[4 * i] = kn[i].x; kk[4 * i + 1] = kn[i].y; kk[4 * i + 2] = kn[i].z; kk[4 * i + 3] = kn[i].w;
+            qq[4 * i] = qn[i].x; qq[4 * i + 1] = qn[i].y; qq[4 * i + 2] = qn[i].z; qq[4 * i + 3] = qn[i].w;
+        }
+        const float v = vn;
+        if (t + 1 < d.n_tokens) {
+#pragma unroll
+            for (int i = 0; i < V4; i++) {
+                kn[i] = ((const float4*)(kbase + (int64_t)(t + 1) * kper))[i];
+                qn[i] = ((const float4*)(qbase + (int64_t)(t + 1) * kper))[i];
+            }
+            vn = vbase[(int64_t)(t + 1) * vper];
+        }
+        const float g = gates[2 * t], beta = gates[2 * t + 1];
+        float pred = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SEG; i++) {
+            row[i] *= g;
+            pred += row[i] * kk[i];
+        }
+        pred += __shfl_xor(pred, 1, 64);
+        pred += __shfl_xor(pred, 2, 64);
+        pred += __shfl_xor(pred, 4, 64);
+        const float delta = beta * (v - pred);
+        float o = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SEG; i++) {
+            row[i] += kk[i] * delta;
+            o += row[i] * (qq[i] * q_scale);
+        }
+        o += __shfl_xor(o, 1, 64);
+        o += __shfl_xor(o, 2, 64);
+        o += __shfl_xor(o, 4, 64);
+        if (seg == 0) out[(int64_t)t * vper + h * dv + j] = o;
+    }
+#pragma unroll
+    for (int i = 0; i < V4; i++)
+        ((float4*)S)[i] = make_float4(row[4 * i], row[4 * i + 1], row[4 * i + 2], row[4 * i + 3]);
+}
+
 void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, hipStream_t s) {
-    (void)exact;
     if (d.n_tokens <= 0) return;
     float q_scale = 1.0f / sqrtf((float)d.head_k_dim);
+    const size_t gate_lds = (size_t)d.n_tokens * 2 * sizeof(float);
+    if (!exact && d.head_v_dim % 32 == 0 && (d.head_k_dim == 64 || d.head_k_dim == 128) && gate_lds <= 48 * 1024) {
+        const int blocks = d.n_v_heads * (d.head_v_dim / 32);
+        if (d.head_k_dim == 64) hipLaunchKernelGGL(delta_rule_fast_k<64>, dim3(blocks), dim3(256), gate_lds, s, d, state, out, q_scale);
+        else hipLaunchKernelGGL(delta_rule_fast_k<128>, dim3(blocks), dim3(256), gate_lds, s, d, state, out, q_scale);
+        return;
+    }
     int blocks = d.n_v_heads * ((d.head_v_dim + 63) / 64);
     switch (d.head_k_dim) {
         case 32: hipLaunchKernelGGL(delta_rule_k<32>, dim3(blocks), dim3(64), 0, s, d, state, out, q_scale); break;

@@ -1,0 +1,98 @@
+"""Fast mode (the mode bench.py measures) op by op against the CPU oracle, through the C ABI.
+
+Fast mode keeps the oracle's integer dots and scale products but sums in wave order, runs
+attention split over the context and the delta rule with rows split over lanes, so results are
+held to rel/abs 1e-3 of the oracle rather than to the bit.  Shapes are the single-op
+configurations of the baseline: GQA decode attention (16 q heads, 2 kv heads, head_dim 256,
+contexts 1024 / 8192 / 32000, q and the result rounded to bf16), the Gated DeltaNet layer
+(16 key / 32 value heads, dk = dv = 128, one decode step and a multi-token batch) and the
+NVFP4 expert matmuls, plus the tiny configuration's shapes.
+"""
+import numpy as np
+import pytest
+
+from util import bf16_round, f16_bits, nvfp4_weights, q8_0_weights, rng
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import inferred_hip as ih
+    be = ih.Hip(exact=False)
+    yield be
+    err = be.take_error()
+    be.close()
+    assert err is None, err
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import binding as ob
+    o = ob.Oracle(threads=8)
+    return o
+
+
+def fresh(hip):
+    hip.drop_mirrors()
+    hip.begin_pass(1)
+
+
+def close(a, b, tol=1e-3):
+    """rel/abs: |a - b| <= tol * max(1, |b|) elementwise."""
+    return np.all(np.abs(a - b) <= tol * np.maximum(1.0, np.abs(b)))
+
+
+def l2n(x, hd):
+    x = x.reshape(-1, hd)
+    return (x / np.linalg.norm(x, axis=1, keepdims=True)).astype(np.float32).reshape(-1)
+
+
+@pytest.mark.parametrize("n_q,n_pos,hd,nh,nkv", [(1, 1024, 256, 16, 2), (1, 8192, 256, 16, 2), (1, 32000, 256, 16, 2),
+                                                  (1, 63, 64, 8, 2), (1, 200, 128, 8, 1), (5, 300, 256, 16, 2),
+                                                  (40, 700, 64, 8, 2)])
+def test_attend_split(hip, orc, n_q, n_pos, hd, nh, nkv):
+    fresh(hip)
+    r = rng(31)
+    kv_dim = nkv * hd
+    q = bf16_round(r.standard_normal(n_q * nh * hd).astype(np.float32))
+    k = f16_bits(r.standard_normal(n_pos * kv_dim)); v = f16_bits(r.standard_normal(n_pos * kv_dim))
+    a, b = np.zeros(n_q * nh * hd, np.float32), np.zeros(n_q * nh * hd, np.float32)
+    sc = 1.0 / np.sqrt(np.float32(hd))
+    hip.attend(q, k, v, kv_dim, n_pos, hd, nh, nkv, sc, a); hip.host_needs(a)
+    orc.attend(q, k, v, kv_dim, n_pos, hd, nh, nkv, sc, b)
+    hip.raise_if_error()
+    assert close(a, b), np.abs(a - b).max()
+    assert close(bf16_round(a), bf16_round(b), 8e-3)     # one bf16 step at most after rounding the result
+
+
+@pytest.mark.parametrize("n_tok,dk,nk,nv", [(1, 128, 16, 32), (64, 128, 16, 32), (380, 128, 16, 32), (1, 64, 4, 8),
+                                            (37, 64, 4, 8)])
+def test_delta_rule_fast(hip, orc, n_tok, dk, nk, nv):
+    fresh(hip)
+    r = rng(32)
+    dv = dk
+    q = l2n(bf16_round(r.standard_normal(n_tok * nk * dk)), dk); k = l2n(bf16_round(r.standard_normal(n_tok * nk * dk)), dk)
+    v = bf16_round(r.standard_normal(n_tok * nv * dv).astype(np.float32))
+    alpha = r.standard_normal(n_tok * nv).astype(np.float32); alpha[0] = 25.0
+    beta = r.standard_normal(n_tok * nv).astype(np.float32)
+    ssm_a = -np.ones(nv, np.float32); dt = np.zeros(nv, np.float32)      # g = -softplus(alpha), as config 4 states it
+    sa = (r.standard_normal(nv * dk * dv) * 0.1).astype(np.float32); sb = sa.copy()
+    a, b = np.zeros(n_tok * nv * dv, np.float32), np.zeros(n_tok * nv * dv, np.float32)
+    hip.delta_rule(q, k, v, alpha, beta, ssm_a, dt, dk, dv, nk, nv, sa, a); hip.host_needs(a); hip.read_state(sa)
+    orc.delta_rule(q, k, v, alpha, beta, ssm_a, dt, dk, dv, nk, nv, sb, b)
+    hip.raise_if_error()
+    assert close(a, b), np.abs(a - b).max()
+    assert close(sa, sb), np.abs(sa - sb).max()
+
+
+@pytest.mark.parametrize("n,nd", [(1, 2048), (33, 2048), (3, 512)])
+def test_rms_norm_fast(hip, orc, n, nd):
+    fresh(hip)
+    r = rng(33)
+    x = r.standard_normal(n * nd).astype(np.float32) * 3
+    w = r.standard_normal(nd).astype(np.float32)
+    a, b = np.zeros_like(x), np.zeros_like(x)
+    hip.rms_norm(x, w, 1e-6, a); hip.host_needs(a)
+    orc.rms_norm(x, w, 1e-6, b)
+    assert close(a, b, 1e-5)
