@@ -203,6 +203,7 @@ __global__ void dense_float_k(const uint8_t* __restrict__ w, const float* __rest
 void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
             float* out, float out_scale, hipStream_t s) {
     if (n_tok <= 0 || w.n_out <= 0) return;
+    if (q8_gemm(w, act_scales, act_quants, n_tok, out, out_scale, s)) return;
     if (w.fmt == W_Q8_0 || w.fmt == W_NVFP4) {
         GemvP p{};
         p.q = (const uint8_t*)w.q;

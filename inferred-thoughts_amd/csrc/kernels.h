@@ -34,6 +34,11 @@ void quantize_q8_0(const float* x, float* scales, int8_t* quants, int64_t n, hip
 void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
             float* out, float out_scale, hipStream_t s);
 
+// The same product for 16 or more tokens on the int8 matrix cores (Q8_0 weights only): bit-identical
+// to `matmul`.  Returns false without launching when the shape or format is not handled.
+bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, int n_tok, float* out, float out_scale,
+             hipStream_t s);
+
 struct ExpertsView {
     const void* q;       // expert e at q + e*q_stride
     const void* scales;  // expert e at scales + e*s_stride

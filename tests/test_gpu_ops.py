@@ -64,7 +64,10 @@ def test_rms_norm_heads_and_l2(hip, orc, heads, hd):
 
 
 @pytest.mark.parametrize("n_in,n_out,n", [(512, 1024, 1), (512, 16, 1), (512, 1, 3), (2048, 8192, 1),
-                                            (4096, 2048, 1), (2048, 512, 7), (256, 512, 4)])
+                                            (4096, 2048, 1), (2048, 512, 7), (256, 512, 4),
+                                            # 16 tokens and more take the int8 matrix-core kernel: ragged rows and tokens
+                                            (2048, 2048, 16), (2048, 1000, 37), (4096, 512, 380), (512, 1024, 129),
+                                            (256, 33, 200), (2048, 8, 64)])
 def test_matmul_q8_0(hip, orc, n_in, n_out, n):
     import inferred_hip as ih
     from oracle import binding as ob
