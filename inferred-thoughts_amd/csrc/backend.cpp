@@ -520,6 +520,26 @@ const float2* it_hip::rope_table(float theta, uint64_t n_rot, uint64_t need_pos)
     return r.dev;
 }
 
+int32_t* it_hip::moe_work_for(size_t picks, size_t n_expert, size_t* ints) {
+    *ints = 0;
+    if (picks < 32) return nullptr;
+    const size_t need = itk::experts_group_work_ints((int)picks, (int)n_expert);
+    if (moe_work_ints < need) {
+        need_eager("expert grouping scratch has to grow");
+        if (moe_work) {
+            check(hipStreamSynchronize(stream), "sync before scratch free");
+            (void)hipFree(moe_work);
+            moe_work = nullptr;
+            moe_work_ints = 0;
+        }
+        const size_t want = need + need / 2;
+        if (!check(hipMalloc((void**)&moe_work, want * sizeof(int32_t)), "hipMalloc(expert grouping scratch)")) return nullptr;
+        moe_work_ints = want;
+    }
+    *ints = moe_work_ints;
+    return moe_work;
+}
+
 float* it_hip::scratch_f32(size_t floats) {
     if (attn_scratch_cap >= floats) return attn_scratch;
     need_eager("attention scratch has to grow");
@@ -1065,13 +1085,18 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    size_t work_ints;
+    int32_t* work = be->moe_work_for(picks, w->n_expert, &work_ints);
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
     rec.i[6] = v.q_stride; rec.i[7] = v.s_stride;
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
-               [=](hipStream_t s) { matmul_experts(v, ids, np, nu, xm, as, aq, dout, s); });
+               [=](hipStream_t s) {
+                   if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
+                       matmul_experts(v, ids, np, nu, xm, as, aq, dout, s);
+               });
     be->expert_lookups += picks;
 }
 
@@ -1103,6 +1128,8 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
+    size_t work_ints;
+    int32_t* work = be->moe_work_for(picks, gate->n_expert, &work_ints);
     it_hip::OpRec rec;
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
@@ -1111,7 +1138,10 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     be->submit(it_hip::FAM_MOE_GLU, 2 * picks * (gate->len / gate->n_expert) + x_len + out_len * 4,
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
-               [=](hipStream_t s) { moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s); });
+               [=](hipStream_t s) {
+                   if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
+                       moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s);
+               });
     be->expert_lookups += 2 * picks;
 }
 

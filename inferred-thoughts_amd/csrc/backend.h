@@ -117,6 +117,10 @@ struct it_hip {
     size_t route_cap = 0;  // picks
     uint64_t route_n_used = 0, route_n_tok = 0;
     bool route_reserve(size_t picks);
+    // scratch of the grouped expert matmuls (expert-sorted pair lists and their tiles)
+    int32_t* moe_work = nullptr;
+    size_t moe_work_ints = 0;
+    int32_t* moe_work_for(size_t picks, size_t n_expert, size_t* ints);
     bool route_stage(const it_route* r, const int32_t** ids, const float** w, uint64_t* n_used, uint64_t* n_tok);
 
     // ---- RoPE tables, built on the host in f64 (naive.rs:205-208)

@@ -11,6 +11,7 @@
 // k = 8 * (l / 16) for both A (weight rows) and B (tokens); it receives D for token l % 16
 // and weight rows 4 * (l / 16) + {0,1,2,3}.
 #include "it_device.h"
+#include "it_dot.h"
 #include "kernels.h"
 
 namespace itk {
@@ -152,6 +153,268 @@ bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, 
     else if (tiles >= 2) IT_GEMM(2);
     else IT_GEMM(1);
 #undef IT_GEMM
+    return true;
+}
+
+}  // namespace itk
+
+// =====================================================================================
+// Grouped expert matmuls for a batch of (token, pick) pairs.
+//
+// The per-pair GEMV reads an expert's matrix once per pair.  Here the pairs are first sorted
+// into per-expert lists ("expert-sorted token lists": moe_group_k), the lists are cut into
+// tiles of up to 16 pairs, and one block multiplies 64 rows of that expert's matrix with the
+// tile's 16 activation rows on the int8 matrix cores, so a matrix is read once per tile.
+// Per pair and row the arithmetic is the GEMV's: per-block integer dots, scaled and added in
+// block order (Q8_0: (float)isum * (dw * dx); NVFP4: (dy * dA) * (float)sa then
+// (dy * dB) * (float)sb per 32-element chunk), then the expert's second scale, then silu-mul
+// for the gate/up pair.  An NVFP4 chunk holds two 16-element sub-blocks with their own
+// scales; each needs its own integer sum, so the chunk takes two MFMAs whose token operand is
+// zeroed outside the sub-block.
+namespace itk {
+namespace {
+
+// One block.  work layout: [0] = number of tiles; tiles as int4 {expert, first slot, pairs, 0};
+// order[slot] = pair index.  The order of pairs inside an expert's list depends on the atomics'
+// arrival order; it only decides which lane computes which pair, never a value.
+__global__ __launch_bounds__(1024) void moe_group_k(const int32_t* __restrict__ ids, int n_picks, int n_expert,
+                                                    int32_t* __restrict__ n_tiles, int4* __restrict__ tiles,
+                                                    int32_t* __restrict__ order) {
+    __shared__ int cnt[1024], off[1024], toff[1024], cur[1024];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < n_expert; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < n_picks; p += 1024) atomicAdd(&cnt[ids[p]], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int o = 0, t = 0;
+        for (int e = 0; e < n_expert; e++) {
+            off[e] = o;
+            toff[e] = t;
+            o += cnt[e];
+            t += (cnt[e] + 15) >> 4;
+        }
+        *n_tiles = t;
+    }
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += 1024) cur[e] = off[e];
+    __syncthreads();
+    for (int p = tid; p < n_picks; p += 1024) {
+        const int slot = atomicAdd(&cur[ids[p]], 1);
+        order[slot] = p;
+    }
+    for (int e = tid; e < n_expert; e += 1024)
+        for (int k = 0; k * 16 < cnt[e]; k++) tiles[toff[e] + k] = make_int4(e, off[e] + 16 * k, min(16, cnt[e] - 16 * k), 0);
+}
+
+struct ExpertsGemmP {
+    const uint8_t *q, *s, *q2, *s2;
+    int64_t q_stride, s_stride;
+    const float *scale2, *scale2_up;
+    const float* act_scales;
+    const int8_t* act_quants;
+    float* out;
+    int n_in, n_out, x_mode, n_used;
+    const int32_t* n_tiles;
+    const int4* tiles;
+    const int32_t* order;
+};
+
+constexpr int NSTR = 64 + 8;  // LDS row stride of an NVFP4 slab (64 nibble bytes + pad)
+
+template <int FMT, bool GLU>
+__global__ __launch_bounds__(GT) void experts_gemm_k(ExpertsGemmP p) {
+    constexpr int NM = GLU ? 2 : 1;
+    constexpr int ASTR = FMT == W_Q8_0 ? LSTR : NSTR;
+    constexpr int SPR = FMT == W_Q8_0 ? 4 : 8;  // scales per row per slab
+    __shared__ __align__(16) int8_t As[2][NM][64 * ASTR];
+    __shared__ float Asc[2][NM][64 * SPR];
+    __shared__ __align__(16) int8_t Bs[2][16 * LSTR];
+    __shared__ float Bsc[2][16 * 4];
+    __shared__ int xrow_s[16], pair_s[16];
+    const int tile = blockIdx.x;
+    if (tile >= *p.n_tiles) return;
+    const int4 td = p.tiles[tile];
+    const int64_t e = td.x;
+    const int cnt = td.z;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.y * 64;
+    const int n_in = p.n_in, nb = n_in >> 5;
+    const int nslab = n_in / SLAB;
+    if (tid < 16) {
+        const int pair = p.order[td.y + min(tid, cnt - 1)];
+        pair_s[tid] = pair;
+        xrow_s[tid] = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
+    }
+    __syncthreads();
+    const uint8_t* wq[2] = {p.q + e * p.q_stride, GLU ? p.q2 + e * p.q_stride : nullptr};
+    const uint8_t* ws[2] = {p.s + e * p.s_stride, GLU ? p.s2 + e * p.s_stride : nullptr};
+
+    uint4 ra[NM][2], rb;
+    float rsa[NM][2], rsb;
+    auto fetch = [&](int s) {
+#pragma unroll
+        for (int mt = 0; mt < NM; mt++) {
+            if (FMT == W_Q8_0) {
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    const int idx = tid + q * GT, row = idx >> 3, seg = idx & 7;
+                    ra[mt][q] = *(const uint4*)(wq[mt] + (int64_t)min(row0 + row, p.n_out - 1) * n_in + s * SLAB + seg * 16);
+                }
+                const int row = tid >> 2, bi = tid & 3;
+                rsa[mt][0] = it_f16_to_f32(((const uint16_t*)ws[mt])[(int64_t)min(row0 + row, p.n_out - 1) * nb + s * 4 + bi]);
+            } else {
+                const int row = tid >> 2, seg = tid & 3;
+                ra[mt][0] = *(const uint4*)(wq[mt] + (int64_t)min(row0 + row, p.n_out - 1) * (n_in >> 1) + s * 64 + seg * 16);
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    const int idx = tid + q * GT, r2 = idx >> 3, k = idx & 7;
+                    rsa[mt][q] = it_ue4m3_to_f32(ws[mt][(int64_t)min(row0 + r2, p.n_out - 1) * (n_in >> 4) + s * 8 + k]);
+                }
+            }
+        }
+        if (tid < 128) {
+            const int pr = tid >> 3, seg = tid & 7;
+            rb = *(const uint4*)(p.act_quants + (int64_t)xrow_s[pr] * n_in + s * SLAB + seg * 16);
+        }
+        if (tid < 64) rsb = p.act_scales[(int64_t)xrow_s[tid >> 2] * nb + s * 4 + (tid & 3)];
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int mt = 0; mt < NM; mt++) {
+            if (FMT == W_Q8_0) {
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    const int idx = tid + q * GT, row = idx >> 3, seg = idx & 7;
+                    *(uint4*)(As[buf][mt] + row * ASTR + seg * 16) = ra[mt][q];
+                }
+                Asc[buf][mt][tid] = rsa[mt][0];
+            } else {
+                const int row = tid >> 2, seg = tid & 3;
+                *(uint4*)(As[buf][mt] + row * ASTR + seg * 16) = ra[mt][0];
+#pragma unroll
+                for (int q = 0; q < 2; q++) Asc[buf][mt][tid + q * GT] = rsa[mt][q];
+            }
+        }
+        if (tid < 128) *(uint4*)(Bs[buf] + (tid >> 3) * LSTR + (tid & 7) * 16) = rb;
+        if (tid < 64) Bsc[buf][tid] = rsb;
+    };
+
+    float acc[NM][4];
+#pragma unroll
+    for (int mt = 0; mt < NM; mt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[mt][i] = 0.0f;
+    const v4i z = {0, 0, 0, 0};
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int s = 0; s < nslab; s++) {
+        const int buf = s & 1;
+        if (s + 1 < nslab) fetch(s + 1);
+#pragma unroll
+        for (int bi = 0; bi < 4; bi++) {
+            const long bv = *(const long*)(Bs[buf] + m * LSTR + bi * 32 + g * 8);
+            const float dx = Bsc[buf][m * 4 + bi];
+#pragma unroll
+            for (int mt = 0; mt < NM; mt++) {
+                if (FMT == W_Q8_0) {
+                    const long a = *(const long*)(As[buf][mt] + (wave * 16 + m) * ASTR + bi * 32 + g * 8);
+                    const v4i d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bv, z, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float dw = Asc[buf][mt][(wave * 16 + 4 * g + i) * 4 + bi];
+                        acc[mt][i] += (float)d[i] * (dw * dx);
+                    }
+                } else {
+                    // lane (m, g): sub-block g / 2 of the chunk, its low (g even) or high nibbles
+                    const uint2 nb8 = *(const uint2*)(As[buf][mt] + (wave * 16 + m) * ASTR + bi * 16 + (g >> 1) * 8);
+                    const int sh = (g & 1) * 4;
+                    const uint32_t lo = fp4x4_to_i8x4((nb8.x >> sh) & 0x0f0f0f0fu), hi = fp4x4_to_i8x4((nb8.y >> sh) & 0x0f0f0f0fu);
+                    const long a = (long)(((unsigned long long)hi << 32) | lo);
+                    const long bA = g < 2 ? bv : 0l, bB = g < 2 ? 0l : bv;
+                    const v4i dA = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bA, z, 0, 0, 0);
+                    const v4i dB = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bB, z, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float sA = Asc[buf][mt][(wave * 16 + 4 * g + i) * 8 + 2 * bi];
+                        const float sB = Asc[buf][mt][(wave * 16 + 4 * g + i) * 8 + 2 * bi + 1];
+                        acc[mt][i] += (dx * sA) * (float)dA[i];
+                        acc[mt][i] += (dx * sB) * (float)dB[i];
+                    }
+                }
+            }
+        }
+        if (s + 1 < nslab) stash(buf ^ 1);
+        __syncthreads();
+    }
+    if (m < cnt) {
+        const int64_t pair = pair_s[m];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int j = row0 + wave * 16 + 4 * g + i;
+            if (j >= p.n_out) continue;
+            float a0 = acc[0][i];
+            if (p.scale2) a0 *= p.scale2[e];
+            if (GLU) {
+                float a1 = acc[NM - 1][i];
+                if (p.scale2_up) a1 *= p.scale2_up[e];
+                a0 = it_silu(a0) * a1;
+            }
+            p.out[pair * p.n_out + j] = a0;
+        }
+    }
+}
+
+}  // namespace
+
+size_t experts_group_work_ints(int n_picks, int n_expert) {
+    return 16 + (size_t)(n_expert + n_picks / 16 + 2) * 4 + (size_t)n_picks;
+}
+
+bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
+                  const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
+                  hipStream_t s) {
+    if (n_picks < 32 || !work || w.n_expert > 1024 || w.n_in % SLAB || (w.fmt != W_Q8_0 && w.fmt != W_NVFP4)) return false;
+    if (work_ints < experts_group_work_ints(n_picks, w.n_expert)) return false;
+    if ((reinterpret_cast<uintptr_t>(w.q) & 15) || w.q_stride % 16 || (reinterpret_cast<uintptr_t>(act_quants) & 15)) return false;
+    if (up && (up->fmt != w.fmt || up->n_in != w.n_in || up->n_out != w.n_out || (reinterpret_cast<uintptr_t>(up->q) & 15)))
+        return false;
+    const int max_tiles = w.n_expert + n_picks / 16 + 1;
+    int32_t* n_tiles = work;
+    int4* tiles = (int4*)(work + 16);
+    int32_t* order = work + 16 + (size_t)(max_tiles + 1) * 4;
+    hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, n_tiles, tiles, order);
+    ExpertsGemmP p{};
+    p.q = (const uint8_t*)w.q;
+    p.s = (const uint8_t*)w.scales;
+    p.q2 = up ? (const uint8_t*)up->q : nullptr;
+    p.s2 = up ? (const uint8_t*)up->scales : nullptr;
+    p.q_stride = w.q_stride;
+    p.s_stride = w.s_stride;
+    p.scale2 = w.scale2;
+    p.scale2_up = up ? up->scale2 : nullptr;
+    p.act_scales = act_scales;
+    p.act_quants = act_quants;
+    p.out = out;
+    p.n_in = w.n_in;
+    p.n_out = w.n_out;
+    p.x_mode = x_mode;
+    p.n_used = n_used < 1 ? 1 : n_used;
+    p.n_tiles = n_tiles;
+    p.tiles = tiles;
+    p.order = order;
+    dim3 grid(max_tiles, (w.n_out + 63) / 64);
+    if (w.fmt == W_Q8_0) {
+        if (up) hipLaunchKernelGGL((experts_gemm_k<W_Q8_0, true>), grid, dim3(GT), 0, s, p);
+        else hipLaunchKernelGGL((experts_gemm_k<W_Q8_0, false>), grid, dim3(GT), 0, s, p);
+    } else {
+        if (up) hipLaunchKernelGGL((experts_gemm_k<W_NVFP4, true>), grid, dim3(GT), 0, s, p);
+        else hipLaunchKernelGGL((experts_gemm_k<W_NVFP4, false>), grid, dim3(GT), 0, s, p);
+    }
     return true;
 }
 

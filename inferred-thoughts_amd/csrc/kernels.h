@@ -50,6 +50,14 @@ struct ExpertsView {
 // (pick i reads row i / n_used), 2 = a single shared row.
 void matmul_experts(const ExpertsView& w, const int32_t* ids, int n_picks, int n_used, int x_mode,
                     const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);
+// The same products (up == null) or the gate/up pair with silu-mul (up != null) for a batch of 32 or more
+// pairs: pairs are grouped by expert and multiplied on the int8 matrix cores, a matrix read once per 16
+// pairs; bit-identical to the per-pair kernels.  `work` is device scratch of experts_group_work_ints ints.
+// Returns false without launching when the shape, format or scratch does not fit.
+size_t experts_group_work_ints(int n_picks, int n_expert);
+bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
+                  const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
+                  hipStream_t s);
 // out[i] = silu(gate_e . x * sg_e) * (up_e . x * su_e)
 void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids, int n_picks, int n_used,
              int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);

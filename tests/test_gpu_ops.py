@@ -299,7 +299,10 @@ def test_route(hip, orc, n_tok, n_expert, n_used):
 
 @pytest.mark.parametrize("fmt", ["q8_0", "nvfp4"])
 @pytest.mark.parametrize("n_tok,n_expert,n_used,nd,ff", [(1, 16, 4, 512, 256), (6, 16, 4, 512, 256),
-                                                         (1, 64, 10, 2048, 512), (3, 64, 10, 2048, 512)])
+                                                         (1, 64, 10, 2048, 512), (3, 64, 10, 2048, 512),
+                                                         # 32 pairs and more: expert-grouped tiles on the matrix cores
+                                                         (37, 16, 4, 512, 256), (200, 16, 4, 512, 256),
+                                                         (48, 64, 10, 2048, 512)])
 def test_moe_stage(hip, orc, fmt, n_tok, n_expert, n_used, nd, ff):
     """moe_glu + matmul_experts(down) + moe_finish, host route, against the oracle's defaults."""
     import inferred_hip as ih
