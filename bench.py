@@ -40,6 +40,7 @@ def main():
     ap.add_argument("--layers", type=int, default=48, help="48 is the baseline config; fewer only for quick checks")
     ap.add_argument("--prompt", type=int, default=5700)
     ap.add_argument("--ctx", type=int, default=8192)
+    XX
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--exact", action="store_true", help="CPU-order reductions (bit-exact mode)")
@@ -63,7 +64,7 @@ def main():
 
     be = ih.Hip(exact=args.exact)
     model = ih.Model(path)
-    eng = ih.Engine(model, be, args.ctx)
+    eng = ih.Engine(model, be, args.ctx, args.max_batch)
     rng = np.random.default_rng(args.seed)
     prompt = rng.integers(0, model.n_vocab, args.prompt).astype(np.uint32)
 
@@ -153,7 +154,7 @@ def main():
         "config": {"workload": "config 5: full 35B-A3B-shaped model, greedy decode after a 5,700-token prefill at ctx 8192"
                                if args.layers == 48 and args.prompt == 5700 else
                                f"REDUCED check run: {args.layers} layers, prompt {args.prompt}",
-                   "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "decode_pos": int(pos0),
+                   "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "prefill_batch": args.max_batch, "decode_pos": int(pos0),
                    "experts": "512 top-10 + shared, NVFP4", "dense": "Q8_0 (router and ssm_alpha/beta Q8_0)",
                    "mode": "exact" if args.exact else "fast", "batch": 1},
         "prefill_tok_s": round(args.prompt / t_prefill, 1),

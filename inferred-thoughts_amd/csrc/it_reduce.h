@@ -33,4 +33,13 @@ __device__ double block_sumsq(const float* buf, int n, int exact, double* red) {
 }
 
 
+// Sum over the 8 lanes of an aligned group with data-parallel-primitive moves (no LDS crossbar):
+// neighbours, then pairs, then the mirrored half.  Every lane of the group ends with the total.
+IT_DEV float sum8_lanes(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+    return v;
+}
+
 }  // namespace itk

@@ -297,17 +297,27 @@ void quantize_q8_0(const float* x, float* scales, int8_t* quants, int64_t n, hip
 }
 
 // ------------------------------------------------------------------ causal conv + silu
-// naive.rs:275-315.  One thread per channel walks the batch in order with the
-// window in registers; state is [channel][kernel-1], oldest first.
+// naive.rs:275-315.  One thread per channel and token chunk, the window in registers;
+// state is [channel][kernel-1], oldest first.
+// Tokens are independent given their window, so the batch is cut into chunks of CONV_TOK tokens
+// (grid.y): a thread rebuilds its window from the inputs before its chunk, or from the state for
+// the first tokens of the batch.  Only chunk 0 reads the old state, and it is the one that
+// writes the new one (the last KEEP inputs), so no block reads what another writes.
+constexpr int CONV_TOK = 16;
 template <int KEEP>
 __global__ void ssm_conv_k(float* __restrict__ state, const float* __restrict__ x, const float* __restrict__ w,
                            int nc, int n_tok, float* __restrict__ out) {
-    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= nc) return;
-    float past[KEEP], wt[KEEP + 1];
-    for (int k = 0; k < KEEP; k++) past[k] = state[(int64_t)c * KEEP + k];
+    const int t0 = blockIdx.y * CONV_TOK, t1 = min(n_tok, t0 + CONV_TOK);
+    float past[KEEP], wt[KEEP + 1], old[KEEP];
+    for (int k = 0; k < KEEP; k++) {
+        const int idx = t0 - KEEP + k;
+        old[k] = blockIdx.y == 0 ? state[(int64_t)c * KEEP + k] : 0.0f;
+        past[k] = idx >= 0 ? x[(int64_t)idx * nc + c] : old[KEEP + idx];
+    }
     for (int k = 0; k <= KEEP; k++) wt[k] = w[(int64_t)c * (KEEP + 1) + k];
-    for (int t = 0; t < n_tok; t++) {
+    for (int t = t0; t < t1; t++) {
         float xv = x[(int64_t)t * nc + c];
         float sum = 0.0f;
         for (int k = 0; k < KEEP; k++) sum += past[k] * wt[k];
@@ -316,13 +326,18 @@ __global__ void ssm_conv_k(float* __restrict__ state, const float* __restrict__ 
         for (int k = 0; k + 1 < KEEP; k++) past[k] = past[k + 1];
         past[KEEP - 1] = xv;
     }
-    for (int k = 0; k < KEEP; k++) state[(int64_t)c * KEEP + k] = past[k];
+    if (blockIdx.y == 0) {
+        for (int k = 0; k < KEEP; k++) {
+            const int idx = n_tok - KEEP + k;
+            state[(int64_t)c * KEEP + k] = idx >= 0 ? x[(int64_t)idx * nc + c] : old[KEEP + idx];
+        }
+    }
 }
 
 void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
               hipStream_t s) {
     if (nc <= 0 || n_tok <= 0) return;
-    dim3 grid((nc + 127) / 128), block(128);
+    dim3 grid((nc + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);
     switch (kernel) {
         case 2: hipLaunchKernelGGL(ssm_conv_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
         case 3: hipLaunchKernelGGL(ssm_conv_k<2>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;

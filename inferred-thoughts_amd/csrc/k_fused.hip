@@ -508,9 +508,7 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
         row[i] *= g;
         pred += row[i] * kk[i];
     }
-    pred += __shfl_xor(pred, 1, 64);
-    pred += __shfl_xor(pred, 2, 64);
-    pred += __shfl_xor(pred, 4, 64);
+    pred = sum8_lanes(pred);
     float delta = beta * (v - pred);
     float o = 0.0f;
 #pragma unroll
@@ -518,9 +516,7 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
         row[i] += kk[i] * delta;
         o += row[i] * (qq[i] * p.q_scale);
     }
-    o += __shfl_xor(o, 1, 64);
-    o += __shfl_xor(o, 2, 64);
-    o += __shfl_xor(o, 4, 64);
+    o = sum8_lanes(o);
 #pragma unroll
     for (int i = 0; i < SEG / 4; i++)
         ((float4*)S)[i] = make_float4(row[4 * i], row[4 * i + 1], row[4 * i + 2], row[4 * i + 3]);

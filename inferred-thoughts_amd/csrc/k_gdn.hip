@@ -10,6 +10,7 @@
 // to the CPU path.  The 64-row tile moves between HBM and registers through a
 // padded LDS tile so both the load and the store are fully coalesced.
 #include "it_device.h"
+#include "it_reduce.h"
 #include "kernels.h"
 
 namespace itk {
@@ -172,9 +173,7 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
             row[i] *= g;
             pred += row[i] * kk[i];
         }
-        pred += __shfl_xor(pred, 1, 64);
-        pred += __shfl_xor(pred, 2, 64);
-        pred += __shfl_xor(pred, 4, 64);
+        pred = sum8_lanes(pred);
         const float delta = beta * (v - pred);
         float o = 0.0f;
 #pragma unroll
@@ -182,9 +181,7 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
             row[i] += kk[i] * delta;
             o += row[i] * (qq[i] * q_scale);
         }
-        o += __shfl_xor(o, 1, 64);
-        o += __shfl_xor(o, 2, 64);
-        o += __shfl_xor(o, 4, 64);
+        o = sum8_lanes(o);
         if (seg == 0) out[(int64_t)t * vper + h * dv + j] = o;
     }
 #pragma unroll

@@ -10,6 +10,7 @@
 //   moe_batch                    src/model/qwen35.rs:1587-1700
 //   KvCache / RecurrentState     src/cache/mod.rs:33-65,215-252, src/cache/recurrent.rs:31-142
 //   Engine run/prefill/generate  src/engine/mod.rs:310-437
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -251,6 +252,7 @@ struct it_engine {
     it_model* m;
     it_hip* be;
     uint64_t n_ctx, max_batch;
+    uint64_t moe_chunk = 512;  // tokens per routed-FFN sub-batch
     uint64_t len = 0;
     uint64_t ring_next = 0;  // next slot of the backend's device token ring this engine files into
     std::vector<uint16_t> k_slabs, v_slabs;
@@ -275,7 +277,7 @@ struct it_engine {
 };
 
 namespace {
-constexpr uint64_t MOE_CHUNK = 512;  // src/model/qwen35.rs:650
+constexpr uint64_t MOE_CHUNK = 512;  // src/model/qwen35.rs:650: the reference's routed-FFN sub-batch; a larger engine batch raises it (it_engine_new)
 
 void fit(it_engine* e, uint64_t n) {
     const Dims& d = e->m->d;
@@ -285,7 +287,7 @@ void fit(it_engine* e, uint64_t n) {
     e->qkv.fit(n * d.conv_dim()); e->z.fit(n * d.value_dim()); e->alpha.fit(n * d.dt_rank); e->beta.fit(n * d.dt_rank);
     e->convo.fit(n * d.conv_dim()); e->q_part.fit(n * d.key_dim()); e->k_part.fit(n * d.key_dim());
     e->v_part.fit(n * d.value_dim()); e->core.fit(n * d.value_dim());
-    uint64_t nt = n < MOE_CHUNK ? n : MOE_CHUNK;
+    uint64_t nt = n < e->moe_chunk ? n : e->moe_chunk;
     uint64_t ff = d.expert_ff > d.shared_ff ? d.expert_ff : d.shared_ff;
     e->router.fit(nt * d.n_expert); e->e_gate.fit(nt * ff); e->e_up.fit(nt * ff); e->e_out.fit(nt * d.n_embd);
     e->e_in.fit(nt * d.n_embd); e->g_all.fit(nt * d.n_used * d.expert_ff); e->u_all.fit(nt * d.n_used * d.expert_ff);
@@ -417,7 +419,7 @@ int forward(it_engine* e, const uint32_t* tokens, uint64_t n, uint64_t start, bo
         e->tr("attn_residual", il, e->x, n * nd);
         it_hip_rms_norm(be, e->x.p(), n * nd, b.ffn_norm.data(), nd, d.eps, e->normed.p(), n * nd);
         for (uint64_t t = 0; t < n;) {
-            uint64_t take = MOE_CHUNK < n - t ? MOE_CHUNK : n - t;
+            uint64_t take = e->moe_chunk < n - t ? e->moe_chunk : n - t;
             moe_batch(e, b, t * nd, take, n);
             t += take;
         }
@@ -491,6 +493,9 @@ it_engine* it_engine_new(it_model* m, it_hip* be, uint64_t n_ctx, uint64_t max_b
     e->n_ctx = n_ctx;
     e->max_batch = max_batch ? max_batch : 512;  // DEFAULT_MAX_BATCH, src/engine/mod.rs:87
     const Dims& d = m->d;
+    // every expert's matrices are read once per routed-FFN sub-batch, so with memory to spare the sub-batch
+    // follows the engine batch (the seam carries at most 65535 pairs per call)
+    e->moe_chunk = std::max<uint64_t>(MOE_CHUNK, std::min<uint64_t>(e->max_batch, 65535 / std::max<uint64_t>(1, d.n_used)));
     e->k_slabs.assign(m->n_kv_layer * n_ctx * d.kv_dim(), 0);
     e->v_slabs.assign(m->n_kv_layer * n_ctx * d.kv_dim(), 0);
     e->conv.assign(d.layers() * d.conv_len(), 0.0f);
