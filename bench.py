@@ -25,6 +25,12 @@ sys.path.insert(0, str(ROOT / "inferred-thoughts_amd"))
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch (fetched + written) of each kernel family, averaged over the full model's per-layer launches,
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 256 MiB copy
+# (profiles/decode_kernels_hbm_traffic_pmc.txt holds the commands and the per-kernel readings)
+PMC_TRAFFIC_BYTES = {"fused_gemv (norm + quantize + dense GEMVs)": 12_190_000, "moe_glu (expert gate+up)": 14_400_000,
+                     "matmul_experts (expert down)": 7_430_000, "gdn_rows (l2 norm + delta rule)": 4_400_000,
+                     "lm_head (norm + GEMV)": 331_660_000}
 
 
 def model_path(args):
@@ -46,6 +52,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--exact", action="store_true", help="CPU-order reductions (bit-exact mode)")
     ap.add_argument("--keep", action="store_true", help="keep the generated GGUF")
+    ap.add_argument("--copy-ref", action="store_true",
+                    help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective; see DESIGN.md "
@@ -63,6 +72,12 @@ def main():
     t_synth = time.time() - t0
     print(f"[bench] model {path} ({path.stat().st_size / 2**30:.1f} GiB) ready in {t_synth:.1f}s", file=sys.stderr, flush=True)
 
+    if args.copy_ref:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src); torch.cuda.synchronize()
+        dst.copy_(src); torch.cuda.synchronize()
+        del src, dst
     be = ih.Hip(exact=args.exact)
     model = ih.Model(path)
     eng = ih.Engine(model, be, args.ctx, args.max_batch)
@@ -124,7 +139,8 @@ def main():
     if dom:
         ach = (dom["bytes"] / 1e9) / (dom["ms"] / 1e3)
         roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                    "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                    "traffic": PMC_TRAFFIC_BYTES.get(dom["name"]) if args.layers == 48 else None,
                     "avg_launch_us": round(1e3 * dom["ms"] / dom["launches"], 2),
                     "bytes_per_launch": dom["bytes"] // dom["launches"]}
 
