@@ -110,20 +110,29 @@ __global__ __launch_bounds__(64) void delta_rule_k(DeltaArgs d, float* __restric
 // ------------------------------------------------------------------ fast form over a batch
 // 32 value rows per block, 8 lanes per row (DK / 8 keys each): the row's dots are reduced
 // with three lane exchanges, so the sums are not in the CPU path's order (fast mode only).
-// The gates of every token of the batch are formed once, up front, in LDS; each token's
-// k, q and v are fetched one token ahead of their use, straight from global memory, so a
-// step needs no block barrier.
+// The gates of every token of the batch are formed once, up front, in LDS.  The batch is
+// walked in chunks of 16 tokens: a chunk's k, q and v are staged into LDS with coalesced
+// loads while the previous chunk is being applied, so a token step touches only LDS and
+// registers and the only block barrier is the one between chunks.
+constexpr int GDN_TCH = 16;
+
 template <int DK>
 __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __restrict__ state,
                                                          float* __restrict__ out, float q_scale) {
     constexpr int SEG = DK / 8;
     constexpr int V4 = SEG / 4;
-    extern __shared__ float gates[];  // [n_tokens][2]: decay g, write strength beta
-    const int tid = threadIdx.x, seg = tid & 7;
+    constexpr int KQ4 = GDN_TCH * DK / 4;          // float4 per chunk of k (and of q)
+    constexpr int KQL = (KQ4 + 255) / 256;          // per thread
+    extern __shared__ __align__(16) float lds[];
+    float* gates = lds;                                               // [n_tokens][2]
+    float* kbuf = lds + (((size_t)d.n_tokens * 2 + 3) & ~(size_t)3);  // [2][TCH][DK]
+    float* qbuf = kbuf + 2 * GDN_TCH * DK;                            // [2][TCH][DK]
+    float* vbuf = qbuf + 2 * GDN_TCH * DK;                            // [2][TCH][32]
+    const int tid = threadIdx.x, seg = tid & 7, r = tid >> 3;
     const int dv = d.head_v_dim;
     const int bph = dv / 32;
     const int h = blockIdx.x / bph, jb = blockIdx.x % bph, kh = h % d.n_k_heads;
-    const int j = jb * 32 + (tid >> 3);
+    const int j = jb * 32 + r;
     const int kper = d.n_k_heads * DK, vper = d.n_v_heads * dv;
     for (int t = tid; t < d.n_tokens; t += 256) {
         const float a = d.alpha[(int64_t)t * d.n_v_heads + h] + d.dt_bias[h];
@@ -138,51 +147,72 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
         const float4 t4 = ((const float4*)S)[i];
         row[4 * i] = t4.x; row[4 * i + 1] = t4.y; row[4 * i + 2] = t4.z; row[4 * i + 3] = t4.w;
     }
-    const float* kbase = d.k + kh * DK + seg * SEG;
-    const float* qbase = d.q + kh * DK + seg * SEG;
-    const float* vbase = d.v + h * dv + j;
-    float4 kn[V4], qn[V4];
-    float vn;
+    float4 rk[KQL], rq[KQL];
+    float rv[2];
+    auto fetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < V4; i++) {
-        kn[i] = ((const float4*)kbase)[i];
-        qn[i] = ((const float4*)qbase)[i];
-    }
-    vn = vbase[0];
-    __syncthreads();
-    for (int t = 0; t < d.n_tokens; t++) {
-        float kk[SEG], qq[SEG];
-#pragma unroll
-        for (int i = 0; i < V4; i++) {
-            kk[4 * i] = kn[i].x; kk[4 * i + 1] = kn[i].y; kk[4 * i + 2] = kn[i].z; kk[4 * i + 3] = kn[i].w;
-            qq[4 * i] = qn[i].x; qq[4 * i + 1] = qn[i].y; qq[4 * i + 2] = qn[i].z; qq[4 * i + 3] = qn[i].w;
+        for (int p = 0; p < KQL; p++) {
+            const int idx = tid + p * 256, tt = idx / (DK / 4), c4 = idx % (DK / 4);
+            const bool ok = idx < KQ4 && t0 + tt < d.n_tokens;
+            rk[p] = ok ? ((const float4*)(d.k + (int64_t)(t0 + tt) * kper + kh * DK))[c4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            rq[p] = ok ? ((const float4*)(d.q + (int64_t)(t0 + tt) * kper + kh * DK))[c4] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        const float v = vn;
-        if (t + 1 < d.n_tokens) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const int idx = tid + p * 256, tt = idx >> 5, rr = idx & 31;
+            rv[p] = t0 + tt < d.n_tokens ? d.v[(int64_t)(t0 + tt) * vper + h * dv + jb * 32 + rr] : 0.0f;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < KQL; p++) {
+            const int idx = tid + p * 256;
+            if (idx < KQ4) {
+                ((float4*)(kbuf + buf * GDN_TCH * DK))[idx] = rk[p];
+                ((float4*)(qbuf + buf * GDN_TCH * DK))[idx] = rq[p];
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 2; p++) vbuf[buf * GDN_TCH * 32 + tid + p * 256] = rv[p];
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int t0 = 0, c = 0; t0 < d.n_tokens; t0 += GDN_TCH, c++) {
+        const int buf = c & 1;
+        if (t0 + GDN_TCH < d.n_tokens) fetch(t0 + GDN_TCH);
+        const int nt = min(GDN_TCH, d.n_tokens - t0);
+        for (int tt = 0; tt < nt; tt++) {
+            const float4* k4 = (const float4*)(kbuf + (buf * GDN_TCH + tt) * DK + seg * SEG);
+            const float4* q4 = (const float4*)(qbuf + (buf * GDN_TCH + tt) * DK + seg * SEG);
+            float kk[SEG], qq[SEG];
 #pragma unroll
             for (int i = 0; i < V4; i++) {
-                kn[i] = ((const float4*)(kbase + (int64_t)(t + 1) * kper))[i];
-                qn[i] = ((const float4*)(qbase + (int64_t)(t + 1) * kper))[i];
+                const float4 a = k4[i], b = q4[i];
+                kk[4 * i] = a.x; kk[4 * i + 1] = a.y; kk[4 * i + 2] = a.z; kk[4 * i + 3] = a.w;
+                qq[4 * i] = b.x; qq[4 * i + 1] = b.y; qq[4 * i + 2] = b.z; qq[4 * i + 3] = b.w;
             }
-            vn = vbase[(int64_t)(t + 1) * vper];
-        }
-        const float g = gates[2 * t], beta = gates[2 * t + 1];
-        float pred = 0.0f;
+            const float v = vbuf[(buf * GDN_TCH + tt) * 32 + r];
+            const float g = gates[2 * (t0 + tt)], beta = gates[2 * (t0 + tt) + 1];
+            float pred = 0.0f;
 #pragma unroll
-        for (int i = 0; i < SEG; i++) {
-            row[i] *= g;
-            pred += row[i] * kk[i];
-        }
-        pred = sum8_lanes(pred);
-        const float delta = beta * (v - pred);
-        float o = 0.0f;
+            for (int i = 0; i < SEG; i++) {
+                row[i] *= g;
+                pred += row[i] * kk[i];
+            }
+            pred = sum8_lanes(pred);
+            const float delta = beta * (v - pred);
+            float o = 0.0f;
 #pragma unroll
-        for (int i = 0; i < SEG; i++) {
-            row[i] += kk[i] * delta;
-            o += row[i] * (qq[i] * q_scale);
+            for (int i = 0; i < SEG; i++) {
+                row[i] += kk[i] * delta;
+                o += row[i] * (qq[i] * q_scale);
+            }
+            o = sum8_lanes(o);
+            if (seg == 0) out[(int64_t)(t0 + tt) * vper + h * dv + j] = o;
         }
-        o = sum8_lanes(o);
-        if (seg == 0) out[(int64_t)t * vper + h * dv + j] = o;
+        if (t0 + GDN_TCH < d.n_tokens) stash(buf ^ 1);
+        __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < V4; i++)
@@ -192,8 +222,8 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
 void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, hipStream_t s) {
     if (d.n_tokens <= 0) return;
     float q_scale = 1.0f / sqrtf((float)d.head_k_dim);
-    const size_t gate_lds = (size_t)d.n_tokens * 2 * sizeof(float);
-    if (!exact && d.head_v_dim % 32 == 0 && (d.head_k_dim == 64 || d.head_k_dim == 128) && gate_lds <= 48 * 1024) {
+    const size_t gate_lds = ((((size_t)d.n_tokens * 2 + 3) & ~(size_t)3) + 4 * GDN_TCH * d.head_k_dim + 2 * GDN_TCH * 32) * sizeof(float);
+    if (!exact && d.head_v_dim % 32 == 0 && (d.head_k_dim == 64 || d.head_k_dim == 128) && gate_lds <= 96 * 1024) {
         const int blocks = d.n_v_heads * (d.head_v_dim / 32);
         if (d.head_k_dim == 64) hipLaunchKernelGGL(delta_rule_fast_k<64>, dim3(blocks), dim3(256), gate_lds, s, d, state, out, q_scale);
         else hipLaunchKernelGGL(delta_rule_fast_k<128>, dim3(blocks), dim3(256), gate_lds, s, d, state, out, q_scale);
