@@ -182,7 +182,7 @@ def main():
         "kernels": kernels,
         "cpu_baseline": cpu,
         "setup_s": {"synth": round(t_synth, 1), "upload_repack": round(t_upload, 1)},
-        "graph": graph_stats, "launches_per_token": launches_per_token,
+        "graph": graph_stats, "seam_ops_per_token": launches_per_token,
     }
     print(json.dumps(line), flush=True)
     eng.close(); model.close(); be.close()

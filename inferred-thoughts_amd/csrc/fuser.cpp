@@ -8,7 +8,6 @@
 // scales — is simply issued op by op.  A fused launch sits at the position of its
 // block's first op; everything it replaces is dropped, except an activation
 // quantization that some unfused op still reads.
-#include <cstdlib>
 #include "backend.h"
 
 using namespace itk;
