@@ -33,6 +33,105 @@ __device__ double block_sumsq(const float* buf, int n, int exact, double* red) {
 }
 
 
+// ------------------------------------------------------------------ lane exchanges without LDS
+// DPP moves reach the lanes of a row of 16: neighbour (quad_perm 1,0,3,2), pair (quad_perm
+// 2,3,0,1), the mirrored half of 8 and the mirrored row of 16.  After the first two steps a
+// quad is uniform, after three a group of 8, so the mirrors pair each lane with one of the
+// other half.  Across rows (offsets 16 and 32) the exchange goes through ds_bpermute.
+IT_DEV float dpp_xor1(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)); }
+IT_DEV float dpp_xor2(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)); }
+IT_DEV float dpp_half_mirror(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)); }
+IT_DEV float dpp_row_mirror(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)); }
+IT_DEV double dpp_f64(double v, int which) {
+    const unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+    int lo = (int)(u & 0xffffffffull), hi = (int)(u >> 32);
+    if (which == 0) {
+        lo = __builtin_amdgcn_update_dpp(0, lo, 0xB1, 0xf, 0xf, true);
+        hi = __builtin_amdgcn_update_dpp(0, hi, 0xB1, 0xf, 0xf, true);
+    } else if (which == 1) {
+        lo = __builtin_amdgcn_update_dpp(0, lo, 0x4E, 0xf, 0xf, true);
+        hi = __builtin_amdgcn_update_dpp(0, hi, 0x4E, 0xf, 0xf, true);
+    } else if (which == 2) {
+        lo = __builtin_amdgcn_update_dpp(0, lo, 0x141, 0xf, 0xf, true);
+        hi = __builtin_amdgcn_update_dpp(0, hi, 0x141, 0xf, 0xf, true);
+    } else {
+        lo = __builtin_amdgcn_update_dpp(0, lo, 0x140, 0xf, 0xf, true);
+        hi = __builtin_amdgcn_update_dpp(0, hi, 0x140, 0xf, 0xf, true);
+    }
+    return __builtin_bit_cast(double, ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
+// sum (or max) over aligned groups of L lanes, L a power of two up to 64; every lane gets the result
+template <int L> IT_DEV float group_sum(float v) {
+    if (L >= 2) v += dpp_xor1(v);
+    if (L >= 4) v += dpp_xor2(v);
+    if (L >= 8) v += dpp_half_mirror(v);
+    if (L >= 16) v += dpp_row_mirror(v);
+    if (L >= 32) v += __shfl_xor(v, 16, 64);
+    if (L >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+template <int L> IT_DEV float group_max(float v) {
+    if (L >= 2) v = fmaxf(v, dpp_xor1(v));
+    if (L >= 4) v = fmaxf(v, dpp_xor2(v));
+    if (L >= 8) v = fmaxf(v, dpp_half_mirror(v));
+    if (L >= 16) v = fmaxf(v, dpp_row_mirror(v));
+    if (L >= 32) v = fmaxf(v, __shfl_xor(v, 16, 64));
+    if (L >= 64) v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+// The same reductions with the result only in the LAST lane of each group: across rows a row's
+// total (its lane 15) is broadcast into the next row (row_bcast15 into rows 1 and 3, row_bcast31
+// into rows 2 and 3), which needs no LDS crossbar at all.
+IT_DEV float dpp_bcast15(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false)); }
+IT_DEV float dpp_bcast31(float v) { return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false)); }
+template <int L> IT_DEV float group_sum_tail(float v) {
+    if (L >= 2) v += dpp_xor1(v);
+    if (L >= 4) v += dpp_xor2(v);
+    if (L >= 8) v += dpp_half_mirror(v);
+    if (L >= 16) v += dpp_row_mirror(v);
+    if (L >= 32) v += dpp_bcast15(v);
+    if (L >= 64) v += dpp_bcast31(v);
+    return v;
+}
+template <int L> IT_DEV float group_max_tail(float v) {
+    if (L >= 2) v = fmaxf(v, dpp_xor1(v));
+    if (L >= 4) v = fmaxf(v, dpp_xor2(v));
+    if (L >= 8) v = fmaxf(v, dpp_half_mirror(v));
+    if (L >= 16) v = fmaxf(v, dpp_row_mirror(v));
+    // a masked-off row receives 0 from the broadcast: harmless for a maximum only when values are
+    // compared through max(v, t) on the rows that do receive, so the other rows keep v
+    if (L >= 32) {
+        const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
+        v = fmaxf(v, t);
+    }
+    if (L >= 64) {
+        const float t = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));
+        v = fmaxf(v, t);
+    }
+    return v;
+}
+// total of the wave in lane 63
+IT_DEV double wave_sum_f64_tail(double v) {
+    v += dpp_f64(v, 0);
+    v += dpp_f64(v, 1);
+    v += dpp_f64(v, 2);
+    v += dpp_f64(v, 3);
+    {
+        const unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+        const int lo = __builtin_amdgcn_update_dpp(0, (int)(u & 0xffffffffull), 0x142, 0xa, 0xf, false);
+        const int hi = __builtin_amdgcn_update_dpp(0, (int)(u >> 32), 0x142, 0xa, 0xf, false);
+        v += __builtin_bit_cast(double, ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+    }
+    {
+        const unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+        const int lo = __builtin_amdgcn_update_dpp(0, (int)(u & 0xffffffffull), 0x143, 0xc, 0xf, false);
+        const int hi = __builtin_amdgcn_update_dpp(0, (int)(u >> 32), 0x143, 0xc, 0xf, false);
+        v += __builtin_bit_cast(double, ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+    }
+    return v;
+}
+
 // Sum over the 8 lanes of an aligned group with data-parallel-primitive moves (no LDS crossbar):
 // neighbours, then pairs, then the mirrored half.  Every lane of the group ends with the total.
 IT_DEV float sum8_lanes(float v) {

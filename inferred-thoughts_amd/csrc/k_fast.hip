@@ -13,6 +13,7 @@
 // lanes, CPL = cpr / L chunks each, so a wave covers P = 64 / L rows per step.
 #include "it_device.h"
 #include "it_dot.h"
+#include "it_reduce.h"
 #include "kernels.h"
 #include "kernels_fused.h"
 
@@ -127,20 +128,15 @@ IT_DEV float dot_chunks(const WChunks<CPL>& t, const XChunks<FMT, CPL>& x) {
     return acc;
 }
 
-template <int L> IT_DEV float reduce_lanes(float v) {
-#pragma unroll
-    for (int o = L / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
+// the row's dot, complete in the LAST lane of its L-lane group
+template <int L> IT_DEV float reduce_lanes(float v) { return group_sum_tail<L>(v); }
 
 // ------------------------------------------------------------------ activation prologue
 // Q8_0 block quantization (naive.rs:652-675) of the quad a thread holds; the 8 threads of a
 // 32-block are neighbours in a wave.  Dead threads pass zeros and write nothing.
 IT_DEV void quant_quad(float4 v, bool live, int qi, int8_t* xq, float* xs) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+    amax = group_max<8>(amax);
     if (!live) return;
     const float d = amax / 127.0f;
     const float id = d != 0.0f ? 1.0f / d : 0.0f;
@@ -187,10 +183,8 @@ __device__ __forceinline__ void stage_activation(const float* x, int n_in, int m
 #pragma unroll
         for (int k = 0; k < 2; k++)
             w[k] = live[k] ? ((const float4*)norm_w)[tid + k * THREADS] : make_float4(0.f, 0.f, 0.f, 0.f);
-        double part = quad_sumsq(v[0]) + quad_sumsq(v[1]);
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-        if ((tid & 63) == 0) red[tid >> 6] = part;
+        double part = wave_sum_f64_tail(quad_sumsq(v[0]) + quad_sumsq(v[1]));
+        if ((tid & 63) == 63) red[tid >> 6] = part;
         __syncthreads();
         double sum = 0.0;
 #pragma unroll
@@ -270,7 +264,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
         for (int r = 0; r < RB; r++) {
             const int row = row0 + r * P + rsub;
             load_w<FMT, CPL, L>(t[r], m.q, m.s, n_in, row, sub, row < m.n_out);
-            if (sub == 0 && row < m.n_out && m.epi == 2) ep[r] = m.out[row];
+            if (sub == L - 1 && row < m.n_out && m.epi == 2) ep[r] = m.out[row];
         }
     };
     // the first group's weights start moving before the activation prologue runs
@@ -294,7 +288,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
         if (g < p.total_groups) fetch(g);
 #pragma unroll
         for (int r = 0; r < RB; r++) acc[r] = reduce_lanes<L>(acc[r]);
-        if (sub == 0) {
+        if (sub == L - 1) {
             const FusedMat& m = p.m[cmi];
 #pragma unroll
             for (int r = 0; r < RB; r++) {
@@ -457,9 +451,8 @@ __device__ __forceinline__ float block_route(const float* logits, int n_expert, 
     }
     if (tid < NW * 16) sh.cand[tid] = 0ull;  // slots a wave does not fill stay empty
     if (tid < 16) wts[tid] = 0.0f;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-    if (lane == 0) sh.redf[wave] = m;
+    m = group_max_tail<64>(m);
+    if (lane == 63) sh.redf[wave] = m;
     __syncthreads();
     m = sh.redf[0];
 #pragma unroll
@@ -472,9 +465,8 @@ __device__ __forceinline__ float block_route(const float* logits, int n_expert, 
         v[k] = (k < K && e < n_expert) ? it_expf(l[k] - m) : 0.0f;
         part += v[k];
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
-    if (lane == 0) sh.redf[NW + wave] = part;
+    part = group_sum_tail<64>(part);
+    if (lane == 63) sh.redf[NW + wave] = part;
     __syncthreads();
     float sum = 0.0f;
 #pragma unroll
@@ -552,7 +544,7 @@ IT_DEV void glu_job(const uint8_t* gq, const uint8_t* gs, const uint8_t* uq, con
         float ag = reduce_lanes<L>(dot_chunks<FMT, CPL>(tg[r], x));
         float au = reduce_lanes<L>(dot_chunks<FMT, CPL>(tu[r], x));
         const int row = row0 + r * P + rsub;
-        if (sub == 0 && row < n_out) {
+        if (sub == L - 1 && row < n_out) {
             ag *= sg;
             au *= su;
             out[row] = it_silu(ag) * au;
@@ -718,7 +710,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
         }
     }
     if (half) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
-    const float x_old = (!half && sub == 0 && live) ? p.x[row] : 0.0f;
+    const float x_old = (!half && sub == L - 1 && live) ? p.x[row] : 0.0f;
     if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
     const float gate = it_sigmoid(p.logit[0]);
     IT_STAMP(1);
@@ -749,7 +741,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     if (half) partial[group][lane] = acc;
     __syncthreads();
     IT_STAMP(5);
-    if (!half && sub == 0 && live) p.x[row] = x_old + (acc + partial[group][lane]);
+    if (!half && sub == L - 1 && live) p.x[row] = x_old + (acc + partial[group][lane]);
     IT_STAMP(6);
 }
 

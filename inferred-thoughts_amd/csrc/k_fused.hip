@@ -419,6 +419,30 @@ __device__ void load_kq_l2(const float* conv, int key_dim, int kh, float eps, in
     }
 }
 
+// Fast form for a block of 256 threads: thread t < DK holds k[t], thread DK + t holds q[t]; each
+// vector's sum of squares is reduced in its own waves, two barriers in all.
+// `v` is the thread's element, loaded by the caller (ahead of its other loads: loads return in order).
+template <int DK>
+__device__ __forceinline__ void l2_kq_fast(float v, float eps, float* kq, double* red) {
+    static_assert(DK == 64 || DK == 128, "one or two waves per vector");
+    constexpr int WPV = DK / 64;  // waves per vector
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const bool live = tid < 2 * DK;
+    const bool is_q = tid >= DK;
+    const int i = is_q ? tid - DK : tid;
+    const double part = wave_sum_f64_tail((double)(v * v));
+    if ((tid & 63) == 63) red[wave] = part;
+    __syncthreads();
+    if (live) {
+        const int w0 = is_q ? WPV : 0;
+        double sum = red[w0];
+        if (WPV == 2) sum += red[w0 + 1];
+        const float scale = 1.0f / fmaxf(sqrtf((float)sum), eps);
+        kq[(is_q ? DK : 0) + i] = v * scale;
+    }
+    __syncthreads();
+}
+
 IT_DEV void gdn_gates(const GdnCoreP& p, int h, float* g, float* beta) {
     float a = p.alpha[h] + p.dt_bias[h];
     float softplus = a > 20.0f ? a : it_logf(1.0f + it_expf(a));
@@ -488,14 +512,18 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
     const int bph = dv / 32;
     const int h = blockIdx.x / bph, jb = blockIdx.x % bph, kh = h % p.n_k_heads;
     const int key_dim = p.n_k_heads * DK;
-    load_kq_l2<DK, 256>(p.conv, key_dim, kh, p.eps, 0, kq, red);
+    // key / query element first, then the state rows: both are in flight while k and q are normalized
+    const float kqv = tid < 2 * DK ? p.conv[(tid >= DK ? 0 : key_dim) + kh * DK + (tid >= DK ? tid - DK : tid)] : 0.0f;
     const int j = jb * 32 + (tid >> 3);
     float* S = p.state + ((int64_t)h * dv + j) * DK + seg * SEG;
+    float4 st[SEG / 4];
+#pragma unroll
+    for (int i = 0; i < SEG / 4; i++) st[i] = ((const float4*)S)[i];
+    l2_kq_fast<DK>(kqv, p.eps, kq, red);
     float row[SEG];
 #pragma unroll
     for (int i = 0; i < SEG / 4; i++) {
-        float4 t = ((const float4*)S)[i];
-        row[4 * i] = t.x; row[4 * i + 1] = t.y; row[4 * i + 2] = t.z; row[4 * i + 3] = t.w;
+        row[4 * i] = st[i].x; row[4 * i + 1] = st[i].y; row[4 * i + 2] = st[i].z; row[4 * i + 3] = st[i].w;
     }
     float g, beta;
     gdn_gates(p, h, &g, &beta);
