@@ -317,10 +317,26 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     // K and V rows of the live context, f16 (the position is the one this pass was recorded at)
     const uint64_t kv_bytes = (uint64_t)at.i[8] * kvd * 2 * 2;
     pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
-    pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
-    if (at.i[6] == 0) {
+    TilePrepP tp{};
+    tp.qg = pp.qg;
+    tp.kproj = pp.k;
+    tp.vproj = pp.v;
+    tp.q_norm = pp.q_norm;
+    tp.k_norm = pp.k_norm;
+    tp.rope = pp.rope;
+    tp.n_rot = pp.n_rot;
+    tp.eps = pp.eps;
+    tp.k_slab = pp.k_slab;
+    tp.v_slab = pp.v_slab;
+    if (at.i[6] == 0 && attend_tile_prep_ok(aa, tp)) {
+        // norm + rotation of q and of the new key, and the slab writes, happen inside the tile kernel
+        pl.add(i, it_hip::FAM_ATTEND, kv_bytes + (uint64_t)(2 * hd * nh + 2 * kvd) * 4,
+               [=](hipStream_t s) { attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s); });
+    } else if (at.i[6] == 0) {
+        pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
         pl.add(i, it_hip::FAM_ATTEND, kv_bytes, [=](hipStream_t s) { attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s); });
     } else {
+        pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
         // the exact attention kernel and its gate stay as they are
         auto run_attend = at.run, run_gate = sg.run, run_gather_gate = gg.run;
         pl.add(i, it_hip::FAM_OTHER, 0, run_gather_gate);

@@ -9,6 +9,7 @@
 // chunk, keeps an online-softmax partial (acc, m, l), and a second kernel merges
 // the partials.  Reordered sums: compared against the exact path at 1e-3.
 #include "it_device.h"
+#include "it_reduce.h"
 #include "kernels.h"
 
 namespace itk {
@@ -193,8 +194,51 @@ __global__ __launch_bounds__(256) void attend_split_k(AttnArgs a, int n_split, f
 // in LDS).  Partial layout as above: [hd acc][m][l] per (t, head, split).
 constexpr int TILE = 64;
 
-template <int HD, int G>
-__global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, float* __restrict__ part) {
+// Per-head rms_norm (weight w) and NeoX rotation at `pos` of one head's HD values, four per lane
+// (lane li of the head's HD / 4 lanes holds dims 4 li .. 4 li + 3): what rms_norm_heads + rope_neox do
+// for a single token (naive.rs:180-218, 633-650), with the sum of squares reduced across the lanes.
+template <int HD>
+IT_DEV float4 head_norm_rope(float4 v, const float* __restrict__ w, float eps, const float2* __restrict__ rope,
+                             int n_rot, int pos, int li) {
+    constexpr int LPH = HD / 4;
+    double part = (double)(v.x * v.x);
+    part += (double)(v.y * v.y);
+    part += (double)(v.z * v.z);
+    part += (double)(v.w * v.w);
+    part += dpp_f64(part, 0);
+    part += dpp_f64(part, 1);
+    part += dpp_f64(part, 2);
+    part += dpp_f64(part, 3);
+    if (LPH >= 32) part += __shfl_xor(part, 16, 64);
+    if (LPH >= 64) part += __shfl_xor(part, 32, 64);
+    const float scale = 1.0f / sqrtf((float)(part / (double)HD) + eps);
+    const float4 ww = ((const float4*)w)[li];
+    v.x = v.x * scale * ww.x;
+    v.y = v.y * scale * ww.y;
+    v.z = v.z * scale * ww.z;
+    v.w = v.w * scale * ww.w;
+    const int half = n_rot >> 1, hl = half >> 2;  // lanes per rotated half (a power of two)
+    float4 o;
+    o.x = __shfl_xor(v.x, hl, 64);
+    o.y = __shfl_xor(v.y, hl, 64);
+    o.z = __shfl_xor(v.z, hl, 64);
+    o.w = __shfl_xor(v.w, hl, 64);
+    if (li < 2 * hl) {
+        const float4* cs = (const float4*)(rope + (int64_t)pos * half + 4 * (li & (hl - 1)));
+        const float4 c01 = cs[0], c23 = cs[1];  // (cos, sin) of dims i, i+1 and i+2, i+3
+        if (li < hl) {  // x0 = mine, x1 = partner
+            v = make_float4(v.x * c01.x - o.x * c01.y, v.y * c01.z - o.y * c01.w, v.z * c23.x - o.z * c23.y,
+                            v.w * c23.z - o.w * c23.w);
+        } else {        // x0 = partner, x1 = mine
+            v = make_float4(o.x * c01.y + v.x * c01.x, o.y * c01.w + v.y * c01.z, o.z * c23.y + v.z * c23.x,
+                            o.w * c23.w + v.w * c23.z);
+        }
+    }
+    return v;
+}
+
+template <int HD, int G, bool PREP>
+__global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, TilePrepP pr, int n_split, float* __restrict__ part) {
     constexpr int CPR = HD / 8;            // 16-byte chunks per K or V row
     constexpr int KSTR = HD * 2 + 16;      // K row stride in LDS: padded so lanes reading rows do not collide
     constexpr int DPL = HD / 64;           // output dimensions per lane
@@ -224,13 +268,16 @@ __global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, fl
         }
         return;
     }
+    // With PREP the block forms its query heads itself, and the block whose tile holds the new position
+    // forms that position's key and value rows: they go to the slabs and straight into the tile.
+    const int new_row = PREP ? (n_pos - 1) - s0 : -1;  // in [0, len) only in the last live tile
     // stage K and V (rows past the context are zero)
     {
         uint4 kr[NLD], vr[NLD];
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
             const int idx = tid + i * 256, pos = idx / CPR, c = idx % CPR;
-            if (pos < len) {
+            if (pos < len && pos != new_row) {
                 const int64_t g = (int64_t)(s0 + pos) * a.kv_dim + off + c * 8;
                 kr[i] = *(const uint4*)(a.k + g);
                 vr[i] = *(const uint4*)(a.v + g);
@@ -239,13 +286,46 @@ __global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, fl
                 vr[i] = make_uint4(0, 0, 0, 0);
             }
         }
-        for (int i = tid; i < G * HD / 4; i += 256)
-            ((float4*)qs)[i] = ((const float4*)(a.q + ((int64_t)t * a.n_head + h0) * HD))[i];
+        if (!PREP) {
+            for (int i = tid; i < G * HD / 4; i += 256)
+                ((float4*)qs)[i] = ((const float4*)(a.q + ((int64_t)t * a.n_head + h0) * HD))[i];
+        } else {
+            constexpr int LPH = HD / 4, HPP = 64 / LPH;  // lanes per head, heads per wave pass
+            const int li = lane % LPH, pos_now = n_pos - 1;
+            for (int g0 = wave * HPP; g0 < G; g0 += 4 * HPP) {
+                const int g = g0 + lane / LPH;  // G is a multiple of HPP or smaller than it
+                if (g < G) {
+                    float4 v = ((const float4*)(pr.qg + (int64_t)(h0 + g) * 2 * HD))[li];
+                    v = head_norm_rope<HD>(v, pr.q_norm, pr.eps, pr.rope, pr.n_rot, pos_now, li);
+                    ((float4*)(qs + g * HD))[li] = v;
+                }
+            }
+            if (new_row >= 0 && new_row < len) {
+                if (wave == 0 && lane < LPH) {
+                    float4 v = ((const float4*)(pr.kproj + (int64_t)h_kv * HD))[li];
+                    v = head_norm_rope<HD>(v, pr.k_norm, pr.eps, pr.rope, pr.n_rot, pos_now, li);
+                    uint2 hv;
+                    hv.x = (uint32_t)it_f32_to_f16(v.x) | ((uint32_t)it_f32_to_f16(v.y) << 16);
+                    hv.y = (uint32_t)it_f32_to_f16(v.z) | ((uint32_t)it_f32_to_f16(v.w) << 16);
+                    *(uint2*)(pr.k_slab + (int64_t)pos_now * a.kv_dim + off + 4 * li) = hv;
+                    *(uint2*)(ktile + new_row * KSTR + 8 * li) = hv;
+                } else if (wave == 1 && lane < LPH) {
+                    const float4 v = ((const float4*)(pr.vproj + (int64_t)h_kv * HD))[li];
+                    uint2 hv;
+                    hv.x = (uint32_t)it_f32_to_f16(v.x) | ((uint32_t)it_f32_to_f16(v.y) << 16);
+                    hv.y = (uint32_t)it_f32_to_f16(v.z) | ((uint32_t)it_f32_to_f16(v.w) << 16);
+                    *(uint2*)(pr.v_slab + (int64_t)pos_now * a.kv_dim + off + 4 * li) = hv;
+                    *(uint2*)(vtile + new_row * HD * 2 + 8 * li) = hv;
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
             const int idx = tid + i * 256, pos = idx / CPR, c = idx % CPR;
-            *(uint4*)(ktile + pos * KSTR + c * 16) = kr[i];
-            *(uint4*)(vtile + pos * HD * 2 + c * 16) = vr[i];
+            if (pos != new_row) {
+                *(uint4*)(ktile + pos * KSTR + c * 16) = kr[i];
+                *(uint4*)(vtile + pos * HD * 2 + c * 16) = vr[i];
+            }
         }
     }
     __syncthreads();
@@ -264,15 +344,11 @@ __global__ __launch_bounds__(256) void attend_tile_k(AttnArgs a, int n_split, fl
                    q1.z * it_f16_to_f32((uint16_t)(kk.w & 0xffff)) + q1.w * it_f16_to_f32((uint16_t)(kk.w >> 16));
         }
         const float sco = lane < len ? acc * a.scale : -INFINITY;
-        float m = sco;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+        const float m = group_max<64>(sco);
         const float p = lane < len ? __expf(sco - m) : 0.0f;
-        float l = p;
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+        const float l = group_sum_tail<64>(p);
         sc[lane * G + g] = p;
-        if (lane == 0) {
+        if (lane == 63) {
             mrow[g] = m;
             lrow[g] = l;
         }
@@ -399,14 +475,41 @@ int attend_split_count(int n_pos_max, int n_q, int head_dim, int group) {
     return (n_pos_max + chunk - 1) / chunk;
 }
 
+bool attend_tile_prep_ok(const AttnArgs& a, const TilePrepP& pr) {
+    const int G = a.n_head / a.n_head_kv, half = pr.n_rot / 2;
+    if (a.n_q != 1 || !tile_path(1, a.head_dim, G) || !a.n_pos_dyn) return false;
+    const int lph = a.head_dim / 4, hpp = 64 / lph;
+    if (G % hpp && G > hpp) return false;
+    // the rotated halves must be whole lanes and a power-of-two number of them, inside the head
+    if (pr.n_rot <= 0 || half % 4 || ((half / 4) & (half / 4 - 1)) || pr.n_rot > a.head_dim) return false;
+    return a.kv_dim % 4 == 0;
+}
+
+static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
+                              const float* gate, int gate_stride, hipStream_t s);
+
 void attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* out, const float* gate,
                         int gate_stride, hipStream_t s) {
+    attend_split_impl(a, nullptr, n_split, scratch, out, gate, gate_stride, s);
+}
+
+void attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
+                             const float* gate, int gate_stride, hipStream_t s) {
+    attend_split_impl(a, &pr, n_split, scratch, out, gate, gate_stride, s);
+}
+
+static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
+                              const float* gate, int gate_stride, hipStream_t s) {
     if (a.n_q <= 0) return;
     const int G = a.n_head / a.n_head_kv;
     dim3 grid(a.n_q * a.n_head_kv, n_split), block(256);
     const bool tile = tile_path(a.n_q, a.head_dim, G);
     if (tile) {
-#define IT_TILE(HD, GG) hipLaunchKernelGGL((attend_tile_k<HD, GG>), grid, block, 0, s, a, n_split, scratch)
+#define IT_TILE(HD, GG)                                                                                      \
+    do {                                                                                                     \
+        if (prep) hipLaunchKernelGGL((attend_tile_k<HD, GG, true>), grid, block, 0, s, a, *prep, n_split, scratch); \
+        else hipLaunchKernelGGL((attend_tile_k<HD, GG, false>), grid, block, 0, s, a, TilePrepP{}, n_split, scratch); \
+    } while (0)
 #define IT_TILE_G(HD)                  \
     switch (G) {                       \
         case 1: IT_TILE(HD, 1); break; \

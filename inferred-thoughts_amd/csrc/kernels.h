@@ -121,6 +121,20 @@ void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s);
 // split-K flash decoding; scratch: n_q*n_head*n_split*(head_dim+2) floats.
 int attend_split_count(int n_pos_max, int n_q, int head_dim, int group);
 void attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);
+// What one decode token's attention needs before it can attend, folded into the tile kernel: the
+// query heads' norm + rotation (every block, for its own heads) and the new position's key
+// (norm + rotation) and value rows, written to the slabs by the block whose tile holds them.
+struct TilePrepP {
+    const float *qg, *kproj, *vproj;  // wq output [n_head][2 * head_dim] (q then gate), k and v projections
+    const float *q_norm, *k_norm;
+    const float2* rope;               // [pos][n_rot / 2] (cos, sin)
+    int n_rot;
+    float eps;
+    uint16_t *k_slab, *v_slab;
+};
+bool attend_tile_prep_ok(const AttnArgs& a, const TilePrepP& pr);
+void attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
+                             const float* gate, int gate_stride, hipStream_t s);
 // the same with the merge multiplying by sigmoid(gate[head * gate_stride + i]) (n_q == 1)
 void attend_split_gated(const AttnArgs& a, int n_split_max, float* scratch, float* out, const float* gate,
                         int gate_stride, hipStream_t s);

@@ -110,6 +110,46 @@ int main() {
         snprintf(nm, sizeof nm, "moe efmt=%d n_in=%d ff=%d glu shared", efmt, n_in, ff); report(nm, shs[0], shs[1]);
         snprintf(nm, sizeof nm, "moe efmt=%d n_in=%d ff=%d down+residual", efmt, n_in, ff); report(nm, xs2[0], xs2[1]);
     }
+    // ---- attention: prep folded into the tile kernel against attn_prep + the plain tile kernel
+    for (int hd : {64, 128, 256}) for (int n_pos : {1, 64, 65, 300}) {
+        const int nh = hd == 256 ? 16 : 8, nkv = 2, kvd = nkv * hd, n_rot = hd / 4, half = n_rot / 2, cap = 512;
+        auto qg = randf((size_t)nh * 2 * hd), kp = randf(kvd), vp = randf(kvd), qn = randf(hd, 0.5f), kn = randf(hd, 0.5f);
+        std::vector<float> tab((size_t)cap * half * 2);
+        for (int p = 0; p < cap; p++) for (int i = 0; i < half; i++) { double a = p * std::pow(1e6, -2.0 * i / n_rot); tab[((size_t)p * half + i) * 2] = (float)std::cos(a); tab[((size_t)p * half + i) * 2 + 1] = (float)std::sin(a); }
+        std::vector<uint16_t> kslab((size_t)cap * kvd), vslab((size_t)cap * kvd);
+        for (auto& x : kslab) x = f2h(std::normal_distribution<float>(0, 1)(rng));
+        for (auto& x : vslab) x = f2h(std::normal_distribution<float>(0, 1)(rng));
+        float *dqg = dev(qg), *dkp = dev(kp), *dvp = dev(vp), *dqn = dev(qn), *dkn = dev(kn); float2* dtab = (float2*)dev(tab);
+        const int pos = n_pos - 1; int* dpos = dev(std::vector<int>{pos}); int* dnpos = dev(std::vector<int>{n_pos});
+        const int n_split = attend_split_count(cap, 1, hd, nh / nkv);
+        std::vector<float> outs[2]; std::vector<uint16_t> krows[2], vrows[2];
+        for (int fused = 0; fused < 2; fused++) {
+            uint16_t *dk = dev(kslab), *dv = dev(vslab);
+            float* dq = dev(std::vector<float>((size_t)nh * hd, 0.f)); float* dout = dev(std::vector<float>((size_t)nh * hd, 0.f));
+            float* scratch = dev(std::vector<float>((size_t)nh * n_split * (hd + 2), 0.f));
+            AttnArgs a{dq, dk, dv, 1, kvd, 0, hd, nh, nkv, 1.0f / std::sqrt((float)hd), dnpos};
+            const float* gate = dqg + hd;
+            if (!fused) {
+                AttnPrepP pp{}; pp.qg = dqg; pp.k = dkp; pp.v = dvp; pp.q_norm = dqn; pp.k_norm = dkn; pp.rope = dtab; pp.pos_dyn = dpos; pp.q = dq;
+                pp.k_slab = dk; pp.v_slab = dv; pp.n_head = nh; pp.n_head_kv = nkv; pp.head_dim = hd; pp.n_rot = n_rot; pp.kv_dim = kvd; pp.exact = 0; pp.eps = 1e-6f;
+                attn_prep(pp, 0);
+                attend_split_gated(a, n_split, scratch, dout, gate, 2 * hd, 0);
+            } else {
+                TilePrepP tp{}; tp.qg = dqg; tp.kproj = dkp; tp.vproj = dvp; tp.q_norm = dqn; tp.k_norm = dkn; tp.rope = dtab; tp.n_rot = n_rot; tp.eps = 1e-6f; tp.k_slab = dk; tp.v_slab = dv;
+                if (!attend_tile_prep_ok(a, tp)) { printf("attention prep hd=%d: fused form refused  MISMATCH\n", hd); g_bad++; break; }
+                attend_split_gated_prep(a, tp, n_split, scratch, dout, gate, 2 * hd, 0);
+            }
+            outs[fused] = host(dout, (size_t)nh * hd);
+            krows[fused] = host(dk + (size_t)pos * kvd, kvd); vrows[fused] = host(dv + (size_t)pos * kvd, kvd);
+        }
+        if (outs[1].empty()) continue;
+        char nm[128];
+        snprintf(nm, sizeof nm, "attention prep folded in, hd=%d n_pos=%d: output", hd, n_pos); report(nm, outs[1], outs[0]);
+        int kd = 0, vd = 0;
+        for (int i = 0; i < kvd; i++) { kd += std::abs((int)krows[0][i] - (int)krows[1][i]) > 1; vd += vrows[0][i] != vrows[1][i]; }
+        printf("attention prep folded in, hd=%d n_pos=%d: new K row %d values off by more than one f16 step, new V row %d differ  %s\n", hd, n_pos, kd, vd, kd || vd ? "MISMATCH" : "ok");
+        if (kd || vd) g_bad++;
+    }
     printf("%d mismatches\n", g_bad);
     return g_bad ? 1 : 0;
 }
