@@ -112,7 +112,7 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     a.exact = exact;
     a.n_mats = 4;
     a.m[0] = mat_of(mqkv, 1, (float*)cv);
-    a.m[1] = mat_of(mz, 0);
+    a.m[1] = mat_of(mz, exact ? 0 : 3);  // fast mode stores silu(z) once here instead of in every block of ssm_out
     a.m[2] = mat_of(ma, 0);
     a.m[3] = mat_of(mb, 0);
     a.conv_state = (float*)conv.p[0];
@@ -141,7 +141,7 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     b.gate = (const float*)z;
     b.eps = rh.f[0];
     b.n_in = (int)vdim;
-    b.mode = 2;
+    b.mode = exact ? 2 : 3;
     b.head_dim = (int)dv;
     b.exact = exact;
     b.n_mats = 1;

@@ -198,7 +198,7 @@ __device__ __forceinline__ void stage_activation(const float* x, int n_in, int m
             v[k].z = v[k].z * scale * w[k].z;
             v[k].w = v[k].w * scale * w[k].w;
         }
-    } else if (mode == 2) {
+    } else if (mode == 2 || mode == 3) {
         const int lh = head_dim >> 2;  // lanes per head
 #pragma unroll
         for (int k = 0; k < 2; k++) {
@@ -209,10 +209,11 @@ __device__ __forceinline__ void stage_activation(const float* x, int n_in, int m
                 const float hs = 1.0f / sqrtf((float)(part / (double)head_dim) + eps);
                 const float4 w = ((const float4*)norm_w)[qi & (lh - 1)];
                 const float4 g = ((const float4*)gate)[qi];
-                v[k].x = it_silu(g.x) * (v[k].x * hs * w.x);
-                v[k].y = it_silu(g.y) * (v[k].y * hs * w.y);
-                v[k].z = it_silu(g.z) * (v[k].z * hs * w.z);
-                v[k].w = it_silu(g.w) * (v[k].w * hs * w.w);
+                // mode 3: the producer already stored silu(gate)
+                v[k].x = (mode == 2 ? it_silu(g.x) : g.x) * (v[k].x * hs * w.x);
+                v[k].y = (mode == 2 ? it_silu(g.y) : g.y) * (v[k].y * hs * w.y);
+                v[k].z = (mode == 2 ? it_silu(g.z) : g.z) * (v[k].z * hs * w.z);
+                v[k].w = (mode == 2 ? it_silu(g.w) : g.w) * (v[k].w * hs * w.w);
             }
         }
     }
@@ -299,6 +300,8 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                     m.out[j] = a;
                 } else if (m.epi == 2) {
                     m.out[j] = cp[r] + a;
+                } else if (m.epi == 3) {
+                    m.out[j] = it_silu(a);
                 } else {
                     // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
                     float* past = p.conv_state + (int64_t)j * 3;
@@ -332,7 +335,7 @@ bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
     if (!g.ok || p.n_in > FT * 8 || p.n_in % 32) return false;
     if (!aligned16(p.x) || !aligned16(p.x_copy) || !aligned16(p.x_copy2)) return false;
     if (p.mode == 1 && !aligned16(p.norm_w)) return false;
-    if (p.mode == 2) {
+    if (p.mode == 2 || p.mode == 3) {
         const int lh = p.head_dim / 4;
         if (p.head_dim % 4 || lh < 1 || lh > 64 || (lh & (lh - 1)) || p.n_in % p.head_dim) return false;
         if (!aligned16(p.norm_w) || !aligned16(p.gate)) return false;

@@ -224,6 +224,8 @@ IT_DEV void finish_rows(const FusedGemvP& p, const FusedMat& m, int row0, int nr
         m.out[j] = acc;
     } else if (m.epi == 2) {
         m.out[j] += acc;
+    } else if (m.epi == 3) {
+        m.out[j] = it_silu(acc);
     } else {
         // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
         float* past = p.conv_state + (int64_t)j * 3;
@@ -276,7 +278,7 @@ __global__ __launch_bounds__(FG_THREADS) void fused_gemv_k(FusedGemvP p) {
         float scale = 1.0f / sqrtf(mean + p.eps);
         for (int i = tid; i < n_in; i += FG_THREADS) xf[i] = xf[i] * scale * p.norm_w[i];
         __syncthreads();
-    } else if (p.mode == 2) {
+    } else if (p.mode == 2 || p.mode == 3) {
         const int hd = p.head_dim, nh = n_in / hd;  // nh <= 64 (checked on the host)
         if (p.exact) {
             if (tid < nh) {
@@ -300,7 +302,7 @@ __global__ __launch_bounds__(FG_THREADS) void fused_gemv_k(FusedGemvP p) {
         __syncthreads();
         for (int i = tid; i < n_in; i += FG_THREADS) {
             float core = xf[i] * hscale[i / hd] * p.norm_w[i % hd];
-            xf[i] = it_silu(p.gate[i]) * core;
+            xf[i] = (p.mode == 2 ? it_silu(p.gate[i]) : p.gate[i]) * core;
         }
         __syncthreads();
     }

@@ -10,13 +10,13 @@ struct FusedMat {
     const uint8_t* s;
     float* out;
     int n_out, fmt;
-    int epi;     // 0 store, 1 causal conv (kernel 4) + silu, 2 accumulate into out
+    int epi;     // 0 store, 1 causal conv (kernel 4) + silu, 2 accumulate into out, 3 store silu (fast kernels only)
     int group0;  // filled by the launcher
 };
 struct FusedGemvP {
     const float* x;       // [n_in] f32
     const float* norm_w;  // rms_norm weight (mode 1: [n_in]; mode 2: [head_dim])
-    const float* gate;    // mode 2: silu gate, [n_in]
+    const float* gate;    // mode 2: silu gate, [n_in]; mode 3 (fast kernels only): the same gate, already silu'd
     float* x_copy;        // optional: the activation after the prologue, f32, written by block 0
     float* x_copy2;       // optional second copy (a whole-row gather of it)
     float eps;

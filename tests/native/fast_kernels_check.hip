@@ -48,7 +48,7 @@ void report(const char* what, const std::vector<float>& a, const std::vector<flo
 int main() {
     int fmts[2] = {W_Q8_0, W_NVFP4};
     // ---- fused_gemv
-    for (int fmt : fmts) for (int n_in : {256, 512, 1024, 2048, 4096}) for (int mode : {0, 1, 2}) for (int epi0 : {0, 1, 2}) {
+    for (int fmt : fmts) for (int n_in : {256, 512, 1024, 2048, 4096}) for (int mode : {0, 1, 2, 3}) for (int epi0 : {0, 1, 2, 3}) {
         int rows[3] = {1000, 512, 9};
         Mat m[3]; for (int i = 0; i < 3; i++) m[i] = make_mat(fmt, rows[i], n_in);
         auto x = randf(n_in), nw = randf(n_in, 0.5f), gate = randf(n_in);

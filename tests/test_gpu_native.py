@@ -18,4 +18,4 @@ def test_fast_kernels_match_order_preserving_kernels():
     r = subprocess.run([str(BIN)], capture_output=True, text=True, timeout=300)
     bad = [l for l in r.stdout.splitlines() if "MISMATCH" in l or "DIFFERENT" in l]
     assert r.returncode == 0 and not bad, "\n".join(bad[:20]) + r.stderr[-2000:]
-    assert r.stdout.count(" ok") > 300
+    assert r.stdout.count(" ok") > 400
