@@ -25,6 +25,8 @@ sys.path.insert(0, str(ROOT / "inferred-thoughts_amd"))
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA, published
+FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch (fetched + written) of each kernel family, averaged over the full model's per-layer launches,
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 256 MiB copy
 # (profiles/decode_kernels_hbm_traffic_pmc.txt holds the commands and the per-kernel readings)
@@ -84,9 +86,10 @@ def main():
     rng = np.random.default_rng(args.seed)
     prompt = rng.integers(0, model.n_vocab, args.prompt).astype(np.uint32)
 
-    # first pass uploads and repacks every weight: charge it to setup, not to prefill
+    # the first pass uploads and repacks every weight and sizes every device buffer for a full-width pass:
+    # charge it to setup, not to prefill
     t1 = time.time()
-    eng.forward(prompt[:1], want_logits=False)
+    eng.forward(prompt[:min(args.prompt, args.max_batch)], want_logits=False)
     be.sync()
     t_upload = time.time() - t1
     eng.reset()
@@ -119,6 +122,34 @@ def main():
     err = be.take_error()
     if err:
         raise SystemExit(f"device error: {err}")
+
+    n_gdn_layers = sum(1 for il in range(args.layers) if (il + 1) % 4 != 0)
+    # per-family device time of one more identical prefill, and the int8 MFMA rate of its three GEMM families
+    eng.reset()
+    be.profile_begin()
+    eng.prefill(prompt, want_logits=False)
+    prows = be.profile_end()
+    err = be.take_error()
+    if err:
+        raise SystemExit(f"device error: {err}")
+    macs = dict(zip(("matmul (dense GEMV/GEMM)", "moe_glu (expert gate+up)", "matmul_experts (expert down)"),
+                    model.token_macs()))
+    prefill_kernels = {}
+    for r in sorted(prows, key=lambda r: -r["ms"]):
+        k = {"launches": r["launches"], "ms": round(r["ms"], 2)}
+        if r["name"] in macs and r["ms"] > 0:
+            tops = 2 * macs[r["name"]] * args.prompt / (r["ms"] / 1e3) / 1e12
+            k["int8_tops"] = round(tops, 1)
+            k["mfma_frac"] = round(tops / INT8_PEAK_TOPS, 4)
+        if r["name"] == "delta_rule" and r["ms"] > 0 and not args.exact:
+            # chunked form, per (64-token chunk, value head): K S^T, Q S^T and the state update (64 x dk x dv each),
+            # T R and P U (lower triangles, 64 x 64 x dv / 2 each), K K^T and Q K^T (64 x 64 x dk / 2 each)
+            C, dk, dv, heads = 64, 128, 128, 32
+            chunk_macs = 3 * C * dk * dv + C * C * dv + C * C * dk
+            flops = 2 * chunk_macs * heads * (args.prompt / C) * n_gdn_layers
+            k["fp32_tflops"] = round(flops / (r["ms"] / 1e3) / 1e12, 1)
+            k["mfma_frac"] = round(flops / (r["ms"] / 1e3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
+        prefill_kernels[r["name"]] = k
 
     # algorithmic bytes of one decode token (weights once + GDN state r+w + KV read)
     n_attn = sum(1 for il in range(args.layers) if (il + 1) % 4 == 0)
@@ -175,6 +206,7 @@ def main():
                    "experts": "512 top-10 + shared, NVFP4", "dense": "Q8_0 (router and ssm_alpha/beta Q8_0)",
                    "mode": "exact" if args.exact else "fast", "batch": 1},
         "prefill_tok_s": round(args.prompt / t_prefill, 1),
+        "prefill_kernels": prefill_kernels,
         "bytes_per_token": int(tok_bytes),
         "token_roofline": {"bound": "hbm", "achieved": round(whole, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": round(whole / HBM_PEAK_GBS, 4)},

@@ -238,6 +238,9 @@ void it_model_close(it_model*);
 void it_model_dims(const it_model*, uint64_t out[10]);
 /* weight bytes one decode token reads (src/model/qwen35.rs:875-939) */
 uint64_t it_model_decode_weight_bytes(const it_model*);
+/* multiply-accumulates of one token's pass without the output head: dense matrices, routed expert gate+up,
+ * routed expert down (the matrices of src/model/qwen35.rs:875-939) */
+void it_model_token_macs(const it_model*, uint64_t out[3]);
 it_engine* it_engine_new(it_model*, it_hip*, uint64_t n_ctx, uint64_t max_batch);
 void it_engine_free(it_engine*);
 void it_engine_reset(it_engine*);

@@ -520,6 +520,21 @@ const float2* it_hip::rope_table(float theta, uint64_t n_rot, uint64_t need_pos)
     return r.dev;
 }
 
+float* it_hip::gdn_work_for(size_t floats) {
+    if (gdn_work_floats < floats) {
+        need_eager("delta rule chunk scratch has to grow");
+        if (gdn_work) {
+            check(hipStreamSynchronize(stream), "sync before scratch free");
+            (void)hipFree(gdn_work);
+            gdn_work = nullptr;
+            gdn_work_floats = 0;
+        }
+        if (!check(hipMalloc((void**)&gdn_work, floats * sizeof(float)), "hipMalloc(delta rule chunk scratch)")) return nullptr;
+        gdn_work_floats = floats;
+    }
+    return gdn_work;
+}
+
 int32_t* it_hip::moe_work_for(size_t picks, size_t n_expert, size_t* ints) {
     *ints = 0;
     if (picks < 32) return nullptr;
@@ -612,6 +627,8 @@ it_hip::~it_hip() {
     if (route_ids) (void)hipFree(route_ids);
     if (route_w) (void)hipFree(route_w);
     if (attn_scratch) (void)hipFree(attn_scratch);
+    if (gdn_work) (void)hipFree(gdn_work);
+    if (moe_work) (void)hipFree(moe_work);
     if (argmax_idx) (void)hipFree(argmax_idx);
     if (argmax_val) (void)hipFree(argmax_val);
     if (argmax_out) (void)hipFree(argmax_out);
@@ -1016,6 +1033,13 @@ void it_hip_delta_rule(it_hip* be, const it_delta* d, float* state, uint64_t sta
     DeltaArgs args{dq, dk, dv, da, db, dssm, ddt, (int)n, (int)d->head_k_dim, (int)d->head_v_dim,
                    (int)d->n_k_heads, (int)d->n_v_heads};
     int exact = be->exact;
+    float* work = nullptr;
+    size_t work_floats = 0;
+    if (!exact && n >= 64 && (d->head_k_dim == 64 || d->head_k_dim == 128) && d->head_v_dim % 16 == 0) {
+        work_floats = itk::gdn_chunk_work_floats((int)n, (int)d->n_v_heads);
+        work = be->gdn_work_for(work_floats);
+        if (!work) return;
+    }
     it_hip::OpRec rec;
     rec.id = OP_DELTA; rec.p[0] = dq; rec.p[1] = dk; rec.p[2] = dv; rec.p[3] = da; rec.p[4] = db; rec.p[5] = dssm;
     rec.p[6] = ddt; rec.p[7] = dstate; rec.p[8] = dout;
@@ -1023,7 +1047,7 @@ void it_hip_delta_rule(it_hip* be, const it_delta* d, float* state, uint64_t sta
     be->submit(it_hip::FAM_DELTA, state_len * 8 + n * (2 * kper + 2 * vper) * 4,
                sig_of(OP_DELTA, dq, dk, dv, da, db, dssm, ddt, args.n_tokens, args.head_k_dim, args.head_v_dim,
                       args.n_k_heads, args.n_v_heads, dstate, dout), rec,
-               [=](hipStream_t s) { delta_rule(args, dstate, dout, exact, s); });
+               [=](hipStream_t s) { delta_rule(args, dstate, dout, exact, work, work_floats, s); });
 }
 
 void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_expert, uint64_t n_used,

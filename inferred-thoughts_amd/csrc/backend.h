@@ -121,6 +121,9 @@ struct it_hip {
     int32_t* moe_work = nullptr;
     size_t moe_work_ints = 0;
     int32_t* moe_work_for(size_t picks, size_t n_expert, size_t* ints);
+    float* gdn_work = nullptr;   // T and P matrices of the chunked delta rule
+    size_t gdn_work_floats = 0;
+    float* gdn_work_for(size_t floats);
     bool route_stage(const it_route* r, const int32_t** ids, const float** w, uint64_t* n_used, uint64_t* n_tok);
 
     // ---- RoPE tables, built on the host in f64 (naive.rs:205-208)

@@ -219,8 +219,9 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
         ((float4*)S)[i] = make_float4(row[4 * i], row[4 * i + 1], row[4 * i + 2], row[4 * i + 3]);
 }
 
-void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, hipStream_t s) {
+void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, float* work, size_t work_floats, hipStream_t s) {
     if (d.n_tokens <= 0) return;
+    if (!exact && delta_rule_chunked(d, state, out, work, work_floats, s)) return;
     float q_scale = 1.0f / sqrtf((float)d.head_k_dim);
     const size_t gate_lds = ((((size_t)d.n_tokens * 2 + 3) & ~(size_t)3) + 4 * GDN_TCH * d.head_k_dim + 2 * GDN_TCH * 32) * sizeof(float);
     if (!exact && d.head_v_dim % 32 == 0 && (d.head_k_dim == 64 || d.head_k_dim == 128) && gate_lds <= 96 * 1024) {

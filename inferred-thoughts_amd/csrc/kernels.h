@@ -105,7 +105,10 @@ struct DeltaArgs {
     const float *q, *k, *v, *alpha, *beta, *ssm_a, *dt_bias;
     int n_tokens, head_k_dim, head_v_dim, n_k_heads, n_v_heads;
 };
-void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, hipStream_t s);
+// work: scratch of gdn_chunk_work_floats() floats for the chunked MFMA form (fast mode, 64 tokens and more); may be null
+void delta_rule(const DeltaArgs& d, float* state, float* out, int exact, float* work, size_t work_floats, hipStream_t s);
+size_t gdn_chunk_work_floats(int n_tokens, int n_v_heads);
+bool delta_rule_chunked(const DeltaArgs& d, float* state, float* out, float* work, size_t work_floats, hipStream_t s);
 
 // ---- attention -------------------------------------------------------------------------
 struct AttnArgs {

@@ -485,6 +485,21 @@ uint64_t it_model_decode_weight_bytes(const it_model* m) {
     return bytes;
 }
 
+void it_model_token_macs(const it_model* m, uint64_t out[3]) {
+    uint64_t dense = 0, glu = 0, down = 0;
+    auto macs = [](const it_weights& w) { return w.n_in * w.n_out; };
+    for (const Block& b : m->blocks) {
+        if (b.recurrent) dense += macs(b.wqkv) + macs(b.wgate) + macs(b.w_alpha) + macs(b.w_beta) + macs(b.w_out);
+        else dense += macs(b.wq) + macs(b.wk) + macs(b.wv) + macs(b.wo);
+        dense += macs(b.router) + macs(b.sh_gate) + macs(b.sh_up) + macs(b.sh_down) + macs(b.sh_gate_inp);
+        glu += m->d.n_used * (b.gate.n_in * b.gate.n_out + b.up.n_in * b.up.n_out);
+        down += m->d.n_used * b.down.n_in * b.down.n_out;
+    }
+    out[0] = dense;
+    out[1] = glu;
+    out[2] = down;
+}
+
 it_engine* it_engine_new(it_model* m, it_hip* be, uint64_t n_ctx, uint64_t max_batch) {
     if (!m || !be || n_ctx == 0) return nullptr;
     it_engine* e = new it_engine();

@@ -92,7 +92,7 @@ it_hip_read_state it_hip_read_kv it_hip_device_report it_hip_reserve_activations
 it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_budget
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
 it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_model_open
-it_model_close it_model_dims it_model_decode_weight_bytes it_engine_new it_engine_free it_engine_reset
+it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
 it_engine_v_slab it_synth_write_gguf""".split()
@@ -183,6 +183,7 @@ def lib() -> C.CDLL:
         "it_model_close": (None, [vp]),
         "it_model_dims": (None, [vp, vp]),
         "it_model_decode_weight_bytes": (u64, [vp]),
+        "it_model_token_macs": (None, [vp, vp]),
         "it_engine_new": (vp, [vp, vp, u64, u64]),
         "it_engine_free": (None, [vp]),
         "it_engine_reset": (None, [vp]),
@@ -427,6 +428,12 @@ class Model:
 
     def decode_weight_bytes(self) -> int:
         return int(self.L.it_model_decode_weight_bytes(self.h))
+
+    def token_macs(self):
+        """(dense, expert gate+up, expert down) multiply-accumulates of one token, output head excluded."""
+        v = (c_u64 * 3)()
+        self.L.it_model_token_macs(self.h, v)
+        return int(v[0]), int(v[1]), int(v[2])
 
     def close(self):
         if self.h:

@@ -66,8 +66,11 @@ def test_attend_split(hip, orc, n_q, n_pos, hd, nh, nkv):
     assert close(bf16_round(a), bf16_round(b), 8e-3)     # one bf16 step at most after rounding the result
 
 
-@pytest.mark.parametrize("n_tok,dk,nk,nv", [(1, 128, 16, 32), (64, 128, 16, 32), (380, 128, 16, 32), (1, 64, 4, 8),
-                                            (37, 64, 4, 8)])
+# up to 63 tokens: rows split over lanes, token by token; 64 and more: chunks of 64 on fp32 MFMA (ragged last chunk,
+# one chunk, the baseline's 5,700-token prefill)
+@pytest.mark.parametrize("n_tok,dk,nk,nv", [(1, 128, 16, 32), (64, 128, 16, 32), (65, 128, 16, 32), (380, 128, 16, 32),
+                                            (2048, 128, 16, 32), (5700, 128, 16, 32), (1, 64, 4, 8), (37, 64, 4, 8),
+                                            (63, 128, 16, 32), (127, 64, 4, 8), (200, 64, 4, 8)])
 def test_delta_rule_fast(hip, orc, n_tok, dk, nk, nv):
     fresh(hip)
     r = rng(32)
@@ -83,6 +86,27 @@ def test_delta_rule_fast(hip, orc, n_tok, dk, nk, nv):
     orc.delta_rule(q, k, v, alpha, beta, ssm_a, dt, dk, dv, nk, nv, sb, b)
     hip.raise_if_error()
     assert close(a, b), np.abs(a - b).max()
+    assert close(sa, sb), np.abs(sa - sb).max()
+
+
+def test_delta_rule_fast_state_carries_over_calls(hip, orc):
+    """Three calls in a row on one state (chunked, token by token, chunked) equal the oracle's."""
+    fresh(hip)
+    r = rng(34)
+    dk = dv = 128; nk, nv = 16, 32
+    ssm_a = -(0.5 + r.random(nv)).astype(np.float32); dt = (r.standard_normal(nv) * 0.3).astype(np.float32)
+    sa = (r.standard_normal(nv * dk * dv) * 0.1).astype(np.float32); sb = sa.copy()
+    for n_tok in (150, 9, 70):
+        q = l2n(r.standard_normal(n_tok * nk * dk).astype(np.float32), dk); k = l2n(r.standard_normal(n_tok * nk * dk).astype(np.float32), dk)
+        v = r.standard_normal(n_tok * nv * dv).astype(np.float32)
+        alpha = r.standard_normal(n_tok * nv).astype(np.float32); beta = r.standard_normal(n_tok * nv).astype(np.float32)
+        a, b = np.zeros(n_tok * nv * dv, np.float32), np.zeros(n_tok * nv * dv, np.float32)
+        hip.begin_pass(n_tok)
+        hip.delta_rule(q, k, v, alpha, beta, ssm_a, dt, dk, dv, nk, nv, sa, a); hip.host_needs(a)
+        orc.delta_rule(q, k, v, alpha, beta, ssm_a, dt, dk, dv, nk, nv, sb, b)
+        hip.raise_if_error()
+        assert close(a, b), (n_tok, np.abs(a - b).max())
+    hip.read_state(sa)
     assert close(sa, sb), np.abs(sa - sb).max()
 
 
