@@ -48,8 +48,9 @@ def main():
     ap.add_argument("--layers", type=int, default=48, help="48 is the baseline config; fewer only for quick checks")
     ap.add_argument("--prompt", type=int, default=5700)
     ap.add_argument("--ctx", type=int, default=8192)
-    ap.add_argument("--max-batch", type=int, default=2048,
-                    help="tokens per prefill pass (the reference's default is 512; expert matrices are read once per pass)")
+    ap.add_argument("--max-batch", type=int, default=8192,
+                    help="tokens per prefill pass; the default takes the 5,700-token prompt through each layer in one "
+                         "pass (layer-at-a-time prefill); the reference's own default is 512")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--exact", action="store_true", help="CPU-order reductions (bit-exact mode)")

@@ -520,6 +520,22 @@ const float2* it_hip::rope_table(float theta, uint64_t n_rot, uint64_t need_pos)
     return r.dev;
 }
 
+void* it_hip::moe_f16_for(size_t bytes) {
+    if (moe_f16_bytes < bytes) {
+        need_eager("expert activation scratch has to grow");
+        if (moe_f16) {
+            check(hipStreamSynchronize(stream), "sync before scratch free");
+            (void)hipFree(moe_f16);
+            moe_f16 = nullptr;
+            moe_f16_bytes = 0;
+        }
+        const size_t want = bytes + bytes / 4;
+        if (!check(hipMalloc(&moe_f16, want), "hipMalloc(expert activation scratch)")) return nullptr;
+        moe_f16_bytes = want;
+    }
+    return moe_f16;
+}
+
 float* it_hip::gdn_work_for(size_t floats) {
     if (gdn_work_floats < floats) {
         need_eager("delta rule chunk scratch has to grow");
@@ -628,6 +644,7 @@ it_hip::~it_hip() {
     if (route_w) (void)hipFree(route_w);
     if (attn_scratch) (void)hipFree(attn_scratch);
     if (gdn_work) (void)hipFree(gdn_work);
+    if (moe_f16) (void)hipFree(moe_f16);
     if (moe_work) (void)hipFree(moe_work);
     if (argmax_idx) (void)hipFree(argmax_idx);
     if (argmax_val) (void)hipFree(argmax_val);
@@ -1111,6 +1128,12 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
     size_t work_ints;
     int32_t* work = be->moe_work_for(picks, w->n_expert, &work_ints);
+    void* fwork = nullptr;
+    size_t fwork_bytes = 0;
+    if (!be->exact && work && v.fmt == itk::W_NVFP4) {
+        fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)w->n_in);
+        fwork = be->moe_f16_for(fwork_bytes);
+    }
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
@@ -1118,6 +1141,8 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
+                   if (fwork && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, s))
+                       return;
                    if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
                        matmul_experts(v, ids, np, nu, xm, as, aq, dout, s);
                });
@@ -1154,6 +1179,12 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
     size_t work_ints;
     int32_t* work = be->moe_work_for(picks, gate->n_expert, &work_ints);
+    void* fwork = nullptr;
+    size_t fwork_bytes = 0;
+    if (!be->exact && work && g.fmt == itk::W_NVFP4) {
+        fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)gate->n_in);
+        fwork = be->moe_f16_for(fwork_bytes);
+    }
     it_hip::OpRec rec;
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
@@ -1163,6 +1194,8 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
                [=](hipStream_t s) {
+                   if (fwork && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, s))
+                       return;
                    if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
                        moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s);
                });

@@ -121,6 +121,9 @@ struct it_hip {
     int32_t* moe_work = nullptr;
     size_t moe_work_ints = 0;
     int32_t* moe_work_for(size_t picks, size_t n_expert, size_t* ints);
+    void* moe_f16 = nullptr;     // f16 hi / lo copies of the expert GEMM's activations
+    size_t moe_f16_bytes = 0;
+    void* moe_f16_for(size_t bytes);
     float* gdn_work = nullptr;   // T and P matrices of the chunked delta rule
     size_t gdn_work_floats = 0;
     float* gdn_work_for(size_t floats);

@@ -177,34 +177,39 @@ namespace {
 // One block.  work layout: [0] = number of tiles; tiles as int4 {expert, first slot, pairs, 0};
 // order[slot] = pair index.  The order of pairs inside an expert's list depends on the atomics'
 // arrival order; it only decides which lane computes which pair, never a value.
+// tile_pairs: most pairs of one tile (16 for the int8 kernels, 128 for the f16 kernel).
 __global__ __launch_bounds__(1024) void moe_group_k(const int32_t* __restrict__ ids, int n_picks, int n_expert,
-                                                    int32_t* __restrict__ n_tiles, int4* __restrict__ tiles,
-                                                    int32_t* __restrict__ order) {
+                                                    int tile_pairs, int32_t* __restrict__ n_tiles,
+                                                    int4* __restrict__ tiles, int32_t* __restrict__ order) {
     __shared__ int cnt[1024], off[1024], toff[1024], cur[1024];
     const int tid = threadIdx.x;
-    for (int e = tid; e < n_expert; e += 1024) cnt[e] = 0;
+    cnt[tid] = 0;
     __syncthreads();
     for (int p = tid; p < n_picks; p += 1024) atomicAdd(&cnt[ids[p]], 1);
     __syncthreads();
-    if (tid == 0) {
-        int o = 0, t = 0;
-        for (int e = 0; e < n_expert; e++) {
-            off[e] = o;
-            toff[e] = t;
-            o += cnt[e];
-            t += (cnt[e] + 15) >> 4;
-        }
-        *n_tiles = t;
-    }
+    // exclusive prefix sums of the pair counts and of the tile counts, all 1024 slots at once
+    const int mine = tid < n_expert ? cnt[tid] : 0;
+    const int my_tiles = (mine + tile_pairs - 1) / tile_pairs;
+    off[tid] = mine;
+    toff[tid] = my_tiles;
     __syncthreads();
-    for (int e = tid; e < n_expert; e += 1024) cur[e] = off[e];
+    for (int d = 1; d < 1024; d <<= 1) {
+        const int a = tid >= d ? off[tid - d] : 0, b = tid >= d ? toff[tid - d] : 0;
+        __syncthreads();
+        off[tid] += a;
+        toff[tid] += b;
+        __syncthreads();
+    }
+    if (tid == 1023) *n_tiles = toff[1023];
+    const int my_off = off[tid] - mine, my_toff = toff[tid] - my_tiles;
+    cur[tid] = my_off;
     __syncthreads();
     for (int p = tid; p < n_picks; p += 1024) {
         const int slot = atomicAdd(&cur[ids[p]], 1);
         order[slot] = p;
     }
-    for (int e = tid; e < n_expert; e += 1024)
-        for (int k = 0; k * 16 < cnt[e]; k++) tiles[toff[e] + k] = make_int4(e, off[e] + 16 * k, min(16, cnt[e] - 16 * k), 0);
+    for (int k = 0; k < my_tiles; k++)
+        tiles[my_toff + k] = make_int4(tid, my_off + tile_pairs * k, min(tile_pairs, mine - tile_pairs * k), 0);
 }
 
 struct ExpertsGemmP {
@@ -387,7 +392,7 @@ bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* id
     int32_t* n_tiles = work;
     int4* tiles = (int4*)(work + 16);
     int32_t* order = work + 16 + (size_t)(max_tiles + 1) * 4;
-    hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, n_tiles, tiles, order);
+    hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, 16, n_tiles, tiles, order);
     ExpertsGemmP p{};
     p.q = (const uint8_t*)w.q;
     p.s = (const uint8_t*)w.scales;
@@ -415,6 +420,329 @@ bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* id
         if (up) hipLaunchKernelGGL((experts_gemm_k<W_NVFP4, true>), grid, dim3(GT), 0, s, p);
         else hipLaunchKernelGGL((experts_gemm_k<W_NVFP4, false>), grid, dim3(GT), 0, s, p);
     }
+    return true;
+}
+
+
+// =====================================================================================
+// NVFP4 expert matmuls on the f16 matrix cores (fast mode).
+//
+// An NVFP4 weight is (doubled e2m1 value) x (halved e4m3 sub-block scale): at most six significant
+// bits, so it is EXACT in f16, and so is every product with an f16 activation in the f32
+// accumulator.  The Q8_0 activation x = q * dx is divided by a power of two that brings its row
+// into [-1, 1] and split into two f16 numbers (x = hi + lo, 22 bits kept); the power of two comes
+// back in the epilogue.  With the scales inside the operands the whole k range accumulates in the
+// MFMA accumulator: no per-block scaling on the vector ALU, which bounds the int8 kernels above.
+// What differs from the CPU path is the f32 summation order and the 2^-22 of the split.
+//
+// A block owns one tile of up to 128 (token, pick) pairs of one expert and 128 rows of the
+// gate AND up matrices (GLU) or 256 rows of one matrix.  A wave owns two sets of 32 rows (gate
+// and up rows of the same index, or two row groups) and every token tile, so a token fragment
+// read from LDS feeds four MFMAs (two sets, hi and lo).  Weight nibbles go from HBM straight to
+// the owning lane's registers (a lane owns 16 contiguous bytes of a row per 64-wide k slab: the
+// k order inside an MFMA is free once the scales are folded in) and are expanded there: a byte
+// permute yields the f16 high bytes of four magnitudes, the sign bit is or-ed in, two more
+// permutes interleave zero low bytes, and v_pk_mul_f16 applies the sub-block scale.
+//
+// MFMA operand layout (32x32x16, f16): lane l supplies 8 k values of row (l % 32), k group
+// l / 32, for both A (weight rows) and B (tokens); it receives D for token l % 32 and weight
+// rows 8 * (i / 4) + 4 * (l / 32) + i % 4, i = 0..15.
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int FK = 64;          // k per slab
+constexpr int FBS = FK + 4;     // LDS row stride of a token slab, in f16 (136 bytes: no bank is hit twice by 16 lanes)
+constexpr int FPAIRS = 128;     // pairs per tile
+
+// rows of f16 hi / lo and the row's power of two, from Q8_0 quants and scales
+__global__ __launch_bounds__(256) void acts_split_f16_k(const int8_t* __restrict__ q, const float* __restrict__ sc,
+                                                         int n_in, uint16_t* __restrict__ xh, uint16_t* __restrict__ xl,
+                                                         float* __restrict__ rscale) {
+    __shared__ float part[4];
+    const int row = blockIdx.x, tid = threadIdx.x, nb = n_in >> 5;
+    float mx = 0.0f;
+    for (int b = tid; b < nb; b += 256) mx = fmaxf(mx, fabsf(sc[(int64_t)row * nb + b]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((tid & 63) == 0) part[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])) * 127.0f;
+    int ex = 0;
+    if (mx > 0.0f) (void)frexpf(mx, &ex);                     // mx = m * 2^ex, m in [0.5, 1)
+    ex = max(-100, min(100, ex));
+    const float down = ldexpf(1.0f, -ex);
+    if (tid == 0) rscale[row] = ldexpf(1.0f, ex);
+    for (int i = tid; i < n_in / 4; i += 256) {
+        const uint32_t qq = ((const uint32_t*)(q + (int64_t)row * n_in))[i];
+        const float d = sc[(int64_t)row * nb + (i >> 3)] * down;
+        uint16_t h[4], l[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float x = (float)(int8_t)(qq >> (8 * k)) * d;
+            const _Float16 hi = (_Float16)x;
+            const _Float16 lo = (_Float16)(x - (float)hi);
+            h[k] = __builtin_bit_cast(uint16_t, hi);
+            l[k] = __builtin_bit_cast(uint16_t, lo);
+        }
+        ((uint2*)(xh + (int64_t)row * n_in))[i] = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+        ((uint2*)(xl + (int64_t)row * n_in))[i] = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+    }
+}
+
+// four nibbles (one per byte, 0..15) -> four f16 weights (two dwords), scaled by the sub-block scale
+__device__ __forceinline__ void fp4x4_to_f16x4(uint32_t v, h2 scale, h2* a, h2* b) {
+    // f16 high bytes of the doubled e2m1 magnitudes 0 1 2 3 4 6 8 12; the low bytes are zero
+    const uint32_t mag = __builtin_amdgcn_perm(0x4a484644u, 0x42403c00u, v & 0x07070707u);
+    const uint32_t hb = mag | ((v & 0x08080808u) << 4);
+    const uint32_t d0 = __builtin_amdgcn_perm(hb, hb, 0x010c000cu);   // bytes 0, hb.0, 0, hb.1
+    const uint32_t d1 = __builtin_amdgcn_perm(hb, hb, 0x030c020cu);   // bytes 0, hb.2, 0, hb.3
+    *a = __builtin_bit_cast(h2, d0) * scale;
+    *b = __builtin_bit_cast(h2, d1) * scale;
+}
+
+struct ExpertsF16P {
+    const uint8_t *q, *s, *q2, *s2;
+    int64_t q_stride, s_stride;
+    const float *scale2, *scale2_up;
+    const uint16_t *xh, *xl;
+    const float* rscale;
+    float* out;
+    int n_in, n_out, x_mode, n_used;
+    const int32_t* n_tiles;
+    const int4* tiles;
+    const int32_t* order;
+};
+
+template <bool GLU, int T>
+__device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int4 td, uint16_t* Bh, uint16_t* Bl,
+                                                 const int* xrow_s, const int* pair_s) {
+    const int64_t e = td.x;
+    const int cnt = td.z;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, kg = lane >> 5;
+    const int n_in = p.n_in, nslab = n_in / FK;
+    // the two row sets of this wave
+    const int rows_per_block = GLU ? 128 : 256;
+    const int rb0 = blockIdx.y * rows_per_block + (GLU ? 32 : 64) * wave;
+    const int rbase[2] = {rb0, GLU ? rb0 : rb0 + 32};
+    const uint8_t* wq[2] = {p.q + e * p.q_stride, GLU ? p.q2 + e * p.q_stride : p.q + e * p.q_stride};
+    const uint8_t* ws[2] = {p.s + e * p.s_stride, GLU ? p.s2 + e * p.s_stride : p.s + e * p.s_stride};
+    const uint8_t* arow[2];
+    const uint8_t* srow[2];
+#pragma unroll
+    for (int z = 0; z < 2; z++) {
+        const int64_t row = min(rbase[z] + r, p.n_out - 1);
+        arow[z] = wq[z] + row * (n_in >> 1) + 16 * kg;
+        srow[z] = ws[z] + row * (n_in >> 4) + 2 * kg;
+    }
+
+    uint4 ra[2];
+    uint16_t rs[2];
+    uint4 rbh[T], rbl[T];   // 32 * T tokens x 8 segments of 16 bytes = 256 * T segments per array
+    auto fetch = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int z = 0; z < 2; z++) {
+            ra[z] = *(const uint4*)(arow[z] + s * 32);
+            rs[z] = *(const uint16_t*)(srow[z] + s * 4);
+        }
+#pragma unroll
+        for (int u = 0; u < T; u++) {
+            const int idx = tid + u * 256, tok = idx >> 3, seg = idx & 7;
+            const int64_t at = (int64_t)xrow_s[tok] * n_in + s * FK + seg * 8;
+            rbh[u] = *(const uint4*)(p.xh + at);
+            rbl[u] = *(const uint4*)(p.xl + at);
+        }
+    };
+    auto stash = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < T; u++) {
+            const int idx = tid + u * 256, tok = idx >> 3, seg = idx & 7;
+            uint16_t* dh = Bh + (buf * FPAIRS + tok) * FBS + seg * 8;
+            uint16_t* dl = Bl + (buf * FPAIRS + tok) * FBS + seg * 8;
+            *(uint2*)dh = make_uint2(rbh[u].x, rbh[u].y);
+            *(uint2*)(dh + 4) = make_uint2(rbh[u].z, rbh[u].w);
+            *(uint2*)dl = make_uint2(rbl[u].x, rbl[u].y);
+            *(uint2*)(dl + 4) = make_uint2(rbl[u].z, rbl[u].w);
+        }
+    };
+
+    v16f acc[2][T];
+#pragma unroll
+    for (int z = 0; z < 2; z++)
+#pragma unroll
+        for (int tt = 0; tt < T; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[z][tt][i] = 0.0f;
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int s = 0; s < nslab; s++) {
+        const int buf = s & 1;
+        // this slab's weights: 32 nibbles per set -> four fragments of 8 f16
+        h8 af[2][4];
+#pragma unroll
+        for (int z = 0; z < 2; z++) {
+            const _Float16 s0 = (_Float16)it_ue4m3_to_f32(rs[z] & 0xffu), s1 = (_Float16)it_ue4m3_to_f32(rs[z] >> 8);
+            const uint32_t wd[4] = {ra[z].x, ra[z].y, ra[z].z, ra[z].w};
+#pragma unroll
+            for (int n = 0; n < 4; n++) {
+                const h2 sc = n < 2 ? h2{s0, s0} : h2{s1, s1};
+                h2 a0, a1, a2, a3;
+                fp4x4_to_f16x4(wd[n] & 0x0f0f0f0fu, sc, &a0, &a1);          // low nibbles: elements i
+                fp4x4_to_f16x4((wd[n] >> 4) & 0x0f0f0f0fu, sc, &a2, &a3);   // high nibbles: elements 8 + i
+                af[z][n] = h8{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
+            }
+        }
+        if (s + 1 < nslab) fetch(s + 1);
+#pragma unroll
+        for (int n = 0; n < 4; n++) {
+            // bytes 16 * kg + 4 * n .. + 3 of the row's slab: sub-block 2 * kg + n / 2, elements 4 * (n % 2) + {0..3}
+            // from the low nibbles and 8 more from the high ones
+            const int k0 = 32 * kg + 16 * (n >> 1) + 4 * (n & 1);
+#pragma unroll
+            for (int tt = 0; tt < T; tt++) {
+                const uint16_t* bh = Bh + (buf * FPAIRS + 32 * tt + r) * FBS + k0;
+                const uint16_t* bl = Bl + (buf * FPAIRS + 32 * tt + r) * FBS + k0;
+                const uint2 h0 = *(const uint2*)bh, h1 = *(const uint2*)(bh + 8);
+                const uint2 l0 = *(const uint2*)bl, l1 = *(const uint2*)(bl + 8);
+                const h8 vh = __builtin_bit_cast(h8, make_uint4(h0.x, h0.y, h1.x, h1.y));
+                const h8 vl = __builtin_bit_cast(h8, make_uint4(l0.x, l0.y, l1.x, l1.y));
+#pragma unroll
+                for (int z = 0; z < 2; z++) {
+                    acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[z][n], vh, acc[z][tt], 0, 0, 0);
+                    acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[z][n], vl, acc[z][tt], 0, 0, 0);
+                }
+            }
+        }
+        if (s + 1 < nslab) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    const float e2a = p.scale2 ? p.scale2[e] : 1.0f;
+    const float e2b = GLU ? (p.scale2_up ? p.scale2_up[e] : 1.0f) : e2a;
+#pragma unroll
+    for (int tt = 0; tt < T; tt++) {
+        const int slot = 32 * tt + r;
+        if (slot >= cnt) continue;
+        const int64_t pair = pair_s[slot];
+        const float rsc = p.rscale[xrow_s[slot]];
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+            if (GLU) {
+                const int row = rbase[0] + 8 * i4 + 4 * kg;
+                if (row >= p.n_out) continue;
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float g = acc[0][tt][4 * i4 + i] * rsc * e2a, u = acc[1][tt][4 * i4 + i] * rsc * e2b;
+                    o[i] = it_silu(g) * u;
+                }
+                *(float4*)(p.out + pair * p.n_out + row) = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int z = 0; z < 2; z++) {
+                    const int row = rbase[z] + 8 * i4 + 4 * kg;
+                    if (row >= p.n_out) continue;
+                    *(float4*)(p.out + pair * p.n_out + row) =
+                        make_float4(acc[z][tt][4 * i4] * rsc * e2a, acc[z][tt][4 * i4 + 1] * rsc * e2a,
+                                    acc[z][tt][4 * i4 + 2] * rsc * e2a, acc[z][tt][4 * i4 + 3] * rsc * e2a);
+                }
+            }
+        }
+    }
+}
+
+template <bool GLU>
+__global__ __launch_bounds__(256) void experts_f16_k(ExpertsF16P p) {
+    extern __shared__ __align__(16) uint16_t flds[];
+    uint16_t* Bh = flds;                          // [2][128][FBS]
+    uint16_t* Bl = flds + 2 * FPAIRS * FBS;       // [2][128][FBS]
+    __shared__ int xrow_s[FPAIRS], pair_s[FPAIRS];
+    const int tile = blockIdx.x;
+    if (tile >= *p.n_tiles) return;
+    const int4 td = p.tiles[tile];
+    const int cnt = td.z;
+    if (threadIdx.x < FPAIRS) {
+        const int pair = p.order[td.y + min((int)threadIdx.x, cnt - 1)];
+        pair_s[threadIdx.x] = pair;
+        xrow_s[threadIdx.x] = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
+    }
+    __syncthreads();
+    switch ((cnt + 31) >> 5) {
+        case 1: experts_f16_body<GLU, 1>(p, td, Bh, Bl, xrow_s, pair_s); break;
+        case 2: experts_f16_body<GLU, 2>(p, td, Bh, Bl, xrow_s, pair_s); break;
+        case 3: experts_f16_body<GLU, 3>(p, td, Bh, Bl, xrow_s, pair_s); break;
+        default: experts_f16_body<GLU, 4>(p, td, Bh, Bl, xrow_s, pair_s); break;
+    }
+}
+
+}  // namespace
+
+size_t experts_f16_work_ints(int n_picks, int n_expert) {
+    return 16 + (size_t)(n_expert + n_picks / FPAIRS + 2) * 4 + (size_t)n_picks;
+}
+size_t experts_f16_work_bytes(int x_rows, int n_in) {
+    return (size_t)x_rows * n_in * 4 + (((size_t)x_rows * 4 + 255) & ~(size_t)255);
+}
+
+bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
+                      int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
+                      size_t work_ints, void* fwork, size_t fwork_bytes, hipStream_t s) {
+    if (n_picks < 32 || !work || !fwork || w.n_expert > 1024 || w.fmt != W_NVFP4 || w.n_in % FK || w.n_out % 4) return false;
+    if (n_used < 1) n_used = 1;
+    const int x_rows = x_mode == 0 ? n_picks : (x_mode == 1 ? (n_picks + n_used - 1) / n_used : 1);
+    if (work_ints < experts_f16_work_ints(n_picks, w.n_expert) || fwork_bytes < experts_f16_work_bytes(x_rows, w.n_in)) return false;
+    if ((reinterpret_cast<uintptr_t>(w.q) & 15) || w.q_stride % 16 || w.s_stride % 2 || (reinterpret_cast<uintptr_t>(w.scales) & 1) ||
+        (reinterpret_cast<uintptr_t>(act_quants) & 3) || (reinterpret_cast<uintptr_t>(out) & 15))
+        return false;
+    if (up && (up->fmt != w.fmt || up->n_in != w.n_in || up->n_out != w.n_out || (reinterpret_cast<uintptr_t>(up->q) & 15) ||
+               (reinterpret_cast<uintptr_t>(up->scales) & 1) || up->q_stride != w.q_stride || up->s_stride != w.s_stride))
+        return false;
+    static bool sized = false;
+    const size_t lds = (size_t)4 * FPAIRS * FBS * sizeof(uint16_t);
+    if (!sized) {
+        if (hipFuncSetAttribute((const void*)experts_f16_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+            hipFuncSetAttribute((const void*)experts_f16_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        sized = true;
+    }
+    const int max_tiles = w.n_expert + n_picks / FPAIRS + 1;
+    int32_t* n_tiles = work;
+    int4* tiles = (int4*)(work + 16);
+    int32_t* order = work + 16 + (size_t)(max_tiles + 1) * 4;
+    hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, FPAIRS, n_tiles, tiles, order);
+    uint16_t* xh = (uint16_t*)fwork;
+    uint16_t* xl = xh + (size_t)x_rows * w.n_in;
+    float* rscale = (float*)(xl + (size_t)x_rows * w.n_in);
+    hipLaunchKernelGGL(acts_split_f16_k, dim3(x_rows), dim3(256), 0, s, act_quants, act_scales, w.n_in, xh, xl, rscale);
+    ExpertsF16P p{};
+    p.q = (const uint8_t*)w.q;
+    p.s = (const uint8_t*)w.scales;
+    p.q2 = up ? (const uint8_t*)up->q : nullptr;
+    p.s2 = up ? (const uint8_t*)up->scales : nullptr;
+    p.q_stride = w.q_stride;
+    p.s_stride = w.s_stride;
+    p.scale2 = w.scale2;
+    p.scale2_up = up ? up->scale2 : nullptr;
+    p.xh = xh;
+    p.xl = xl;
+    p.rscale = rscale;
+    p.out = out;
+    p.n_in = w.n_in;
+    p.n_out = w.n_out;
+    p.x_mode = x_mode;
+    p.n_used = n_used;
+    p.n_tiles = n_tiles;
+    p.tiles = tiles;
+    p.order = order;
+    if (up) hipLaunchKernelGGL(experts_f16_k<true>, dim3(max_tiles, (w.n_out + 127) / 128), dim3(256), lds, s, p);
+    else hipLaunchKernelGGL(experts_f16_k<false>, dim3(max_tiles, (w.n_out + 255) / 256), dim3(256), lds, s, p);
     return true;
 }
 

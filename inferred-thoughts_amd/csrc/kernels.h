@@ -55,6 +55,14 @@ void matmul_experts(const ExpertsView& w, const int32_t* ids, int n_picks, int n
 // pairs; bit-identical to the per-pair kernels.  `work` is device scratch of experts_group_work_ints ints.
 // Returns false without launching when the shape, format or scratch does not fit.
 size_t experts_group_work_ints(int n_picks, int n_expert);
+// NVFP4 only, fast mode: the same products on the f16 matrix cores, weights expanded exactly to f16 and the
+// Q8_0 activations as an f16 hi/lo pair; results agree with the int8 kernels to ~1e-6 relative.
+// work: experts_f16_work_ints ints; fwork: experts_f16_work_bytes bytes, 16-byte aligned.
+size_t experts_f16_work_ints(int n_picks, int n_expert);
+size_t experts_f16_work_bytes(int x_rows, int n_in);
+bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
+                      int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
+                      size_t work_ints, void* fwork, size_t fwork_bytes, hipStream_t s);
 bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
                   const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
                   hipStream_t s);

@@ -110,6 +110,46 @@ def test_delta_rule_fast_state_carries_over_calls(hip, orc):
     assert close(sa, sb), np.abs(sa - sb).max()
 
 
+# NVFP4 expert matmuls over a batch: pairs grouped by expert and multiplied on the f16 matrix cores (weights exact
+# in f16, activations as an f16 hi/lo pair).  Tiles of 1..4 token groups, an expert with more than one tile,
+# experts with no pair at all, ragged row counts.
+@pytest.mark.parametrize("n_tok,n_expert,n_used,nd,ff", [(48, 64, 10, 2048, 512), (200, 16, 4, 512, 256),
+                                                         (600, 64, 10, 2048, 512), (700, 16, 4, 512, 256),
+                                                         (33, 512, 10, 2048, 512), (90, 8, 2, 256, 192)])
+def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
+    import inferred_hip as ih
+    from oracle import binding as ob
+    fresh(hip)
+    hip.begin_pass(n_tok)
+    r = rng(40)
+    mk = lambda rows, n_in: nvfp4_weights(r, rows, n_in)
+    code = ih.NVFP4
+    scales = [(r.random(n_expert).astype(np.float32) * 0.01 + 0.002) for _ in range(3)]
+    gate, up, down = mk(n_expert * ff, nd), mk(n_expert * ff, nd), mk(n_expert * nd, ff)
+    # token magnitudes over four decades (a Q8_0 block scale is an f16: the gate/up products must stay below 8e6)
+    x = (r.standard_normal(n_tok * nd) * np.repeat(10.0 ** r.uniform(-2.5, 1.5, n_tok), nd)).astype(np.float32)
+    ids = np.stack([r.permutation(n_expert)[:n_used] for _ in range(n_tok)]).astype(np.uint32).reshape(-1)
+    w = r.random(n_tok * n_used).astype(np.float32)
+    pairs = n_tok * n_used
+    route = ih.Hip.host_route(ids, w, n_used)
+    ga, gb = np.zeros(pairs * ff, np.float32), np.zeros(pairs * ff, np.float32)
+    sa, sb = np.zeros(pairs * ff, np.float32), np.zeros(pairs * ff, np.float32)
+    hip.moe_glu(ih.experts(gate, code, nd, ff, n_expert, scales[0]), ih.experts(up, code, nd, ff, n_expert, scales[1]),
+                route, x, ga, sa)
+    orc.moe_glu(ob.experts(gate, code, nd, ff, n_expert, scales[0]), ob.experts(up, code, nd, ff, n_expert, scales[1]),
+                ids, n_used, x, gb, sb)
+    hip.host_needs(ga); hip.raise_if_error()
+    scale = np.repeat(np.abs(gb.reshape(pairs, ff)).max(axis=1) + 1e-30, ff)
+    assert np.all(np.abs(ga - gb) <= 1e-3 * np.maximum(scale, np.abs(gb))), (np.abs(ga - gb) / scale).max()
+    oa, obuf = np.zeros(pairs * nd, np.float32), np.zeros(pairs * nd, np.float32)
+    hip.matmul_experts(ih.experts(down, code, ff, nd, n_expert, scales[2]), route, gb, oa)
+    orc.matmul_experts(ob.experts(down, code, ff, nd, n_expert, scales[2]), ids, n_used, gb, obuf)
+    hip.host_needs(oa); hip.raise_if_error()
+    assert np.isfinite(obuf).all()
+    scale = np.repeat(np.abs(obuf.reshape(pairs, nd)).max(axis=1) + 1e-30, nd)
+    assert np.all(np.abs(oa - obuf) <= 1e-3 * np.maximum(scale, np.abs(obuf))), (np.abs(oa - obuf) / scale).max()
+
+
 @pytest.mark.parametrize("n,nd", [(1, 2048), (33, 2048), (3, 512)])
 def test_rms_norm_fast(hip, orc, n, nd):
     fresh(hip)
