@@ -125,7 +125,7 @@ def main():
         raise SystemExit(f"device error: {err}")
 
     n_gdn_layers = sum(1 for il in range(args.layers) if (il + 1) % 4 != 0)
-    # per-family device time of one more identical prefill, and the int8 MFMA rate of its three GEMM families
+    # per-family device time of one more identical prefill, and the matrix-core rate of each family that uses them
     eng.reset()
     be.profile_begin()
     eng.prefill(prompt, want_logits=False)
@@ -133,24 +133,44 @@ def main():
     err = be.take_error()
     if err:
         raise SystemExit(f"device error: {err}")
-    macs = dict(zip(("matmul (dense GEMV/GEMM)", "moe_glu (expert gate+up)", "matmul_experts (expert down)"),
-                    model.token_macs()))
+    dense_macs, glu_macs, down_macs = model.token_macs()
+    n_attn_layers = args.layers - n_gdn_layers
+    F16_PEAK = 2500.0
     prefill_kernels = {}
     for r in sorted(prows, key=lambda r: -r["ms"]):
         k = {"launches": r["launches"], "ms": round(r["ms"], 2)}
-        if r["name"] in macs and r["ms"] > 0:
-            tops = 2 * macs[r["name"]] * args.prompt / (r["ms"] / 1e3) / 1e12
-            k["int8_tops"] = round(tops, 1)
-            k["mfma_frac"] = round(tops / INT8_PEAK_TOPS, 4)
-        if r["name"] == "delta_rule" and r["ms"] > 0 and not args.exact:
+        sec = r["ms"] / 1e3
+        if sec <= 0:
+            prefill_kernels[r["name"]] = k
+            continue
+        name = r["name"]
+        if name.startswith("matmul (dense"):
+            # Q8_0 x Q8_0 on the int8 matrix cores, both modes
+            tops = 2 * dense_macs * args.prompt / sec / 1e12
+            k.update(unit="int8 MFMA", tops=round(tops, 1), mfma_frac=round(tops / INT8_PEAK_TOPS, 4))
+        elif name.startswith("moe_glu") or name.startswith("matmul_experts"):
+            m = glu_macs if name.startswith("moe_glu") else down_macs
+            useful = 2 * m * args.prompt / sec / 1e12
+            if args.exact:
+                k.update(unit="int8 MFMA", tops=round(useful, 1), mfma_frac=round(useful / INT8_PEAK_TOPS, 4))
+            else:
+                # f16 matrix cores, every product issued twice (activation hi and lo halves)
+                k.update(unit="f16 MFMA", useful_tops=round(useful, 1), tflops=round(2 * useful, 1),
+                         mfma_frac=round(2 * useful / F16_PEAK, 4))
+        elif name == "delta_rule" and not args.exact:
             # chunked form, per (64-token chunk, value head): K S^T, Q S^T and the state update (64 x dk x dv each),
             # T R and P U (lower triangles, 64 x 64 x dv / 2 each), K K^T and Q K^T (64 x 64 x dk / 2 each)
             C, dk, dv, heads = 64, 128, 128, 32
             chunk_macs = 3 * C * dk * dv + C * C * dv + C * C * dk
             flops = 2 * chunk_macs * heads * (args.prompt / C) * n_gdn_layers
-            k["fp32_tflops"] = round(flops / (r["ms"] / 1e3) / 1e12, 1)
-            k["mfma_frac"] = round(flops / (r["ms"] / 1e3) / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
-        prefill_kernels[r["name"]] = k
+            k.update(unit="fp32 MFMA", tflops=round(flops / sec / 1e12, 1),
+                     mfma_frac=round(flops / sec / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4))
+        elif name == "attend" and not args.exact:
+            # causal pairs x head_dim x (scores with the query's hi and lo halves + weighted values)
+            pairs = args.prompt * (args.prompt + 1) / 2
+            flops = 2 * pairs * model.n_head * model.head_dim * 3 * n_attn_layers
+            k.update(unit="f16 MFMA", tflops=round(flops / sec / 1e12, 1), mfma_frac=round(flops / sec / 1e12 / F16_PEAK, 4))
+        prefill_kernels[name] = k
 
     # algorithmic bytes of one decode token (weights once + GDN state r+w + KV read)
     n_attn = sum(1 for il in range(args.layers) if (il + 1) % 4 == 0)

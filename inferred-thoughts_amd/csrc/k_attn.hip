@@ -460,6 +460,7 @@ __global__ __launch_bounds__(1024) void attend_merge_k(const float* __restrict__
 }
 
 void attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hipStream_t s) {
+    if (attend_prefill(a, out, s)) return;
     attend_split_gated(a, n_split, scratch, out, nullptr, 0, s);
 }
 

@@ -50,7 +50,13 @@ def l2n(x, hd):
 
 @pytest.mark.parametrize("n_q,n_pos,hd,nh,nkv", [(1, 1024, 256, 16, 2), (1, 8192, 256, 16, 2), (1, 32000, 256, 16, 2),
                                                   (1, 63, 64, 8, 2), (1, 200, 128, 8, 1), (5, 300, 256, 16, 2),
-                                                  (40, 700, 64, 8, 2)])
+                                                  (16, 300, 256, 16, 2),
+                                                  # more than 16 queries: one pass over the keys on the f16 matrix cores
+                                                  # (whole prompt; a batch at an offset; ragged last query tile; one
+                                                  # to sixteen query heads per KV head)
+                                                  (40, 700, 64, 8, 2), (17, 17, 256, 16, 2), (64, 64, 64, 8, 2),
+                                                  (300, 300, 256, 16, 2), (100, 450, 128, 8, 1), (130, 130, 128, 4, 4),
+                                                  (33, 1000, 256, 16, 2), (70, 70, 64, 16, 1), (1500, 1500, 256, 16, 2)])
 def test_attend_split(hip, orc, n_q, n_pos, hd, nh, nkv):
     fresh(hip)
     r = rng(31)
