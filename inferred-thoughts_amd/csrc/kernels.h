@@ -59,6 +59,10 @@ size_t experts_group_work_ints(int n_picks, int n_expert);
 // Q8_0 activations as an f16 hi/lo pair; results agree with the int8 kernels to ~1e-6 relative.
 // work: experts_f16_work_ints ints; fwork: experts_f16_work_bytes bytes, 16-byte aligned.
 size_t experts_f16_work_ints(int n_picks, int n_expert);
+// pairs sorted into per-expert lists cut into tiles of at most tile_pairs: n_tiles[0] = tile count, tiles = {expert,
+// first slot, pairs, 0}, order[slot] = pair
+void moe_group(const int32_t* ids, int n_picks, int n_expert, int tile_pairs, int32_t* n_tiles, int4* tiles,
+               int32_t* order, hipStream_t s);
 size_t experts_f16_work_bytes(int x_rows, int n_in);
 bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
                       int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
