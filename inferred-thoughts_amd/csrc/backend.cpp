@@ -480,6 +480,7 @@ bool it_hip::route_stage(const it_route* r, const int32_t** ids, const float** w
         check(hipStreamSynchronize(stream), "upload route");
         route_n_used = r->n_used;
         route_n_tok = r->n_tok;
+        route_gen++;
         // remember the ids for bounds checks
     }
     *ids = route_ids;
@@ -551,6 +552,21 @@ float* it_hip::gdn_work_for(size_t floats) {
     return gdn_work;
 }
 
+// true when moe_work already holds this grouping (the gate/up and down products of one MoE layer share it);
+// records the grouping as held otherwise.  Eager passes only: a recorded launch may run later.
+bool it_hip::group_cached(int picks, int n_expert, int tile) {
+    if (mode != Mode::Eager) {
+        group_gen = ~0ull;
+        return false;
+    }
+    const bool hit = group_gen == route_gen && group_picks == picks && group_experts == n_expert && group_tile == tile;
+    group_gen = route_gen;
+    group_picks = picks;
+    group_experts = n_expert;
+    group_tile = tile;
+    return hit;
+}
+
 int32_t* it_hip::moe_work_for(size_t picks, size_t n_expert, size_t* ints) {
     *ints = 0;
     if (picks < 32) return nullptr;
@@ -564,6 +580,7 @@ int32_t* it_hip::moe_work_for(size_t picks, size_t n_expert, size_t* ints) {
             moe_work_ints = 0;
         }
         const size_t want = need + need / 2;
+        group_gen = ~0ull;
         if (!check(hipMalloc((void**)&moe_work, want * sizeof(int32_t)), "hipMalloc(expert grouping scratch)")) return nullptr;
         moe_work_ints = want;
     }
@@ -1089,6 +1106,7 @@ void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_exper
                [=](hipStream_t s) { route_topk(dp, nt, ne, nu, ids, rw, s); });
     be->route_n_used = n_used;
     be->route_n_tok = n_tok;
+    be->route_gen++;
 }
 
 static int x_mode_of(uint64_t rows, uint64_t picks) { return rows == picks ? 0 : (rows > 1 ? 1 : 2); }
@@ -1134,6 +1152,9 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
         fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)w->n_in);
         fwork = be->moe_f16_for(fwork_bytes);
     }
+    // the tile size the launch below will group for: 128 pairs for the f16 kernel, 16 for the int8 one
+    const bool f16_shape = fwork && itk::experts_f16_takes(v, nullptr, np, aq, dout);
+    const bool grouped = work && be->group_cached(np, (int)w->n_expert, f16_shape ? 128 : 16);
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
@@ -1141,9 +1162,9 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
-                   if (fwork && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, s))
+                   if (f16_shape && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
-                   if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
+                   if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
                        matmul_experts(v, ids, np, nu, xm, as, aq, dout, s);
                });
     be->expert_lookups += picks;
@@ -1185,6 +1206,8 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
         fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)gate->n_in);
         fwork = be->moe_f16_for(fwork_bytes);
     }
+    const bool f16_shape = fwork && itk::experts_f16_takes(g, &u, np, aq, dout);
+    const bool grouped = work && be->group_cached(np, (int)gate->n_expert, f16_shape ? 128 : 16);
     it_hip::OpRec rec;
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
@@ -1194,9 +1217,9 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
                [=](hipStream_t s) {
-                   if (fwork && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, s))
+                   if (f16_shape && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
-                   if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, s))
+                   if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
                        moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s);
                });
     be->expert_lookups += 2 * picks;
@@ -1219,6 +1242,7 @@ void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, ui
         be->check(hipStreamSynchronize(be->stream), "upload weights");
         be->route_n_used = route->n_used;
         be->route_n_tok = route->n_tok;
+        be->route_gen++;
         rw = be->route_w;
         n_used = route->n_used;
         n_tok = route->n_tok;

@@ -116,6 +116,11 @@ struct it_hip {
     float* route_w = nullptr;
     size_t route_cap = 0;  // picks
     uint64_t route_n_used = 0, route_n_tok = 0;
+    uint64_t route_gen = 0;   // bumped whenever the device route ids are rewritten
+    // the expert grouping that moe_work holds: valid for one route generation, pick count, expert count and tile size
+    uint64_t group_gen = ~0ull;
+    int group_picks = 0, group_experts = 0, group_tile = 0;
+    bool group_cached(int picks, int n_expert, int tile);
     bool route_reserve(size_t picks);
     // scratch of the grouped expert matmuls (expert-sorted pair lists and their tiles)
     int32_t* moe_work = nullptr;

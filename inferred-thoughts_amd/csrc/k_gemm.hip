@@ -391,7 +391,7 @@ size_t experts_group_work_ints(int n_picks, int n_expert) {
 
 bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
                   const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
-                  hipStream_t s) {
+                  bool grouped, hipStream_t s) {
     if (n_picks < 32 || !work || w.n_expert > 1024 || w.n_in % SLAB || (w.fmt != W_Q8_0 && w.fmt != W_NVFP4)) return false;
     if (work_ints < experts_group_work_ints(n_picks, w.n_expert)) return false;
     if ((reinterpret_cast<uintptr_t>(w.q) & 15) || w.q_stride % 16 || (reinterpret_cast<uintptr_t>(act_quants) & 15)) return false;
@@ -401,7 +401,7 @@ bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* id
     int32_t* n_tiles = work;
     int4* tiles = (int4*)(work + 16);
     int32_t* order = work + 16 + (size_t)(max_tiles + 1) * 4;
-    hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, 16, n_tiles, tiles, order);
+    if (!grouped) hipLaunchKernelGGL(moe_group_k, dim3(1), dim3(1024), 0, s, ids, n_picks, w.n_expert, 16, n_tiles, tiles, order);
     ExpertsGemmP p{};
     p.q = (const uint8_t*)w.q;
     p.s = (const uint8_t*)w.scales;

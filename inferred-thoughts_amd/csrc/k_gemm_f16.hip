@@ -380,34 +380,38 @@ size_t experts_f16_work_bytes(int x_rows, int n_in) {
     return (size_t)x_rows * n_in * 4 + (((size_t)x_rows * 4 + 255) & ~(size_t)255);
 }
 
-bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
-                      int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
-                      size_t work_ints, void* fwork, size_t fwork_bytes, hipStream_t s) {
-    if (n_picks < 32 || !work || !fwork || w.n_expert > 1024 || w.fmt != W_NVFP4 || w.n_in % FSUPER || w.n_out % 4) return false;
-    if (n_used < 1) n_used = 1;
-    const int x_rows = x_mode == 0 ? n_picks : (x_mode == 1 ? (n_picks + n_used - 1) / n_used : 1);
-    if (work_ints < experts_f16_work_ints(n_picks, w.n_expert) || fwork_bytes < experts_f16_work_bytes(x_rows, w.n_in)) return false;
+bool experts_f16_takes(const ExpertsView& w, const ExpertsView* up, int n_picks, const int8_t* act_quants, const float* out) {
+    if (n_picks < 32 || w.n_expert > 1024 || w.fmt != W_NVFP4 || w.n_in % FSUPER || w.n_out % 4) return false;
     if ((reinterpret_cast<uintptr_t>(w.q) & 15) || w.q_stride % 16 || w.s_stride % 16 || (reinterpret_cast<uintptr_t>(w.scales) & 15) ||
         (reinterpret_cast<uintptr_t>(act_quants) & 3) || (reinterpret_cast<uintptr_t>(out) & 15))
         return false;
     if (up && (up->fmt != w.fmt || up->n_in != w.n_in || up->n_out != w.n_out || (reinterpret_cast<uintptr_t>(up->q) & 15) ||
                (reinterpret_cast<uintptr_t>(up->scales) & 15) || up->q_stride != w.q_stride || up->s_stride != w.s_stride))
         return false;
-    static bool sized = false;
-    const size_t lds = (size_t)4 * FPAIRS * FBS * sizeof(uint16_t) + (size_t)2 * 256 * (FWS + 16);
+    static int sized = 0;   // 0 unknown, 1 yes, -1 the LDS size was refused
     if (!sized) {
-        if (hipFuncSetAttribute((const void*)experts_f16_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
-            hipFuncSetAttribute((const void*)experts_f16_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-            (void)hipGetLastError();
-            return false;
-        }
-        sized = true;
+        const size_t lds = (size_t)4 * FPAIRS * FBS * sizeof(uint16_t) + (size_t)2 * 256 * (FWS + 16);
+        sized = hipFuncSetAttribute((const void*)experts_f16_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess &&
+                        hipFuncSetAttribute((const void*)experts_f16_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess
+                    ? 1 : -1;
+        if (sized < 0) (void)hipGetLastError();
     }
+    return sized > 0;
+}
+
+bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
+                      int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
+                      size_t work_ints, void* fwork, size_t fwork_bytes, bool grouped, hipStream_t s) {
+    if (!work || !fwork || !experts_f16_takes(w, up, n_picks, act_quants, out)) return false;
+    if (n_used < 1) n_used = 1;
+    const int x_rows = x_mode == 0 ? n_picks : (x_mode == 1 ? (n_picks + n_used - 1) / n_used : 1);
+    if (work_ints < experts_f16_work_ints(n_picks, w.n_expert) || fwork_bytes < experts_f16_work_bytes(x_rows, w.n_in)) return false;
+    const size_t lds = (size_t)4 * FPAIRS * FBS * sizeof(uint16_t) + (size_t)2 * 256 * (FWS + 16);
     const int max_tiles = w.n_expert + n_picks / FPAIRS + 1;
     int32_t* n_tiles = work;
     int4* tiles = (int4*)(work + 16);
     int32_t* order = work + 16 + (size_t)(max_tiles + 1) * 4;
-    moe_group(ids, n_picks, w.n_expert, FPAIRS, n_tiles, tiles, order, s);
+    if (!grouped) moe_group(ids, n_picks, w.n_expert, FPAIRS, n_tiles, tiles, order, s);
     uint16_t* xh = (uint16_t*)fwork;
     uint16_t* xl = xh + (size_t)x_rows * w.n_in;
     float* rscale = (float*)(xl + (size_t)x_rows * w.n_in);

@@ -64,12 +64,14 @@ size_t experts_f16_work_ints(int n_picks, int n_expert);
 void moe_group(const int32_t* ids, int n_picks, int n_expert, int tile_pairs, int32_t* n_tiles, int4* tiles,
                int32_t* order, hipStream_t s);
 size_t experts_f16_work_bytes(int x_rows, int n_in);
+// whether experts_gemm_f16 takes these operands (shape, format, alignment), given scratch of the sizes above
+bool experts_f16_takes(const ExpertsView& w, const ExpertsView* up, int n_picks, const int8_t* act_quants, const float* out);
 bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
                       int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
-                      size_t work_ints, void* fwork, size_t fwork_bytes, hipStream_t s);
+                      size_t work_ints, void* fwork, size_t fwork_bytes, bool grouped, hipStream_t s);
 bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
                   const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
-                  hipStream_t s);
+                  bool grouped, hipStream_t s);
 // out[i] = silu(gate_e . x * sg_e) * (up_e . x * su_e)
 void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids, int n_picks, int n_used,
              int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);

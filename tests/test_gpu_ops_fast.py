@@ -121,7 +121,11 @@ def test_delta_rule_fast_state_carries_over_calls(hip, orc):
 # experts with no pair at all, ragged row counts.
 @pytest.mark.parametrize("n_tok,n_expert,n_used,nd,ff", [(48, 64, 10, 2048, 512), (200, 16, 4, 512, 256),
                                                          (600, 64, 10, 2048, 512), (700, 16, 4, 512, 256),
-                                                         (33, 512, 10, 2048, 512), (90, 8, 2, 256, 192)])
+                                                         (33, 512, 10, 2048, 512), (90, 8, 2, 256, 192),
+                                                         # the baseline's single-op expert FFN: 512 experts top-10,
+                                                         # hidden 2048, inter 512, token sweep (1 token: test_gpu_ops)
+                                                         (8, 512, 10, 2048, 512), (64, 512, 10, 2048, 512),
+                                                         (512, 512, 10, 2048, 512)])
 def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
     import inferred_hip as ih
     from oracle import binding as ob
