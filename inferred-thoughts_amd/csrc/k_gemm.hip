@@ -148,8 +148,9 @@ bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, 
 #define IT_GEMM(NT)                                                                                                  \
     hipLaunchKernelGGL((q8_gemm_k<NT>), dim3(gx, (tiles + NT - 1) / NT), dim3(GT), 0, s, wq, ws, act_quants, act_scales, \
                        out, w.n_in, w.n_out, n_tok, out_scale)
-    if (tiles >= 8) IT_GEMM(8);
-    else if (tiles >= 4) IT_GEMM(4);
+    // 64 tokens per block at most: four blocks fit a CU (38 KB of LDS, 98 VGPRs) and hide each other's LDS and
+    // barrier waits; 128 tokens per block (two blocks per CU) measured 20 % slower despite reading the weights half as often
+    if (tiles >= 4) IT_GEMM(4);
     else if (tiles >= 2) IT_GEMM(2);
     else IT_GEMM(1);
 #undef IT_GEMM
