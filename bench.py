@@ -37,7 +37,7 @@ PMC_TRAFFIC_BYTES = {"fused_gemv (norm + quantize + dense GEMVs)": 12_190_000, "
 
 def model_path(args):
     base = Path("/dev/shm") if Path("/dev/shm").is_dir() and os.access("/dev/shm", os.W_OK) else Path("/tmp")
-    return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}.gguf"
+    return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}{'_f32router' if args.router_f32 else ''}.gguf"
 
 
 def main():
@@ -47,6 +47,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=48, help="48 is the baseline config; fewer only for quick checks")
     ap.add_argument("--prompt", type=int, default=5700)
+    ap.add_argument("--router-f32", action="store_true",
+                    help="router, shared-expert gate and ssm alpha / beta matrices in F32 (as real files keep them) "
+                         "instead of the baseline's Q8_0: a variant, not the baseline workload")
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--max-batch", type=int, default=8192,
                     help="tokens per prefill pass; the default takes the 5,700-token prompt through each layer in one "
@@ -70,6 +73,8 @@ def main():
     t0 = time.time()
     path = model_path(args)
     cfg = ih.big_config(seed=args.seed, n_layer=args.layers, n_threads=min(16, os.cpu_count() or 8))
+    if args.router_f32:
+        cfg.router_type = ih.ROUTER_F32
     if not path.exists():
         ih.synth_write_gguf(path, cfg)
     t_synth = time.time() - t0
@@ -221,8 +226,9 @@ def main():
         "vs_baseline": None, "dtype": "int8 dot / f32 accumulate (NVFP4 + Q8_0 weights, Q8_0 activations)",
         "data": "synthetic",
         "config": {"workload": "config 5: full 35B-A3B-shaped model, greedy decode after a 5,700-token prefill at ctx 8192"
-                               if args.layers == 48 and args.prompt == 5700 else
-                               f"REDUCED check run: {args.layers} layers, prompt {args.prompt}",
+                               if args.layers == 48 and args.prompt == 5700 and not args.router_f32 else
+                               f"VARIANT / reduced check run: {args.layers} layers, prompt {args.prompt}, "
+                               f"router {'F32' if args.router_f32 else 'Q8_0'}",
                    "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "prefill_batch": args.max_batch, "decode_pos": int(pos0),
                    "experts": "512 top-10 + shared, NVFP4", "dense": "Q8_0 (router and ssm_alpha/beta Q8_0)",
                    "mode": "exact" if args.exact else "fast", "batch": 1},

@@ -265,6 +265,7 @@ const uint16_t* it_engine_v_slab(it_engine*, uint64_t slot, uint64_t* len);
 
 /* ---- synthetic GGUF writer (the reference ships none; its model tests need real
  * files, tests/common/mod.rs:10-44) ---- */
+#define IT_SYNTH_ROUTER_F32 0xffffffffu
 typedef struct {
     uint64_t n_layer, n_embd, n_vocab;
     uint64_t n_head, n_head_kv, head_dim, n_rot;
@@ -274,7 +275,8 @@ typedef struct {
     float rope_theta, rms_eps;
     uint32_t dense_type;  /* IT_Q8_0 */
     uint32_t expert_type; /* IT_Q8_0 or IT_NVFP4 */
-    uint32_t router_type; /* IT_Q8_0 or IT_F32 */
+    uint32_t router_type; /* router, shared-gate and ssm alpha/beta matrices: 0 = as dense_type, IT_Q8_0, or
+                             IT_SYNTH_ROUTER_F32 for F32 (what real files keep them in; IT_F32 itself is 0) */
     uint32_t _pad;
     uint64_t seed;
     float weight_std; /* N(0, std) for Q8_0 matrices */

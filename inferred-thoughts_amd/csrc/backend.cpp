@@ -833,12 +833,13 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int nt = (int)n;
+    const int exact = be->exact;
     it_hip::OpRec rec;
     rec.id = OP_MATMUL; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = dx; rec.p[3] = as; rec.p[4] = aq; rec.p[5] = dout;
     rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = nt;
     be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
                sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout), rec,
-               [=](hipStream_t s) { matmul(v, dx, as, aq, nt, dout, 1.0f, s); });
+               [=](hipStream_t s) { matmul(v, dx, as, aq, nt, dout, 1.0f, exact, s); });
 }
 
 void it_hip_matmul(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, float* out,

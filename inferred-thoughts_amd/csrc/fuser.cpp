@@ -42,8 +42,12 @@ struct Plan {
 
 bool quantized_fmt(int64_t f) { return f == W_Q8_0 || f == W_NVFP4; }
 
-// bytes of `rows` repacked rows of n_in weights (Q8_0: 34 per 32, NVFP4: 9 per 16)
+bool float_fmt(int64_t f) { return f == W_F32 || f == W_F16 || f == W_BF16; }
+
+// bytes of `rows` repacked rows of n_in weights (Q8_0: 34 per 32, NVFP4: 9 per 16; unquantized rows as stored)
 uint64_t rows_bytes(int fmt, uint64_t rows, uint64_t n_in) {
+    if (fmt == W_F32) return rows * n_in * 4;
+    if (fmt == W_F16 || fmt == W_BF16) return rows * n_in * 2;
     return fmt == W_NVFP4 ? rows * n_in * 9 / 16 : rows * n_in * 34 / 32;
 }
 uint64_t gemv_bytes(const FusedGemvP& p) {
@@ -56,6 +60,12 @@ uint64_t gemv_bytes(const FusedGemvP& p) {
 bool mm_reads(const Op& m, const void* x, const Op& q) {
     return m.id == OP_MATMUL && m.p[2] == x && m.p[3] == q.p[1] && m.p[4] == q.p[2] && m.i[3] == 1 &&
            quantized_fmt(m.i[0]) && m.i[1] == q.i[0];
+}
+
+// MATMUL `m` with unquantized weights (the router and ssm alpha / beta of real files are F32) reads the f32
+// activation `x` itself, one token.  Only the fast kernels take such a matrix into a fused launch.
+bool mm_reads_f32(const Op& m, const void* x, int64_t n_in, int exact) {
+    return !exact && m.id == OP_MATMUL && m.p[2] == x && m.i[3] == 1 && float_fmt(m.i[0]) && m.i[1] == n_in;
 }
 
 FusedMat mat_of(const Op& m, int epi, float* out_override = nullptr) {
@@ -80,9 +90,9 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     const Op &dl = o[i + 12], &rh = o[i + 13], &sm = o[i + 14], &q2 = o[i + 15], &mo = o[i + 16], &add = o[i + 17];
     const void* normed = rms.p[2];
     if (rms.i[0] != 1 || q1.p[0] != normed || q1.i[0] != rms.i[1]) return false;
-    if (!mm_reads(mqkv, normed, q1) || !mm_reads(mz, normed, q1) || !mm_reads(ma, normed, q1) ||
-        !mm_reads(mb, normed, q1))
-        return false;
+    if (!mm_reads(mqkv, normed, q1) || !mm_reads(mz, normed, q1)) return false;
+    if (!mm_reads(ma, normed, q1) && !mm_reads_f32(ma, normed, rms.i[1], exact)) return false;
+    if (!mm_reads(mb, normed, q1) && !mm_reads_f32(mb, normed, rms.i[1], exact)) return false;
     int64_t dk = dl.i[1], dv = dl.i[2], nk = dl.i[3], nv = dl.i[4];
     int64_t kdim = nk * dk, vdim = nv * dv, cdim = 2 * kdim + vdim;
     if (dl.i[0] != 1 || dk != dv || (dk != 64 && dk != 128)) return false;
@@ -117,6 +127,7 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     a.m[3] = mat_of(mb, 0);
     a.conv_state = (float*)conv.p[0];
     a.conv_w = (const float*)conv.p[2];
+    if ((float_fmt(ma.i[0]) || float_fmt(mb.i[0])) && !fused_gemv_fast_takes(a)) return false;
 
     GdnCoreP c{};
     c.conv = (const float*)cv;
@@ -349,18 +360,28 @@ bool match_attn(Plan& pl, size_t i, int exact) {
 
 // routed FFN: 17 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
 bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
-    if (!pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT, OP_EXPERTS,
-                    OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW}))
-        return false;
+    // With a quantized router the activation is quantized before the router matmul; with an unquantized one
+    // (F32 in real files) the first reader of the quantized form is the expert gate/up product, after the route.
+    const bool q_first = pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT,
+                                    OP_EXPERTS, OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW});
+    const bool q_late = !q_first && !exact &&
+                        pl.ids(i, {OP_RMS, OP_GATHER, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_QUANT, OP_GLU, OP_QUANT,
+                                   OP_EXPERTS, OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW});
+    if (!q_first && !q_late) return false;
     auto& o = pl.ops;
-    const Op &rms = o[i], &ga = o[i + 1], &q1 = o[i + 2], &mr = o[i + 3], &ml = o[i + 4], &sm = o[i + 5], &rt = o[i + 6];
+    const Op &rms = o[i], &ga = o[i + 1];
+    const Op &q1 = q_first ? o[i + 2] : o[i + 6];
+    const Op &mr = q_first ? o[i + 3] : o[i + 2], &ml = q_first ? o[i + 4] : o[i + 3];
+    const Op &sm = q_first ? o[i + 5] : o[i + 4], &rt = q_first ? o[i + 6] : o[i + 5];
     const Op &glu = o[i + 7], &q2 = o[i + 8], &ex = o[i + 9], &sgm = o[i + 10], &sum_ = o[i + 11], &sil = o[i + 12];
     const Op &q3 = o[i + 13], &sdm = o[i + 14], &fin = o[i + 15], &add = o[i + 16];
     int64_t nd = rms.i[1];
     if (rms.i[0] != 1) return false;
     if (ga.p[0] != rms.p[2] || ga.i[0] != nd || ga.i[2] != 0 || ga.i[3] != nd) return false;
     const void* x = ga.p[1];
-    if (q1.p[0] != x || q1.i[0] != nd || !mm_reads(mr, x, q1) || !mm_reads(ml, x, q1) || ml.i[2] != 1) return false;
+    if (q1.p[0] != x || q1.i[0] != nd || ml.i[2] != 1) return false;
+    if (q_first ? !mm_reads(mr, x, q1) : !mm_reads_f32(mr, x, nd, exact)) return false;
+    if (!mm_reads(ml, x, q1) && !mm_reads_f32(ml, x, nd, exact)) return false;
     int64_t ne = mr.i[2];
     const void* router = mr.p[5];
     if (sm.p[0] != router || sm.i[0] != 1 || sm.i[1] != ne) return false;
@@ -404,6 +425,7 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     a.n_used = (int)nu;
     a.route_ids = (int32_t*)rt.p[1];
     a.route_w = (float*)rt.p[2];
+    if ((float_fmt(mr.i[0]) || float_fmt(ml.i[0])) && !fused_gemv_fast_takes(a)) return false;
 
     MoeGluP g{};
     g.x = (const float*)x;

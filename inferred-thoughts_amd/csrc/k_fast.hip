@@ -167,7 +167,8 @@ IT_DEV double quad_sumsq(float4 v) {
 // Ends with a block barrier; xq / xs are then complete.
 template <int THREADS>
 __device__ __forceinline__ void stage_activation(const float* x, int n_in, int mode, const float* norm_w, const float* gate, int head_dim,
-                                 float eps, float* copy1, float* copy2, int8_t* xq, float* xs, double* red) {
+                                 float eps, float* copy1, float* copy2, int8_t* xq, float* xs, double* red,
+                                 float* xf = nullptr) {
     const int tid = threadIdx.x;
     const int nq = n_in >> 2;
     float4 v[2];
@@ -223,6 +224,7 @@ __device__ __forceinline__ void stage_activation(const float* x, int n_in, int m
         if (live[k]) {
             if (copy1) ((float4*)copy1)[qi] = v[k];
             if (copy2) ((float4*)copy2)[qi] = v[k];
+            if (xf) ((float4*)xf)[qi] = v[k];   // the f32 activation in LDS, for unquantized matrices
         }
         quant_quad(v[k], live[k], qi, xq, xs);
     }
@@ -246,6 +248,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     __shared__ __align__(16) int8_t xq[FT * 8];
     __shared__ float xs[FT * 8 / 32];
     __shared__ double red[FW];
+    __shared__ __align__(16) float xf[FT * 8];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sub = lane % L, rsub = lane / L;
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
 
     const bool first = blockIdx.x == 0;
     stage_activation<FT>(p.x, n_in, p.mode, p.norm_w, p.gate, p.head_dim, p.eps, first ? p.x_copy : nullptr,
-                         first ? p.x_copy2 : nullptr, xq, xs, red);
+                         first ? p.x_copy2 : nullptr, xq, xs, red, p.n_fmats ? xf : nullptr);
     XChunks<FMT, CPL> x;
     load_x<FMT, CPL, L>(x, xq, xs, sub);
 
@@ -320,16 +323,63 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
             }
         }
     }
+
+    // unquantized matrices (the router and ssm alpha / beta of real files are F32): one wave per row, the row sum
+    // split over the lanes
+    for (int fr = blockIdx.x * FW + wave; fr < p.total_frows; fr += gstride) {
+        int k = p.n_mats, j = fr;
+        while (k + 1 < p.n_mats + p.n_fmats && j >= p.m[k].n_out) {
+            j -= p.m[k].n_out;
+            k++;
+        }
+        const FusedMat& m = p.m[k];
+        const int esz = m.fmt == W_F32 ? 4 : 2;
+        const uint8_t* row = m.q + (int64_t)j * n_in * esz;
+        float acc = 0.0f;
+        for (int i = lane * 4; i < n_in; i += 256) {
+            float4 wv;
+            if (m.fmt == W_F32) {
+                wv = *(const float4*)(row + (int64_t)i * 4);
+            } else {
+                const uint2 h = *(const uint2*)(row + (int64_t)i * 2);
+                wv = m.fmt == W_F16 ? make_float4(it_f16_to_f32(h.x & 0xffffu), it_f16_to_f32(h.x >> 16), it_f16_to_f32(h.y & 0xffffu), it_f16_to_f32(h.y >> 16))
+                                    : make_float4(it_bf16_to_f32(h.x & 0xffffu), it_bf16_to_f32(h.x >> 16), it_bf16_to_f32(h.y & 0xffffu), it_bf16_to_f32(h.y >> 16));
+            }
+            const float4 xv = *(const float4*)(xf + i);
+            acc = fmaf(wv.x, xv.x, fmaf(wv.y, xv.y, fmaf(wv.z, xv.z, fmaf(wv.w, xv.w, acc))));
+        }
+        acc = reduce_lanes<64>(acc);
+        if (lane == 63) m.out[j] = acc;
+    }
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline bool float_fmt(int f) { return f == W_F32 || f == W_F16 || f == W_BF16; }
 
 }  // namespace
 
-bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
+// checks p and fills the launch fields (matrix order, groups); false: not a case for the fast kernel
+static bool fused_gemv_fast_prepare(FusedGemvP& p, Geo* geo, int* fmt_out, int* blocks_out) {
     if (p.exact || p.route_counter || p.n_mats < 1) return false;
-    const int fmt = p.m[0].fmt;
-    for (int i = 1; i < p.n_mats; i++)
+    // quantized matrices first, unquantized ones behind them
+    FusedMat qm[4], fm[4];
+    int nq = 0, nf = 0;
+    for (int i = 0; i < p.n_mats; i++) {
+        if (float_fmt(p.m[i].fmt)) fm[nf++] = p.m[i];
+        else qm[nq++] = p.m[i];
+    }
+    for (int i = 0; i < nq; i++) p.m[i] = qm[i];
+    for (int i = 0; i < nf; i++) p.m[nq + i] = fm[i];
+    p.n_mats = nq;
+    p.n_fmats = nf;
+    p.total_frows = 0;
+    for (int i = 0; i < nf; i++) {
+        if (fm[i].epi != 0 || !aligned16(fm[i].q) || p.n_in % 4) return false;
+        p.total_frows += fm[i].n_out;
+    }
+    const int fmt = nq ? p.m[0].fmt : (int)W_Q8_0;
+    if (fmt != W_Q8_0 && fmt != W_NVFP4) return false;
+    for (int i = 1; i < nq; i++)
         if (p.m[i].fmt != fmt) return false;
     const Geo g = geo_of(fmt, p.n_in);
     if (!g.ok || p.n_in > FT * 8 || p.n_in % 32) return false;
@@ -340,21 +390,38 @@ bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
         if (p.head_dim % 4 || lh < 1 || lh > 64 || (lh & (lh - 1)) || p.n_in % p.head_dim) return false;
         if (!aligned16(p.norm_w) || !aligned16(p.gate)) return false;
     }
-    for (int i = 0; i < p.n_mats; i++) {
+    for (int i = 0; i < nq; i++) {
         if (!aligned16(p.m[i].q) || (reinterpret_cast<uintptr_t>(p.m[i].s) & 1)) return false;
         if (p.m[i].epi == 1 && !aligned16(p.conv_w)) return false;
     }
     const int P = 64 / g.l, RB = g.cpl >= 4 ? 1 : 4 / g.cpl, RG = RB * P;
     int groups = 0;
-    for (int i = 0; i < p.n_mats; i++) {
+    for (int i = 0; i < nq; i++) {
         p.m[i].group0 = groups;
         groups += (p.m[i].n_out + RG - 1) / RG;
     }
     p.total_groups = groups;
     p.rows_per_wave = RG;
-    int blocks = (groups + FW - 1) / FW;
+    int blocks = (max(groups, p.total_frows) + FW - 1) / FW;
     if (blocks > 1024) blocks = 1024;  // four resident blocks per CU; larger matrices loop
     if (blocks < 1) blocks = 1;
+    *geo = g;
+    *fmt_out = fmt;
+    *blocks_out = blocks;
+    return true;
+}
+
+bool fused_gemv_fast_takes(const FusedGemvP& p) {
+    FusedGemvP q = p;
+    Geo g;
+    int fmt, blocks;
+    return fused_gemv_fast_prepare(q, &g, &fmt, &blocks);
+}
+
+bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
+    Geo g;
+    int fmt, blocks;
+    if (!fused_gemv_fast_prepare(p, &g, &fmt, &blocks)) return false;
 #define IT_LAUNCH(F, C, LL) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL>), dim3(blocks), dim3(FT), 0, s, p)
     if (fmt == W_Q8_0) {
         if (g.l == 64 && g.cpl == 1) IT_LAUNCH(W_Q8_0, 1, 64);

@@ -200,8 +200,120 @@ __global__ void dense_float_k(const uint8_t* __restrict__ w, const float* __rest
     out[t * n_out + j] = sum;
 }
 
+// Unquantized weights, fast mode: the row sum is split over a wave (not the CPU path's serial order).
+// Up to 8 tokens per launch row: one wave per weight row, lanes stride the row in 4-element pieces that are read
+// once and used for every token.
+template <int FMT>
+IT_DEV float4 load_w4(const uint8_t* row, int i) {
+    if (FMT == W_F32) return *(const float4*)((const float*)row + i);
+    const uint2 h = *(const uint2*)((const uint16_t*)row + i);
+    if (FMT == W_F16)
+        return make_float4(it_f16_to_f32(h.x & 0xffffu), it_f16_to_f32(h.x >> 16), it_f16_to_f32(h.y & 0xffffu), it_f16_to_f32(h.y >> 16));
+    return make_float4(it_bf16_to_f32(h.x & 0xffffu), it_bf16_to_f32(h.x >> 16), it_bf16_to_f32(h.y & 0xffffu), it_bf16_to_f32(h.y >> 16));
+}
+
+template <int FMT, int NT>
+__global__ __launch_bounds__(256) void float_gemv_fast_k(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ out, int n_in, int n_out, int n_tok, int tok0,
+                                                         float out_scale) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = blockIdx.x * 4 + wave;
+    if (j >= n_out) return;
+    const uint8_t* row = w + (int64_t)j * n_in * (FMT == W_F32 ? 4 : 2);
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0.0f;
+    for (int i = lane * 4; i < n_in; i += 256) {
+        const float4 wv = load_w4<FMT>(row, i);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            if (tok0 + t < n_tok) {
+                const float4 xv = *(const float4*)(x + (int64_t)(tok0 + t) * n_in + i);
+                acc[t] = fmaf(wv.x, xv.x, fmaf(wv.y, xv.y, fmaf(wv.z, xv.z, fmaf(wv.w, xv.w, acc[t]))));
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        float v = acc[t];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (lane == 0 && tok0 + t < n_tok) out[(int64_t)(tok0 + t) * n_out + j] = out_scale != 1.0f ? v * out_scale : v;
+    }
+}
+
+// More tokens: a block owns 64 weight rows x 64 tokens, stages 16-wide k slabs of both operands in LDS and every
+// thread keeps a 4 x 4 tile of sums.
+template <int FMT>
+__global__ __launch_bounds__(256) void float_gemm_fast_k(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ out, int n_in, int n_out, int n_tok,
+                                                         float out_scale) {
+    constexpr int KS = 16;
+    __shared__ float Ws[KS][64 + 4], Xs[KS][64 + 4];
+    const int tid = threadIdx.x, tr = tid & 15, tc = tid >> 4;   // rows 4 tr .. + 3, tokens 4 tc .. + 3
+    const int row0 = blockIdx.x * 64, tok0 = blockIdx.y * 64;
+    const int lr = tid >> 2, lk = (tid & 3) * 4;                 // staging: row (or token) lr, k lk .. + 3
+    const int64_t wrow = min(row0 + lr, n_out - 1);
+    const int64_t xrow = min(tok0 + lr, n_tok - 1);
+    const uint8_t* wp = w + wrow * n_in * (FMT == W_F32 ? 4 : 2);
+    const float* xp = x + xrow * n_in;
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = 0.0f;
+    for (int k0 = 0; k0 < n_in; k0 += KS) {
+        const float4 wv = load_w4<FMT>(wp, k0 + lk);
+        const float4 xv = *(const float4*)(xp + k0 + lk);
+        __syncthreads();
+        Ws[lk][lr] = wv.x; Ws[lk + 1][lr] = wv.y; Ws[lk + 2][lr] = wv.z; Ws[lk + 3][lr] = wv.w;
+        Xs[lk][lr] = xv.x; Xs[lk + 1][lr] = xv.y; Xs[lk + 2][lr] = xv.z; Xs[lk + 3][lr] = xv.w;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < KS; k++) {
+            const float4 a = *(const float4*)&Ws[k][4 * tr];
+            const float4 b = *(const float4*)&Xs[k][4 * tc];
+            const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int ia = 0; ia < 4; ia++)
+#pragma unroll
+                for (int ib = 0; ib < 4; ib++) acc[ia][ib] = fmaf(av[ia], bv[ib], acc[ia][ib]);
+        }
+    }
+#pragma unroll
+    for (int ib = 0; ib < 4; ib++) {
+        const int t = tok0 + 4 * tc + ib;
+        if (t >= n_tok) continue;
+#pragma unroll
+        for (int ia = 0; ia < 4; ia++) {
+            const int j = row0 + 4 * tr + ia;
+            if (j < n_out) out[(int64_t)t * n_out + j] = out_scale != 1.0f ? acc[ia][ib] * out_scale : acc[ia][ib];
+        }
+    }
+}
+
+template <int FMT>
+static bool float_matmul_fast(const WView& w, const float* x, int n_tok, float* out, float out_scale, hipStream_t s) {
+    if (w.n_in % 16 || (reinterpret_cast<uintptr_t>(w.q) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return false;
+    const uint8_t* wp = (const uint8_t*)w.q;
+    if (n_tok > 16) {
+        hipLaunchKernelGGL(float_gemm_fast_k<FMT>, dim3((w.n_out + 63) / 64, (n_tok + 63) / 64), dim3(256), 0, s, wp, x, out,
+                           w.n_in, w.n_out, n_tok, out_scale);
+        return true;
+    }
+    for (int t0 = 0; t0 < n_tok; t0 += 8) {
+        if (n_tok - t0 == 1)
+            hipLaunchKernelGGL((float_gemv_fast_k<FMT, 1>), dim3((w.n_out + 3) / 4), dim3(256), 0, s, wp, x, out, w.n_in, w.n_out,
+                               n_tok, t0, out_scale);
+        else
+            hipLaunchKernelGGL((float_gemv_fast_k<FMT, 8>), dim3((w.n_out + 3) / 4), dim3(256), 0, s, wp, x, out, w.n_in, w.n_out,
+                               n_tok, t0, out_scale);
+    }
+    return true;
+}
+
 void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
-            float* out, float out_scale, hipStream_t s) {
+            float* out, float out_scale, int exact, hipStream_t s) {
     if (n_tok <= 0 || w.n_out <= 0) return;
     if (q8_gemm(w, act_scales, act_quants, n_tok, out, out_scale, s)) return;
     if (w.fmt == W_Q8_0 || w.fmt == W_NVFP4) {
@@ -219,6 +331,11 @@ void matmul(const WView& w, const float* x, const float* act_scales, const int8_
         if (w.fmt == W_Q8_0) launch_gemv<W_Q8_0, false>(p, n_tok, s);
         else launch_gemv<W_NVFP4, false>(p, n_tok, s);
         return;
+    }
+    if (!exact) {
+        if (w.fmt == W_F32 && float_matmul_fast<W_F32>(w, x, n_tok, out, out_scale, s)) return;
+        if (w.fmt == W_F16 && float_matmul_fast<W_F16>(w, x, n_tok, out, out_scale, s)) return;
+        if (w.fmt == W_BF16 && float_matmul_fast<W_BF16>(w, x, n_tok, out, out_scale, s)) return;
     }
     int64_t total = (int64_t)w.n_out * n_tok;
     dim3 grid((unsigned)((total + 127) / 128)), block(128);

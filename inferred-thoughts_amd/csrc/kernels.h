@@ -32,7 +32,7 @@ void quantize_q8_0(const float* x, float* scales, int8_t* quants, int64_t n, hip
 // ---- matmul family -------------------------------------------------------------
 // out[t][j] = dot(w.row(j), x[t]); act is the Q8_0 form of x for quantized formats.
 void matmul(const WView& w, const float* x, const float* act_scales, const int8_t* act_quants, int n_tok,
-            float* out, float out_scale, hipStream_t s);
+            float* out, float out_scale, int exact, hipStream_t s);
 
 // The same product for 16 or more tokens on the int8 matrix cores (Q8_0 weights only): bit-identical
 // to `matmul`.  Returns false without launching when the shape or format is not handled.

@@ -22,6 +22,9 @@ struct FusedGemvP {
     float eps;
     int n_in, mode, head_dim, exact, n_mats, rows_per_wave, total_groups;
     FusedMat m[4];
+    // fast kernels only: the launcher moves unquantized (F32 / F16 / BF16) matrices behind the quantized ones;
+    // m[n_mats .. n_mats + n_fmats) are those, total_frows rows in all (epi 0 only)
+    int n_fmats, total_frows;
     float* conv_state;    // epi 1
     const float* conv_w;
     // optional: matrix 0 is the router; the last block to finish picks the experts
@@ -31,6 +34,8 @@ struct FusedGemvP {
     float* route_w;
 };
 void fused_gemv(FusedGemvP p, hipStream_t s);
+// whether the fast kernel takes p (formats, shapes, alignment); unquantized matrices are taken by the fast kernel only
+bool fused_gemv_fast_takes(const FusedGemvP& p);
 
 struct GdnCoreP {
     const float* conv;  // [q | k | v] after conv + silu

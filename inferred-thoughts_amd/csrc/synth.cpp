@@ -97,7 +97,7 @@ extern "C" int it_synth_write_gguf(const char* path, const it_synth_config* c, c
     const uint64_t d_inner = dk * nv, key_dim = dk * nk, conv_dim = 2 * key_dim + d_inner;
     const uint64_t qd = c->head_dim * c->n_head, kvd = c->head_dim * c->n_head_kv;
     const uint32_t D = c->dense_type ? c->dense_type : IT_Q8_0;
-    const uint32_t R = c->router_type ? c->router_type : D;
+    const uint32_t R = c->router_type == IT_SYNTH_ROUTER_F32 ? (uint32_t)IT_F32 : (c->router_type ? c->router_type : D);
     std::vector<Spec> specs;
     auto add = [&](const std::string& n, std::vector<uint64_t> dims, uint32_t ty, int kind) {
         specs.push_back(Spec{n, dims, ty, kind});

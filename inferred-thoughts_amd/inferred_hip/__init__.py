@@ -72,6 +72,9 @@ class ProfileRow(C.Structure):
     _fields_ = [("name", C.c_char * 48), ("launches", c_u64), ("ms_total", C.c_double), ("bytes_total", c_u64)]
 
 
+ROUTER_F32 = 0xffffffff   # SynthConfig.router_type: F32 router / shared-gate / ssm alpha, beta matrices
+
+
 class SynthConfig(C.Structure):
     _fields_ = [(n, c_u64) for n in ("n_layer", "n_embd", "n_vocab", "n_head", "n_head_kv", "head_dim", "n_rot",
                                       "n_expert", "n_expert_used", "expert_ff", "shared_ff", "ssm_d_conv",

@@ -37,6 +37,16 @@ def mid_gguf(tmp_path_factory):
 
 
 @pytest.fixture(scope="session")
+def tiny_f32_router_gguf(tmp_path_factory):
+    """The tiny shape with the router, the shared-expert gate and ssm alpha / beta in F32, as real files keep them
+    (the matrices that decide which experts run), and NVFP4 experts."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "tiny_f32_router.gguf"
+    ih.synth_write_gguf(str(p), ih.tiny_config(seed=3, expert_type=ih.NVFP4, router_type=ih.ROUTER_F32))
+    return p
+
+
+@pytest.fixture(scope="session")
 def tiny_nvfp4_gguf(tmp_path_factory):
     """The tiny shape with NVFP4 experts and per-expert scales (exercises config 5's formats)."""
     import inferred_hip as ih

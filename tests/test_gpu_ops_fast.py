@@ -160,6 +160,33 @@ def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
     assert np.all(np.abs(oa - obuf) <= 1e-3 * np.maximum(scale, np.abs(obuf))), (np.abs(oa - obuf) / scale).max()
 
 
+# unquantized weights (the router and ssm alpha / beta of real files are F32): wave-split row sums for up to 16
+# tokens, LDS-tiled products for more
+@pytest.mark.parametrize("ty", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("n_in,n_out,n", [(2048, 512, 1), (2048, 32, 1), (2048, 1, 5), (512, 16, 16), (2048, 512, 100),
+                                          (512, 70, 17), (2048, 33, 300)])
+def test_matmul_float_types_fast(hip, orc, ty, n_in, n_out, n):
+    import inferred_hip as ih
+    from oracle import binding as ob
+    fresh(hip)
+    hip.begin_pass(n)
+    r = rng(41)
+    w = r.standard_normal((n_out, n_in)).astype(np.float32)
+    if ty == "f32":
+        wb, code = w.view(np.uint8).reshape(-1).copy(), ih.F32
+    elif ty == "f16":
+        wb, code = w.astype(np.float16).view(np.uint8).reshape(-1).copy(), ih.F16
+    else:
+        wb, code = (w.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(-1).copy(), ih.BF16
+    x = r.standard_normal(n * n_in).astype(np.float32)
+    a = np.zeros(n * n_out, np.float32); b = np.zeros_like(a)
+    hip.matmul(ih.weights(wb, code, n_in, n_out), x, a); hip.host_needs(a)
+    orc.matmul(ob.weights(wb, code, n_in, n_out), x, b)
+    hip.raise_if_error()
+    assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(np.abs(b), np.sqrt(n_in))), np.abs(a - b).max()
+    assert np.abs(a - b).max() <= 2e-4 * np.sqrt(n_in)     # f32 rounding of a different sum order, no more
+
+
 @pytest.mark.parametrize("n,nd", [(1, 2048), (33, 2048), (3, 512)])
 def test_rms_norm_fast(hip, orc, n, nd):
     fresh(hip)
