@@ -60,9 +60,63 @@ __global__ __launch_bounds__(256) void route_topk_k(const float* __restrict__ pr
     }
 }
 
+// The same rule with one wave per token (up to 1024 experts, 16 picks): a probability is non-negative, so its
+// bit pattern orders like its value; a pick is compared as the 64-bit key (probability bits, ~id): the largest key
+// is the largest probability and, among equals, the smallest id.  A lane holds the keys of experts lane, lane + 64,
+// ...; each round takes the wave's largest key and retires it.  Same picks and weights as route_topk_k, bit for bit.
+template <int K>
+__global__ __launch_bounds__(256) void route_topk_wave_k(const float* __restrict__ probs, int n_tok, int n_expert, int n_used,
+                                                         int32_t* __restrict__ ids, float* __restrict__ weights) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tok) return;
+    const float* row = probs + (int64_t)t * n_expert;
+    unsigned long long key[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int e = lane + 64 * k;
+        key[k] = e < n_expert ? ((unsigned long long)__float_as_uint(row[e]) << 32) | (0xffffffffu - (unsigned)e) : 0ull;
+    }
+    float sum = 0.0f;
+    float mine = 0.0f;     // lane r keeps pick r's probability
+    int mine_id = 0;
+    for (int r = 0; r < n_used; r++) {
+        unsigned long long m = key[0];
+#pragma unroll
+        for (int k = 1; k < K; k++) m = key[k] > m ? key[k] : m;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const unsigned long long other = __shfl_xor(m, o, 64);
+            m = other > m ? other : m;
+        }
+#pragma unroll
+        for (int k = 0; k < K; k++)
+            if (key[k] == m) key[k] = 0ull;
+        const float pv = __uint_as_float((unsigned)(m >> 32));
+        sum += pv;                         // pick order, as the CPU path adds them
+        if (lane == r) {
+            mine = pv;
+            mine_id = (int)(0xffffffffu - (unsigned)(m & 0xffffffffu));
+        }
+    }
+    const float denom = fmaxf(sum, 6.103515625e-5f);
+    if (lane < n_used) {
+        ids[(int64_t)t * n_used + lane] = mine_id;
+        weights[(int64_t)t * n_used + lane] = mine / denom;
+    }
+}
+
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,
                 hipStream_t s) {
     if (n_tok <= 0) return;
+    if (n_used <= 16 && n_used <= n_expert && n_expert <= 1024) {
+        const dim3 grid((n_tok + 3) / 4), block(256);
+        if (n_expert <= 64) hipLaunchKernelGGL(route_topk_wave_k<1>, grid, block, 0, s, probs, n_tok, n_expert, n_used, ids, weights);
+        else if (n_expert <= 256) hipLaunchKernelGGL(route_topk_wave_k<4>, grid, block, 0, s, probs, n_tok, n_expert, n_used, ids, weights);
+        else if (n_expert <= 512) hipLaunchKernelGGL(route_topk_wave_k<8>, grid, block, 0, s, probs, n_tok, n_expert, n_used, ids, weights);
+        else hipLaunchKernelGGL(route_topk_wave_k<16>, grid, block, 0, s, probs, n_tok, n_expert, n_used, ids, weights);
+        return;
+    }
     hipLaunchKernelGGL(route_topk_k, dim3(n_tok), dim3(256), n_expert * sizeof(float), s, probs, n_expert, n_used,
                        ids, weights);
 }

@@ -256,7 +256,8 @@ def planted_probs(r, n_tok, n_expert):
     return p
 
 
-@pytest.mark.parametrize("n_tok,n_expert,n_used", [(1, 16, 4), (9, 16, 4), (1, 512, 10), (5, 512, 10), (2, 256, 8)])
+@pytest.mark.parametrize("n_tok,n_expert,n_used", [(1, 16, 4), (9, 16, 4), (1, 512, 10), (5, 512, 10), (2, 256, 8),
+                                                     (301, 512, 10), (70, 1000, 16), (33, 100, 5)])
 def test_route(hip, orc, n_tok, n_expert, n_used):
     import ctypes as C
     fresh(hip)
