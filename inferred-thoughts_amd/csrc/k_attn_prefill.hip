@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void attend_prefill_k(AttnArgs a, float* __res
         }
 #pragma unroll
         for (int u = 0; u < VU; u++) {
-            const int unit = tid + u * 256, ka = unit / (HD / 8), b = unit % (HD / 8);
+            const int unit = tid + u * 256, ka = unit % (KT / 4), b = unit / (KT / 4);   // 16 key groups across lanes: the transposed LDS writes of a wave hit every bank once
             if (unit < UNITS) {
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void attend_prefill_k(AttnArgs a, float* __res
         }
 #pragma unroll
         for (int u = 0; u < VU; u++) {
-            const int unit = tid + u * 256, ka = unit / (HD / 8), b = unit % (HD / 8);
+            const int unit = tid + u * 256, ka = unit % (KT / 4), b = unit / (KT / 4);   // 16 key groups across lanes: the transposed LDS writes of a wave hit every bank once
             if (unit >= UNITS) continue;
             const uint32_t x[4][4] = {{rv[u][0].x, rv[u][0].y, rv[u][0].z, rv[u][0].w},
                                       {rv[u][1].x, rv[u][1].y, rv[u][1].z, rv[u][1].w},
