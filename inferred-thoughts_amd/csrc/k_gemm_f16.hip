@@ -117,7 +117,9 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     const int64_t e = td.x;
     const int cnt = td.z;
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave8 & 3;      // which 32 (GLU) or 64 rows of the block
+    const int th = wave8 >> 2;       // which half of the tile's token groups: T groups each
     const int r = lane & 31, kg = lane >> 5;
     const int n_in = p.n_in, nslab = n_in / FK;
     // the two row sets of this wave
@@ -128,21 +130,22 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     const uint8_t* ws[2] = {p.s + e * p.s_stride, GLU ? p.s2 + e * p.s_stride : p.s + e * p.s_stride};
     // this wave's row segments in the block's weight buffer: GLU [set][wave][row], else [wave][set][row]
     const int myseg[2] = {GLU ? 32 * wave + r : 64 * wave + r, GLU ? 128 + 32 * wave + r : 64 * wave + 32 + r};
-    // the segments this thread loads (eight rows, one 16-byte piece of each row's 128 nibble bytes) and
-    // the segment whose 16 scale bytes it loads
+    // the segments this thread loads (four rows, one 16-byte piece of each row's 128 nibble bytes) and, for the
+    // first 256 threads, the segment whose 16 scale bytes it loads
     const int piece = tid & 7;
-    const uint8_t* wload[8];
+    const uint8_t* wload[4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int seg = (tid >> 3) + 32 * i;
+    for (int i = 0; i < 4; i++) {
+        const int seg = (tid >> 3) + 64 * i;
         const int z = GLU ? seg >> 7 : 0;
         const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? seg & 127 : seg), p.n_out - 1);
         wload[i] = wq[z] + row * (n_in >> 1) + piece * 16;
     }
     const uint8_t* sload;
     {
-        const int z = GLU ? tid >> 7 : 0;
-        const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? tid & 127 : tid), p.n_out - 1);
+        const int st = tid & 255;
+        const int z = GLU ? st >> 7 : 0;
+        const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? st & 127 : st), p.n_out - 1);
         sload = ws[z] + row * (n_in >> 4);
     }
 
@@ -153,30 +156,30 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     // ahead through registers into the other LDS token buffer.  Inside a slab the token fragments of the
     // next MFMA group are read from LDS while the current group is on the matrix unit.
     const int n_super = n_in / FSUPER;
-    uint4 rw[8], rsw;
-    uint4 rbh[T], rbl[T];   // 32 * T tokens x 8 segments of 16 bytes = 256 * T segments per array
+    uint4 rw[4], rsw;
+    uint4 rbh[T], rbl[T];   // 64 * T tokens x 8 segments of 16 bytes = 512 * T segments per array
     rsw = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 8; i++) rw[i] = rsw;
+    for (int i = 0; i < 4; i++) rw[i] = rsw;
     // the token rows this thread stages: fixed for the whole k loop
     const uint16_t* xhp[T];
     const uint16_t* xlp[T];
 #pragma unroll
     for (int u = 0; u < T; u++) {
-        const int idx = tid + u * 256, tok = idx >> 3, seg = idx & 7;
+        const int idx = tid + u * 512, tok = idx >> 3, seg = idx & 7;
         const int64_t at = (int64_t)xrow_s[tok] * n_in + seg * 8;
         xhp[u] = p.xh + at;
         xlp[u] = p.xl + at;
     }
     auto fetch_w = [&](int S) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) rw[i] = *(const uint4*)(wload[i] + S * (FSUPER / 2));
+        for (int i = 0; i < 4; i++) rw[i] = *(const uint4*)(wload[i] + S * (FSUPER / 2));
         rsw = *(const uint4*)(sload + S * (FSUPER / 16));
     };
     // The same loads one at a time, to be issued between MFMA groups: a burst of 16-byte loads from all four
     // waves backs up the load unit (about 200 cycles an instruction) and the matrix unit idles behind it.
-    // q < 2 T: piece q of the next slab's tokens; then the nine loads of the next super-slab.
-    constexpr int N_LOADS = 2 * T + 9, LPG = (N_LOADS + 4 * T - 1) / (4 * T);
+    // q < 2 T: piece q of the next slab's tokens; then the five loads of the next super-slab.
+    constexpr int N_LOADS = 2 * T + 5, LPG = (N_LOADS + 4 * T - 1) / (4 * T);
     auto fetch_one = [&](int q, int s_next, int S_next, bool x_on, bool w_on) __attribute__((always_inline)) {
         if (q < 2 * T) {
             if (x_on) {
@@ -185,14 +188,14 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
             }
         } else if (q < N_LOADS && w_on) {
             const int i = q - 2 * T;
-            if (i < 8) rw[i] = *(const uint4*)(wload[i] + S_next * (FSUPER / 2));
+            if (i < 4) rw[i] = *(const uint4*)(wload[i] + S_next * (FSUPER / 2));
             else rsw = *(const uint4*)(sload + S_next * (FSUPER / 16));
         }
     };
     auto stash_w = [&](int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) *(uint4*)(Wn + (b * 256 + (tid >> 3) + 32 * i) * FWS + piece * 16) = rw[i];
-        *(uint4*)(Wsc + (b * 256 + tid) * 16) = rsw;
+        for (int i = 0; i < 4; i++) *(uint4*)(Wn + (b * 256 + (tid >> 3) + 64 * i) * FWS + piece * 16) = rw[i];
+        if (tid < 256) *(uint4*)(Wsc + (b * 256 + tid) * 16) = rsw;
     };
     auto fetch_x = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
@@ -204,7 +207,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     auto stash_x = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < T; u++) {
-            const int idx = tid + u * 256, tok = idx >> 3, seg = idx & 7;
+            const int idx = tid + u * 512, tok = idx >> 3, seg = idx & 7;
             uint16_t* dh = Bh + (buf * FPAIRS + tok) * FBS + seg * 8;
             uint16_t* dl = Bl + (buf * FPAIRS + tok) * FBS + seg * 8;
             *(uint2*)dh = make_uint2(rbh[u].x, rbh[u].y);
@@ -238,8 +241,8 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
         // bytes 16 * kg + 4 * n .. + 3 of the row's slab: sub-block 2 * kg + n / 2, elements 4 * (n % 2) + {0..3}
         // from the low nibbles and 8 more from the high ones
         const int k0 = 32 * kg + 16 * (n >> 1) + 4 * (n & 1);
-        const uint16_t* bh = Bh + (buf * FPAIRS + 32 * tt + r) * FBS + k0;
-        const uint16_t* bl = Bl + (buf * FPAIRS + 32 * tt + r) * FBS + k0;
+        const uint16_t* bh = Bh + (buf * FPAIRS + 32 * (T * th + tt) + r) * FBS + k0;
+        const uint16_t* bl = Bl + (buf * FPAIRS + 32 * (T * th + tt) + r) * FBS + k0;
         const uint2 h0 = *(const uint2*)bh, h1 = *(const uint2*)(bh + 8);
         const uint2 l0 = *(const uint2*)bl, l1 = *(const uint2*)(bl + 8);
         return Tok{__builtin_bit_cast(h8, make_uint4(h0.x, h0.y, h1.x, h1.y)),
@@ -315,7 +318,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     const float e2b = GLU ? (p.scale2_up ? p.scale2_up[e] : 1.0f) : e2a;
 #pragma unroll
     for (int tt = 0; tt < T; tt++) {
-        const int slot = 32 * tt + r;
+        const int slot = 32 * (T * th + tt) + r;
         if (slot >= cnt) continue;
         const int64_t pair = pair_s[slot];
         const float rsc = p.rscale[xrow_s[slot]];
@@ -346,7 +349,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
 }
 
 template <bool GLU>
-__global__ __launch_bounds__(256) void experts_f16_k(ExpertsF16P p) {
+__global__ __launch_bounds__(512) void experts_f16_k(ExpertsF16P p) {
     extern __shared__ __align__(16) uint16_t flds[];
     uint16_t* Bh = flds;                          // [2][128][FBS]
     uint16_t* Bl = flds + 2 * FPAIRS * FBS;       // [2][128][FBS]
@@ -363,12 +366,9 @@ __global__ __launch_bounds__(256) void experts_f16_k(ExpertsF16P p) {
         xrow_s[threadIdx.x] = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
     }
     __syncthreads();
-    switch ((cnt + 31) >> 5) {
-        case 1: experts_f16_body<GLU, 1>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s); break;
-        case 2: experts_f16_body<GLU, 2>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s); break;
-        case 3: experts_f16_body<GLU, 3>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s); break;
-        default: experts_f16_body<GLU, 4>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s); break;
-    }
+    // waves 0..3 take the first T token groups of the tile, waves 4..7 the next T
+    if (cnt <= 64) experts_f16_body<GLU, 1>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
+    else experts_f16_body<GLU, 2>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
 }
 
 }  // namespace
@@ -436,8 +436,8 @@ bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t
     p.n_tiles = n_tiles;
     p.tiles = tiles;
     p.order = order;
-    if (up) hipLaunchKernelGGL(experts_f16_k<true>, dim3(max_tiles, (w.n_out + 127) / 128), dim3(256), lds, s, p);
-    else hipLaunchKernelGGL(experts_f16_k<false>, dim3(max_tiles, (w.n_out + 255) / 256), dim3(256), lds, s, p);
+    if (up) hipLaunchKernelGGL(experts_f16_k<true>, dim3(max_tiles, (w.n_out + 127) / 128), dim3(512), lds, s, p);
+    else hipLaunchKernelGGL(experts_f16_k<false>, dim3(max_tiles, (w.n_out + 255) / 256), dim3(512), lds, s, p);
     return true;
 }
 
