@@ -141,6 +141,13 @@ def main():
     dense_macs, glu_macs, down_macs = model.token_macs()
     n_attn_layers = args.layers - n_gdn_layers
     F16_PEAK = 2500.0
+    # this card's own ceilings: back-to-back MFMA instructions with no memory in the loop, in TOP/s (TFLOP/s)
+    ceilings = {kind: round(be.mfma_ceiling(kind) / 1e12, 1) for kind in ih.Hip.MFMA_KINDS}
+    # the instruction each family issues
+    family_inst = {"matmul (dense": "int8_16x16x32", "moe_glu": "f16_32x32x16", "matmul_experts": "f16_32x32x16",
+                   "delta_rule": "f32_16x16x4", "attend": "f16_32x32x16"}
+    if args.exact:
+        family_inst.update({"moe_glu": "int8_16x16x32", "matmul_experts": "int8_16x16x32"})
     prefill_kernels = {}
     for r in sorted(prows, key=lambda r: -r["ms"]):
         k = {"launches": r["launches"], "ms": round(r["ms"], 2)}
@@ -175,6 +182,10 @@ def main():
             pairs = args.prompt * (args.prompt + 1) / 2
             flops = 2 * pairs * model.n_head * model.head_dim * 3 * n_attn_layers
             k.update(unit="f16 MFMA", tflops=round(flops / sec / 1e12, 1), mfma_frac=round(flops / sec / 1e12 / F16_PEAK, 4))
+        rate = k.get("tflops", k.get("tops"))
+        inst = next((v for f, v in family_inst.items() if name.startswith(f)), None)
+        if rate is not None and inst is not None:
+            k.update(instruction=inst, measured_ceiling=ceilings[inst], frac_of_measured=round(rate / ceilings[inst], 4))
         prefill_kernels[name] = k
 
     # algorithmic bytes of one decode token (weights once + GDN state r+w + KV read)
@@ -234,6 +245,7 @@ def main():
                    "mode": "exact" if args.exact else "fast", "batch": 1},
         "prefill_tok_s": round(args.prompt / t_prefill, 1),
         "prefill_kernels": prefill_kernels,
+        "mfma_ceilings_measured": ceilings,
         "bytes_per_token": int(tok_bytes),
         "token_roofline": {"bound": "hbm", "achieved": round(whole, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": round(whole / HBM_PEAK_GBS, 4)},

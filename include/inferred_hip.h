@@ -224,6 +224,12 @@ void it_hip_drop_mirrors(it_hip*);
 uint64_t it_hip_launch_count(it_hip*);
 /* decode graphs: captures, replays, fallbacks to eager, kernel launches in the captured graph */
 void it_hip_graph_stats(it_hip*, uint64_t out[4]);
+/* This card's matrix-core ceiling, measured: back-to-back MFMA instructions on eight independent
+ * accumulators per wave, two waves on every SIMD, no memory in the loop (the method of the reference's
+ * own ceilings, tests/cuda_ops.rs:56-72).  kind: 0 int8 16x16x64, 1 int8 16x16x32, 2 f16 32x32x16,
+ * 3 f16 16x16x32, 4 f32 16x16x4; iters = instructions per accumulator.  Writes operations per second
+ * (2 per multiply-accumulate).  0 = ok, 1 = bad argument, 2 = device error */
+int it_hip_mfma_ceiling(it_hip*, int kind, int iters, double* ops_per_s);
 
 /* ---- model + engine: the host side of the loop over this backend ----------
  * Qwen35::load / forward (src/model/qwen35.rs:755-858, 956-1127) and

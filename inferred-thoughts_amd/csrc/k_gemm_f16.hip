@@ -10,9 +10,11 @@
 // What differs from the CPU path is the f32 summation order and the 2^-22 of the split.
 //
 // A block owns one tile of up to 128 (token, pick) pairs of one expert and 128 rows of the
-// gate AND up matrices (GLU) or 256 rows of one matrix.  A wave owns two sets of 32 rows (gate
-// and up rows of the same index, or two row groups) and every token tile, so a token fragment
-// read from LDS feeds four MFMAs (two sets, hi and lo).  Weight nibbles go from HBM straight to
+// gate AND up matrices (GLU) or 256 rows of one matrix, with eight waves.  A wave owns two sets of
+// 32 rows (gate and up rows of the same index, or two row groups) and half of the token tiles
+// (waves 0-3 the first one or two groups of 32 pairs, waves 4-7 the next), so a token fragment
+// read from LDS feeds four MFMAs (two sets, hi and lo) and the f32 sums of a wave stay within the
+// registers that two waves per SIMD leave.  Weight nibbles go through LDS as full 128-byte lines to
 // the owning lane's registers (a lane owns 16 contiguous bytes of a row per 64-wide k slab: the
 // k order inside an MFMA is free once the scales are folded in) and are expanded there: a byte
 // permute yields the f16 high bytes of four magnitudes, the sign bit is or-ed in, two more

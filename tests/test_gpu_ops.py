@@ -380,3 +380,18 @@ def test_shape_errors_are_sticky_not_fatal(hip):
     hip.rms_norm(x, w, 1e-6, out)
     assert "rms_norm" in (hip.take_error() or "")
     assert hip.take_error() is None
+
+
+def test_mfma_ceilings_are_measured(hip):
+    """The back-to-back MFMA loop gives a rate for every instruction kind; the rates sit below the published
+    dense peaks (5 POP/s int8, 2.5 PFLOP/s f16, 157.3 TFLOP/s fp32 with some slack for clocks above nominal)
+    and above a tenth of them, and the 64-deep int8 instruction is not slower than the 32-deep one."""
+    import inferred_hip as ih
+    peak = {"int8_16x16x64": 5000e12, "int8_16x16x32": 5000e12, "f16_32x32x16": 2500e12, "f16_16x16x32": 2500e12,
+            "f32_16x16x4": 157.3e12}
+    got = {k: hip.mfma_ceiling(k, 4000) for k in ih.Hip.MFMA_KINDS}
+    for k, v in got.items():
+        assert 0.1 * peak[k] < v < 1.25 * peak[k], (k, v)
+    assert got["int8_16x16x64"] >= 0.95 * got["int8_16x16x32"]
+    with pytest.raises(KeyError):
+        hip.mfma_ceiling("f64_16x16x4")
