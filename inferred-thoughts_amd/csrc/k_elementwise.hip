@@ -60,14 +60,68 @@ __global__ __launch_bounds__(64) void head_norm_k(float* __restrict__ x, const f
     }
 }
 
+// The same for many heads when the order of the sum is free: a wave per head, PER neighbouring elements per
+// lane held in registers, the f64 partial sums added across the wave by lane moves (no LDS, no barrier).
+template <int PER>
+__global__ __launch_bounds__(256) void head_norm_wave_k(float* __restrict__ x, const float* __restrict__ w,
+                                                        int64_t n_heads, float eps, int mode) {
+    constexpr int HD = 64 * PER;
+    const int lane = threadIdx.x & 63;
+    const int64_t h = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (h >= n_heads) return;
+    float* at = x + h * HD + lane * PER;
+    float v[PER];
+    if constexpr (PER == 4) {
+        const float4 t = *(const float4*)at;
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else if constexpr (PER == 2) {
+        const float2 t = *(const float2*)at;
+        v[0] = t.x; v[1] = t.y;
+    } else {
+        v[0] = at[0];
+    }
+    double part = 0.0;
+#pragma unroll
+    for (int e = 0; e < PER; e++) part += (double)(v[e] * v[e]);
+    const double sum = __shfl(wave_sum_f64_tail(part), 63, 64);
+    float o[PER];
+    if (mode == 0) {
+        const float mean = (float)(sum / (double)HD);
+        const float scale = 1.0f / sqrtf(mean + eps);
+#pragma unroll
+        for (int e = 0; e < PER; e++) o[e] = v[e] * scale * w[lane * PER + e];
+    } else {
+        const float nrm = sqrtf((float)sum);
+        const float scale = 1.0f / fmaxf(nrm, eps);
+#pragma unroll
+        for (int e = 0; e < PER; e++) o[e] = v[e] * scale;
+    }
+    if constexpr (PER == 4) *(float4*)at = make_float4(o[0], o[1], o[2], o[3]);
+    else if constexpr (PER == 2) *(float2*)at = make_float2(o[0], o[1]);
+    else at[0] = o[0];
+}
+
+static bool head_norm_wave(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int mode, hipStream_t s) {
+    if (n_heads < 256 || ((uintptr_t)x & 15) != 0) return false;
+    const dim3 grid((unsigned)((n_heads + 3) / 4)), block(256);
+    switch (head_dim) {
+        case 64: hipLaunchKernelGGL(head_norm_wave_k<1>, grid, block, 0, s, x, w, n_heads, eps, mode); return true;
+        case 128: hipLaunchKernelGGL(head_norm_wave_k<2>, grid, block, 0, s, x, w, n_heads, eps, mode); return true;
+        case 256: hipLaunchKernelGGL(head_norm_wave_k<4>, grid, block, 0, s, x, w, n_heads, eps, mode); return true;
+        default: return false;
+    }
+}
+
 void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int exact,
                     hipStream_t s) {
     if (n_heads <= 0) return;
+    if (!exact && head_norm_wave(x, w, head_dim, eps, n_heads, 0, s)) return;
     hipLaunchKernelGGL(head_norm_k, dim3((unsigned)n_heads), dim3(64), head_dim * sizeof(float), s, x, w,
                        head_dim, eps, 0, exact);
 }
 void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s) {
     if (n_heads <= 0) return;
+    if (!exact && head_norm_wave(x, nullptr, head_dim, eps, n_heads, 1, s)) return;
     hipLaunchKernelGGL(head_norm_k, dim3((unsigned)n_heads), dim3(64), head_dim * sizeof(float), s, x,
                        (const float*)nullptr, head_dim, eps, 1, exact);
 }
@@ -223,14 +277,65 @@ __global__ void fill_zero_k(uint32_t* p, int64_t n_words) {
         p[i] = 0u;
 }
 
+// Four elements per lane for the long batches: the same arithmetic per element, 16-byte accesses.
+__global__ void silu_mul4_k(float4* __restrict__ g, const float4* __restrict__ u, int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 a = g[i];
+        const float4 b = u[i];
+        a.x = it_silu(a.x) * b.x; a.y = it_silu(a.y) * b.y; a.z = it_silu(a.z) * b.z; a.w = it_silu(a.w) * b.w;
+        g[i] = a;
+    }
+}
+__global__ void sigmoid_mul4_k(float4* __restrict__ x, const float4* __restrict__ g, int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 a = x[i];
+        const float4 b = g[i];
+        a.x *= it_sigmoid(b.x); a.y *= it_sigmoid(b.y); a.z *= it_sigmoid(b.z); a.w *= it_sigmoid(b.w);
+        x[i] = a;
+    }
+}
+__global__ void add_assign4_k(float4* __restrict__ a, const float4* __restrict__ b, int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 v = a[i];
+        const float4 w = b[i];
+        v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+        a[i] = v;
+    }
+}
+// chunk, stride and offset in units of four floats, every index below 2^31
+__global__ void gather_chunks4_k(const float4* __restrict__ src, uint32_t chunk4, uint32_t stride4, uint32_t offset4,
+                                 float4* __restrict__ out, uint32_t out_len4) {
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < out_len4; i += gridDim.x * blockDim.x) {
+        const uint32_t c = i / chunk4, j = i - c * chunk4;
+        out[i] = src[c * stride4 + offset4 + j];
+    }
+}
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+constexpr int64_t VEC_MIN = 1 << 14;  // below this one pass of scalar lanes is as quick
+
 #define EW_LAUNCH(kern, n, ...)                                                              \
     do {                                                                                     \
         if ((n) > 0) hipLaunchKernelGGL(kern, dim3(blocks_for((n), 256)), dim3(256), 0, s, __VA_ARGS__); \
     } while (0)
 
-void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s) { EW_LAUNCH(silu_mul_k, n, gate, up, n); }
-void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s) { EW_LAUNCH(sigmoid_mul_k, n, x, g, n); }
-void add_assign(float* a, const float* b, int64_t n, hipStream_t s) { EW_LAUNCH(add_assign_k, n, a, b, n); }
+void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s) {
+    if (n >= VEC_MIN && n % 4 == 0 && aligned16(gate) && aligned16(up))
+        EW_LAUNCH(silu_mul4_k, n / 4, (float4*)gate, (const float4*)up, n / 4);
+    else
+        EW_LAUNCH(silu_mul_k, n, gate, up, n);
+}
+void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s) {
+    if (n >= VEC_MIN && n % 4 == 0 && aligned16(x) && aligned16(g))
+        EW_LAUNCH(sigmoid_mul4_k, n / 4, (float4*)x, (const float4*)g, n / 4);
+    else
+        EW_LAUNCH(sigmoid_mul_k, n, x, g, n);
+}
+void add_assign(float* a, const float* b, int64_t n, hipStream_t s) {
+    if (n >= VEC_MIN && n % 4 == 0 && aligned16(a) && aligned16(b))
+        EW_LAUNCH(add_assign4_k, n / 4, (float4*)a, (const float4*)b, n / 4);
+    else
+        EW_LAUNCH(add_assign_k, n, a, b, n);
+}
 void scale(float* a, float v, int64_t n, hipStream_t s) { EW_LAUNCH(scale_k, n, a, v, n); }
 void add_scaled(float* a, const float* b, float v, int64_t n, hipStream_t s) {
     EW_LAUNCH(add_scaled_k, n, a, b, v, n);
@@ -244,6 +349,13 @@ void add_scaled_sigmoid(float* acc, const float* b, int64_t n, const float* logi
 }
 void gather_chunks(const float* src, int64_t chunk, int64_t stride, int64_t offset, float* out,
                    int64_t out_len, hipStream_t s) {
+    const int64_t n_chunks = chunk > 0 ? (out_len + chunk - 1) / chunk : 0;
+    if (out_len >= VEC_MIN && chunk % 4 == 0 && stride % 4 == 0 && offset % 4 == 0 && out_len % 4 == 0 && offset >= 0 &&
+        aligned16(src) && aligned16(out) && (n_chunks * stride + offset) / 4 < (1ll << 31) && out_len / 4 < (1ll << 31)) {
+        EW_LAUNCH(gather_chunks4_k, out_len / 4, (const float4*)src, (uint32_t)(chunk / 4), (uint32_t)(stride / 4),
+                  (uint32_t)(offset / 4), (float4*)out, (uint32_t)(out_len / 4));
+        return;
+    }
     EW_LAUNCH(gather_chunks_k, out_len, src, chunk, stride, offset, out, out_len);
 }
 void scatter_chunks(const float* src, int64_t src_len, int64_t chunk, int64_t stride, int64_t offset,
@@ -334,9 +446,73 @@ __global__ void ssm_conv_k(float* __restrict__ state, const float* __restrict__ 
     }
 }
 
+// The same for four neighbouring channels per lane: 16-byte accesses, the chunk's inputs all in flight at once.
+template <int KEEP>
+__global__ __launch_bounds__(128) void ssm_conv4_k(float* __restrict__ state, const float* __restrict__ x,
+                                                   const float* __restrict__ w, int nc, int n_tok,
+                                                   float* __restrict__ out) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (c >= nc) return;
+    const int t0 = blockIdx.y * CONV_TOK, t1 = min(n_tok, t0 + CONV_TOK);
+    float past[KEEP][4], wt[KEEP + 1][4];
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        if (blockIdx.y == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) past[k][e] = state[(int64_t)(c + e) * KEEP + k];
+        } else {
+            const float4 v = *(const float4*)(x + (int64_t)(t0 - KEEP + k) * nc + c);
+            past[k][0] = v.x; past[k][1] = v.y; past[k][2] = v.z; past[k][3] = v.w;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k <= KEEP; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) wt[k][e] = w[(int64_t)(c + e) * (KEEP + 1) + k];
+    float4 xin[CONV_TOK];
+#pragma unroll
+    for (int i = 0; i < CONV_TOK; i++)
+        xin[i] = t0 + i < t1 ? *(const float4*)(x + (int64_t)(t0 + i) * nc + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < CONV_TOK; i++) {
+        if (t0 + i >= t1) break;
+        const float xv[4] = {xin[i].x, xin[i].y, xin[i].z, xin[i].w};
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KEEP; k++) sum += past[k][e] * wt[k][e];
+            sum += xv[e] * wt[KEEP][e];
+            o[e] = it_silu(sum);
+#pragma unroll
+            for (int k = 0; k + 1 < KEEP; k++) past[k][e] = past[k + 1][e];
+            past[KEEP - 1][e] = xv[e];
+        }
+        *(float4*)(out + (int64_t)(t0 + i) * nc + c) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+    // the batch is longer than the window (the launcher sees to it): the new state is its last KEEP inputs
+    if (blockIdx.y == 0) {
+#pragma unroll
+        for (int k = 0; k < KEEP; k++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) state[(int64_t)(c + e) * KEEP + k] = x[(int64_t)(n_tok - KEEP + k) * nc + c + e];
+    }
+}
+
 void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
               hipStream_t s) {
     if (nc <= 0 || n_tok <= 0) return;
+    if (n_tok >= 64 && nc % 4 == 0 && aligned16(x) && aligned16(out) && kernel >= 2 && kernel <= 5) {
+        dim3 grid((nc / 4 + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);
+        switch (kernel) {
+            case 2: hipLaunchKernelGGL(ssm_conv4_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+            case 3: hipLaunchKernelGGL(ssm_conv4_k<2>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+            case 4: hipLaunchKernelGGL(ssm_conv4_k<3>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+            default: hipLaunchKernelGGL(ssm_conv4_k<4>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+        }
+        return;
+    }
     dim3 grid((nc + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);
     switch (kernel) {
         case 2: hipLaunchKernelGGL(ssm_conv_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;

@@ -137,10 +137,63 @@ __global__ void moe_finish_k(float* __restrict__ out, int64_t at, int n, const f
     out[at + t * n + j] = v;
 }
 
+// Four neighbouring outputs per lane with the picks' rows all in flight at once (NU = picks per token, 0 = any):
+// the same sum per output, in pick order.
+template <int NU>
+__global__ __launch_bounds__(256) void moe_finish4_k(float* __restrict__ out, int64_t at, int n4,
+                                                     const float4* __restrict__ rows, const float* __restrict__ weights,
+                                                     int n_tok, int n_used, const float4* __restrict__ shared,
+                                                     const float* __restrict__ logit, int64_t logit_at) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)n_tok * n4) return;
+    const int64_t t = idx / n4;
+    const int j = (int)(idx - t * n4);
+    const int nu = NU ? NU : n_used;
+    const float g = it_sigmoid(logit[logit_at + t]);
+    const float* w = weights + t * nu;
+    const float4* r = rows + t * nu * n4 + j;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if constexpr (NU > 0) {
+        float4 rr[NU];
+#pragma unroll
+        for (int e = 0; e < NU; e++) rr[e] = r[(int64_t)e * n4];
+#pragma unroll
+        for (int e = 0; e < NU; e++) {
+            const float we = w[e];
+            v.x += we * rr[e].x; v.y += we * rr[e].y; v.z += we * rr[e].z; v.w += we * rr[e].w;
+        }
+    } else {
+        for (int e = 0; e < nu; e++) {
+            const float we = w[e];
+            const float4 re = r[(int64_t)e * n4];
+            v.x += we * re.x; v.y += we * re.y; v.z += we * re.z; v.w += we * re.w;
+        }
+    }
+    const float4 sh = shared[t * n4 + j];
+    v.x += sh.x * g; v.y += sh.y * g; v.z += sh.z * g; v.w += sh.w * g;
+    *(float4*)(out + at + t * (int64_t)n4 * 4 + j * 4) = v;
+}
+
 void moe_finish(float* out, int64_t at, int n, const float* rows, const float* weights, int n_tok, int n_used,
                 const float* shared, const float* logit, int64_t logit_at, hipStream_t s) {
     int64_t total = (int64_t)n_tok * n;
     if (total <= 0) return;
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    if (n_tok >= 16 && n % 4 == 0 && at % 4 == 0 && al(out) && al(rows) && al(shared)) {
+        const int n4 = n / 4;
+        const dim3 grid((unsigned)((total / 4 + 255) / 256)), block(256);
+#define IT_FIN(NU)                                                                                             \
+    hipLaunchKernelGGL(moe_finish4_k<NU>, grid, block, 0, s, out, at, n4, (const float4*)rows, weights, n_tok, \
+                       n_used, (const float4*)shared, logit, logit_at)
+        switch (n_used) {
+            case 4: IT_FIN(4); break;
+            case 8: IT_FIN(8); break;
+            case 10: IT_FIN(10); break;
+            default: IT_FIN(0); break;
+        }
+#undef IT_FIN
+        return;
+    }
     hipLaunchKernelGGL(moe_finish_k, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, out, at, n, rows,
                        weights, n_tok, n_used, shared, logit, logit_at);
 }

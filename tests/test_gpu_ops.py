@@ -142,10 +142,10 @@ def test_softmax(hip, orc, n, row):
     assert_bits_equal(a, b, "softmax")
 
 
-def test_elementwise(hip, orc):
+@pytest.mark.parametrize("n", [4096 + 3, 65536, 65536 + 4])  # the long ones take four elements per lane
+def test_elementwise(hip, orc, n):
     fresh(hip)
     r = rng(8)
-    n = 4096 + 3
     g = (r.standard_normal(n) * 5).astype(np.float32); u = r.standard_normal(n).astype(np.float32)
     for name in ["silu_mul", "sigmoid_mul", "add_assign"]:
         a, b = g.copy(), g.copy()
@@ -184,6 +184,14 @@ def test_gather_scatter(hip, orc):
     hip.scatter_chunks(a, 64, 128, 64, da); hip.host_needs(da)
     orc.scatter_chunks(b, 64, 128, 64, db)
     assert_bits_equal(da, db, "scatter_chunks")
+    # long batches move 16 bytes per lane: a slice of every row, as the model cuts q, k, v and gates apart
+    for rows, chunk, stride, offset in [(300, 256, 1024, 512), (64, 512, 516, 4), (200, 128, 1024, 130)]:
+        fresh(hip)
+        src = rng(10).standard_normal(rows * stride).astype(np.float32)
+        a, b = np.zeros(rows * chunk, np.float32), np.zeros(rows * chunk, np.float32)
+        hip.gather_chunks(src, chunk, stride, offset, a); hip.host_needs(a)
+        orc.gather_chunks(src, chunk, stride, offset, b)
+        assert_bits_equal(a, b, f"gather_chunks {rows}x{chunk}")
 
 
 def test_kv_write(hip, orc):
@@ -196,16 +204,19 @@ def test_kv_write(hip, orc):
     assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("n_tok,nc", [(1, 1024), (6, 1024), (1, 8192), (3, 8192)])
-def test_ssm_conv(hip, orc, n_tok, nc):
+@pytest.mark.parametrize("n_tok,nc,kernel", [(1, 1024, 4), (6, 1024, 4), (1, 8192, 4), (3, 8192, 4),
+                                              # token chunks, and from 64 tokens on four channels per lane
+                                              (40, 1024, 4), (70, 1024, 4), (130, 8192, 4), (97, 512, 2), (64, 512, 3),
+                                              (81, 1028, 5), (66, 1022, 4)])
+def test_ssm_conv(hip, orc, n_tok, nc, kernel):
     fresh(hip)
     r = rng(11)
-    sa = r.standard_normal(nc * 3).astype(np.float32); sb = sa.copy()
+    sa = r.standard_normal(nc * (kernel - 1)).astype(np.float32); sb = sa.copy()
     x = r.standard_normal(n_tok * nc).astype(np.float32)
-    w = r.standard_normal(nc * 4).astype(np.float32)
+    w = r.standard_normal(nc * kernel).astype(np.float32)
     a, b = np.zeros_like(x), np.zeros_like(x)
-    hip.ssm_conv(sa, x, w, 4, a); hip.host_needs(a); hip.read_state(sa)
-    orc.ssm_conv(sb, x, w, 4, b)
+    hip.ssm_conv(sa, x, w, kernel, a); hip.host_needs(a); hip.read_state(sa)
+    orc.ssm_conv(sb, x, w, kernel, b)
     assert_bits_equal(a, b, "ssm_conv out")
     assert_bits_equal(sa, sb, "ssm_conv state")
 
@@ -340,6 +351,22 @@ def test_moe_stage(hip, orc, fmt, n_tok, n_expert, n_used, nd, ff):
     fa, fb = np.zeros(n_tok * nd, np.float32), np.zeros(n_tok * nd, np.float32)
     hip.moe_finish(fa, 0, nd, oa, route, shared, logit, 0); hip.host_needs(fa)
     orc.moe_finish(fb, 0, nd, obuf, w, n_used, shared, logit, 0)
+    assert_bits_equal(fa, fb, "moe_finish")
+
+
+@pytest.mark.parametrize("n_tok,n_used,nd", [(20, 8, 512), (33, 5, 256), (16, 10, 2048), (40, 4, 516), (15, 8, 512)])
+def test_moe_finish_batches(hip, orc, n_tok, n_used, nd):
+    """The weighted sum of the picks' rows plus the gated shared expert, in pick order, for the batch shapes
+    that take four outputs per lane and the ones that do not."""
+    import inferred_hip as ih
+    fresh(hip)
+    r = rng(21)
+    rows = r.standard_normal(n_tok * n_used * nd).astype(np.float32)
+    ids = np.zeros(n_tok * n_used, np.uint32); w = r.random(n_tok * n_used).astype(np.float32)
+    shared = r.standard_normal(n_tok * nd).astype(np.float32); logit = r.standard_normal(n_tok + 2).astype(np.float32)
+    fa, fb = np.zeros(n_tok * nd + 8, np.float32), np.zeros(n_tok * nd + 8, np.float32)
+    hip.moe_finish(fa, 8, nd, rows, ih.Hip.host_route(ids, w, n_used), shared, logit, 2); hip.host_needs(fa)
+    orc.moe_finish(fb, 8, nd, rows, w, n_used, shared, logit, 2)
     assert_bits_equal(fa, fb, "moe_finish")
 
 

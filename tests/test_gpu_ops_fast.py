@@ -197,3 +197,23 @@ def test_rms_norm_fast(hip, orc, n, nd):
     hip.rms_norm(x, w, 1e-6, a); hip.host_needs(a)
     orc.rms_norm(x, w, 1e-6, b)
     assert close(a, b, 1e-5)
+
+
+@pytest.mark.parametrize("heads,hd", [(8, 64), (300, 64), (1000 * 16 + 3, 128), (257, 256), (40 * 32, 128)])
+def test_head_norms_fast(hip, orc, heads, hd):
+    """rms and l2 norms over heads: batches of 256 heads and more take a wave per head with the sum of
+    squares added across lanes; the f64 sum only changes its order, so results stay within a few ulp."""
+    fresh(hip)
+    r = rng(31)
+    x = (r.standard_normal(heads * hd) * 3).astype(np.float32)
+    w = r.standard_normal(hd).astype(np.float32)
+    a, b = x.copy(), x.copy()
+    hip.rms_norm_heads(a, w, hd, 1e-6); hip.host_needs(a)
+    orc.rms_norm_heads(b, w, hd, 1e-6)
+    assert np.all(np.abs(a - b) <= 1e-6 * np.maximum(1.0, np.abs(b)))
+    a, b = x.copy(), x.copy()
+    a[:hd] = 0; b[:hd] = 0  # the eps clamp
+    fresh(hip)
+    hip.l2_norm_heads(a, hd, 1e-6); hip.host_needs(a)
+    orc.l2_norm_heads(b, hd, 1e-6)
+    assert np.all(np.abs(a - b) <= 1e-6 * np.maximum(1.0, np.abs(b)))
