@@ -506,19 +506,26 @@ __device__ __attribute__((noinline)) void wave_rank_many(const unsigned long lon
         if (k < K && key[k] != 0ull && rank[k] < n_used) cand[rank[k]] = key[k];
 }
 
+// this thread's logits (up to four experts, THREADS apart): fetched ahead of the activation prologue so that the
+// two loads share one trip to memory
 template <int THREADS>
-__device__ __forceinline__ float block_route(const float* logits, int n_expert, int n_used, RouteLds<THREADS>& sh, int* ids, float* wts) {
+__device__ __forceinline__ void route_fetch(const float* logits, int n_expert, float l[4]) {
+    const int K = (n_expert + THREADS - 1) / THREADS;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int e = threadIdx.x + k * THREADS;
+        l[k] = (k < K && e < n_expert) ? logits[e] : -INFINITY;
+    }
+}
+
+template <int THREADS>
+__device__ __forceinline__ float block_route(const float l[4], int n_expert, int n_used, RouteLds<THREADS>& sh, int* ids, float* wts) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int NW = THREADS / 64;
     const int K = (n_expert + THREADS - 1) / THREADS;  // experts per thread that can be live
-    float l[4];
     float m = -INFINITY;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const int e = tid + k * THREADS;
-        l[k] = (k < K && e < n_expert) ? logits[e] : -INFINITY;
-        m = fmaxf(m, l[k]);
-    }
+    for (int k = 0; k < 4; k++) m = fmaxf(m, l[k]);
     if (tid < NW * 16) sh.cand[tid] = 0ull;  // slots a wave does not fill stay empty
     if (tid < 16) wts[tid] = 0.0f;
     m = group_max_tail<64>(m);
@@ -652,9 +659,11 @@ __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
         }
     }
 
+    float logit[4];
+    if (p.logits) route_fetch<FT>(p.logits, p.n_expert, logit);
     stage_activation<FT>(p.x, n_in, 0, nullptr, nullptr, 0, 0.0f, nullptr, nullptr, xq, xs, red);
     if (p.logits) {
-        const float denom = block_route<FT>(p.logits, p.n_expert, p.n_used, route_sh, ids, wts);
+        const float denom = block_route<FT>(logit, p.n_expert, p.n_used, route_sh, ids, wts);
         if (blockIdx.x == 0 && tid < p.n_used) {
             p.route_ids_out[tid] = ids[tid];
             p.route_w_out[tid] = wts[tid] / denom;
