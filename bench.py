@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle baseline")
     ap.add_argument("--exact", action="store_true", help="CPU-order reductions (bit-exact mode)")
     ap.add_argument("--keep", action="store_true", help="keep the generated GGUF")
+    ap.add_argument("--no-single-ops", action="store_true",
+                    help="skip the single-op configurations (expert FFN sweep, decode attention, Gated DeltaNet)")
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -86,6 +88,12 @@ def main():
         dst.copy_(src); torch.cuda.synchronize()
         dst.copy_(src); torch.cuda.synchronize()
         del src, dst
+    single = None
+    if not args.no_single_ops and args.layers == 48:
+        from inferred_hip import single_ops
+        t_s = time.time()
+        single = single_ops.run(ih, seed=args.seed, exact=args.exact)
+        print(f"[bench] single-op configurations in {time.time() - t_s:.1f}s", file=sys.stderr, flush=True)
     be = ih.Hip(exact=args.exact)
     model = ih.Model(path)
     eng = ih.Engine(model, be, args.ctx, args.max_batch)
@@ -246,6 +254,7 @@ def main():
         "prefill_tok_s": round(args.prompt / t_prefill, 1),
         "prefill_kernels": prefill_kernels,
         "mfma_ceilings_measured": ceilings,
+        "single_op": single,
         "bytes_per_token": int(tok_bytes),
         "token_roofline": {"bound": "hbm", "achieved": round(whole, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": round(whole / HBM_PEAK_GBS, 4)},

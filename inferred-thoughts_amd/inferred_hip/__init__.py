@@ -391,6 +391,10 @@ class Hip:
         return [dict(name=rows[i].name.decode(), launches=int(rows[i].launches), ms=float(rows[i].ms_total),
                      bytes=int(rows[i].bytes_total)) for i in range(n)]
 
+    def release(self, buf):
+        """Forget the device copy of one host buffer (call before the buffer is freed)."""
+        self.L.it_hip_release(self.h, _p(buf))
+
     def drop_mirrors(self):
         self.L.it_hip_drop_mirrors(self.h)
 
