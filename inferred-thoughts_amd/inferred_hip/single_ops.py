@@ -67,7 +67,7 @@ def _timed(be, fn, reps):
 
 def _line(bytes_, ms, launches, **extra):
     gbs = bytes_ / 1e9 / (ms / 1e3)
-    d = dict(algorithmic_mb=round(bytes_ / 1e6, 2), us=round(ms * 1e3, 1), launches=round(launches, 1),
+    d = dict(algorithmic_mb=round(bytes_ / 1e6, 2), us=round(ms * 1e3, 1), ops=round(launches, 1),
              gb_s=round(gbs, 1), hbm_frac=round(gbs / HBM_PEAK_GBS, 4))
     d.update(extra)
     return d
