@@ -211,10 +211,10 @@ __device__ __forceinline__ void stage_activation(const float* x, int n_in, int m
                 const float4 w = ((const float4*)norm_w)[qi & (lh - 1)];
                 const float4 g = ((const float4*)gate)[qi];
                 // mode 3: the producer already stored silu(gate)
-                v[k].x = (mode == 2 ? it_silu(g.x) : g.x) * (v[k].x * hs * w.x);
-                v[k].y = (mode == 2 ? it_silu(g.y) : g.y) * (v[k].y * hs * w.y);
-                v[k].z = (mode == 2 ? it_silu(g.z) : g.z) * (v[k].z * hs * w.z);
-                v[k].w = (mode == 2 ? it_silu(g.w) : g.w) * (v[k].w * hs * w.w);
+                v[k].x = (mode == 2 ? fx_silu(g.x) : g.x) * (v[k].x * hs * w.x);
+                v[k].y = (mode == 2 ? fx_silu(g.y) : g.y) * (v[k].y * hs * w.y);
+                v[k].z = (mode == 2 ? fx_silu(g.z) : g.z) * (v[k].z * hs * w.z);
+                v[k].w = (mode == 2 ? fx_silu(g.w) : g.w) * (v[k].w * hs * w.w);
             }
         }
     }
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                 } else if (m.epi == 2) {
                     m.out[j] = cp[r] + a;
                 } else if (m.epi == 3) {
-                    m.out[j] = it_silu(a);
+                    m.out[j] = fx_silu(a);
                 } else {
                     // causal conv (kernel 4) + silu on channel j, state [channel][3] oldest first
                     float* past = p.conv_state + (int64_t)j * 3;
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                     sum += p1 * w.y;
                     sum += p2 * w.z;
                     sum += a * w.w;
-                    m.out[j] = it_silu(sum);
+                    m.out[j] = fx_silu(sum);
                     past[0] = p1;
                     past[1] = p2;
                     past[2] = a;
@@ -539,7 +539,7 @@ __device__ __forceinline__ float block_route(const float l[4], int n_expert, int
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int e = tid + k * THREADS;
-        v[k] = (k < K && e < n_expert) ? it_expf(l[k] - m) : 0.0f;
+        v[k] = (k < K && e < n_expert) ? fx_expf(l[k] - m) : 0.0f;
         part += v[k];
     }
     part = group_sum_tail<64>(part);
@@ -567,7 +567,7 @@ __device__ __forceinline__ float block_route(const float l[4], int n_expert, int
         int cnt = 0;
 #pragma unroll
         for (int c2 = 0; c2 < NW * 2; c2++) {
-            const ulonglong2 q = ((const ulonglong2*)sh.cand)[part * NW * 2 + c2];
+            const ulonglong2 q = ((const ulonglong2*)sh.cand)[c2 * 4 + part];  // the four threads of a slot read neighbouring 16-byte pieces: no bank is hit twice
             cnt += q.x > me ? 1 : 0;
             cnt += q.y > me ? 1 : 0;
         }
@@ -624,7 +624,7 @@ IT_DEV void glu_job(const uint8_t* gq, const uint8_t* gs, const uint8_t* uq, con
         if (sub == L - 1 && row < n_out) {
             ag *= sg;
             au *= su;
-            out[row] = it_silu(ag) * au;
+            out[row] = fx_silu(ag) * au;
         }
     }
 }
@@ -791,7 +791,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     if (half) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
     const float x_old = (!half && sub == L - 1 && live) ? p.x[row] : 0.0f;
     if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
-    const float gate = it_sigmoid(p.logit[0]);
+    const float gate = fx_sigmoid(p.logit[0]);
     IT_STAMP(1);
 
 #pragma unroll

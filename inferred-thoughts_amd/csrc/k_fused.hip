@@ -451,6 +451,13 @@ IT_DEV void gdn_gates(const GdnCoreP& p, int h, float* g, float* beta) {
     *g = it_expf(softplus * p.ssm_a[h]);
     *beta = 1.0f / (1.0f + it_expf(-p.beta[h]));
 }
+// the same on the transcendental unit, for the kernel that reorders its sums anyway
+IT_DEV void gdn_gates_fast(const GdnCoreP& p, int h, float* g, float* beta) {
+    float a = p.alpha[h] + p.dt_bias[h];
+    float softplus = a > 20.0f ? a : fx_logf(1.0f + fx_expf(a));
+    *g = fx_expf(softplus * p.ssm_a[h]);
+    *beta = fx_sigmoid(p.beta[h]);
+}
 
 // Exact form: one lane owns one value row, the three sweeps run in the CPU path's order.
 template <int DK>
@@ -528,7 +535,7 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
         row[4 * i] = st[i].x; row[4 * i + 1] = st[i].y; row[4 * i + 2] = st[i].z; row[4 * i + 3] = st[i].w;
     }
     float g, beta;
-    gdn_gates(p, h, &g, &beta);
+    gdn_gates_fast(p, h, &g, &beta);
     float v = p.conv[2 * key_dim + h * dv + j];
     const float* kk = kq + seg * SEG;
     const float* qq = kq + DK + seg * SEG;
