@@ -958,10 +958,11 @@ static void ew2(it_hip* be, float* a, uint64_t a_len, const float* b, uint64_t b
     int64_t n = (int64_t)a_len;
     it_hip::OpRec rec;
     rec.id = OP_EW; rec.p[0] = da; rec.p[1] = db; rec.i[0] = op; rec.i[1] = n; rec.f[0] = v;
+    const int exact = be->exact;
     be->submit(it_hip::FAM_OTHER, a_len * 12, sig_of(OP_EW, op, da, db, n, v), rec, [=](hipStream_t s) {
         switch (op) {
-            case 0: silu_mul(da, db, n, s); break;
-            case 1: sigmoid_mul(da, db, n, s); break;
+            case 0: silu_mul(da, db, n, exact, s); break;
+            case 1: sigmoid_mul(da, db, n, exact, s); break;
             case 2: add_assign(da, db, n, s); break;
             case 3: add_scaled(da, db, v, n, s); break;
         }
@@ -1009,7 +1010,7 @@ void it_hip_ssm_conv(it_hip* be, float* state, uint64_t state_len, const float* 
     it_hip::OpRec rec;
     rec.id = OP_CONV; rec.p[0] = dstate; rec.p[1] = dx; rec.p[2] = dw; rec.p[3] = dout; rec.i[0] = k; rec.i[1] = c; rec.i[2] = nt;
     be->submit(it_hip::FAM_OTHER, x_len * 8 + state_len * 8, sig_of(OP_CONV, dstate, dx, dw, k, c, nt, dout), rec,
-               [=](hipStream_t s) { ssm_conv(dstate, dx, dw, k, c, nt, dout, s); });
+               [=, exact = (int)be->exact](hipStream_t s) { ssm_conv(dstate, dx, dw, k, c, nt, dout, exact, s); });
 }
 
 void it_hip_gather_chunks(it_hip* be, const float* src, uint64_t src_len, uint64_t chunk, uint64_t stride,
@@ -1268,7 +1269,7 @@ void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, ui
     rec.id = OP_FINISH; rec.p[0] = dout; rec.p[1] = dr; rec.p[2] = rw; rec.p[3] = ds; rec.p[4] = dl;
     rec.i[0] = a64; rec.i[1] = ni; rec.i[2] = nt; rec.i[3] = nu; rec.i[4] = la;
     be->submit(it_hip::FAM_OTHER, rows_len * 4 + n_tok * n * 8, sig_of(OP_FINISH, dout, a64, ni, dr, rw, nt, nu, ds, dl, la), rec,
-               [=](hipStream_t s) { moe_finish(dout, a64, ni, dr, rw, nt, nu, ds, dl, la, s); });
+               [=, exact = (int)be->exact](hipStream_t s) { moe_finish(dout, a64, ni, dr, rw, nt, nu, ds, dl, la, exact, s); });
 }
 
 void it_hip_add_scaled_rows(it_hip* be, float* acc, uint64_t acc_len, const float* rows, uint64_t rows_len,

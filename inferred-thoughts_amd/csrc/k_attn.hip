@@ -624,7 +624,7 @@ __global__ __launch_bounds__(1024) void attend_merge_k(const float* __restrict__
     __syncthreads();
     if (g == 0) {
         float r = ((accs[i] + accs[hd + i]) + (accs[2 * hd + i] + accs[3 * hd + i])) / l;
-        if (gate) r *= it_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + i]);
+        if (gate) r *= fx_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + i]);
         out[(int64_t)blockIdx.x * hd + i] = r;
     }
 }
@@ -676,7 +676,7 @@ __global__ __launch_bounds__(256) void attend_merge_wide_k(const float* __restri
     __syncthreads();
     if (tid < 32) {
         float r = (((accs[0][i] + accs[1][i]) + (accs[2][i] + accs[3][i])) + ((accs[4][i] + accs[5][i]) + (accs[6][i] + accs[7][i]))) / l;
-        if (gate) r *= it_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + d0 + i]);
+        if (gate) r *= fx_sigmoid(gate[(int64_t)blockIdx.x * gate_stride + d0 + i]);
         out[(int64_t)blockIdx.x * hd + d0 + i] = r;
     }
 }

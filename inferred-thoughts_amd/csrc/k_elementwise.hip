@@ -278,19 +278,24 @@ __global__ void fill_zero_k(uint32_t* p, int64_t n_words) {
 }
 
 // Four elements per lane for the long batches: the same arithmetic per element, 16-byte accesses.
+// FX: the exponential on the transcendental unit (fast mode) instead of the CPU path's libm form
+template <bool FX> IT_DEV float silu_of(float v) { return FX ? fx_silu(v) : it_silu(v); }
+template <bool FX> IT_DEV float sigmoid_of(float v) { return FX ? fx_sigmoid(v) : it_sigmoid(v); }
+template <bool FX>
 __global__ void silu_mul4_k(float4* __restrict__ g, const float4* __restrict__ u, int64_t n4) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
         float4 a = g[i];
         const float4 b = u[i];
-        a.x = it_silu(a.x) * b.x; a.y = it_silu(a.y) * b.y; a.z = it_silu(a.z) * b.z; a.w = it_silu(a.w) * b.w;
+        a.x = silu_of<FX>(a.x) * b.x; a.y = silu_of<FX>(a.y) * b.y; a.z = silu_of<FX>(a.z) * b.z; a.w = silu_of<FX>(a.w) * b.w;
         g[i] = a;
     }
 }
+template <bool FX>
 __global__ void sigmoid_mul4_k(float4* __restrict__ x, const float4* __restrict__ g, int64_t n4) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
         float4 a = x[i];
         const float4 b = g[i];
-        a.x *= it_sigmoid(b.x); a.y *= it_sigmoid(b.y); a.z *= it_sigmoid(b.z); a.w *= it_sigmoid(b.w);
+        a.x *= sigmoid_of<FX>(b.x); a.y *= sigmoid_of<FX>(b.y); a.z *= sigmoid_of<FX>(b.z); a.w *= sigmoid_of<FX>(b.w);
         x[i] = a;
     }
 }
@@ -318,16 +323,18 @@ constexpr int64_t VEC_MIN = 1 << 14;  // below this one pass of scalar lanes is 
         if ((n) > 0) hipLaunchKernelGGL(kern, dim3(blocks_for((n), 256)), dim3(256), 0, s, __VA_ARGS__); \
     } while (0)
 
-void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s) {
-    if (n >= VEC_MIN && n % 4 == 0 && aligned16(gate) && aligned16(up))
-        EW_LAUNCH(silu_mul4_k, n / 4, (float4*)gate, (const float4*)up, n / 4);
-    else
+void silu_mul(float* gate, const float* up, int64_t n, int exact, hipStream_t s) {
+    if (n >= VEC_MIN && n % 4 == 0 && aligned16(gate) && aligned16(up)) {
+        if (exact) EW_LAUNCH(silu_mul4_k<false>, n / 4, (float4*)gate, (const float4*)up, n / 4);
+        else EW_LAUNCH(silu_mul4_k<true>, n / 4, (float4*)gate, (const float4*)up, n / 4);
+    } else
         EW_LAUNCH(silu_mul_k, n, gate, up, n);
 }
-void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s) {
-    if (n >= VEC_MIN && n % 4 == 0 && aligned16(x) && aligned16(g))
-        EW_LAUNCH(sigmoid_mul4_k, n / 4, (float4*)x, (const float4*)g, n / 4);
-    else
+void sigmoid_mul(float* x, const float* g, int64_t n, int exact, hipStream_t s) {
+    if (n >= VEC_MIN && n % 4 == 0 && aligned16(x) && aligned16(g)) {
+        if (exact) EW_LAUNCH(sigmoid_mul4_k<false>, n / 4, (float4*)x, (const float4*)g, n / 4);
+        else EW_LAUNCH(sigmoid_mul4_k<true>, n / 4, (float4*)x, (const float4*)g, n / 4);
+    } else
         EW_LAUNCH(sigmoid_mul_k, n, x, g, n);
 }
 void add_assign(float* a, const float* b, int64_t n, hipStream_t s) {
@@ -447,7 +454,7 @@ __global__ void ssm_conv_k(float* __restrict__ state, const float* __restrict__ 
 }
 
 // The same for four neighbouring channels per lane: 16-byte accesses, the chunk's inputs all in flight at once.
-template <int KEEP>
+template <int KEEP, bool FX>
 __global__ __launch_bounds__(128) void ssm_conv4_k(float* __restrict__ state, const float* __restrict__ x,
                                                    const float* __restrict__ w, int nc, int n_tok,
                                                    float* __restrict__ out) {
@@ -484,7 +491,7 @@ __global__ __launch_bounds__(128) void ssm_conv4_k(float* __restrict__ state, co
 #pragma unroll
             for (int k = 0; k < KEEP; k++) sum += past[k][e] * wt[k][e];
             sum += xv[e] * wt[KEEP][e];
-            o[e] = it_silu(sum);
+            o[e] = silu_of<FX>(sum);
 #pragma unroll
             for (int k = 0; k + 1 < KEEP; k++) past[k][e] = past[k + 1][e];
             past[KEEP - 1][e] = xv[e];
@@ -500,17 +507,23 @@ __global__ __launch_bounds__(128) void ssm_conv4_k(float* __restrict__ state, co
     }
 }
 
-void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
+void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out, int exact,
               hipStream_t s) {
     if (nc <= 0 || n_tok <= 0) return;
     if (n_tok >= 64 && nc % 4 == 0 && aligned16(x) && aligned16(out) && kernel >= 2 && kernel <= 5) {
         dim3 grid((nc / 4 + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);
+#define IT_CONV4(KEEP)                                                                                        \
+    do {                                                                                                      \
+        if (exact) hipLaunchKernelGGL((ssm_conv4_k<KEEP, false>), grid, block, 0, s, state, x, w, nc, n_tok, out); \
+        else hipLaunchKernelGGL((ssm_conv4_k<KEEP, true>), grid, block, 0, s, state, x, w, nc, n_tok, out);   \
+    } while (0)
         switch (kernel) {
-            case 2: hipLaunchKernelGGL(ssm_conv4_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
-            case 3: hipLaunchKernelGGL(ssm_conv4_k<2>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
-            case 4: hipLaunchKernelGGL(ssm_conv4_k<3>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
-            default: hipLaunchKernelGGL(ssm_conv4_k<4>, grid, block, 0, s, state, x, w, nc, n_tok, out); break;
+            case 2: IT_CONV4(1); break;
+            case 3: IT_CONV4(2); break;
+            case 4: IT_CONV4(3); break;
+            default: IT_CONV4(4); break;
         }
+#undef IT_CONV4
         return;
     }
     dim3 grid((nc + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);

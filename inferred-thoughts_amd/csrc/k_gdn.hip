@@ -136,9 +136,9 @@ __global__ __launch_bounds__(256) void delta_rule_fast_k(DeltaArgs d, float* __r
     const int kper = d.n_k_heads * DK, vper = d.n_v_heads * dv;
     for (int t = tid; t < d.n_tokens; t += 256) {
         const float a = d.alpha[(int64_t)t * d.n_v_heads + h] + d.dt_bias[h];
-        const float softplus = a > 20.0f ? a : it_logf(1.0f + it_expf(a));
-        gates[2 * t] = it_expf(softplus * d.ssm_a[h]);
-        gates[2 * t + 1] = 1.0f / (1.0f + it_expf(-d.beta[(int64_t)t * d.n_v_heads + h]));
+        const float softplus = a > 20.0f ? a : fx_logf(1.0f + fx_expf(a));
+        gates[2 * t] = fx_expf(softplus * d.ssm_a[h]);
+        gates[2 * t + 1] = fx_sigmoid(d.beta[(int64_t)t * d.n_v_heads + h]);
     }
     float* S = state + ((int64_t)h * dv + j) * DK + seg * SEG;
     float row[SEG];

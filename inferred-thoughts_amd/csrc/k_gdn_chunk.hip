@@ -79,9 +79,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_k(DeltaArgs d, float* __re
         float lg = 0.0f, beta = 0.0f;
         if (ok) {
             const float a = d.alpha[(int64_t)t * d.n_v_heads + h] + d.dt_bias[h];
-            const float softplus = a > 20.0f ? a : it_logf(1.0f + it_expf(a));
+            const float softplus = a > 20.0f ? a : fx_logf(1.0f + fx_expf(a));
             lg = softplus * d.ssm_a[h];
-            beta = 1.0f / (1.0f + it_expf(-d.beta[(int64_t)t * d.n_v_heads + h]));
+            beta = 1.0f / (1.0f + fx_expf(-d.beta[(int64_t)t * d.n_v_heads + h]));
         }
         float x = lg;
 #pragma unroll
@@ -92,10 +92,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_k(DeltaArgs d, float* __re
         const float xc = __shfl(x, 63, 64);
         cum[lane] = x;
         bet[lane] = beta;
-        ws[WS_GAM + lane] = it_expf(x);
-        ws[WS_DEC + lane] = it_expf(xc - x);
+        ws[WS_GAM + lane] = fx_expf(x);
+        ws[WS_DEC + lane] = fx_expf(xc - x);
         ws[WS_BET + lane] = beta;
-        ws[WS_GC + lane] = it_expf(xc);
+        ws[WS_GC + lane] = fx_expf(xc);
     }
     for (int idx = tid; idx < GC * DK / 4; idx += 256) {
         const int tt = idx / (DK / 4), c4 = idx % (DK / 4);

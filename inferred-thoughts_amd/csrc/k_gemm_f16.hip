@@ -333,7 +333,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float g = acc[0][tt][4 * i4 + i] * rsc * e2a, u = acc[1][tt][4 * i4 + i] * rsc * e2b;
-                    o[i] = it_silu(g) * u;
+                    o[i] = fx_silu(g) * u;
                 }
                 *(float4*)(p.out + pair * p.n_out + row) = make_float4(o[0], o[1], o[2], o[3]);
             } else {

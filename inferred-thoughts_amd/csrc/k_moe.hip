@@ -139,7 +139,7 @@ __global__ void moe_finish_k(float* __restrict__ out, int64_t at, int n, const f
 
 // Four neighbouring outputs per lane with the picks' rows all in flight at once (NU = picks per token, 0 = any):
 // the same sum per output, in pick order.
-template <int NU>
+template <int NU, bool FX>
 __global__ __launch_bounds__(256) void moe_finish4_k(float* __restrict__ out, int64_t at, int n4,
                                                      const float4* __restrict__ rows, const float* __restrict__ weights,
                                                      int n_tok, int n_used, const float4* __restrict__ shared,
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void moe_finish4_k(float* __restrict__ out, in
     const int64_t t = idx / n4;
     const int j = (int)(idx - t * n4);
     const int nu = NU ? NU : n_used;
-    const float g = it_sigmoid(logit[logit_at + t]);
+    const float g = FX ? fx_sigmoid(logit[logit_at + t]) : it_sigmoid(logit[logit_at + t]);
     const float* w = weights + t * nu;
     const float4* r = rows + t * nu * n4 + j;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -175,16 +175,20 @@ __global__ __launch_bounds__(256) void moe_finish4_k(float* __restrict__ out, in
 }
 
 void moe_finish(float* out, int64_t at, int n, const float* rows, const float* weights, int n_tok, int n_used,
-                const float* shared, const float* logit, int64_t logit_at, hipStream_t s) {
+                const float* shared, const float* logit, int64_t logit_at, int exact, hipStream_t s) {
     int64_t total = (int64_t)n_tok * n;
     if (total <= 0) return;
     auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
     if (n_tok >= 16 && n % 4 == 0 && at % 4 == 0 && al(out) && al(rows) && al(shared)) {
         const int n4 = n / 4;
         const dim3 grid((unsigned)((total / 4 + 255) / 256)), block(256);
-#define IT_FIN(NU)                                                                                             \
-    hipLaunchKernelGGL(moe_finish4_k<NU>, grid, block, 0, s, out, at, n4, (const float4*)rows, weights, n_tok, \
-                       n_used, (const float4*)shared, logit, logit_at)
+#define IT_FIN(NU)                                                                                                      \
+    do {                                                                                                                \
+        if (exact) hipLaunchKernelGGL((moe_finish4_k<NU, false>), grid, block, 0, s, out, at, n4, (const float4*)rows, weights, \
+                                      n_tok, n_used, (const float4*)shared, logit, logit_at);                           \
+        else hipLaunchKernelGGL((moe_finish4_k<NU, true>), grid, block, 0, s, out, at, n4, (const float4*)rows, weights, \
+                                n_tok, n_used, (const float4*)shared, logit, logit_at);                                 \
+    } while (0)
         switch (n_used) {
             case 4: IT_FIN(4); break;
             case 8: IT_FIN(8); break;

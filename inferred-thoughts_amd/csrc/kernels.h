@@ -81,7 +81,7 @@ void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,
                 hipStream_t s);
 void moe_finish(float* out, int64_t at, int n, const float* rows, const float* weights, int n_tok, int n_used,
-                const float* shared, const float* logit, int64_t logit_at, hipStream_t s);
+                const float* shared, const float* logit, int64_t logit_at, int exact, hipStream_t s);
 
 // ---- norms and elementwise ------------------------------------------------------
 void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
@@ -91,8 +91,9 @@ void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n
 void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s);
 void rope_neox(float* x, const float2* table, int table_half, int64_t n_tok, int pos, const int* pos_dyn,
                int head_dim, int n_rot, int n_heads, hipStream_t s);
-void silu_mul(float* gate, const float* up, int64_t n, hipStream_t s);
-void sigmoid_mul(float* x, const float* g, int64_t n, hipStream_t s);
+// exact = 0: long batches take the exponential on the transcendental unit (fast mode)
+void silu_mul(float* gate, const float* up, int64_t n, int exact, hipStream_t s);
+void sigmoid_mul(float* x, const float* g, int64_t n, int exact, hipStream_t s);
 void add_assign(float* a, const float* b, int64_t n, hipStream_t s);
 void scale(float* a, float v, int64_t n, hipStream_t s);
 void add_scaled(float* a, const float* b, float v, int64_t n, hipStream_t s);
@@ -113,7 +114,7 @@ void embed_row(const WView& w, const int32_t* token, float* x, int32_t* ring, in
                hipStream_t s);
 
 // ---- gated delta net ---------------------------------------------------------------
-void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out,
+void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out, int exact,
               hipStream_t s);
 struct DeltaArgs {
     const float *q, *k, *v, *alpha, *beta, *ssm_a, *dt_bias;
