@@ -1550,11 +1550,10 @@ int it_hip_embed_argmax(it_hip* be, const it_weights* table, const float* logits
     int64_t n = (int64_t)logits_len;
     it_hip::OpRec rec;
     rec.id = OP_EMBED; rec.p[0] = dl; rec.p[1] = dx; rec.p[2] = w.q; rec.i[0] = n; rec.i[1] = w.n_in;
-    be->launches += 2;
+    be->launches += 1;
     be->submit(it_hip::FAM_OTHER, logits_len * 4 + x_len * 6, sig_of(OP_EMBED, dl, dx, w.q, w.scales, w.fmt, n, w.n_in, dyn ? 1 : 0),
                rec, [=](hipStream_t s) {
-                   argmax(dl, n, out, idx, val, s);
-                   embed_row(w, out, dx, ring, slot, dyn, s);
+                   argmax_embed(dl, n, out, idx, val, w, dx, ring, slot, dyn, s);
                });
     return 1;
 }

@@ -578,21 +578,33 @@ __global__ __launch_bounds__(256) void argmax_part_k(const float* __restrict__ x
         pval[blockIdx.x] = sv[0];
     }
 }
-__global__ void argmax_final_k(const int32_t* __restrict__ pidx, const float* __restrict__ pval, int n_part,
-                               int32_t* __restrict__ out) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+// the first strict maximum among the partial results, found by one wave: every lane ends with the winner
+IT_DEV int argmax_of_parts(const int32_t* __restrict__ pidx, const float* __restrict__ pval, int n_part, int lane) {
     float bv = 0.f;
     int bi = 0x7fffffff;
-    for (int p = 0; p < n_part; p++) {
-        int oi = pidx[p];
-        float ov = pval[p];
-        if (oi == 0x7fffffff) continue;
-        if (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi)) {
+    for (int p = lane; p < n_part; p += 64) {
+        const int oi = pidx[p];
+        const float ov = pval[p];
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
             bv = ov;
             bi = oi;
         }
     }
-    out[0] = bi == 0x7fffffff ? 0 : bi;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    return bi == 0x7fffffff ? 0 : bi;
+}
+__global__ __launch_bounds__(64) void argmax_final_k(const int32_t* __restrict__ pidx, const float* __restrict__ pval, int n_part,
+                                                     int32_t* __restrict__ out) {
+    const int bi = argmax_of_parts(pidx, pval, n_part, threadIdx.x);
+    if (threadIdx.x == 0) out[0] = bi;
 }
 
 void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s) {
@@ -625,6 +637,52 @@ __global__ __launch_bounds__(256) void embed_row_k(WView w, const int32_t* __res
         }
         x[i] = v;
     }
+}
+
+// The last step of the arg-max and the embedding of its result in one launch: every block's first wave picks the
+// winner among the partial results (the same in every block), block 0 files it, and the blocks share the row.
+__global__ __launch_bounds__(256) void argmax_embed_k(const int32_t* __restrict__ pidx, const float* __restrict__ pval, int n_part,
+                                                      int32_t* __restrict__ out, WView w, float* __restrict__ x,
+                                                      int32_t* __restrict__ ring, int ring_idx, const int* __restrict__ ring_dyn) {
+    __shared__ int winner;
+    if (threadIdx.x < 64) {
+        const int bi = argmax_of_parts(pidx, pval, n_part, threadIdx.x);
+        if (threadIdx.x == 0) {
+            winner = bi;
+            if (blockIdx.x == 0) {
+                out[0] = bi;
+                if (ring) ring[ring_dyn ? *ring_dyn : ring_idx] = bi;
+            }
+        }
+    }
+    __syncthreads();
+    const int64_t tok = winner;
+    const int n_in = w.n_in;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n_in; i += gridDim.x * 256) {
+        float v;
+        if (w.fmt == W_Q8_0) {
+            const int8_t q = ((const int8_t*)w.q)[tok * n_in + i];
+            const uint16_t d = ((const uint16_t*)w.scales)[tok * (n_in >> 5) + (i >> 5)];
+            v = it_f16_to_f32(d) * (float)q;
+        } else if (w.fmt == W_F16) {
+            v = it_f16_to_f32(((const uint16_t*)w.q)[tok * n_in + i]);
+        } else if (w.fmt == W_BF16) {
+            v = it_bf16_to_f32(((const uint16_t*)w.q)[tok * n_in + i]);
+        } else {
+            v = ((const float*)w.q)[tok * n_in + i];
+        }
+        x[i] = v;
+    }
+}
+
+void argmax_embed(const float* logits, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, const WView& w,
+                  float* x, int32_t* ring, int ring_idx, const int* ring_dyn, hipStream_t s) {
+    const int parts = 64;
+    hipLaunchKernelGGL(argmax_part_k, dim3(parts), dim3(256), 0, s, logits, n, scratch_idx, scratch_val);
+    int blocks = (w.n_in + 255) / 256;
+    if (blocks > 64) blocks = 64;
+    hipLaunchKernelGGL(argmax_embed_k, dim3(blocks), dim3(256), 0, s, scratch_idx, scratch_val, parts, out, w, x, ring, ring_idx,
+                       ring_dyn);
 }
 
 void embed_row(const WView& w, const int32_t* token, float* x, int32_t* ring, int ring_idx, const int* ring_dyn,

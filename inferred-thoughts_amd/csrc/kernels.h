@@ -110,6 +110,9 @@ void fill_zero(void* p, int64_t bytes, hipStream_t s);
 void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s);
 // x = dequantized row `*token` of an embedding table (Q8_0 repacked, F16, BF16 or F32); the id goes to
 // ring[ring_dyn ? *ring_dyn : ring_idx] when ring is non-null
+// arg-max of the logits and the embedding row of the winner (the two above) in two launches instead of three
+void argmax_embed(const float* logits, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, const WView& w,
+                  float* x, int32_t* ring, int ring_idx, const int* ring_dyn, hipStream_t s);
 void embed_row(const WView& w, const int32_t* token, float* x, int32_t* ring, int ring_idx, const int* ring_dyn,
                hipStream_t s);
 
