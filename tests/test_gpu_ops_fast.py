@@ -50,6 +50,12 @@ def l2n(x, hd):
 
 @pytest.mark.parametrize("n_q,n_pos,hd,nh,nkv", [(1, 1024, 256, 16, 2), (1, 8192, 256, 16, 2), (1, 32000, 256, 16, 2),
                                                   (1, 63, 64, 8, 2), (1, 200, 128, 8, 1), (5, 300, 256, 16, 2),
+                                                  # the few-query kernel's edges: one key, fewer keys than a group of
+                                                  # 16, a query that sees a single position, every group size it takes,
+                                                  # more key ranges than the 256 splits (two tiles per block)
+                                                  (1, 1, 256, 16, 2), (1, 5, 64, 8, 2), (1, 16, 128, 8, 8), (1, 17, 256, 16, 2),
+                                                  (5, 5, 256, 16, 2), (16, 16, 64, 8, 2), (3, 129, 128, 4, 2), (2, 700, 64, 2, 2),
+                                                  (1, 20000, 64, 8, 2), (4, 33000, 128, 8, 1),
                                                   (16, 300, 256, 16, 2),
                                                   # more than 16 queries: one pass over the keys on the f16 matrix cores
                                                   # (whole prompt; a batch at an offset; ragged last query tile; one
