@@ -224,6 +224,9 @@ void it_hip_drop_mirrors(it_hip*);
 uint64_t it_hip_launch_count(it_hip*);
 /* decode graphs: captures, replays, fallbacks to eager, kernel launches in the captured graph */
 void it_hip_graph_stats(it_hip*, uint64_t out[4]);
+/* The caller has zeroed the host copy of every recurrent-state slab (a sequence reset): the device copies are
+ * zeroed in place, where forget_state (mod.rs:1360-1419) would upload the zeros again at their next use. */
+void it_hip_zero_state(it_hip*);
 /* This card's matrix-core ceiling, measured: back-to-back MFMA instructions on eight independent
  * accumulators per wave, two waves on every SIMD, no memory in the loop (the method of the reference's
  * own ceilings, tests/cuda_ops.rs:56-72).  kind: 0 int8 16x16x64, 1 int8 16x16x32, 2 f16 32x32x16,

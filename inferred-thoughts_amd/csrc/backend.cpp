@@ -1394,6 +1394,19 @@ void it_hip_forget_state(it_hip* be) {
         if (kv.second.is_state) kv.second.dev_owned = false;
 }
 
+void it_hip_zero_state(it_hip* be) {
+    // the host copies were just zeroed: zero the device copies in place instead of uploading zeros at the next use
+    for (auto& kv : be->slabs) {
+        if (!kv.second.is_state) continue;
+        if (kv.second.dev) {
+            fill_zero(kv.second.dev, (int64_t)kv.second.bytes, be->stream);
+            kv.second.dev_owned = true;
+        } else {
+            kv.second.dev_owned = false;
+        }
+    }
+}
+
 void it_hip_read_state(it_hip* be, float* host, uint64_t len) {
     be->need_eager("a state slab is read");
     auto it = be->slabs.find(host);

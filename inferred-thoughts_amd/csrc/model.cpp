@@ -542,7 +542,7 @@ void it_engine_reset(it_engine* e) {
     e->len = 0;
     std::fill(e->conv.begin(), e->conv.end(), 0.0f);
     std::fill(e->ssm.begin(), e->ssm.end(), 0.0f);
-    it_hip_forget_state(e->be);
+    it_hip_zero_state(e->be);
 }
 void it_engine_set_trace(it_engine* e, it_trace_fn fn, void* user) {
     e->trace = fn;
