@@ -928,7 +928,14 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
                    [=](hipStream_t s) { attend_exact(args, sc, dout, s); });
     } else {
         int n_split = attend_split_count((int)n_pos_cap, (int)n_q, (int)a->head_dim, (int)group);
-        float* sc = be->scratch_f32((size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2));
+        // the one-pass kernel of a large batch (never a graphed pass) keeps no partial results: what is reserved is
+        // what the single-token passes that follow will ask for (the whole slab's splits), so that they do not grow it
+        AttnArgs probe{dq, dk, dv, (int)n_q, (int)a->kv_dim, (int)a->n_pos, (int)a->head_dim, (int)a->n_head, (int)a->n_head_kv,
+                       a->scale, nullptr};
+        const bool one_pass = !graphed && attend_prefill_takes(probe, dout);
+        const size_t decode_floats = (size_t)a->n_head * attend_split_count((int)(a->kv_len / a->kv_dim), 1, (int)a->head_dim, (int)group) *
+                                     (a->head_dim + 2);
+        float* sc = be->scratch_f32(one_pass ? decode_floats : (size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2));
         if (!sc) return;
         const int* dyn = be->dyn_slot((int)a->n_pos);
         AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? 0 : (int)a->n_pos, (int)a->head_dim,

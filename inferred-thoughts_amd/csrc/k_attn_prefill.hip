@@ -258,12 +258,20 @@ bool launch_prefill_g(const AttnArgs& a, float* out, hipStream_t s) {
 
 }  // namespace
 
-// false: not a shape this kernel takes (the caller uses the split kernels)
-bool attend_prefill(const AttnArgs& a, float* out, hipStream_t s) {
-    if (a.n_pos_dyn || a.n_q <= 16 || a.n_pos < a.n_q || a.n_head % a.n_head_kv) return false;
+// whether the one-pass kernel takes the shape (then the split kernels' scratch is not needed)
+bool attend_prefill_takes(const AttnArgs& a, const float* out) {
+    if (a.n_pos_dyn || a.n_q <= 16 || a.n_pos < a.n_q || a.n_head_kv <= 0 || a.n_head % a.n_head_kv) return false;
     if (a.kv_dim % 8 || (reinterpret_cast<uintptr_t>(a.k) & 15) || (reinterpret_cast<uintptr_t>(a.v) & 15) ||
         (reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(out) & 15))
         return false;
+    const int G = a.n_head / a.n_head_kv;
+    if (G != 1 && G != 2 && G != 4 && G != 8 && G != 16) return false;
+    return a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256;
+}
+
+// false: not a shape this kernel takes (the caller uses the split kernels)
+bool attend_prefill(const AttnArgs& a, float* out, hipStream_t s) {
+    if (!attend_prefill_takes(a, out)) return false;
     switch (a.head_dim) {
         case 64: return launch_prefill_g<64>(a, out, s);
         case 128: return launch_prefill_g<128>(a, out, s);

@@ -144,6 +144,7 @@ int attend_split_count(int n_pos_max, int n_q, int head_dim, int group);
 void attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);
 // more than 16 queries, fast mode: one pass over the keys on the f16 matrix cores; false when the shape is not taken
 bool attend_prefill(const AttnArgs& a, float* out, hipStream_t s);
+bool attend_prefill_takes(const AttnArgs& a, const float* out);
 // What one decode token's attention needs before it can attend, folded into the tile kernel: the
 // query heads' norm + rotation (every block, for its own heads) and the new position's key
 // (norm + rotation) and value rows, written to the slabs by the block whose tile holds them.
