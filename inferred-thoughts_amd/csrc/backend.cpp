@@ -1130,6 +1130,12 @@ static bool host_ids_in_range(it_hip* be, const it_route* r, uint64_t n_expert, 
     return true;
 }
 
+// Expert-sorted tiles read an expert's rows once for all of its pairs; the per-pair kernels read them once per
+// pair but stream them at several times the rate.  Measured on the 512-expert shape (pairs per expert 0.08 .. 5):
+// the tiles win from about 3.5 pairs per expert on (a batch of 128 tokens at top-10 still takes 653 us per pair
+// against 772 us tiled; at 256 tokens it is 1,180 against 848).
+static bool expert_tiles_pay(uint64_t picks, uint64_t n_expert) { return picks >= 32 && 2 * picks >= 7 * n_expert; }
+
 void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* route, const float* x,
                            uint64_t x_len, float* out, uint64_t out_len) {
     ExpertsView v;
@@ -1153,8 +1159,8 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
-    size_t work_ints;
-    int32_t* work = be->moe_work_for(picks, w->n_expert, &work_ints);
+    size_t work_ints = 0;
+    int32_t* work = expert_tiles_pay(picks, w->n_expert) ? be->moe_work_for(picks, w->n_expert, &work_ints) : nullptr;
     void* fwork = nullptr;
     size_t fwork_bytes = 0;
     if (!be->exact && work && v.fmt == itk::W_NVFP4) {
@@ -1207,8 +1213,8 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     float* dout = be->act_out(out, out_len);
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
-    size_t work_ints;
-    int32_t* work = be->moe_work_for(picks, gate->n_expert, &work_ints);
+    size_t work_ints = 0;
+    int32_t* work = expert_tiles_pay(picks, gate->n_expert) ? be->moe_work_for(picks, gate->n_expert, &work_ints) : nullptr;
     void* fwork = nullptr;
     size_t fwork_bytes = 0;
     if (!be->exact && work && g.fmt == itk::W_NVFP4) {
