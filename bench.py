@@ -43,7 +43,7 @@ def model_path(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--steps", type=int, default=256, help="greedy decode tokens timed (the baseline workload decodes 256)")
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=48, help="48 is the baseline config; fewer only for quick checks")
     ap.add_argument("--prompt", type=int, default=5700)
