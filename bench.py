@@ -65,8 +65,8 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path has no collective; see DESIGN.md "
-              "for how it would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (the path has no collective: experts, layers or heads "
+              "would shard across GPUs, none of which is built); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import inferred_hip as ih
