@@ -251,6 +251,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
                    __builtin_bit_cast(h8, make_uint4(l0.x, l0.y, l1.x, l1.y))};
     };
 
+    const bool live_half = __builtin_amdgcn_readfirstlane(32 * T * th < cnt ? 1 : 0) != 0;
     v16f acc[2][T];
 #pragma unroll
     for (int z = 0; z < 2; z++)
@@ -298,10 +299,12 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
 #pragma unroll
                     for (int q = (g1 - 1) * LPG; q < g1 * LPG; q++) fetch_one(q, s + 1, S + 1, more, j == 0 && more_w);
                     __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of the products they overlap
+                    if (live_half) {   // a wave set whose token groups lie past the tile's pairs only helps with the staging
 #pragma unroll
-                    for (int z = 0; z < 2; z++) {
-                        acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[par][z][n], cur.h, acc[z][tt], 0, 0, 0);
-                        acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[par][z][n], cur.l, acc[z][tt], 0, 0, 0);
+                        for (int z = 0; z < 2; z++) {
+                            acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[par][z][n], cur.h, acc[z][tt], 0, 0, 0);
+                            acc[z][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[par][z][n], cur.l, acc[z][tt], 0, 0, 0);
+                        }
                     }
                     cur = nxt;
                 }
