@@ -186,7 +186,15 @@ __global__ __launch_bounds__(1024) void moe_group_k(const int32_t* __restrict__ 
     const int tid = threadIdx.x;
     cnt[tid] = 0;
     __syncthreads();
-    for (int p = tid; p < n_picks; p += 1024) atomicAdd(&cnt[ids[p]], 1);
+    // eight picks' ids in flight per thread: the walk is bound by the latency of these loads
+    for (int p0 = tid; p0 < n_picks; p0 += 8 * 1024) {
+        int e[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) e[u] = p0 + u * 1024 < n_picks ? ids[p0 + u * 1024] : -1;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (e[u] >= 0) atomicAdd(&cnt[e[u]], 1);
+    }
     __syncthreads();
     // exclusive prefix sums of the pair counts and of the tile counts, all 1024 slots at once
     const int mine = tid < n_expert ? cnt[tid] : 0;
@@ -205,9 +213,13 @@ __global__ __launch_bounds__(1024) void moe_group_k(const int32_t* __restrict__ 
     const int my_off = off[tid] - mine, my_toff = toff[tid] - my_tiles;
     cur[tid] = my_off;
     __syncthreads();
-    for (int p = tid; p < n_picks; p += 1024) {
-        const int slot = atomicAdd(&cur[ids[p]], 1);
-        order[slot] = p;
+    for (int p0 = tid; p0 < n_picks; p0 += 8 * 1024) {
+        int e[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) e[u] = p0 + u * 1024 < n_picks ? ids[p0 + u * 1024] : -1;
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (e[u] >= 0) order[atomicAdd(&cur[e[u]], 1)] = p0 + u * 1024;
     }
     for (int k = 0; k < my_tiles; k++)
         tiles[my_toff + k] = make_int4(tid, my_off + tile_pairs * k, min(tile_pairs, mine - tile_pairs * k), 0);
