@@ -255,6 +255,15 @@ void it_engine_free(it_engine*);
 void it_engine_reset(it_engine*);
 void it_engine_set_trace(it_engine*, it_trace_fn fn, void* user);
 uint64_t it_engine_pos(const it_engine*);
+/* Engine::checkpoint / restore / rewind (src/engine/mod.rs:223-294).  state_sizes: floats of the conv and ssm slabs
+ * (all layers).  checkpoint: brings the device's recurrent state home (read_state per layer), copies both slabs out
+ * and returns the position.  restore: 0 = ok; truncates the sequence to pos, reloads the slabs and has the backend
+ * forget its copies; the next token must be fed from the host (it_engine_forward).  rewind: 1 = done, 0 = refused
+ * (always refused when the model has recurrent layers). */
+void it_engine_state_sizes(const it_engine*, uint64_t out[2]);
+uint64_t it_engine_checkpoint(it_engine*, float* conv_out, float* ssm_out);
+int it_engine_restore(it_engine*, uint64_t pos, const float* conv_in, const float* ssm_in);
+int it_engine_rewind(it_engine*, uint64_t len);
 /* one forward pass at the current position; logits (n_vocab) may be NULL. 0 = ok */
 int it_engine_forward(it_engine*, const uint32_t* tokens, uint64_t n, float* logits);
 /* chunked prefill; logits of the last token (may be NULL) */

@@ -544,6 +544,48 @@ void it_engine_reset(it_engine* e) {
     std::fill(e->ssm.begin(), e->ssm.end(), 0.0f);
     it_hip_zero_state(e->be);
 }
+// Engine::checkpoint / restore / rewind, src/engine/mod.rs:223-294.  The device owns the recurrent state once it has
+// touched it: a checkpoint brings every layer's slabs home through read_state first, a restore writes the host slabs
+// and tells the backend to forget its copies.  The KV needs no stored copy: positions past `pos` are no longer part of
+// the sequence and the next pass overwrites them.
+void it_engine_state_sizes(const it_engine* e, uint64_t out[2]) {
+    out[0] = e->conv.size();
+    out[1] = e->ssm.size();
+}
+uint64_t it_engine_checkpoint(it_engine* e, float* conv_out, float* ssm_out) {
+    const Dims& d = e->m->d;
+    for (uint64_t il = 0; il < d.layers(); il++) {
+        if (!d.recurrent(il)) continue;
+        it_hip_read_state(e->be, e->conv_of(il), d.conv_len());
+        it_hip_read_state(e->be, e->ssm_of(il), d.ssm_len());
+    }
+    if (conv_out) memcpy(conv_out, e->conv.data(), e->conv.size() * sizeof(float));
+    if (ssm_out) memcpy(ssm_out, e->ssm.data(), e->ssm.size() * sizeof(float));
+    return e->len;
+}
+int it_engine_restore(it_engine* e, uint64_t pos, const float* conv_in, const float* ssm_in) {
+    if (pos > e->n_ctx) {
+        e->err = "checkpoint stands at " + std::to_string(pos) + " positions, context is " + std::to_string(e->n_ctx);
+        return -1;
+    }
+    if (!conv_in || !ssm_in) {
+        e->err = "restore: null state";
+        return -2;
+    }
+    e->len = pos;
+    memcpy(e->conv.data(), conv_in, e->conv.size() * sizeof(float));
+    memcpy(e->ssm.data(), ssm_in, e->ssm.size() * sizeof(float));
+    it_hip_forget_state(e->be);  // after both halves
+    return 0;
+}
+int it_engine_rewind(it_engine* e, uint64_t len) {
+    const Dims& d = e->m->d;
+    for (uint64_t il = 0; il < d.layers(); il++)
+        if (d.recurrent(il)) return 0;  // a recurrent state is not a log: it cannot drop tokens
+    if (len > e->len) return 0;
+    e->len = len;
+    return 1;
+}
 void it_engine_set_trace(it_engine* e, it_trace_fn fn, void* user) {
     e->trace = fn;
     e->trace_user = user;

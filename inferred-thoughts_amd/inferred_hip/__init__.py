@@ -96,7 +96,7 @@ it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_bu
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
 it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_hip_zero_state it_hip_mfma_ceiling it_model_open
 it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
-it_engine_set_trace it_engine_pos it_engine_forward it_engine_prefill it_engine_generate
+it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_engine_restore it_engine_rewind it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
 it_engine_v_slab it_synth_write_gguf""".split()
 
@@ -194,6 +194,10 @@ def lib() -> C.CDLL:
         "it_engine_reset": (None, [vp]),
         "it_engine_set_trace": (None, [vp, vp, vp]),
         "it_engine_pos": (u64, [vp]),
+        "it_engine_state_sizes": (None, [vp, vp]),
+        "it_engine_checkpoint": (u64, [vp, vp, vp]),
+        "it_engine_restore": (C.c_int, [vp, u64, vp, vp]),
+        "it_engine_rewind": (C.c_int, [vp, u64]),
         "it_engine_forward": (C.c_int, [vp, vp, u64, vp]),
         "it_engine_prefill": (C.c_int, [vp, vp, u64, vp]),
         "it_engine_generate": (C.c_int64, [vp, vp, u64, u64, vp, vp]),
@@ -480,6 +484,23 @@ class Engine:
     @property
     def pos(self) -> int:
         return int(self.L.it_engine_pos(self.h))
+
+    def checkpoint(self):
+        """(position, conv slab, ssm slab): Engine::checkpoint of the reference."""
+        n = (c_u64 * 2)()
+        self.L.it_engine_state_sizes(self.h, n)
+        conv, ssm = np.empty(int(n[0]), np.float32), np.empty(int(n[1]), np.float32)
+        pos = int(self.L.it_engine_checkpoint(self.h, _p(conv), _p(ssm)))
+        return pos, conv, ssm
+
+    def restore(self, ckpt):
+        pos, conv, ssm = ckpt
+        rc = self.L.it_engine_restore(self.h, pos, _p(conv), _p(ssm))
+        if rc:
+            self._err(rc)
+
+    def rewind(self, n) -> bool:
+        return bool(self.L.it_engine_rewind(self.h, n))
 
     def forward(self, tokens, want_logits=True):
         t = np.ascontiguousarray(tokens, dtype=np.uint32)

@@ -220,3 +220,56 @@ def test_fast_mode_on_baseline_layer_shapes(mid_gguf):
     assert st["captures"] == 1 and st["replays"] >= 5 and st["aborts"] == 0
     assert be.take_error() is None
     he.close(); hm.close(); be.close(); oe.close(); om.close()
+
+
+@pytest.mark.parametrize("exact", [True, False])
+def test_checkpoint_restore_continues_identically(tiny_gguf, exact):
+    """Engine::checkpoint / restore (src/engine/mod.rs:242-294): the recurrent state comes home through read_state,
+    goes back through forget_state, and the sequence continues exactly as it did the first time, whether the passes in
+    between were eager, captured or replayed.  A rewind is refused: the model has recurrent layers.  In exact mode the
+    run is also the oracle's, token for token."""
+    import inferred_hip as ih
+    from oracle import binding as ob
+    be = ih.Hip(exact=exact)
+    m = ih.Model(tiny_gguf); e = ih.Engine(m, be, 128)
+    prompt = prompt_ids(20, seed=11)
+    logits = e.forward(prompt)
+    toks = [int(np.argmax(logits))]
+    for _ in range(5):
+        toks.append(int(np.argmax(e.forward([toks[-1]]))))
+    ck = e.checkpoint()
+    assert ck[0] == 25 and e.pos == 25
+    assert not e.rewind(10)
+    first, first_logits = [], None
+    nxt = toks[-1]
+    for _ in range(8):
+        first_logits = e.forward([nxt]); nxt = int(np.argmax(first_logits)); first.append(nxt)
+    state_after = e.ssm_state(0).copy()
+    e.restore(ck)
+    assert e.pos == 25
+    again, again_logits = [], None
+    nxt = toks[-1]
+    for _ in range(8):
+        again_logits = e.forward([nxt]); nxt = int(np.argmax(again_logits)); again.append(nxt)
+    assert again == first
+    if exact:
+        assert_bits_equal(again_logits, first_logits, "logits after restore")
+        assert_bits_equal(e.ssm_state(0), state_after, "ssm state after restore")
+    else:
+        # the first run went through eager, captured and replayed passes, the second only replays the graph: the fused
+        # and the one-op-per-launch fast kernels differ in their last bits
+        assert _rel(again_logits, first_logits) <= 1e-3
+        assert _rel(e.ssm_state(0), state_after) <= 1e-3
+    # a checkpoint that does not fit the context is refused, and the engine stays where it was
+    with pytest.raises(ih.HipError):
+        e.restore((129, ck[1], ck[2]))
+    assert e.pos == 33
+    if exact:
+        om = ob.Model(tiny_gguf); oe = ob.Engine(om, 128)
+        lo = oe.forward(prompt); ot = [int(np.argmax(lo))]
+        for _ in range(5 + 8):
+            ot.append(int(np.argmax(oe.forward([ot[-1]]))))
+        assert ot == toks + first
+        oe.close(); om.close()
+    assert be.take_error() is None
+    e.close(); m.close(); be.close()
