@@ -101,7 +101,11 @@ IT_DEV void load_w(WChunks<CPL>& t, const uint8_t* q, const uint8_t* s, int n_in
 #pragma unroll
     for (int k = 0; k < CPL; k++) {
         const int c = k * L + sub;
-        t.w[k] = *(const uint4*)(rp + c * 16);
+        {   // read once per token: no reason to keep it in the caches
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+            const v4u nt = __builtin_nontemporal_load((const v4u*)(rp + c * 16));
+            t.w[k] = make_uint4(nt.x, nt.y, nt.z, nt.w);
+        }
         t.sc[k] = FMT == W_Q8_0 ? sp[c >> 1] : sp[c];
     }
 }
