@@ -40,6 +40,59 @@ def model_path(args):
     return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}{'_f32router' if args.router_f32 else ''}.gguf"
 
 
+def config1(ih, ob, seed, tmp_dir):
+    """Config 1 beside the headline run: the tiny all-Q8_0 model, 32 random prompt ids, 64 greedy tokens.  The GPU's
+    exact mode must give the CPU path's token ids; the CPU path is timed on one thread (the reference's bit-exact
+    naive run) and on the spin pool, the GPU in both modes."""
+    path = Path(tmp_dir) / f"inferred_hip_config1_seed{seed}.gguf"
+    ih.synth_write_gguf(path, ih.tiny_config(seed=seed))
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, 4096, 32).astype(np.uint32)
+    out = {"workload": "4 layers (3 GDN + 1 attention), hidden 512, vocab 4096, 16 experts top-4 + shared, all Q8_0; "
+                       "32 prompt ids, 64 greedy tokens"}
+    om = ob.Model(path)
+    cpu_ids = None
+    for name, threads in (("cpu_naive_1_thread", 1), ("cpu_spin", min(16, os.cpu_count() or 1))):
+        ob.lib().orc_set_threads(threads)
+        oe = ob.Engine(om, 128)
+        oe.forward(prompt[:-1])
+        t = time.perf_counter()
+        ids, _ = oe.generate(prompt[-1:], 64)
+        dt = time.perf_counter() - t
+        out[name] = {"decode_tok_s": round(64 / dt, 1), "threads": threads}
+        if cpu_ids is not None:
+            out["cpu_spin"]["ids_equal_naive"] = bool(np.array_equal(cpu_ids, ids))
+        cpu_ids = np.asarray(ids)
+        oe.close()
+    ob.lib().orc_set_threads(1)
+    om.close()
+    for mode, exact in (("gpu_exact", True), ("gpu_fast", False)):
+        be = ih.Hip(exact=exact)
+        model = ih.Model(path)
+        eng = ih.Engine(model, be, 256, 64)
+        eng.generate(prompt, 8)      # upload, buffer sizes, graph capture
+        eng.reset()
+        t = time.perf_counter()
+        eng.prefill(prompt, want_logits=False)
+        be.sync()
+        t_pre = time.perf_counter() - t
+        t = time.perf_counter()
+        ids = eng.decode_greedy(64)   # device-fed: one wait at the end
+        be.sync()
+        dt = time.perf_counter() - t
+        out[mode] = {"decode_tok_s": round(64 / dt, 1), "prefill_32_ms": round(1e3 * t_pre, 3),
+                     "ids_equal_cpu": bool(np.array_equal(cpu_ids, np.asarray(ids)))}
+        err = be.take_error()
+        if err:
+            raise SystemExit(f"device error in the config 1 run: {err}")
+        eng.close(); model.close(); be.close()
+    try:
+        path.unlink()
+    except OSError:
+        pass
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -221,6 +274,7 @@ def main():
                     "bytes_per_launch": dom["bytes"] // dom["launches"]}
 
     cpu = None
+    c1 = None
     if not args.no_cpu:
         from oracle import binding as ob
         cores = min(16, os.cpu_count() or 1)
@@ -237,6 +291,7 @@ def main():
                          f"{n_pre}..{n_pre + n_dec} (context {n_pre + n_dec}, not 5,700), spin-split rows over {cores} threads"}
         oe.close(); om.close()
         ob.lib().orc_set_threads(1)
+        c1 = config1(ih, ob, args.seed, path.parent)
 
     line = {
         "metric": "decode tok/s & % HBM roofline, 35B-A3B-shape NVFP4 synthetic; prefill tok/s",
@@ -261,6 +316,7 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
         "cpu_baseline": cpu,
+        "config1": c1,
         "setup_s": {"synth": round(t_synth, 1), "upload_repack": round(t_upload, 1)},
         "graph": graph_stats, "seam_ops_per_token": launches_per_token,
     }
