@@ -537,6 +537,23 @@ void* it_hip::moe_f16_for(size_t bytes) {
     return moe_f16;
 }
 
+const int32_t* it_hip::zero_ids_for(size_t n) {
+    if (zero_ids_n < n) {
+        need_eager("the one-expert id list has to grow");
+        if (zero_ids) {
+            check(hipStreamSynchronize(stream), "sync before scratch free");
+            (void)hipFree(zero_ids);
+            zero_ids = nullptr;
+            zero_ids_n = 0;
+        }
+        const size_t want = n + n / 2;
+        if (!check(hipMalloc((void**)&zero_ids, want * sizeof(int32_t)), "hipMalloc(one-expert id list)")) return nullptr;
+        if (!check(hipMemset(zero_ids, 0, want * sizeof(int32_t)), "hipMemset(one-expert id list)")) return nullptr;
+        zero_ids_n = want;
+    }
+    return zero_ids;
+}
+
 float* it_hip::gdn_work_for(size_t floats) {
     if (gdn_work_floats < floats) {
         need_eager("delta rule chunk scratch has to grow");
@@ -662,6 +679,7 @@ it_hip::~it_hip() {
     if (attn_scratch) (void)hipFree(attn_scratch);
     if (gdn_work) (void)hipFree(gdn_work);
     if (moe_f16) (void)hipFree(moe_f16);
+    if (zero_ids) (void)hipFree(zero_ids);
     if (moe_work) (void)hipFree(moe_work);
     if (argmax_idx) (void)hipFree(argmax_idx);
     if (argmax_val) (void)hipFree(argmax_val);
@@ -834,12 +852,35 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     if (!dout) return;
     int nt = (int)n;
     const int exact = be->exact;
+    // A dense NVFP4 matrix over a batch (the shared expert of an NVFP4 file during prefill) has no int8 tile kernel
+    // of its own; in fast mode it runs as a batch of one expert on the f16 tile kernel instead of one GEMV per token.
+    ExpertsView ev{};
+    const int32_t* zids = nullptr;
+    int32_t* work = nullptr;
+    void* fwork = nullptr;
+    size_t work_ints = 0, fwork_bytes = 0;
+    bool one_expert = false, grouped = false;
+    if (!exact && v.fmt == W_NVFP4 && n >= 32) {
+        ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
+        ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr;
+        zids = be->zero_ids_for(n);
+        work = be->moe_work_for(n, 1, &work_ints);
+        fwork_bytes = itk::experts_f16_work_bytes(nt, v.n_in);
+        fwork = be->moe_f16_for(fwork_bytes);
+        one_expert = zids && work && fwork && itk::experts_f16_takes(ev, nullptr, nt, aq, dout);
+        if (one_expert) grouped = be->group_cached(nt, 1, 128);
+    }
     it_hip::OpRec rec;
     rec.id = OP_MATMUL; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = dx; rec.p[3] = as; rec.p[4] = aq; rec.p[5] = dout;
     rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = nt;
     be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
                sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout), rec,
-               [=](hipStream_t s) { matmul(v, dx, as, aq, nt, dout, 1.0f, exact, s); });
+               [=](hipStream_t s) {
+                   if (one_expert && experts_gemm_f16(ev, nullptr, zids, nt, 1, 0, as, aq, dout, work, work_ints, fwork,
+                                                      fwork_bytes, grouped, s))
+                       return;
+                   matmul(v, dx, as, aq, nt, dout, 1.0f, exact, s);
+               });
 }
 
 void it_hip_matmul(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, float* out,

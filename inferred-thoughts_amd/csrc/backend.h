@@ -127,6 +127,9 @@ struct it_hip {
     size_t moe_work_ints = 0;
     int32_t* moe_work_for(size_t picks, size_t n_expert, size_t* ints);
     void* moe_f16 = nullptr;     // f16 hi / lo copies of the expert GEMM's activations
+    int32_t* zero_ids = nullptr;  // expert id 0 for every token: a dense NVFP4 matrix run as a one-expert batch
+    size_t zero_ids_n = 0;
+    const int32_t* zero_ids_for(size_t n);
     size_t moe_f16_bytes = 0;
     void* moe_f16_for(size_t bytes);
     float* gdn_work = nullptr;   // T and P matrices of the chunked delta rule

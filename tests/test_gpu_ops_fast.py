@@ -166,6 +166,33 @@ def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
     assert np.all(np.abs(oa - obuf) <= 1e-3 * np.maximum(scale, np.abs(obuf))), (np.abs(oa - obuf) / scale).max()
 
 
+# A dense NVFP4 matrix over a batch (the shared expert of an NVFP4 file during prefill): from 32 tokens on it runs as
+# a one-expert batch on the f16 tile kernel; below that, and in exact mode, one GEMV per token.  Ragged token counts,
+# a row count that is not a multiple of the tile, the baseline's shared-expert shapes at the baseline's prompt length.
+@pytest.mark.parametrize("n_in,n_out,n", [(2048, 512, 31), (2048, 512, 32), (2048, 512, 129), (512, 2048, 300),
+                                          (512, 260, 77), (2048, 512, 5700), (512, 2048, 5700)])
+def test_matmul_nvfp4_batched_fast(hip, orc, n_in, n_out, n):
+    import inferred_hip as ih
+    from oracle import binding as ob
+    fresh(hip)
+    hip.begin_pass(n)
+    r = rng(43)
+    wb = nvfp4_weights(r, n_out, n_in)
+    x = (r.standard_normal(n * n_in) * np.repeat(10.0 ** r.uniform(-2.0, 1.0, n), n_in)).astype(np.float32)
+    a = np.zeros(n * n_out, np.float32); b = np.zeros_like(a)
+    hip.matmul(ih.weights(wb, ih.NVFP4, n_in, n_out), x, a); hip.host_needs(a)
+    orc.matmul(ob.weights(wb, ih.NVFP4, n_in, n_out), x, b)
+    hip.raise_if_error()
+    assert np.isfinite(b).all()
+    scale = np.repeat(np.abs(b.reshape(n, n_out)).max(axis=1) + 1e-30, n_out)
+    assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(scale, np.abs(b))), (np.abs(a - b) / scale).max()
+    # a second call in the same pass (the shared expert's up after its gate) reuses the token grouping
+    a2 = np.zeros_like(a)
+    hip.matmul(ih.weights(wb, ih.NVFP4, n_in, n_out), x, a2); hip.host_needs(a2)
+    hip.raise_if_error()
+    assert np.array_equal(a, a2)
+
+
 # unquantized weights (the router and ssm alpha / beta of real files are F32): wave-split row sums for up to 16
 # tokens, LDS-tiled products for more
 @pytest.mark.parametrize("ty", ["f32", "f16", "bf16"])
