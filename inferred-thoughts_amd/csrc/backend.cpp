@@ -860,7 +860,9 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     void* fwork = nullptr;
     size_t work_ints = 0, fwork_bytes = 0;
     bool one_expert = false, grouped = false;
-    if (!exact && v.fmt == W_NVFP4 && n >= 32) {
+    // (from 513 tokens on: a call costs 55-80 us for the grouping, the f16 split and a latency-bound handful of
+    // tiles, which the GEMVs reach at about 512 tokens)
+    if (!exact && v.fmt == W_NVFP4 && n > 512) {
         ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
         ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr;
         zids = be->zero_ids_for(n);

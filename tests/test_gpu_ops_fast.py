@@ -166,11 +166,11 @@ def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
     assert np.all(np.abs(oa - obuf) <= 1e-3 * np.maximum(scale, np.abs(obuf))), (np.abs(oa - obuf) / scale).max()
 
 
-# A dense NVFP4 matrix over a batch (the shared expert of an NVFP4 file during prefill): from 32 tokens on it runs as
+# A dense NVFP4 matrix over a batch (the shared expert of an NVFP4 file during prefill): from 513 tokens on it runs as
 # a one-expert batch on the f16 tile kernel; below that, and in exact mode, one GEMV per token.  Ragged token counts,
 # a row count that is not a multiple of the tile, the baseline's shared-expert shapes at the baseline's prompt length.
-@pytest.mark.parametrize("n_in,n_out,n", [(2048, 512, 31), (2048, 512, 32), (2048, 512, 129), (512, 2048, 300),
-                                          (512, 260, 77), (2048, 512, 5700), (512, 2048, 5700)])
+@pytest.mark.parametrize("n_in,n_out,n", [(2048, 512, 129), (2048, 512, 512), (2048, 512, 513), (512, 2048, 700),
+                                          (512, 260, 641), (2048, 512, 5700), (512, 2048, 5700)])
 def test_matmul_nvfp4_batched_fast(hip, orc, n_in, n_out, n):
     import inferred_hip as ih
     from oracle import binding as ob
