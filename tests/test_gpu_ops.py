@@ -401,6 +401,36 @@ def test_argmax_ties_to_lower_index(hip, orc):
     assert hip.argmax(x) == 0
 
 
+def test_empty_inputs_launch_nothing(hip, orc):
+    """Zero tokens / zero elements: every op returns without an error and without a launch, as the reference's
+    loops over empty slices do (ops/naive.rs walks `chunks_exact` of empty slices; ops/cuda/ops/mod.rs:91-110 checks
+    shapes before any launch)."""
+    import inferred_hip as ih
+    fresh(hip)
+    r = rng(5)
+    e = np.zeros(0, np.float32)
+    e2 = np.zeros(0, np.float32)
+    before = hip.launch_count()
+    hip.rms_norm(e, np.ones(512, np.float32), 1e-6, e2)
+    hip.rms_norm_heads(e, np.ones(64, np.float32), 64, 1e-6)
+    hip.l2_norm_heads(e, 64, 1e-6)
+    hip.softmax(e, 16)
+    hip.silu_mul(e, e2)
+    hip.sigmoid_mul(e, e2)
+    hip.add_assign(e, e2)
+    hip.scale(e, 2.0)
+    hip.rope_neox(e, 0, 64, 16, 8, 1e6)
+    w = ih.weights(q8_0_weights(orc, r, 32, 512), ih.Q8_0, 512, 32)
+    hip.matmul(w, e, e2)
+    state = np.zeros(1024 * 3, np.float32)
+    s0 = state.copy()
+    hip.ssm_conv(state, e, np.ones(1024 * 4, np.float32), 4, e2)
+    assert hip.take_error() is None
+    assert hip.launch_count() == before
+    hip.host_needs(state)
+    assert np.array_equal(state, s0)
+
+
 def test_shape_errors_are_sticky_not_fatal(hip):
     """A bad shape records an error and launches nothing (ops/cuda/ops/mod.rs:91-110)."""
     x = np.zeros(100, np.float32); w = np.zeros(64, np.float32); out = np.zeros(100, np.float32)
