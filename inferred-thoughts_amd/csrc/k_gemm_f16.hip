@@ -282,12 +282,12 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
             const bool more = j < 3 || more_w;
             GEMM_STAMP(0);
             GEMM_STAMP(1);
-            if (more) read_nib(j < 3 ? wb : wb ^ 1, j < 3 ? j + 1 : 0);
+            if (more && live_half) read_nib(j < 3 ? wb : wb ^ 1, j < 3 ? j + 1 : 0);
             Tok cur = read_tok(par, 0, 0);
 #pragma unroll
             for (int n = 0; n < 4; n++) {
                 // one fragment pair of the next slab between the MFMA groups of this one
-                if (more) {
+                if (more && live_half) {   // a wave set without pairs expands nothing: its SIMD belongs to the wave that has them
 #pragma unroll
                     for (int z = 0; z < 2; z++) af[par ^ 1][z][n] = expand(z, n);
                 }
