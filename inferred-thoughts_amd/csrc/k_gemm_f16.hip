@@ -91,8 +91,9 @@ __global__ __launch_bounds__(256) void acts_split_f16_k(const int8_t* __restrict
 
 // four nibbles (one per byte, 0..15) -> four f16 weights (two dwords), scaled by the sub-block scale
 __device__ __forceinline__ void fp4x4_to_f16x4(uint32_t v, h2 scale, h2* a, h2* b) {
-    // f16 high bytes of the doubled e2m1 magnitudes 0 1 2 3 4 6 8 12; the low bytes are zero
-    const uint32_t mag = __builtin_amdgcn_perm(0x4a484644u, 0x42403c00u, v & 0x07070707u);
+    // f16 high bytes of 128 x the doubled e2m1 magnitudes 0 1 2 3 4 6 8 12 (the low bytes are zero): the 128 pays
+    // for the 2^-8 the scale carries (see expand) and the halving that goes with the doubled magnitudes
+    const uint32_t mag = __builtin_amdgcn_perm(0x66646260u, 0x5e5c5800u, v & 0x07070707u);
     const uint32_t hb = mag | ((v & 0x08080808u) << 4);
     const uint32_t d0 = __builtin_amdgcn_perm(hb, hb, 0x010c000cu);   // bytes 0, hb.0, 0, hb.1
     const uint32_t d1 = __builtin_amdgcn_perm(hb, hb, 0x030c020cu);   // bytes 0, hb.2, 0, hb.3
@@ -230,7 +231,12 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     };
     // fragment n of set z from ra / rs
     auto expand = [&](int z, int n) __attribute__((always_inline)) -> h8 {
-        const _Float16 sv = (_Float16)it_ue4m3_to_f32(n < 2 ? (rs[z] & 0xffu) : (rs[z] >> 8));
+        // An e4m3 code shifted into an f16's exponent and mantissa fields IS the scale times 2^-8, subnormal codes
+        // included (4 exponent bits with bias 7 against 5 with bias 15; f16 subnormals are computed with, not flushed):
+        // no conversion arithmetic.  The magnitudes carry the 2^7 back; code 0x7f (not a number) counts as zero, as
+        // in the CPU path.
+        const uint32_t em = (n < 2 ? rs[z] : rs[z] >> 8) & 0x7fu;
+        const _Float16 sv = __builtin_bit_cast(_Float16, (uint16_t)(em == 0x7fu ? 0u : em << 7));
         const h2 sc = h2{sv, sv};
         const uint32_t wd = n == 0 ? ra[z].x : n == 1 ? ra[z].y : n == 2 ? ra[z].z : ra[z].w;
         h2 a0, a1, a2, a3;

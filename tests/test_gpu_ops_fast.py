@@ -193,6 +193,37 @@ def test_matmul_nvfp4_batched_fast(hip, orc, n_in, n_out, n):
     assert np.array_equal(a, a2)
 
 
+def test_nvfp4_tiles_keep_subnormal_and_extreme_scales(hip, orc):
+    """The f16 tile kernel takes an e4m3 scale code straight into an f16's bit fields (times 2^-8, the magnitudes
+    carry the factor back): the subnormal codes 1..7, the largest code 0x7e and the not-a-number code 0x7f (zero in
+    the CPU path) must come out as the CPU path has them."""
+    import inferred_hip as ih
+    from oracle import binding as ob
+    fresh(hip)
+    n_in, n_out, n = 512, 256, 600
+    hip.begin_pass(n)
+    r = rng(44)
+    wb = nvfp4_weights(r, n_out, n_in).reshape(-1, 36)
+    kinds = r.integers(0, 4, wb.shape[0])
+    wb[kinds == 0, :4] = r.integers(1, 8, (int((kinds == 0).sum()), 4), dtype=np.uint8)        # subnormal scales
+    wb[kinds == 1, :4] = 0x7e                                                                   # 448
+    wb[kinds == 2, :4] = r.choice(np.array([0x7f, 0x00, 0x08], np.uint8), (int((kinds == 2).sum()), 4))
+    wb = wb.reshape(-1).copy()
+    # every row of one run is made of subnormal-scale blocks only: nothing larger hides a flushed scale
+    sub = nvfp4_weights(r, n_out, n_in).reshape(-1, 36)
+    sub[:, :4] = r.integers(1, 8, (sub.shape[0], 4), dtype=np.uint8)
+    sub = sub.reshape(-1).copy()
+    x = r.standard_normal(n * n_in).astype(np.float32)
+    for w_bytes in (wb, sub):
+        a = np.zeros(n * n_out, np.float32); b = np.zeros_like(a)
+        hip.matmul(ih.weights(w_bytes, ih.NVFP4, n_in, n_out), x, a); hip.host_needs(a)
+        orc.matmul(ob.weights(w_bytes, ih.NVFP4, n_in, n_out), x, b)
+        hip.raise_if_error()
+        assert np.isfinite(b).all() and np.abs(b).max() > 0
+        scale = np.repeat(np.abs(b.reshape(n, n_out)).max(axis=1) + 1e-30, n_out)
+        assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(scale, np.abs(b))), (np.abs(a - b) / scale).max()
+
+
 # unquantized weights (the router and ssm alpha / beta of real files are F32): wave-split row sums for up to 16
 # tokens, LDS-tiled products for more
 @pytest.mark.parametrize("ty", ["f32", "f16", "bf16"])
