@@ -18,7 +18,8 @@
 // the owning lane's registers (a lane owns 16 contiguous bytes of a row per 64-wide k slab: the
 // k order inside an MFMA is free once the scales are folded in) and are expanded there: a byte
 // permute yields the f16 high bytes of four magnitudes, the sign bit is or-ed in, two more
-// permutes interleave zero low bytes, and v_pk_mul_f16 applies the sub-block scale.
+// permutes interleave zero low bytes, and v_pk_mul_f16 applies the sub-block scale (the scale code's bits moved
+// into an f16's fields are the scale times 2^-8; the magnitudes are stored times 2^7, which also takes the halving).
 //
 // MFMA operand layout (32x32x16, f16): lane l supplies 8 k values of row (l % 32), k group
 // l / 32, for both A (weight rows) and B (tokens); it receives D for token l % 32 and weight
