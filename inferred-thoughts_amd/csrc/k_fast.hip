@@ -244,10 +244,11 @@ IT_DEV int fast_mat_index(const FusedGemvP& p, int g) {
     return mi;
 }
 
-template <int FMT, int CPL, int L>
+// ONE: one step per group (a matrix of few rows spreads over more blocks, i.e. more CUs pull its weights)
+template <int FMT, int CPL, int L, bool ONE = false>
 __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     constexpr int P = 64 / L;
-    constexpr int RB = CPL >= 4 ? 1 : 4 / CPL;  // steps per group: four chunk loads per lane in flight
+    constexpr int RB = ONE || CPL >= 4 ? 1 : 4 / CPL;  // steps per group: four chunk loads per lane in flight
     constexpr int RG = RB * P;
     __shared__ __align__(16) int8_t xq[FT * 8];
     __shared__ float xs[FT * 8 / 32];
@@ -398,11 +399,22 @@ static bool fused_gemv_fast_prepare(FusedGemvP& p, Geo* geo, int* fmt_out, int* 
         if (!aligned16(p.m[i].q) || (reinterpret_cast<uintptr_t>(p.m[i].s) & 1)) return false;
         if (p.m[i].epi == 1 && !aligned16(p.conv_w)) return false;
     }
-    const int P = 64 / g.l, RB = g.cpl >= 4 ? 1 : 4 / g.cpl, RG = RB * P;
+    const int P = 64 / g.l;
+    int RB = g.cpl >= 4 ? 1 : 4 / g.cpl, RG = RB * P;
     int groups = 0;
-    for (int i = 0; i < nq; i++) {
-        p.m[i].group0 = groups;
-        groups += (p.m[i].n_out + RG - 1) / RG;
+    auto count_groups = [&]() {
+        groups = 0;
+        for (int i = 0; i < nq; i++) {
+            p.m[i].group0 = groups;
+            groups += (p.m[i].n_out + RG - 1) / RG;
+        }
+    };
+    count_groups();
+    // few rows (the router's 513): one step per group, so that twice or four times as many CUs pull the weights
+    if (RB > 1 && (groups + FW - 1) / FW < 128) {
+        RB = 1;
+        RG = P;
+        count_groups();
     }
     p.total_groups = groups;
     p.rows_per_wave = RG;
@@ -436,7 +448,12 @@ bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
     Geo g;
     int fmt, blocks;
     if (!fused_gemv_fast_prepare(p, &g, &fmt, &blocks)) return false;
-#define IT_LAUNCH(F, C, LL) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL>), dim3(blocks), dim3(FT), 0, s, p)
+    const bool one = p.rows_per_wave == 64 / g.l && g.cpl < 4;
+#define IT_LAUNCH(F, C, LL)                                                                          \
+    do {                                                                                             \
+        if (one) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, true>), dim3(blocks), dim3(FT), 0, s, p); \
+        else hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL>), dim3(blocks), dim3(FT), 0, s, p);      \
+    } while (0)
     if (fmt == W_Q8_0) {
         if (g.l == 64 && g.cpl == 1) IT_LAUNCH(W_Q8_0, 1, 64);
         else if (g.l == 64 && g.cpl == 2) IT_LAUNCH(W_Q8_0, 2, 64);
