@@ -509,21 +509,23 @@ __global__ __launch_bounds__(64) void gdn_rows_exact_k(GdnCoreP p) {
     p.core[h * dv + j] = o;
 }
 
-// Fast form: 8 lanes share a row (each a contiguous DK/8 slice, so a row is one 512-byte
-// coalesced read), partial dots meet through xor shuffles.  Reordered sums: 1e-3 class.
-template <int DK>
+// Fast form: LPR lanes share a row (each a contiguous DK/LPR slice, so a row is one 512-byte coalesced read), partial
+// dots meet through DPP moves.  Reordered sums: 1e-3 class.  LPR = 8 gives 32 rows per block, LPR = 16 gives 16: the
+// launcher takes the one that puts a block on every CU (32 value heads of 128 rows: 256 blocks with LPR = 16).
+template <int DK, int LPR>
 __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
-    constexpr int SEG = DK / 8;
+    constexpr int SEG = DK / LPR;
+    constexpr int ROWS = 256 / LPR;
     __shared__ __align__(16) float kq[2 * DK];
     __shared__ double red[5];
-    const int tid = threadIdx.x, seg = tid & 7;
+    const int tid = threadIdx.x, seg = tid % LPR;
     const int dv = DK;
-    const int bph = dv / 32;
+    const int bph = dv / ROWS;
     const int h = blockIdx.x / bph, jb = blockIdx.x % bph, kh = h % p.n_k_heads;
     const int key_dim = p.n_k_heads * DK;
     // key / query element first, then the state rows: both are in flight while k and q are normalized
     const float kqv = tid < 2 * DK ? p.conv[(tid >= DK ? 0 : key_dim) + kh * DK + (tid >= DK ? tid - DK : tid)] : 0.0f;
-    const int j = jb * 32 + (tid >> 3);
+    const int j = jb * ROWS + tid / LPR;
     float* S = p.state + ((int64_t)h * dv + j) * DK + seg * SEG;
     float4 st[SEG / 4];
 #pragma unroll
@@ -545,7 +547,7 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
         row[i] *= g;
         pred += row[i] * kk[i];
     }
-    pred = sum8_lanes(pred);
+    pred = group_sum<LPR>(pred);
     float delta = beta * (v - pred);
     float o = 0.0f;
 #pragma unroll
@@ -553,7 +555,7 @@ __global__ __launch_bounds__(256) void gdn_rows_fast_k(GdnCoreP p) {
         row[i] += kk[i] * delta;
         o += row[i] * (qq[i] * p.q_scale);
     }
-    o = sum8_lanes(o);
+    o = group_sum<LPR>(o);
 #pragma unroll
     for (int i = 0; i < SEG / 4; i++)
         ((float4*)S)[i] = make_float4(row[4 * i], row[4 * i + 1], row[4 * i + 2], row[4 * i + 3]);
@@ -566,9 +568,13 @@ void gdn_core(const GdnCoreP& p, int dk, hipStream_t s) {
         if (dk == 64) hipLaunchKernelGGL(gdn_rows_exact_k<64>, dim3(blocks), dim3(64), 0, s, p);
         else if (dk == 128) hipLaunchKernelGGL(gdn_rows_exact_k<128>, dim3(blocks), dim3(64), 0, s, p);
     } else {
-        int blocks = p.n_v_heads * (dk / 32);
-        if (dk == 64) hipLaunchKernelGGL(gdn_rows_fast_k<64>, dim3(blocks), dim3(256), 0, s, p);
-        else if (dk == 128) hipLaunchKernelGGL(gdn_rows_fast_k<128>, dim3(blocks), dim3(256), 0, s, p);
+        // sixteen lanes a row while that still leaves at most a block per CU (256 on this chip), eight otherwise
+        const bool wide = p.n_v_heads * (dk / 16) <= 256;
+        const int blocks = p.n_v_heads * (dk / (wide ? 16 : 32));
+        if (dk == 64 && wide) hipLaunchKernelGGL((gdn_rows_fast_k<64, 16>), dim3(blocks), dim3(256), 0, s, p);
+        else if (dk == 64) hipLaunchKernelGGL((gdn_rows_fast_k<64, 8>), dim3(blocks), dim3(256), 0, s, p);
+        else if (dk == 128 && wide) hipLaunchKernelGGL((gdn_rows_fast_k<128, 16>), dim3(blocks), dim3(256), 0, s, p);
+        else if (dk == 128) hipLaunchKernelGGL((gdn_rows_fast_k<128, 8>), dim3(blocks), dim3(256), 0, s, p);
     }
 }
 
