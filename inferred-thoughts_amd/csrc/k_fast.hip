@@ -782,14 +782,15 @@ namespace {
 
 // ------------------------------------------------------------------ moe_down, fast
 // x[j] += sum_y w_y * scale2_y * (down_y[j] . g_y) + sigmoid(logit) * (shared_down[j] . g_sh)
-// A wave step covers P = 64 / L output rows.  Two waves share a row group: the even picks go
-// to one, the odd picks and the shared expert to the other, and the two partial sums meet in
-// LDS in a fixed order.  Loads are issued in the order they can be consumed: the small
-// intermediates first (they are quantized while the weights are still on their way), then
-// every weight chunk of the wave and the residual it will add to.
-constexpr int DT = 256, DW = DT / 64;
-constexpr int MAXU = 16, HALFU = MAXU / 2;
+// Loads are issued in the order they can be consumed: the small intermediates first (they are quantized while the
+// weights are still on their way), then every weight chunk of the wave and the residual it will add to.
+constexpr int DT = 512, DW = DT / 64;
+constexpr int MAXU = 16, QUARTU = MAXU / 4;
 
+// A wave step covers P = 64 / L output rows.  Four waves share a row group: wave q of the four takes the picks
+// y = q, q + 4, ..., the last of them the shared expert as well, and the four partial sums meet in LDS in a fixed
+// order.  Eight waves a block (two row groups): the block-wide quantization of the intermediates is three quads a
+// thread, and two waves a SIMD cover each other's waits.
 template <int EF, int ECPL, int L, int SF, int SCPL>
 __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -799,18 +800,18 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     int8_t* xq = (int8_t*)smem;
     float* xs = (float*)(smem + ((total + 15) & ~15));
     __shared__ float coef[MAXU];
-    __shared__ float partial[DW / 2][64];
+    __shared__ float partial[DW / 4][3][64];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int half = wave & 1, group = wave >> 1;
+    const int quarter = wave & 3, group = wave >> 2;
     const int sub = lane % L, rsub = lane / L;
-    const int row = (blockIdx.x * (DW / 2) + group) * P + rsub;
+    const int row = (blockIdx.x * (DW / 4) + group) * P + rsub;
     const bool live = row < p.n_out;
     IT_STAMP(0);
 
-    // the intermediates: up to six quads per thread (24 floats) cover 6144 floats per block
+    // the intermediates: up to three quads per thread (12 floats) cover 6144 floats per block
     const int nq = total >> 2, nq_routed = (NU * n_in) >> 2;
-    constexpr int QR = 6;
+    constexpr int QR = 3;
     float4 v[QR];
 #pragma unroll
     for (int k = 0; k < QR; k++) {
@@ -818,19 +819,19 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
         v[k] = qi >= nq ? make_float4(0.f, 0.f, 0.f, 0.f)
                         : qi < nq_routed ? ((const float4*)p.g_all)[qi] : ((const float4*)p.g_shared)[qi - nq_routed];
     }
-    // this wave's picks: y = 2 * k + half
-    WChunks<ECPL> t[HALFU];
+    // this wave's picks: y = 4 * k + quarter
+    WChunks<ECPL> t[QUARTU];
     WChunks<SCPL> tsh;
 #pragma unroll
-    for (int k = 0; k < HALFU; k++) {
-        const int y = 2 * k + half;
+    for (int k = 0; k < QUARTU; k++) {
+        const int y = 4 * k + quarter;
         if (y < NU) {
             const int64_t e = p.route_ids[y];
             load_w<EF, ECPL, L>(t[k], p.q + e * p.q_stride, p.s + e * p.s_stride, n_in, row, sub, live);
         }
     }
-    if (half) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
-    const float x_old = (!half && sub == L - 1 && live) ? p.x[row] : 0.0f;
+    if (quarter == 3) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
+    const float x_old = (!quarter && sub == L - 1 && live) ? p.x[row] : 0.0f;
     if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
     const float gate = fx_sigmoid(p.logit[0]);
     IT_STAMP(1);
@@ -843,25 +844,26 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
 
     float acc = 0.0f;
 #pragma unroll
-    for (int k = 0; k < HALFU; k++) {
-        const int y = 2 * k + half;
+    for (int k = 0; k < QUARTU; k++) {
+        const int y = 4 * k + quarter;
         if (y < NU) {
             XChunks<EF, ECPL> x;
             load_x<EF, ECPL, L>(x, xq + y * n_in, xs + y * (n_in >> 5), sub);
             acc += coef[y] * dot_chunks<EF, ECPL>(t[k], x);
         }
     }
-    if (half) {
+    if (quarter == 3) {
         XChunks<SF, SCPL> x;
         load_x<SF, SCPL, L>(x, xq + NU * n_in, xs + NU * (n_in >> 5), sub);
         acc += gate * dot_chunks<SF, SCPL>(tsh, x);
     }
     IT_STAMP(4);
     acc = reduce_lanes<L>(acc);
-    if (half) partial[group][lane] = acc;
+    if (quarter) partial[group][quarter - 1][lane] = acc;
     __syncthreads();
     IT_STAMP(5);
-    if (!half && sub == L - 1 && live) p.x[row] = x_old + (acc + partial[group][lane]);
+    if (!quarter && sub == L - 1 && live)
+        p.x[row] = x_old + ((acc + partial[group][0][lane]) + (partial[group][1][lane] + partial[group][2][lane]));
     IT_STAMP(6);
 }
 
@@ -883,9 +885,9 @@ bool moe_down_fast(MoeDownP p, hipStream_t s) {
         return false;
     const int total = p.n_used * p.n_in + p.sh_n_in;
     const size_t lds = (size_t)((total + 15) & ~15) + (size_t)(total / 32) * 4;
-    if (lds > 60 * 1024 || total > 6 * DT * 4) return false;
+    if (lds > 60 * 1024 || total > 3 * DT * 4) return false;
     const int P = 64 / L;
-    const int blocks = (p.n_out + (DW / 2) * P - 1) / ((DW / 2) * P);
+    const int blocks = (p.n_out + (DW / 4) * P - 1) / ((DW / 4) * P);
 #define IT_LAUNCH(EF, LL, SF, SC) hipLaunchKernelGGL((moe_down_fast_k<EF, 1, LL, SF, SC>), dim3(blocks), dim3(DT), lds, s, p)
 #define IT_BY_L(EF, SF, SC)                      \
     do {                                         \
