@@ -234,6 +234,23 @@ void it_hip_zero_state(it_hip*);
  * (2 per multiply-accumulate).  0 = ok, 1 = bad argument, 2 = device error */
 int it_hip_mfma_ceiling(it_hip*, int kind, int iters, double* ops_per_s);
 
+/* ---- one entry point that allocates nothing ----
+ * No counterpart in the reference (its device backend sizes its pools with the driver's allocator as it goes,
+ * src/ops/cuda/mod.rs:1011-1158).  For callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The computation is it_hip_attend's split-K form (fast mode) for at most 16
+ * query rows: same kernels, same split count, bit-identical output.  Differences from it_hip_attend:
+ *  - every pointer in `a`, and `out`, is a DEVICE pointer the caller owns (nothing is mirrored or copied);
+ *  - `stream` is a hipStream_t (NULL = the null stream); the call only enqueues work on it;
+ *  - the split-K partial results live in a fixed array of IT_HIP_NOALLOC_SCRATCH_BYTES inside the library's code
+ *    object, one copy per GPU, held until the process ends and shared by every call on that GPU: calls that overlap
+ *    on one GPU race.  A problem whose partials (n_q * n_head * n_split * (head_dim + 2) floats; n_split =
+ *    ceil(n_pos / 64) capped at 256 for head_dim 64, 128 and 256, ceil(n_pos / 128) otherwise) do not fit is refused;
+ *  - it calls no hipMalloc, hipFree or allocating library routine, and needs no it_hip handle.
+ * Returns 0 = enqueued, 1 = bad argument, 2 = too large for the fixed scratch, 3 = device error; the message goes to
+ * err. */
+#define IT_HIP_NOALLOC_SCRATCH_BYTES (8ull << 20)
+int it_hip_attend_noalloc(const it_attn* a, float* out, uint64_t out_len, void* stream, char* err, size_t err_len);
+
 /* ---- model + engine: the host side of the loop over this backend ----------
  * Qwen35::load / forward (src/model/qwen35.rs:755-858, 956-1127) and
  * Engine::{new, prefill, decode, generate, reset} (src/engine/mod.rs:147-437). */

@@ -697,6 +697,8 @@ it_hip::~it_hip() {
 }
 
 // =================================================================== C ABI
+extern "C" int it_hip_noalloc_setup(void);  // k_noalloc.hip
+
 extern "C" {
 
 it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
@@ -732,6 +734,11 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
         return bad("cannot allocate the position staging buffers");
     }
     be->dyn_host = be->dyn_hosts[0];
+    // the allocation-free attention entry point looks up its fixed scratch once per device, here
+    if (it_hip_noalloc_setup() != 0) {
+        delete be;
+        return bad("cannot resolve the fixed attention scratch on this device");
+    }
     if (hipMalloc((void**)&be->route_counter, sizeof(unsigned)) != hipSuccess ||
         hipMemset(be->route_counter, 0, sizeof(unsigned)) != hipSuccess) {
         delete be;

@@ -98,7 +98,7 @@ it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sy
 it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_engine_restore it_engine_rewind it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
-it_engine_v_slab it_synth_write_gguf""".split()
+it_engine_v_slab it_synth_write_gguf it_hip_attend_noalloc""".split()
 
 _lib = None
 
@@ -208,6 +208,7 @@ def lib() -> C.CDLL:
         "it_engine_k_slab": (vp, [vp, u64, vp]),
         "it_engine_v_slab": (vp, [vp, u64, vp]),
         "it_synth_write_gguf": (C.c_int, [C.c_char_p, vp, C.c_char_p, C.c_size_t]),
+        "it_hip_attend_noalloc": (C.c_int, [vp, vp, u64, vp, C.c_char_p, C.c_size_t]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -236,6 +237,20 @@ def experts(data: np.ndarray, ty: int, n_in: int, n_out: int, n_expert: int, sca
 
 class HipError(RuntimeError):
     pass
+
+
+NOALLOC_SCRATCH_BYTES = 8 << 20
+
+
+def attend_noalloc(q_ptr: int, q_len: int, k_ptr: int, v_ptr: int, kv_len: int, kv_dim: int, n_pos: int,
+                   head_dim: int, n_head: int, n_head_kv: int, scale: float, out_ptr: int, out_len: int,
+                   stream: int = 0):
+    """it_hip_attend_noalloc over DEVICE addresses (q, out: f32; k, v: f16 bits).  Returns (code, message):
+    0 = enqueued on `stream`, 1 = bad argument, 2 = too large for the fixed scratch, 3 = device error."""
+    a = Attn(q_ptr, q_len, k_ptr, v_ptr, kv_len, kv_dim, n_pos, head_dim, n_head, n_head_kv, scale)
+    err = C.create_string_buffer(512)
+    rc = lib().it_hip_attend_noalloc(C.addressof(a), out_ptr, out_len, stream, err, 512)
+    return int(rc), err.value.decode()
 
 
 class Hip:

@@ -49,3 +49,57 @@ def assert_bits_equal(a, b, what=""):
         bad = np.flatnonzero(a != b)
         raise AssertionError(f"{what}: {bad.size} of {a.size} values differ bitwise; first at {bad[0]}: "
                              f"{a.view(np.float32)[bad[0]]!r} vs {b.view(np.float32)[bad[0]]!r}")
+
+
+class Hiprt:
+    """The few HIP runtime calls a test needs to hold device memory of its own (hipMalloc, copies, free), through
+    ctypes on the runtime the product library is linked against, so a test of an entry point that takes device
+    pointers needs nothing but the library under test."""
+
+    def __init__(self):
+        import ctypes as C
+        import inferred_hip as ih
+        ih.lib()                                  # maps libamdhip64 into the process
+        self.C = C
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        self.rt.hipFree.argtypes = [C.c_void_p]
+        self.rt.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        self.rt.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        self.rt.hipGetErrorString.restype = C.c_char_p
+        self.rt.hipGetErrorString.argtypes = [C.c_int]
+        self.held = []
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what}: {self.rt.hipGetErrorString(rc).decode()}")
+
+    def last_error(self):
+        rc = self.rt.hipGetLastError()
+        return None if rc == 0 else self.rt.hipGetErrorString(rc).decode()
+
+    def upload(self, a):
+        """Device copy of a contiguous numpy array; returns the device address."""
+        p = self.C.c_void_p()
+        self.check(self.rt.hipMalloc(self.C.byref(p), max(a.nbytes, 16)), "hipMalloc")
+        self.held.append(p.value)
+        self.check(self.rt.hipMemcpy(p, a.ctypes.data, a.nbytes, 1), "hipMemcpy(host to device)")
+        return p.value
+
+    def filled(self, nbytes, byte):
+        p = self.C.c_void_p()
+        self.check(self.rt.hipMalloc(self.C.byref(p), max(nbytes, 16)), "hipMalloc")
+        self.held.append(p.value)
+        self.check(self.rt.hipMemset(p, byte, nbytes), "hipMemset")
+        return p.value
+
+    def download(self, dev, like):
+        out = np.empty_like(like)
+        self.check(self.rt.hipDeviceSynchronize(), "hipDeviceSynchronize")
+        self.check(self.rt.hipMemcpy(out.ctypes.data, dev, out.nbytes, 2), "hipMemcpy(device to host)")
+        return out
+
+    def free_all(self):
+        for p in self.held:
+            self.rt.hipFree(p)
+        self.held = []
