@@ -16,8 +16,8 @@
 // final ulp), so the oracle fixes one definition: the table-driven double
 // precision algorithm published with glibc >= 2.27 (sysdeps/ieee754/flt-32/
 // e_expf.c, e_logf.c; ARM optimized-routines math/expf.c, logf.c), evaluated
-// without contraction.  tests/test_oracle_math.py measures how often it differs
-// from this machine's libm.
+// without contraction.  tests/test_oracle_golden.py (test_expf_logf_against_libm_and_float64)
+// measures how often it differs from this machine's libm.
 #pragma once
 #include <stdint.h>
 #include <string.h>

@@ -338,3 +338,114 @@ def test_threaded_backend_is_bit_identical(orc):
         orc.matmul(W, x, o2); orc.attend(q, k, v, 32, 100, 16, 4, 2, 0.25, a2)
         assert np.array_equal(o1, o2) and np.array_equal(a1, a2)
     orc.set_threads(1)
+
+
+# ---- hand values for the small ops: each case is built so that a swapped operand, a dropped offset or a
+# ---- wrong stride gives a different number
+
+def test_silu_mul_and_sigmoid_mul_operand_roles(orc):
+    ln3 = np.float32(np.log(3.0))
+    # silu_mul(gate, up): gate <- gate / (1 + e^-gate) * up (src/ops/naive.rs:317-327; sigmoid(ln 3) = 3/4)
+    gate = np.array([ln3, 0.0, -ln3, 2.0], np.float32); up = np.array([2.0, 5.0, 4.0, 0.0], np.float32)
+    g = gate.copy(); u0 = up.copy()
+    orc.silu_mul(g, up)
+    assert np.allclose(g, [ln3 * 0.75 * 2.0, 0.0, -ln3 * 0.25 * 4.0, 0.0], rtol=1e-6, atol=0)
+    assert np.array_equal(up, u0)                       # `up` is read only
+    # with the roles swapped element 0 would be 2 * sigmoid(2) * ln 3 = 1.935, not 1.648
+    assert abs(g[0] - 1.6479184) < 1e-6
+    # sigmoid_mul(x, g): x <- x * sigmoid(g) (naive.rs:339-345)
+    x = np.array([8.0, -4.0, 1.0], np.float32); gg = np.array([ln3, -ln3, 0.0], np.float32)
+    g0 = gg.copy()
+    orc.sigmoid_mul(x, gg)
+    assert np.allclose(x, [6.0, -1.0, 0.5], rtol=1e-6) and np.array_equal(gg, g0)
+
+
+def test_scale_and_the_add_scaled_family(orc):
+    a = np.array([1.0, 2.0, 3.0], np.float32)
+    orc.scale(a, 0.5)
+    assert np.array_equal(a, [0.5, 1.0, 1.5])
+    b = np.array([10.0, 20.0, 30.0], np.float32)
+    orc.add_scaled(a, b, 0.25)                          # a += b * s (ops/mod.rs:1265-1270)
+    assert np.array_equal(a, [3.0, 6.0, 9.0]) and np.array_equal(b, [10.0, 20.0, 30.0])
+    # add_scaled_rows WRITES acc = sum_e scales[e] * rows[e * n + j] (ops/mod.rs:1228-1238): the old contents go
+    acc = np.array([100.0, 100.0], np.float32)
+    rows = np.array([1.0, 2.0, 10.0, 20.0, 100.0, 200.0], np.float32)     # three rows of two
+    orc.add_scaled_rows(acc, rows, np.array([1.0, 0.5, 0.25], np.float32))
+    assert np.array_equal(acc, [1.0 + 5.0 + 25.0, 2.0 + 10.0 + 50.0])
+    # add_scaled_sigmoid: acc += b * sigmoid(logit[0]) (ops/mod.rs:1250-1253); only the first logit counts
+    acc = np.array([1.0, 1.0], np.float32)
+    orc.add_scaled_sigmoid(acc, np.array([4.0, 8.0], np.float32), np.array([np.log(3.0), -30.0], np.float32))
+    assert np.allclose(acc, [4.0, 7.0], rtol=1e-6)
+    a = np.array([1.0, 2.0], np.float32)
+    orc.add_assign(a, np.array([0.5, -2.0], np.float32))
+    assert np.array_equal(a, [1.5, 0.0])
+
+
+def test_gather_and_scatter_chunks_with_offset_and_stride(orc):
+    src = np.arange(20, dtype=np.float32)
+    out = np.full(6, -1, np.float32)
+    orc.gather_chunks(src, 2, 7, 3, out)                # chunk c reads src[c * 7 + 3 ..][:2] (naive.rs:220-232)
+    assert np.array_equal(out, [3, 4, 10, 11, 17, 18])
+    # the attention split: q and gate interleaved per head with stride 2 * head_dim (qwen35.rs:1176-1177)
+    qg = np.arange(16, dtype=np.float32)                # two heads of [q q q q | g g g g]
+    q = np.zeros(8, np.float32); g = np.zeros(8, np.float32)
+    orc.gather_chunks(qg, 4, 8, 0, q); orc.gather_chunks(qg, 4, 8, 4, g)
+    assert np.array_equal(q, [0, 1, 2, 3, 8, 9, 10, 11]) and np.array_equal(g, [4, 5, 6, 7, 12, 13, 14, 15])
+    dst = np.full(12, -1, np.float32)
+    orc.scatter_chunks(np.array([1, 2, 3, 4], np.float32), 2, 5, 1, dst)  # block i -> dst[1 + i * 5 ..][:2]
+    assert np.array_equal(dst, [-1, 1, 2, -1, -1, -1, 3, 4, -1, -1, -1, -1])
+
+
+def test_rms_norm_heads_normalizes_each_head_by_its_own_mean_square(orc):
+    # three heads of four with very different magnitudes and a per-dimension weight: a kernel that normalized the
+    # whole row, or indexed the weight by the flat position, gives other numbers
+    w = np.array([1.0, 2.0, 0.5, -1.0], np.float32)
+    x = np.array([3, 4, 0, 0,   30, 40, 0, 0,   0, 0, 0, 6], np.float32)
+    orc.rms_norm_heads(x, w, 4, 0.0)
+    # head 0: mean square 25/4 -> scale 0.4; head 1: 2500/4 -> 0.04; head 2: 36/4 -> 1/3
+    want = np.array([1.2, 3.2, 0, 0,   1.2, 3.2, 0, 0,   0, 0, 0, -2.0], np.float32)
+    assert np.allclose(x, want, rtol=1e-6, atol=0)
+    # against float64 on random heads, eps inside the root
+    r = rng(21)
+    x = r.standard_normal(5 * 64).astype(np.float32) * np.repeat(10.0 ** np.arange(5), 64).astype(np.float32)
+    w = r.standard_normal(64).astype(np.float32)
+    ref = (x.reshape(5, 64).astype(np.float64) / np.sqrt((x.reshape(5, 64).astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6) * w).reshape(-1)
+    orc.rms_norm_heads(x, w, 64, 1e-6)
+    assert np.allclose(x, ref, rtol=2e-6, atol=0)
+
+
+def test_kv_write_lands_at_the_offset_as_round_to_nearest_even_f16(orc):
+    slab = np.full(16, 0x1234, np.uint16)
+    src = np.array([1.0, -2.5, 65520.0, 1e-8, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11], np.float32)
+    orc.kv_write(slab, 5, src)                          # slab[5 + i] = f16(src[i]) (ops/mod.rs:1421-1425)
+    assert (slab[:5] == 0x1234).all() and (slab[11:] == 0x1234).all()
+    # 65520 is the midpoint above f16's largest finite value: overflow to infinity; 1e-8 is below half the smallest
+    # subnormal: zero; 1 + 2^-11 is a tie that goes to the even mantissa (1.0), 1 + 3 * 2^-11 to 1 + 2^-9
+    assert list(slab[5:11]) == [0x3c00, 0xc100, 0x7c00, 0x0000, 0x3c00, 0x3c02]
+    with np.errstate(over="ignore"):
+        assert np.array_equal(slab[5:11], src.astype(np.float16).view(np.uint16))
+
+
+def test_moe_glu_is_two_expert_products_and_a_silu_mul(orc):
+    r = rng(22)
+    n_in, ff, n_expert, n_used, n_tok = 64, 32, 6, 2, 3
+    gate = q8_0_weights(orc, r, n_expert * ff, n_in, std=1.0); up = q8_0_weights(orc, r, n_expert * ff, n_in, std=1.0)
+    gs = (r.random(n_expert) + 0.5).astype(np.float32); us = (r.random(n_expert) + 0.5).astype(np.float32)
+    G = ob.experts(gate, ob.Q8_0, n_in, ff, n_expert, gs); U = ob.experts(up, ob.Q8_0, n_in, ff, n_expert, us)
+    ids = np.array([4, 0, 5, 5, 1, 2], np.uint32)
+    x = r.standard_normal(n_tok * n_in).astype(np.float32)
+    out = np.zeros(ids.size * ff, np.float32); scratch = np.zeros_like(out)
+    orc.moe_glu(G, U, ids, n_used, x, out, scratch)
+    a = np.zeros_like(out); b = np.zeros_like(out)
+    orc.matmul_experts(G, ids, n_used, x, a); orc.matmul_experts(U, ids, n_used, x, b)
+    orc.silu_mul(a, b)                                  # ops/mod.rs:1105-1117: gate product, up product, silu_mul
+    assert np.array_equal(out.view(np.uint32), a.view(np.uint32))
+    # and against float64 from the dequantized weights and the Q8_0-rounded activation: the per-expert scales sit
+    # between the dot and the silu (ops/mod.rs:1082-1086)
+    sc, q = orc.quantize_q8_0(x)
+    xq = (q.reshape(-1, 32).astype(np.float64) * sc[:, None]).reshape(n_tok, n_in)
+    gw = orc.dequantize(ob.Q8_0, gate, n_expert * ff * n_in).reshape(n_expert, ff, n_in).astype(np.float64)
+    uw = orc.dequantize(ob.Q8_0, up, n_expert * ff * n_in).reshape(n_expert, ff, n_in).astype(np.float64)
+    for i, e in enumerate(ids):
+        g = gw[e] @ xq[i // n_used] * gs[e]; u = uw[e] @ xq[i // n_used] * us[e]
+        assert np.allclose(out[i * ff:(i + 1) * ff], g / (1 + np.exp(-g)) * u, rtol=2e-5, atol=1e-5)
