@@ -985,7 +985,10 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         const bool one_pass = !graphed && attend_prefill_takes(probe, dout);
         const size_t decode_floats = (size_t)a->n_head * attend_split_count((int)(a->kv_len / a->kv_dim), 1, (int)a->head_dim, (int)group) *
                                      (a->head_dim + 2);
-        float* sc = be->scratch_f32(one_pass ? decode_floats : (size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2));
+        // a few-query call reserves the decode size too, so that the first graphed pass after it (whose split count is
+        // the whole slab's) does not have to grow the scratch in the middle of a capture
+        const size_t call_floats = (size_t)(n_q * a->n_head) * n_split * (a->head_dim + 2);
+        float* sc = be->scratch_f32(one_pass ? decode_floats : std::max(call_floats, decode_floats));
         if (!sc) return;
         const int* dyn = be->dyn_slot((int)a->n_pos);
         AttnArgs args{dq, dk, dv, (int)n_q, (int)a->kv_dim, dyn ? 0 : (int)a->n_pos, (int)a->head_dim,
