@@ -16,27 +16,12 @@ the integer block dots are the oracle's).
 import numpy as np
 import pytest
 
-from util import f16_bits, q8_0_weights, rng
+from util import close, f16_bits, q8_0_weights, rng, worst
 
 pytestmark = pytest.mark.gpu
 
 ND, EPS = 2048, 1e-6
 PASSES = 5          # 2 eager + 1 captured + 2 replayed
-
-
-def _bound(b, tol):
-    """rel/abs: tol * |b_i|, with an absolute floor of tol * min(1, largest entry) for the entries near zero."""
-    b = np.abs(np.asarray(b, np.float64))
-    return tol * np.maximum(b, min(1.0, float(b.max())))
-
-
-def close(a, b, tol=1e-3):
-    return bool(np.all(np.abs(a.astype(np.float64) - b) <= _bound(b, tol)))
-
-
-def worst(a, b):
-    """largest error in units of the bound at tol = 1 (so 1e-3 means: at the limit)"""
-    return float((np.abs(a.astype(np.float64) - b) / _bound(b, 1.0)).max())
 
 
 def nvfp4_rows(r, n_out, n_in):

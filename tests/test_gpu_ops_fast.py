@@ -130,7 +130,7 @@ def test_delta_rule_fast_state_carries_over_calls(hip, orc):
                                                          (33, 512, 10, 2048, 512), (90, 8, 2, 256, 192),
                                                          # the baseline's single-op expert FFN: 512 experts top-10,
                                                          # hidden 2048, inter 512, token sweep (1 token: test_gpu_ops)
-                                                         (8, 512, 10, 2048, 512), (64, 512, 10, 2048, 512),
+                                                         (1, 512, 10, 2048, 512), (8, 512, 10, 2048, 512), (64, 512, 10, 2048, 512),
                                                          (512, 512, 10, 2048, 512)])
 def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
     import inferred_hip as ih

@@ -103,3 +103,22 @@ class Hiprt:
         for p in self.held:
             self.rt.hipFree(p)
         self.held = []
+
+
+def bound(b, tol):
+    """The rel/abs bound of the fast-mode tests: tol * |b_i|, with an absolute floor of tol * min(1, largest |b|) for
+    entries near zero (never looser than tol * max(1, |b_i|))."""
+    b = np.abs(np.asarray(b, np.float64))
+    top = float(b.max()) if b.size else 0.0
+    return tol * np.maximum(b, min(1.0, top))
+
+
+def close(a, b, tol=1e-3):
+    return bool(np.all(np.abs(np.asarray(a, np.float64) - b) <= bound(b, tol)))
+
+
+def worst(a, b):
+    """largest error as a multiple of the bound at tol = 1 (1e-3 means: exactly at a 1e-3 limit)"""
+    if np.asarray(b).size == 0:
+        return 0.0
+    return float((np.abs(np.asarray(a, np.float64) - b) / np.maximum(bound(b, 1.0), 1e-300)).max())
