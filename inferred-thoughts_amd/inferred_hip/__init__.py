@@ -482,6 +482,9 @@ class Model:
             self.h = None
 
 
+TRACE_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_char_p, C.c_uint32, C.POINTER(C.c_float), C.c_uint64)
+
+
 class Engine:
     def __init__(self, model: Model, be: Hip, n_ctx: int, max_batch: int = 512):
         self.L = lib()
@@ -495,6 +498,20 @@ class Engine:
 
     def reset(self):
         self.L.it_engine_reset(self.h)
+
+    def set_trace(self, fn):
+        """fn(name, layer, values) after every named intermediate of a pass (Ctx::trace of the reference,
+        src/profile.rs:439-456); None removes the hook.  A traced pass reads device buffers mid-pass, so it runs
+        eagerly."""
+        if fn is None:
+            self._trace_cb = None
+            self.L.it_engine_set_trace(self.h, None, None)
+            return
+
+        def cb(_user, name, layer, data, n):
+            fn(name.decode(), int(layer), np.ctypeslib.as_array(data, shape=(int(n),)).copy())
+        self._trace_cb = TRACE_FN(cb)
+        self.L.it_engine_set_trace(self.h, C.cast(self._trace_cb, C.c_void_p), None)
 
     @property
     def pos(self) -> int:

@@ -258,6 +258,18 @@ class Engine:
     def reset(self):
         self.L.orc_engine_reset(self.h)
 
+    def set_trace(self, fn):
+        """fn(name, layer, values) after every named intermediate of a pass; None removes the hook."""
+        if fn is None:
+            self._trace_cb = None
+            self.L.orc_engine_set_trace(self.h, None, None)
+            return
+
+        def cb(_user, name, layer, data, n):
+            fn(name.decode(), int(layer), np.ctypeslib.as_array(data, shape=(int(n),)).copy())
+        self._trace_cb = TRACE_FN(cb)
+        self.L.orc_engine_set_trace(self.h, C.cast(self._trace_cb, vp), None)
+
     @property
     def pos(self):
         return int(self.L.orc_engine_pos(self.h))
