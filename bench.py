@@ -113,6 +113,10 @@ def main():
     ap.add_argument("--keep", action="store_true", help="keep the generated GGUF")
     ap.add_argument("--no-single-ops", action="store_true",
                     help="skip the single-op configurations (expert FFN sweep, decode attention, Gated DeltaNet)")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="stop after the timed decode stretch (no per-kernel events, no second prefill, no CPU leg): the "
+                         "run to put under rocprofv3 --kernel-trace, whose last steps x graph-kernels records are then "
+                         "the replayed decode graph and nothing else")
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -178,6 +182,20 @@ def main():
     assert len(ids) == args.steps
     tok_s = args.steps / dt
     graph_stats = be.graph_stats()
+    if args.decode_only:
+        err = be.take_error()
+        if err:
+            raise SystemExit(f"device error: {err}")
+        print(json.dumps({"metric": "decode tok/s (decode-only run for a kernel trace)", "value": round(tok_s, 2),
+                          "unit": "tok/s", "steps": args.steps, "warmup": args.warmup,
+                          "ms_per_step": round(1e3 * dt / args.steps, 4), "graph": graph_stats}), flush=True)
+        eng.close(); model.close(); be.close()
+        if not args.keep:
+            try:
+                path.unlink()
+            except OSError:
+                pass
+        return
     l0 = be.launch_count(); eng.decode_greedy(1); launches_per_token = be.launch_count() - l0
 
     # per-kernel device time over a second identical stretch: the launches the decode graph holds, issued

@@ -179,12 +179,33 @@ size_t it_hip_config_report(it_hip*, char* buf, size_t buf_len);
 uint64_t it_hip_setup_cost(it_hip*, char* label, size_t label_len);
 void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x, uint64_t x_len, uint64_t k);
 
-/* ---- expert cache API, all-resident tier (src/ops/cuda/ops/placement.rs:15-363) ---- */
-void it_hip_set_expert_budget(it_hip*, uint64_t bytes);
-void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes);
-void it_hip_set_expert_slots(it_hip*, uint64_t n);
-void it_hip_set_expert_pool(it_hip*, uint64_t n);
+/* ---- expert cache API, all-resident tier (src/ops/cuda/ops/placement.rs:15-363) ----
+ * 288 GB of device memory hold every expert of the models this backend serves, so the cache is one tier: each expert
+ * matrix of a pooled tensor takes a slot at first sight of its tensor and is never evicted.  The slab keeps the
+ * reference's shape: one uniform slot size (the bytes of one expert matrix; a tensor of another size is refused,
+ * experts.rs:890-901), a capacity in slots fixed when the first pooled tensor arrives (set_expert_slots, else
+ * set_expert_budget, else free device memory minus the reserves), and per-expert read counters on the device that
+ * the expert kernels write.  A pool larger than the capacity is refused with a sticky error: the pinned-host and SSD
+ * tiers are not part of this backend. */
+void it_hip_set_expert_budget(it_hip*, uint64_t bytes);      /* placement.rs:178 */
+void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes); /* placement.rs:322; kept and reported, no host tier */
+void it_hip_set_expert_slots(it_hip*, uint64_t n);           /* placement.rs:157; 0 = by budget */
+void it_hip_set_expert_pool(it_hip*, uint64_t n);            /* sizes the read counters, experts.rs:424-438 */
+void it_hip_reserve_for_weights(it_hip*, uint64_t dense_bytes); /* placement.rs:203 */
+void it_hip_reserve_for_kv(it_hip*, uint64_t bytes);         /* placement.rs:341 */
+void it_hip_set_prefetch(it_hip*, int on);                   /* placement.rs:164; nothing to fetch when all resident */
+void it_hip_set_model_path(it_hip*, const char* path);       /* placement.rs:357 */
+void it_hip_set_map_base(it_hip*, uint64_t base);            /* placement.rs:363 */
+/* lookups / hits come from the device counters (waits for the device), placement.rs:15 */
 void it_hip_expert_stats(it_hip*, it_expert_stats* out);
+/* share of all expert reads taken by the busiest slab-many matrices, and the reads counted (placement.rs:347,
+ * experts.rs:861-873); 0 = ok, 1 = no pooled tensor yet */
+int it_hip_expert_coverage(it_hip*, double* fraction, uint64_t* total_reads);
+/* re-place the pool by the reads counted so far; returns the experts moved (always 0 here), -1 on a device error
+ * (placement.rs:113) */
+int64_t it_hip_replace_experts_by_counts(it_hip*);
+/* extension: the per-expert read counts of one tensor (keyed on its data pointer), expert order; returns entries */
+uint64_t it_hip_expert_counts(it_hip*, const uint8_t* tensor_data, uint32_t* out, uint64_t cap);
 /* GCLOCK victim choice (src/ops/cuda/experts.rs:2215-2233) as a pure function over a
  * ring of heat counters and lease flags; returns the victim index or -1 when every
  * slot is leased.  Never selects a victim in the all-resident tier; kept for tests. */

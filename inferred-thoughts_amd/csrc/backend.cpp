@@ -374,13 +374,43 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
         return false;
     }
     bool fresh = weights.find(w->data) == weights.end();
+    if (fresh) {
+        // the slab's slot is one expert matrix of the first pooled tensor; a tensor of another size does not fit
+        // the arena (src/ops/cuda/experts.rs:890-901, 1621-1630)
+        const uint64_t one = type_row_bytes(w->ty, w->n_in) * w->n_out;
+        if (one == 0 || w->len != one * w->n_expert) {
+            fail(std::string(who) + ": expert tensor length is not n_expert matrices of its shape");
+            return false;
+        }
+        if (expert_resident && expert_slot_bytes != one) {
+            fail(std::string(who) + ": expert matrix is " + std::to_string(one) + " bytes but the slab's slot is " +
+                 std::to_string(expert_slot_bytes) + "; the pool is not uniform, which this arena assumes");
+            return false;
+        }
+        if (!expert_resident) {
+            // sized at the first pooled tensor, from what is free then (placement.rs:294-312, 423-453)
+            expert_slot_bytes = one;
+            size_t fr = 0, tot = 0;
+            (void)hipMemGetInfo(&fr, &tot);
+            const uint64_t by_budget = expert_budget ? expert_budget : (fr > expert_reserve ? fr - expert_reserve : 0);
+            expert_slots_cap = expert_slots_req ? expert_slots_req : by_budget / one;
+        }
+        if (expert_resident + w->n_expert > expert_slots_cap) {
+            fail(std::string(who) + ": the expert pool needs " + std::to_string(expert_resident + w->n_expert) +
+                 " slots of " + std::to_string(one) + " bytes but the device tier holds " + std::to_string(expert_slots_cap) +
+                 "; tiers beyond device memory (pinned host, SSD) are not part of this backend");
+            return false;
+        }
+        if (!expert_counters_reserve(expert_counted + w->n_expert)) return false;
+    }
     const Resident* r = resident(w->data, w->len, w->ty, w->n_in, w->n_out * w->n_expert, who);
     if (!r) return false;
     if (fresh) {
         // all-resident tier: every expert of the tensor is placed at first sight
         expert_resident += w->n_expert;
-        expert_slot_bytes = type_row_bytes(w->ty, w->n_in) * w->n_out;
         if (expert_pool < expert_resident) expert_pool = expert_resident;
+        weights[w->data].counter_base = (int64_t)expert_counted;
+        expert_counted += w->n_expert;
     }
     Resident* rw = &weights[w->data];
     if (w->scale && w->scale_len && !rw->scale2) {
@@ -405,6 +435,49 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
         out->s_stride = (int64_t)(w->n_out * (w->n_in / 16));
     }
     out->scale2 = (w->scale && w->scale_len) ? rw->scale2 : nullptr;
+    out->counts = rw->counter_base >= 0 ? expert_counts + rw->counter_base : nullptr;
+    return true;
+}
+
+// the device read counters hold at least `entries` (tensor, expert) entries; existing counts survive a growth
+bool it_hip::expert_counters_reserve(size_t entries) {
+    if (!expert_tally) {
+        if (!check(hipMalloc((void**)&expert_tally, 2 * sizeof(unsigned long long)), "hipMalloc(expert tally)") ||
+            !check(hipMemset(expert_tally, 0, 2 * sizeof(unsigned long long)), "hipMemset(expert tally)"))
+            return false;
+    }
+    if (entries <= expert_counts_cap) return true;
+    need_eager("the expert read counters have to grow");
+    drop_graph();  // a captured graph holds the old array
+    size_t cap = std::max<size_t>({entries, 2 * expert_counts_cap, (size_t)expert_pool, (size_t)4096});
+    uint32_t* fresh = nullptr;
+    if (!check(hipMalloc((void**)&fresh, cap * sizeof(uint32_t)), "hipMalloc(expert read counters)") ||
+        !check(hipMemset(fresh, 0, cap * sizeof(uint32_t)), "hipMemset(expert read counters)"))
+        return false;
+    if (expert_counts) {
+        check(hipStreamSynchronize(stream), "sync before the counters move");
+        check(hipMemcpy(fresh, expert_counts, expert_counts_cap * sizeof(uint32_t), hipMemcpyDeviceToDevice), "copy expert read counters");
+        (void)hipFree(expert_counts);
+    }
+    expert_counts = fresh;
+    expert_counts_cap = cap;
+    return true;
+}
+
+// Bring the device-side read counters home (absorb_expert_counters, placement.rs:130-152); costs a synchronize
+bool it_hip::expert_counters_read(std::vector<uint32_t>* counts, uint64_t tally[2]) {
+    tally[0] = tally[1] = 0;
+    if (counts) counts->assign(expert_counted, 0);
+    if (!expert_tally || !expert_counted) return true;
+    if (in_pass) finish_pass();
+    if (!check(hipStreamSynchronize(stream), "sync before reading the expert counters")) return false;
+    unsigned long long t[2] = {0, 0};
+    if (!check(hipMemcpy(t, expert_tally, sizeof t, hipMemcpyDeviceToHost), "download expert tally")) return false;
+    tally[0] = t[0];
+    tally[1] = t[1];
+    if (counts && !check(hipMemcpy(counts->data(), expert_counts, expert_counted * sizeof(uint32_t), hipMemcpyDeviceToHost),
+                         "download expert read counters"))
+        return false;
     return true;
 }
 
@@ -667,7 +740,13 @@ void it_hip::drop_all() {
         if (kv.second.dev) (void)hipFree(kv.second.dev);
     slabs.clear();
     mirror_bytes = quant_bytes = const_bytes = weight_bytes = kv_bytes = 0;
+    // the pool is gone with the weights: the next pooled tensor sizes a new slab; counters start over
     expert_resident = 0;
+    expert_slot_bytes = 0;
+    expert_slots_cap = 0;
+    expert_counted = 0;
+    if (expert_counts) (void)hipMemset(expert_counts, 0, expert_counts_cap * sizeof(uint32_t));
+    if (expert_tally) (void)hipMemset(expert_tally, 0, 2 * sizeof(unsigned long long));
 }
 
 it_hip::~it_hip() {
@@ -688,6 +767,8 @@ it_hip::~it_hip() {
     for (auto e : prof_pool) (void)hipEventDestroy(e);
     if (dyn_dev) (void)hipFree(dyn_dev);
     if (route_counter) (void)hipFree(route_counter);
+    if (expert_counts) (void)hipFree(expert_counts);
+    if (expert_tally) (void)hipFree(expert_tally);
     for (int i = 0; i < 2; i++) {
         if (dyn_hosts[i]) (void)hipHostFree(dyn_hosts[i]);
         if (dyn_evt[i]) (void)hipEventDestroy(dyn_evt[i]);
@@ -871,7 +952,7 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     // tiles, which the GEMVs reach at about 512 tokens)
     if (!exact && v.fmt == W_NVFP4 && n > 512) {
         ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
-        ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr;
+        ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr; ev.counts = nullptr;
         zids = be->zero_ids_for(n);
         work = be->moe_work_for(n, 1, &work_ints);
         fwork_bytes = itk::experts_f16_work_bytes(nt, v.n_in);
@@ -1226,16 +1307,18 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
-    rec.i[6] = v.q_stride; rec.i[7] = v.s_stride;
+    rec.i[6] = v.q_stride; rec.i[7] = v.s_stride; rec.p[7] = v.counts;
+    unsigned long long* tally = be->expert_tally;
+    uint32_t* counts = v.counts;
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
+                   expert_count(ids, np, counts, tally, s);
                    if (f16_shape && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
                        matmul_experts(v, ids, np, nu, xm, as, aq, dout, s);
                });
-    be->expert_lookups += picks;
 }
 
 void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, const it_route* route,
@@ -1280,17 +1363,20 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
     rec.i[0] = g.fmt; rec.i[1] = g.n_in; rec.i[2] = g.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
-    rec.i[6] = g.q_stride; rec.i[7] = g.s_stride;
+    rec.i[6] = g.q_stride; rec.i[7] = g.s_stride; rec.p[10] = g.counts; rec.p[11] = u.counts;
+    unsigned long long* tally = be->expert_tally;
+    uint32_t *cg = g.counts, *cu = u.counts;
     be->submit(it_hip::FAM_MOE_GLU, 2 * picks * (gate->len / gate->n_expert) + x_len + out_len * 4,
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
                [=](hipStream_t s) {
+                   expert_count(ids, np, cg, tally, s);
+                   expert_count(ids, np, cu, tally, s);
                    if (f16_shape && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
                        moe_glu(g, u, ids, np, nu, xm, as, aq, dout, s);
                });
-    be->expert_lookups += 2 * picks;
 }
 
 void it_hip_moe_finish(it_hip* be, float* out, uint64_t out_len, uint64_t at, uint64_t n, const float* rows,
@@ -1511,9 +1597,12 @@ int it_hip_tier_counters(it_hip* be, it_tier_counters* out) {
     (void)hipMemGetInfo(&fr, &tot);
     out->vram_free = fr;
     out->vram_total = tot;
-    out->lookups = be->expert_lookups;
+    uint64_t tally[2];
+    be->expert_counters_read(nullptr, tally);
+    out->lookups = tally[0] + tally[1];
+    out->host_reads = tally[1];
     out->slot_bytes = be->expert_slot_bytes;
-    out->slots = be->expert_resident;
+    out->slots = be->expert_slots_cap;
     out->mirrors = be->acts.size();
     out->mirror_bytes = be->mirror_bytes;
     out->weight_bytes = be->weight_bytes;
@@ -1522,15 +1611,21 @@ int it_hip_tier_counters(it_hip* be, it_tier_counters* out) {
     out->pool_bytes = be->attn_scratch_cap * 4;
     out->resident_bytes = be->weight_bytes + be->kv_bytes + be->quant_bytes + be->mirror_bytes +
                           be->const_bytes + out->pool_bytes;
-    out->oversubscribed = 0;
+    out->oversubscribed = be->expert_resident > be->expert_slots_cap;
     return 1;
 }
 
 size_t it_hip_config_report(it_hip* be, char* buf, size_t buf_len) {
     int n = snprintf(buf, buf_len,
-                     "backend=hip gfx950\nreductions=%s\ndecode graph=%s\nattention=%s\nexpert tier=all-resident\n",
+                     "backend=hip gfx950\nreductions=%s\ndecode graph=%s\nattention=%s\nexpert tier=all-resident\n"
+                     "expert slots=%llu of %llu bytes (%s)\nexpert host budget=%llu (no host tier)\nexpert prefetch=%s (nothing to fetch)\n"
+                     "model path=%s\n",
                      be->exact ? "serial (CPU order)" : "tree / split-K", be->allow_graph ? "on" : "off",
-                     be->exact ? "exact" : "split-K flash decoding (128-position chunks)");
+                     be->exact ? "exact" : "split-K flash decoding (128-position chunks)",
+                     (unsigned long long)be->expert_slots_cap, (unsigned long long)be->expert_slot_bytes,
+                     be->expert_slots_req ? "fixed" : be->expert_budget ? "by budget" : "by free device memory",
+                     (unsigned long long)be->expert_host_budget, be->expert_prefetch ? "on" : "off",
+                     be->model_path.empty() ? "(not set)" : be->model_path.c_str());
     return n < 0 ? 0 : (size_t)n;
 }
 
@@ -1542,19 +1637,87 @@ void it_hip_prefetch_hint(it_hip* be, const it_weights* w, const float* x, uint6
     (void)be; (void)w; (void)x; (void)x_len; (void)k;  // every expert is resident: nothing to fetch
 }
 
+// Cap the expert slab, in bytes; 0 restores sizing from free device memory (placement.rs:178-189).  Like the
+// reference's, read once: when the first pooled tensor sizes the slab.
 void it_hip_set_expert_budget(it_hip* be, uint64_t bytes) { be->expert_budget = bytes; }
+// The pinned-host tier behind the slab (placement.rs:322-326).  This backend has no host tier: the value is kept and
+// reported, and a pool that does not fit the device tier is refused instead of spilling.
 void it_hip_set_expert_host_budget(it_hip* be, uint64_t bytes) { be->expert_host_budget = bytes; }
+// Fix the slab at n slots whatever the budget says; 0 restores sizing by budget (placement.rs:157-159)
 void it_hip_set_expert_slots(it_hip* be, uint64_t n) { be->expert_slots_req = n; }
-void it_hip_set_expert_pool(it_hip* be, uint64_t n) { be->expert_pool = n; }
+// How many expert matrices the model has: sizes the device read counters up front (placement.rs, experts.rs:424-438)
+void it_hip_set_expert_pool(it_hip* be, uint64_t n) {
+    be->expert_pool = n;
+    if (n) be->expert_counters_reserve((size_t)n);
+}
+// Leave room for the permanent weights / the KV cache when the slab is sized automatically (placement.rs:203-209,
+// 341-343): weights raise the reserve to at least dense + 1 GiB, KV adds to it.  No effect on an explicit budget.
+void it_hip_reserve_for_weights(it_hip* be, uint64_t dense_bytes) {
+    if (be->expert_budget) return;
+    be->expert_reserve = std::max<uint64_t>(be->expert_reserve, dense_bytes + (1ull << 30));
+}
+void it_hip_reserve_for_kv(it_hip* be, uint64_t bytes) { be->expert_reserve += bytes; }
+// Lookahead prefetch of the next layer's experts (placement.rs:164-168): nothing to fetch when every expert is
+// resident; the switch is kept and reported.
+void it_hip_set_prefetch(it_hip* be, int on) { be->expert_prefetch = on != 0; }
+void it_hip_set_model_path(it_hip* be, const char* path) { be->model_path = path ? path : ""; }
+void it_hip_set_map_base(it_hip* be, uint64_t base) { be->map_base = base; }
+
 void it_hip_expert_stats(it_hip* be, it_expert_stats* out) {
     if (!out) return;
     memset(out, 0, sizeof *out);
-    out->slots = be->expert_resident;
+    uint64_t tally[2];
+    be->expert_counters_read(nullptr, tally);
+    out->slots = be->expert_slots_cap;
     out->slot_bytes = be->expert_slot_bytes;
     out->resident = be->expert_resident;
     out->pool = be->expert_pool;
-    out->lookups = be->expert_lookups;
-    out->hits = be->expert_lookups;
+    out->lookups = tally[0] + tally[1];
+    out->hits = tally[0];
+    out->host_slots = 0;
+    out->oversubscribed = be->expert_resident > be->expert_slots_cap;
+}
+
+// What fraction of all expert reads the busiest slab-many matrices took, and the reads counted
+// (ExpertCache::coverage, experts.rs:861-873).  0 = ok, 1 = no pooled tensor seen yet.
+int it_hip_expert_coverage(it_hip* be, double* fraction, uint64_t* total_reads) {
+    std::vector<uint32_t> counts;
+    uint64_t tally[2];
+    if (!be->expert_counted || !be->expert_counters_read(&counts, tally)) return 1;
+    std::sort(counts.begin(), counts.end(), [](uint32_t a, uint32_t b) { return a > b; });
+    uint64_t total = 0, top = 0;
+    for (size_t i = 0; i < counts.size(); i++) {
+        total += counts[i];
+        if (i < be->expert_slots_cap) top += counts[i];
+    }
+    if (fraction) *fraction = total ? (double)top / (double)total : 0.0;
+    if (total_reads) *total_reads = total;
+    return 0;
+}
+
+// Re-place the pool by the reads counted so far (placement.rs:113-128): with every expert in device memory no host
+// expert can be busier than a resident one, so nothing moves.  Returns the experts moved, or -1 on a device error.
+int64_t it_hip_replace_experts_by_counts(it_hip* be) {
+    uint64_t tally[2];
+    if (!be->expert_counters_read(nullptr, tally)) return -1;
+    return 0;
+}
+
+// per-expert read counts of one tensor, in expert order (the rows of `counts` the gather wrote for it); returns the
+// number of entries written, 0 when the tensor has not been seen
+uint64_t it_hip_expert_counts(it_hip* be, const uint8_t* tensor_data, uint32_t* out, uint64_t cap) {
+    auto it = be->weights.find(tensor_data);
+    if (it == be->weights.end() || it->second.counter_base < 0) return 0;
+    std::vector<uint32_t> counts;
+    uint64_t tally[2];
+    if (!be->expert_counters_read(&counts, tally)) return 0;
+    // the tensor's entries run to the next tensor's base (or the end)
+    size_t lo = (size_t)it->second.counter_base, hi = counts.size();
+    for (auto& kv : be->weights)
+        if (kv.second.counter_base > (int64_t)lo && (size_t)kv.second.counter_base < hi) hi = (size_t)kv.second.counter_base;
+    uint64_t n = std::min<uint64_t>(hi - lo, cap);
+    for (uint64_t i = 0; i < n; i++) out[i] = counts[lo + i];
+    return n;
 }
 
 // GCLOCK (src/ops/cuda/experts.rs:2215-2233): sweep from the hand, skipping leased

@@ -94,6 +94,7 @@ struct it_hip {
         int fmt = 0;
         uint64_t n_in = 0, rows = 0;
         float* scale2 = nullptr;  // experts' per-expert second scale
+        int64_t counter_base = -1;  // first of this tensor's entries in expert_counts (expert tensors only)
     };
     std::unordered_map<const void*, Resident> weights;
     const Resident* resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in, uint64_t rows,
@@ -263,8 +264,21 @@ struct it_hip {
     uint64_t launches = 0, h2d = 0, d2h = 0, h2d_bytes = 0, d2h_bytes = 0;
     uint64_t weight_bytes = 0, kv_bytes = 0, quant_bytes = 0, mirror_bytes = 0, const_bytes = 0;
     uint64_t setup_us = 0;
-    uint64_t expert_lookups = 0, expert_resident = 0, expert_slot_bytes = 0, expert_pool = 0;
-    uint64_t expert_budget = 0, expert_host_budget = 0, expert_slots_req = 0;
+    // ---- expert cache, all-resident tier (src/ops/cuda/ops/placement.rs, experts.rs)
+    // Every expert matrix of a pooled tensor is placed in device memory at first sight of the tensor.  The slab has
+    // one uniform slot size (the bytes of one expert matrix in the file); its capacity in slots comes from
+    // set_expert_slots, else set_expert_budget, else free device memory minus the reserves, and a pool that does not
+    // fit is refused (the pinned-host and SSD tiers are not part of this backend).  Reads are counted on the device.
+    uint64_t expert_resident = 0, expert_slot_bytes = 0, expert_pool = 0, expert_slots_cap = 0;
+    uint64_t expert_budget = 0, expert_host_budget = 0, expert_slots_req = 0, expert_reserve = 1ull << 30;
+    bool expert_prefetch = true;
+    std::string model_path;
+    uint64_t map_base = 0;
+    uint32_t* expert_counts = nullptr;            // device: reads per (tensor, expert), in placement order
+    size_t expert_counts_cap = 0, expert_counted = 0;
+    unsigned long long* expert_tally = nullptr;   // device: [0] reads served from device memory, [1] from a host tier
+    bool expert_counters_reserve(size_t entries);
+    bool expert_counters_read(std::vector<uint32_t>* counts, uint64_t tally[2]);
 
     void drop_all();
     void drop_graph();

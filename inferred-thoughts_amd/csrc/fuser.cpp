@@ -359,7 +359,7 @@ bool match_attn(Plan& pl, size_t i, int exact) {
 }
 
 // routed FFN: 17 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
-bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
+bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long long* tally) {
     // With a quantized router the activation is quantized before the router matmul; with an unquantized one
     // (F32 in real files) the first reader of the quantized form is the expert gate/up product, after the route.
     const bool q_first = pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT,
@@ -479,6 +479,10 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter) {
     d.route_w = (const float*)rt.p[2];
     d.logit = (const float*)ml.p[5];
     d.x = (float*)rms.p[0];
+    d.counts_gate = (uint32_t*)glu.p[10];
+    d.counts_up = (uint32_t*)glu.p[11];
+    d.counts_down = (uint32_t*)ex.p[7];
+    d.tally = tally;
 
     pl.take(i, 17);
     const uint64_t glu_b = 2 * rows_bytes(g.fmt, (uint64_t)nu * ff, nd) + 2 * rows_bytes(g.sh_fmt, sff, nd) + (uint64_t)nd * 4 +
@@ -506,7 +510,7 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
             if (pl.consumed[i]) continue;
             if (match_gdn(pl, i, exact)) continue;
             if (match_attn(pl, i, exact)) continue;
-            if (match_ffn(pl, i, exact, route_counter)) continue;
+            if (match_ffn(pl, i, exact, route_counter, expert_tally)) continue;
             if (match_final(pl, i, exact)) continue;
             if (match_norm_matmuls(pl, i, exact)) continue;
             if (match_matmul_residual(pl, i, exact)) continue;

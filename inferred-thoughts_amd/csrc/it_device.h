@@ -14,6 +14,20 @@
 
 #define IT_DEV __device__ __forceinline__
 
+// the expert cache's device-side read counters: one token's picks on the three tensors of a routed FFN
+IT_DEV void it_count_expert_reads(const int32_t* ids, int n_used, uint32_t* cg, uint32_t* cu, uint32_t* cd,
+                                  unsigned long long* tally) {
+    if (blockIdx.x != 0 || blockIdx.y != 0 || !tally) return;
+    const int t = threadIdx.x;
+    if (t < n_used) {
+        const int e = ids[t];
+        if (cg) atomicAdd(cg + e, 1u);
+        if (cu) atomicAdd(cu + e, 1u);
+        if (cd) atomicAdd(cd + e, 1u);
+    }
+    if (t == 0) atomicAdd(tally, (unsigned long long)((cg ? 1 : 0) + (cu ? 1 : 0) + (cd ? 1 : 0)) * n_used);
+}
+
 IT_DEV float it_f16_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 IT_DEV uint16_t it_f32_to_f16(float f) { return __half_as_ushort(__float2half_rn(f)); }
 IT_DEV float it_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }

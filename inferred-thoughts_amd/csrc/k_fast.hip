@@ -808,6 +808,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     const int row = (blockIdx.x * (DW / 4) + group) * P + rsub;
     const bool live = row < p.n_out;
     IT_STAMP(0);
+    it_count_expert_reads(p.route_ids, NU, p.counts_gate, p.counts_up, p.counts_down, p.tally);
 
     // the intermediates: up to three quads per thread (12 floats) cover 6144 floats per block
     const int nq = total >> 2, nq_routed = (NU * n_in) >> 2;

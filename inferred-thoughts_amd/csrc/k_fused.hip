@@ -684,6 +684,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_k(MoeDownP p) {
     int8_t* xq = (int8_t*)(xs + ((NU * nb + sh_nb + 3) & ~3));    // NU*n_in + sh_in quants
     float* terms_all = (float*)(xq + ((NU * n_in + sh_in + 15) & ~15));
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    it_count_expert_reads(p.route_ids, NU, p.counts_gate, p.counts_up, p.counts_down, p.tally);
     constexpr int MAXU = 16;  // n_used <= 16 (checked on the host)
     const int R = p.rows_per_wave;  // R * (n_in / 32) <= 64: one item per lane per expert
     const int T = p.fmt == W_NVFP4 ? nb * 2 : nb;

@@ -106,6 +106,18 @@ __global__ __launch_bounds__(256) void route_topk_wave_k(const float* __restrict
     }
 }
 
+__global__ void expert_count_k(const int32_t* __restrict__ ids, int n_picks, uint32_t* __restrict__ counts,
+                               unsigned long long* __restrict__ tally) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_picks) atomicAdd(counts + ids[i], 1u);
+    if (i == 0) atomicAdd(tally, (unsigned long long)n_picks);
+}
+
+void expert_count(const int32_t* ids, int n_picks, uint32_t* counts, unsigned long long* tally, hipStream_t s) {
+    if (n_picks <= 0 || !counts || !tally) return;
+    hipLaunchKernelGGL(expert_count_k, dim3((n_picks + 255) / 256), dim3(256), 0, s, ids, n_picks, counts, tally);
+}
+
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,
                 hipStream_t s) {
     if (n_tok <= 0) return;

@@ -45,6 +45,7 @@ struct ExpertsView {
     int64_t q_stride, s_stride;
     int fmt, n_in, n_out, n_expert;
     const float* scale2;  // per-expert second scale or null
+    uint32_t* counts;     // this tensor's per-expert read counters (device), or null
 };
 // One matmul per pick.  x rows: mode 0 = one row per pick, 1 = one row per token
 // (pick i reads row i / n_used), 2 = a single shared row.
@@ -75,6 +76,11 @@ bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* id
 // out[i] = silu(gate_e . x * sg_e) * (up_e . x * su_e)
 void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids, int n_picks, int n_used,
              int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);
+
+// ---- expert read counters -------------------------------------------------------
+// counts[ids[i]] += 1 for every pick and tally[0] += n_picks: the device-side read counters of the expert cache
+// (reads served from device memory; tally[1], reads served from a host tier, stays 0 when every expert is resident)
+void expert_count(const int32_t* ids, int n_picks, uint32_t* counts, unsigned long long* tally, hipStream_t s);
 
 // ---- router ----------------------------------------------------------------------
 void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);

@@ -79,6 +79,10 @@ struct MoeDownP {
     const float* route_w;
     const float* logit;     // shared expert gate logit
     float* x;               // residual stream, accumulated into
+    // expert read counters (optional): the gate, up and down tensors' per-expert counts and the tally of reads
+    // served from device memory; block 0 adds this token's picks
+    uint32_t *counts_gate, *counts_up, *counts_down;
+    unsigned long long* tally;
 };
 void moe_down_fused(MoeDownP p, hipStream_t s);
 

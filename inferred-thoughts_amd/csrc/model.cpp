@@ -263,6 +263,7 @@ struct it_engine {
     HostBuf x, normed, mixed, ffn_out, qg, q, g, k, v, attn, qkv, z, alpha, beta, convo, q_part, k_part, v_part,
         core, router, e_gate, e_up, e_out, e_in, g_all, u_all, o_all, shexp_logit, last, final_norm, logits;
 
+    uint64_t kv_reserved = 0;  // bytes this engine asked the backend to keep free of the expert slab
     uint64_t slab_len() const { return n_ctx * m->d.kv_dim(); }
     uint16_t* k_slab(uint64_t slot) { return k_slabs.data() + slot * slab_len(); }
     uint16_t* v_slab(uint64_t slot) { return v_slabs.data() + slot * slab_len(); }
@@ -515,6 +516,20 @@ it_engine* it_engine_new(it_model* m, it_hip* be, uint64_t n_ctx, uint64_t max_b
     e->v_slabs.assign(m->n_kv_layer * n_ctx * d.kv_dim(), 0);
     e->conv.assign(d.layers() * d.conv_len(), 0.0f);
     e->ssm.assign(d.layers() * d.ssm_len(), 0.0f);
+    // what the reference's CLI tells its device backend before the first pass (src/main.rs:545-560): the permanent
+    // weights and the KV cache the expert slab must leave room for, and the size of the expert pool (one read
+    // counter per expert matrix)
+    uint64_t dense = m->output.len + m->tok_embd.len;
+    for (const Block& b : m->blocks) {
+        if (b.recurrent) dense += b.wqkv.len + b.wgate.len + b.w_alpha.len + b.w_beta.len + b.w_out.len;
+        else dense += b.wq.len + b.wk.len + b.wv.len + b.wo.len;
+        dense += b.router.len + b.sh_gate.len + b.sh_up.len + b.sh_down.len + b.sh_gate_inp.len;
+    }
+    it_hip_reserve_for_weights(be, dense);
+    it_hip_set_expert_pool(be, d.layers() * 3 * d.n_expert);
+    e->kv_reserved = 2 * m->n_kv_layer * n_ctx * d.kv_dim() * sizeof(uint16_t) +
+                     (d.layers() * (d.conv_len() + d.ssm_len())) * sizeof(float);
+    it_hip_reserve_for_kv(be, e->kv_reserved);
     return e;
 }
 void it_engine_free(it_engine* e) {
@@ -534,6 +549,8 @@ void it_engine_free(it_engine* e) {
         it_hip_release(e->be, e->conv_of(il));
         it_hip_release(e->be, e->ssm_of(il));
     }
+    // the reserve is additive (placement.rs:341-343): give this engine's share back (unsigned wrap-around subtracts)
+    it_hip_reserve_for_kv(e->be, (uint64_t)0 - e->kv_reserved);
     delete e;
 }
 

@@ -98,7 +98,9 @@ it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sy
 it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_engine_restore it_engine_rewind it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
-it_engine_v_slab it_synth_write_gguf it_hip_attend_noalloc""".split()
+it_engine_v_slab it_synth_write_gguf it_hip_attend_noalloc it_hip_reserve_for_weights it_hip_reserve_for_kv
+it_hip_set_prefetch it_hip_set_model_path it_hip_set_map_base it_hip_expert_coverage it_hip_replace_experts_by_counts
+it_hip_expert_counts""".split()
 
 _lib = None
 
@@ -173,6 +175,14 @@ def lib() -> C.CDLL:
         "it_hip_set_expert_slots": (None, [vp, u64]),
         "it_hip_set_expert_pool": (None, [vp, u64]),
         "it_hip_expert_stats": (None, [vp, vp]),
+        "it_hip_reserve_for_weights": (None, [vp, u64]),
+        "it_hip_reserve_for_kv": (None, [vp, u64]),
+        "it_hip_set_prefetch": (None, [vp, C.c_int]),
+        "it_hip_set_model_path": (None, [vp, C.c_char_p]),
+        "it_hip_set_map_base": (None, [vp, u64]),
+        "it_hip_expert_coverage": (C.c_int, [vp, vp, vp]),
+        "it_hip_replace_experts_by_counts": (C.c_int64, [vp]),
+        "it_hip_expert_counts": (u64, [vp, vp, vp, u64]),
         "it_hip_clock_pick": (C.c_int64, [vp, vp, u64, vp]),
         "it_hip_argmax": (u32, [vp, vp, u64]),
         "it_hip_sync": (None, [vp]),
@@ -448,6 +458,50 @@ class Hip:
         s = ExpertStats()
         self.L.it_hip_expert_stats(self.h, C.addressof(s))
         return s
+
+    def set_expert_budget(self, nbytes):
+        self.L.it_hip_set_expert_budget(self.h, nbytes)
+
+    def set_expert_host_budget(self, nbytes):
+        self.L.it_hip_set_expert_host_budget(self.h, nbytes)
+
+    def set_expert_slots(self, n):
+        self.L.it_hip_set_expert_slots(self.h, n)
+
+    def set_expert_pool(self, n):
+        self.L.it_hip_set_expert_pool(self.h, n)
+
+    def reserve_for_weights(self, nbytes):
+        self.L.it_hip_reserve_for_weights(self.h, nbytes)
+
+    def reserve_for_kv(self, nbytes):
+        self.L.it_hip_reserve_for_kv(self.h, nbytes)
+
+    def set_prefetch(self, on):
+        self.L.it_hip_set_prefetch(self.h, 1 if on else 0)
+
+    def set_model_path(self, path):
+        self.L.it_hip_set_model_path(self.h, str(path).encode())
+
+    def set_map_base(self, base):
+        self.L.it_hip_set_map_base(self.h, base)
+
+    def expert_coverage(self):
+        """(share of reads taken by the busiest slab-many expert matrices, reads counted), or None before any
+        pooled tensor was seen."""
+        f, n = C.c_double(0.0), c_u64(0)
+        if self.L.it_hip_expert_coverage(self.h, C.byref(f), C.byref(n)):
+            return None
+        return float(f.value), int(n.value)
+
+    def replace_experts_by_counts(self) -> int:
+        return int(self.L.it_hip_replace_experts_by_counts(self.h))
+
+    def expert_counts(self, tensor: np.ndarray, n_expert: int) -> np.ndarray:
+        """Per-expert device read counts of one expert tensor (the array its Experts struct points at)."""
+        out = np.zeros(n_expert, np.uint32)
+        n = self.L.it_hip_expert_counts(self.h, _p(tensor), _p(out), n_expert)
+        return out[:int(n)]
 
     def config_report(self) -> str:
         b = C.create_string_buffer(2048)
