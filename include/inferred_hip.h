@@ -159,6 +159,43 @@ void it_hip_add_scaled(it_hip*, float* a, uint64_t a_len, const float* b, uint64
 void it_hip_kv_write(it_hip*, uint16_t* slab, uint64_t slab_len, uint64_t offset, const float* src,
                      uint64_t src_len); /* mod.rs:1421 */
 
+/* ---- methods only the qwen4exp architecture calls (mod.rs:705-966): hyper-connection streams, PLE, QSA sparse
+ * attention.  That architecture is outside this backend's path; each entry point exists so that a binding covers the
+ * whole trait, launches nothing, and records the sticky error "<op>: qwen4exp-only op, not implemented by the hip
+ * backend" (the reference refuses unsupported work the same way: first error kept, polled after the run). ---- */
+typedef struct {
+    uint64_t from, to, ratio, dim;
+    const float* norm;
+    uint64_t norm_len;
+    float eps;
+    uint32_t _pad;
+    uint64_t n_rot;
+    float theta;
+    uint32_t _pad2;
+} it_qsa_pool; /* struct QsaPool, mod.rs:279-289 */
+typedef struct {
+    uint64_t n_head, dim, n_blocks, start_pos, ratio, budget;
+} it_qsa_select; /* struct QsaSelect, mod.rs:294-305 */
+void it_hip_mean_streams(it_hip*, const float* src, uint64_t src_len, uint64_t n_stream, uint64_t nd, float inv,
+                         float* out, uint64_t out_len); /* mod.rs:705 */
+void it_hip_mul_rows(it_hip*, float* x, uint64_t x_len, const float* w, uint64_t w_len); /* mod.rs:801 */
+void it_hip_silu(it_hip*, float* x, uint64_t x_len);                                       /* mod.rs:811 */
+void it_hip_sigmoid(it_hip*, float* x, uint64_t x_len);                                    /* mod.rs:818 */
+void it_hip_mul_streams(it_hip*, float* out, uint64_t out_len, const float* h, uint64_t h_len, const float* w,
+                        uint64_t w_len, uint64_t n_stream); /* mod.rs:828 */
+void it_hip_row_dot(it_hip*, const float* a, uint64_t a_len, const float* b, uint64_t b_len, uint64_t width,
+                    float* out, uint64_t out_len); /* mod.rs:846 */
+void it_hip_signed_sqrt_sigmoid(it_hip*, float* s, uint64_t s_len); /* mod.rs:861 */
+void it_hip_dilated_conv(it_hip*, float* state, uint64_t state_len, const float* x, uint64_t x_len, const float* weight,
+                         uint64_t w_len, uint64_t kernel, uint64_t dilation, float* out, uint64_t out_len); /* :884 */
+void it_hip_qsa_pool(it_hip*, const uint16_t* raw, uint64_t raw_len, float* pooled, uint64_t pooled_len,
+                     const it_qsa_pool* p); /* mod.rs:941 */
+void it_hip_qsa_select(it_hip*, const float* q, uint64_t q_len, const float* pooled, uint64_t pooled_len,
+                       const it_qsa_select* s, float* scores, uint64_t scores_len, uint32_t* cells,
+                       uint64_t cells_len); /* mod.rs:954 */
+void it_hip_attend_sparse(it_hip*, const it_attn* a, const uint32_t* cells, uint64_t cells_len,
+                          const it_qsa_select* sel, float* out, uint64_t out_len); /* mod.rs:966 */
+
 /* ---- residency protocol (mod.rs:1360-1419) ---- */
 void it_hip_host_wrote(it_hip*, const float* buf, uint64_t len);
 void it_hip_host_needs(it_hip*, float* buf, uint64_t len);

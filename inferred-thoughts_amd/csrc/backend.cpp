@@ -25,6 +25,19 @@ uint64_t type_row_bytes(uint32_t ty, uint64_t n_in) {
         default: return 0;
     }
 }
+// A cheap identity of a host weight: its length and 48 sampled bytes.  Resident copies are keyed on the host address,
+// and a second model file mapped where the first one was has the same addresses, types and shapes.
+uint64_t weight_ident(const uint8_t* data, uint64_t len) {
+    uint64_t h = 0xcbf29ce484222325ull ^ len;
+    auto mix = [&](const uint8_t* p, uint64_t n) {
+        for (uint64_t i = 0; i < n; i++) h = (h ^ p[i]) * 0x100000001b3ull;
+    };
+    const uint64_t n = len < 16 ? len : 16;
+    mix(data, n);
+    mix(data + (len - n) / 2, n);
+    mix(data + len - n, n);
+    return h;
+}
 uint64_t now_us() {
     return (uint64_t)std::chrono::duration_cast<std::chrono::microseconds>(
                std::chrono::steady_clock::now().time_since_epoch())
@@ -74,6 +87,7 @@ void it_hip::drop_graph() {
     graph.graph = nullptr;
     graph.valid = false;
     graph.signature.clear();
+    graph.attn_slots.clear();
     stable_passes = 0;
 }
 
@@ -123,6 +137,7 @@ void it_hip::finish_pass() {
                 graph.graph = g;
                 graph.exec = ex;
                 graph.signature = pass_signature;
+                graph.attn_slots = fused_attn_slots;
                 graph.valid = true;
                 graph_captures++;
                 stable_passes = 1;
@@ -144,6 +159,11 @@ void it_hip::finish_pass() {
             need_eager("the pass ended early");
             return;
         }
+        if (!attn_positions_agree(graph.attn_slots)) {
+            mode = Mode::Replay;
+            need_eager("a fused attention block's rope, cache-write and context positions do not agree");
+            return;
+        }
     }
     for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
     precopies.clear();
@@ -156,6 +176,16 @@ void it_hip::finish_pass() {
         graph_launches++;
     }
     pending.clear();
+}
+
+bool it_hip::attn_positions_agree(const std::vector<std::array<int, 4>>& slots) const {
+    for (const auto& t : slots) {
+        for (int i : t)
+            if (i < 0 || (size_t)i >= dyn_count) return false;
+        const int pos = dyn_host[t[0]];
+        if (dyn_host[t[1]] != pos || dyn_host[t[2]] != pos || dyn_host[t[3]] != pos + 1) return false;
+    }
+    return true;
 }
 
 void it_hip::fail(const std::string& what) {
@@ -263,9 +293,12 @@ bool it_hip::act_quantized(const float* host, size_t len, const float** scales, 
 
 const float* it_hip::const_in(const float* host, size_t len) {
     auto it = consts.find(host);
-    if (it != consts.end() && it->second.len >= len) return it->second.dev;
+    const uint64_t ident = weight_ident((const uint8_t*)host, len * sizeof(float));
+    if (it != consts.end() && it->second.len == len && it->second.ident == ident) return it->second.dev;
     need_eager("a constant is uploaded for the first time");
+    if (it != consts.end()) drop_graph();  // a captured graph holds the copy that is about to go
     Const c;
+    c.ident = ident;
     if (!check(hipMalloc((void**)&c.dev, len * sizeof(float)), "hipMalloc(constant)")) return nullptr;
     if (!check(hipMemcpyAsync(c.dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream), "upload constant"))
         return nullptr;
@@ -282,12 +315,6 @@ const float* it_hip::const_in(const float* host, size_t len) {
 // ------------------------------------------------------------------ weights
 const it_hip::Resident* it_hip::resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in,
                                          uint64_t rows, const char* who) {
-    auto it = weights.find(data);
-    if (it != weights.end()) {
-        if (it->second.fmt == (int)ty && it->second.n_in == n_in && it->second.rows == rows) return &it->second;
-        fail(std::string(who) + ": a weight address was seen before with a different shape");
-        return nullptr;
-    }
     uint64_t row_bytes = type_row_bytes(ty, n_in);
     if (row_bytes == 0) {
         fail(std::string(who) + ": unsupported weight type or row length not a whole number of blocks");
@@ -297,12 +324,35 @@ const it_hip::Resident* it_hip::resident(const uint8_t* data, uint64_t len, uint
         fail(std::string(who) + ": weight byte length does not match its shape");
         return nullptr;
     }
+    auto it = weights.find(data);
+    if (it != weights.end()) {
+        const bool same_shape = it->second.fmt == (int)ty && it->second.n_in == n_in && it->second.rows == rows;
+        if (same_shape && it->second.ident == weight_ident(data, len)) return &it->second;
+        if (same_shape && it->second.counter_base < 0) {
+            // the same address, type and shape but other bytes: another file was mapped where the last one was.
+            // The stale copy goes and the weight is uploaded again.  (An expert tensor keeps its slots and counters
+            // for the life of the pool: that case is refused below.)
+            need_eager("a resident weight no longer matches its host bytes");
+            drop_graph();
+            check(hipStreamSynchronize(stream), "sync before a stale weight is freed");
+            weight_bytes -= it->second.q_bytes + it->second.s_bytes;
+            if (it->second.q) (void)hipFree(it->second.q);
+            if (it->second.scales) (void)hipFree(it->second.scales);
+            if (it->second.scale2) (void)hipFree(it->second.scale2);
+            weights.erase(it);
+        } else {
+            fail(std::string(who) + (same_shape ? ": a pooled expert tensor changed under its address; call drop_mirrors when a model file is unmapped"
+                                                : ": a weight address was seen before with a different shape"));
+            return nullptr;
+        }
+    }
     need_eager("a weight is uploaded for the first time");
     uint64_t t0 = now_us();
     Resident r;
     r.fmt = (int)ty;
     r.n_in = n_in;
     r.rows = rows;
+    r.ident = weight_ident(data, len);
     void* raw = nullptr;
     if (!check(hipMalloc(&raw, len), "hipMalloc(weight upload)")) return nullptr;
     if (!check(hipMemcpyAsync(raw, data, len, hipMemcpyHostToDevice, stream), "upload weight")) return nullptr;
@@ -1082,7 +1132,15 @@ void it_hip_attend(it_hip* be, const it_attn* a, float* out, uint64_t out_len) {
         be->submit(it_hip::FAM_ATTEND, bytes,
                    sig_of(OP_ATTEND, 1, dq, dk, dv, args.n_q, args.kv_dim, args.head_dim, args.n_head, args.n_head_kv,
                           args.scale, dyn, dyn ? n_split : 0, sc, dout), rec,
-                   [=](hipStream_t s) { attend_split(args, n_split, sc, dout, s); });
+                   [=](hipStream_t s) {
+                       // a one-pass prefill reserved the decode passes' scratch only: it must not fall into the split
+                       // kernels, whose partials for the whole batch would not fit there
+                       if (one_pass) {
+                           if (!attend_prefill(args, dout, s)) be->fail("attend: the one-pass prefill kernel could not be launched");
+                       } else if (!attend_split_gated(args, n_split, sc, dout, nullptr, 0, s)) {
+                           be->fail("attend: the split-K kernels could not be launched");
+                       }
+                   });
     }
 }
 
@@ -1481,6 +1539,24 @@ void it_hip_kv_write(it_hip* be, uint16_t* slab, uint64_t slab_len, uint64_t off
                [=](hipStream_t s) { kv_write(dslab, off, dyn, mul, ds, n, s); });
 }
 
+
+// ------------------------------------------------------------------ qwen4exp-only methods (mod.rs:705-966)
+// Outside this backend's path: nothing is launched, the first such call leaves its name in the sticky error.
+#define IT_UNSUPPORTED(name) be->fail(name ": qwen4exp-only op, not implemented by the hip backend")
+void it_hip_mean_streams(it_hip* be, const float*, uint64_t, uint64_t, uint64_t, float, float*, uint64_t) { IT_UNSUPPORTED("mean_streams"); }
+void it_hip_mul_rows(it_hip* be, float*, uint64_t, const float*, uint64_t) { IT_UNSUPPORTED("mul_rows"); }
+void it_hip_silu(it_hip* be, float*, uint64_t) { IT_UNSUPPORTED("silu"); }
+void it_hip_sigmoid(it_hip* be, float*, uint64_t) { IT_UNSUPPORTED("sigmoid"); }
+void it_hip_mul_streams(it_hip* be, float*, uint64_t, const float*, uint64_t, const float*, uint64_t, uint64_t) { IT_UNSUPPORTED("mul_streams"); }
+void it_hip_row_dot(it_hip* be, const float*, uint64_t, const float*, uint64_t, uint64_t, float*, uint64_t) { IT_UNSUPPORTED("row_dot"); }
+void it_hip_signed_sqrt_sigmoid(it_hip* be, float*, uint64_t) { IT_UNSUPPORTED("signed_sqrt_sigmoid"); }
+void it_hip_dilated_conv(it_hip* be, float*, uint64_t, const float*, uint64_t, const float*, uint64_t, uint64_t, uint64_t, float*,
+                         uint64_t) { IT_UNSUPPORTED("dilated_conv"); }
+void it_hip_qsa_pool(it_hip* be, const uint16_t*, uint64_t, float*, uint64_t, const it_qsa_pool*) { IT_UNSUPPORTED("qsa_pool"); }
+void it_hip_qsa_select(it_hip* be, const float*, uint64_t, const float*, uint64_t, const it_qsa_select*, float*, uint64_t, uint32_t*,
+                       uint64_t) { IT_UNSUPPORTED("qsa_select"); }
+void it_hip_attend_sparse(it_hip* be, const it_attn*, const uint32_t*, uint64_t, const it_qsa_select*, float*, uint64_t) { IT_UNSUPPORTED("attend_sparse"); }
+#undef IT_UNSUPPORTED
 
 // ------------------------------------------------------------------ residency
 void it_hip_host_wrote(it_hip* be, const float* buf, uint64_t len) {

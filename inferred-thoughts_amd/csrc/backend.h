@@ -9,6 +9,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <array>
 #include <cstdint>
 #include <cstring>
 #include <functional>
@@ -82,6 +83,7 @@ struct it_hip {
     struct Const {
         float* dev = nullptr;
         size_t len = 0;
+        uint64_t ident = 0;  // as for weights: the vectors of another model may sit at the same host address
     };
     std::unordered_map<const void*, Const> consts;
     const float* const_in(const float* host, size_t len);
@@ -95,6 +97,7 @@ struct it_hip {
         uint64_t n_in = 0, rows = 0;
         float* scale2 = nullptr;  // experts' per-expert second scale
         int64_t counter_base = -1;  // first of this tensor's entries in expert_counts (expert tensors only)
+        uint64_t ident = 0;         // length and a sample of the host bytes: another file mapped at the same address differs
     };
     std::unordered_map<const void*, Resident> weights;
     const Resident* resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in, uint64_t rows,
@@ -168,6 +171,10 @@ struct it_hip {
         hipGraphExec_t exec = nullptr;
         std::vector<uint64_t> signature;  // hash of each seam call's static arguments
         bool valid = false;
+        // position slots of every fused attention block: {rope, key write, value write, attend}.  The fused kernel
+        // takes ONE position for all four, so a replay is only valid while write row == rope position and the
+        // context length == position + 1 (the seam does not tie them together; the model loop does)
+        std::vector<std::array<int, 4>> attn_slots;
     };
     Graph graph;
     enum class Mode { Eager, Capture, Replay } mode = Mode::Eager;
@@ -190,6 +197,8 @@ struct it_hip {
     unsigned* route_counter = nullptr;  // device word used by the fused router (zero between launches)
     uint64_t fused_launches = 0;  // launches in the captured graph after fusion
     void run_fused(std::vector<OpRec>& ops);
+    std::vector<std::array<int, 4>> fused_attn_slots;  // filled by run_fused for the pass being captured
+    bool attn_positions_agree(const std::vector<std::array<int, 4>>& slots) const;
     struct PreCopy {
         void* dev;
         const void* host;

@@ -16,6 +16,7 @@ using Op = it_hip::OpRec;
 namespace {
 
 struct Plan {
+    it_hip* be;
     std::vector<Op>& ops;
     std::vector<char> consumed;
     struct Launch {
@@ -27,7 +28,12 @@ struct Plan {
     void add(size_t i, int fam, uint64_t bytes, std::function<void(hipStream_t)> fn) {
         at[i].push_back(Launch{fam, bytes, std::move(fn)});
     }
-    explicit Plan(std::vector<Op>& o) : ops(o), consumed(o.size(), 0), at(o.size()) {}
+    Plan(it_hip* b, std::vector<Op>& o) : be(b), ops(o), consumed(o.size(), 0), at(o.size()) {}
+    // slot of a position scalar in the pass's device array, -1 when the pointer is not one
+    int dyn_index(const void* p) const {
+        const int* q = (const int*)p;
+        return q >= be->dyn_dev && q < be->dyn_dev + it_hip::DYN_CAP ? (int)(q - be->dyn_dev) : -1;
+    }
     bool ids(size_t i, std::initializer_list<int> want) const {
         if (i + want.size() > ops.size()) return false;
         size_t k = i;
@@ -272,6 +278,11 @@ bool match_attn(Plan& pl, size_t i, int exact) {
         wv.i[2] != kvd || wk.p[0] != at.p[1] || wv.p[0] != at.p[2])
         return false;
     if (at.p[0] != qb) return false;
+    // One position feeds the fused block's rotation, cache writes and context length.  The seam passes them
+    // separately, so they are compared here (this pass's values) and again before every replay.
+    const std::array<int, 4> slots = {pl.dyn_index(rq.p[2]), pl.dyn_index(wk.p[1]), pl.dyn_index(wv.p[1]), pl.dyn_index(at.p[3])};
+    if (pl.dyn_index(rk.p[2]) < 0 || pl.be->dyn_host[pl.dyn_index(rk.p[2])] != pl.be->dyn_host[slots[0] < 0 ? 0 : slots[0]]) return false;
+    if (!pl.be->attn_positions_agree({slots})) return false;
     const void* attn = at.p[5];
     if (sg.i[0] != 1 || sg.p[0] != attn || sg.p[1] != gb || sg.i[1] != hd * nh) return false;
     if (q2.p[0] != attn || q2.i[0] != hd * nh || !mm_reads(mo, attn, q2)) return false;
@@ -325,6 +336,8 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
 
     pl.take(i, 18);
+    pl.be->fused_attn_slots.push_back(slots);
+    it_hip* be = pl.be;
     // K and V rows of the live context, f16 (the position is the one this pass was recorded at)
     const uint64_t kv_bytes = (uint64_t)at.i[8] * kvd * 2 * 2;
     pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
@@ -342,10 +355,16 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     if (at.i[6] == 0 && attend_tile_prep_ok(aa, tp)) {
         // norm + rotation of q and of the new key, and the slab writes, happen inside the tile kernel
         pl.add(i, it_hip::FAM_ATTEND, kv_bytes + (uint64_t)(2 * hd * nh + 2 * kvd) * 4,
-               [=](hipStream_t s) { attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s); });
+               [=](hipStream_t s) {
+                   if (!attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s))
+                       be->fail("attend: the split-K kernels could not be launched");
+               });
     } else if (at.i[6] == 0) {
         pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
-        pl.add(i, it_hip::FAM_ATTEND, kv_bytes, [=](hipStream_t s) { attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s); });
+        pl.add(i, it_hip::FAM_ATTEND, kv_bytes, [=](hipStream_t s) {
+            if (!attend_split_gated(aa, n_split, scratch, attn_out, gate, gate_stride, s))
+                be->fail("attend: the split-K kernels could not be launched");
+        });
     } else {
         pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
         // the exact attention kernel and its gate stay as they are
@@ -504,7 +523,8 @@ bool references(const Op& op, const void* a, const void* b) {
 }  // namespace
 
 void it_hip::run_fused(std::vector<OpRec>& ops) {
-    Plan pl(ops);
+    Plan pl(this, ops);
+    fused_attn_slots.clear();
     if (fuse_enabled) {
         for (size_t i = 0; i < ops.size(); i++) {
             if (pl.consumed[i]) continue;

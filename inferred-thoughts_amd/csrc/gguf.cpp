@@ -19,6 +19,14 @@ uint64_t type_bytes(uint32_t ty, uint64_t n) {
     }
 }
 
+bool type_bytes_checked(uint32_t ty, uint64_t n, uint64_t* out) {
+    switch (ty) {
+        case 0: return !__builtin_mul_overflow(n, (uint64_t)4, out);
+        case 1: case 30: return !__builtin_mul_overflow(n, (uint64_t)2, out);
+        default: *out = type_bytes(ty, n); return true;  // block formats shrink: n / 32 * 34 and n / 64 * 36 cannot wrap
+    }
+}
+
 namespace {
 struct Reader {
     const uint8_t* p;
@@ -116,6 +124,7 @@ bool File::open(const std::string& path, std::string* err) {
             uint64_t n = r.take<uint64_t>();
             if (et == 5) {
                 std::vector<int32_t> v;
+                if (n > (uint64_t)(r.end - r.p) / 4) return bad("array longer than the file at " + key);
                 for (uint64_t k = 0; k < n && r.ok; k++) v.push_back(r.take<int32_t>());
                 meta_[key] = std::move(v);
             } else if (et == 8) {
@@ -123,7 +132,9 @@ bool File::open(const std::string& path, std::string* err) {
             } else {
                 size_t w = width_of(et);
                 if (w == 0) return bad("unknown array element type at " + key);
-                r.skip(w * n);
+                uint64_t bytes = 0;
+                if (__builtin_mul_overflow((uint64_t)w, n, &bytes)) return bad("array length overflows at " + key);
+                r.skip(bytes);
             }
         } else {
             Value v;
@@ -148,15 +159,25 @@ bool File::open(const std::string& path, std::string* err) {
     uint64_t align = 32;
     get_uint("general.alignment", &align);
     if (align == 0) return bad("zero alignment");
-    size_t pos = (size_t)(r.p - base_);
-    data_start_ = (pos + align - 1) / align * align;
+    if (align > (1ull << 30)) return bad("implausible alignment");
+    const uint64_t pos = (uint64_t)(r.p - base_);
+    uint64_t start = 0;
+    if (__builtin_add_overflow(pos, align - 1, &start)) return bad("header end overflows");
+    start = start / align * align;
+    if (start > size_) return bad("the data blob starts past the end of the file");
+    data_start_ = (size_t)start;
+    const uint64_t blob = size_ - data_start_;
+    // Every size below comes from the file: each product and sum is checked, so that a huge dimension or offset
+    // cannot wrap round into a small number that passes the bounds test and later indexes outside the mapping.
     for (const Tensor& t : tensors_) {
-        uint64_t nb = type_bytes(t.ty, t.n_elems());
-        if (nb == 0 && t.n_elems() != 0) return bad("tensor " + t.name + " has an unsupported type or partial blocks");
+        uint64_t n = 0, nb = 0;
+        if (!t.n_elems_checked(&n)) return bad("tensor " + t.name + ": element count overflows");
+        if (!type_bytes_checked(t.ty, n, &nb)) return bad("tensor " + t.name + ": byte size overflows");
+        if (nb == 0 && n != 0) return bad("tensor " + t.name + " has an unsupported type or partial blocks");
         if (t.dims.empty() || (t.ty == 8 && t.dims[0] % 32) || (t.ty == 40 && t.dims[0] % 64))
             return bad("tensor " + t.name + ": row length is not a whole number of blocks");
         if (t.offset % align) return bad("tensor " + t.name + " is misaligned");
-        if (data_start_ + t.offset + nb > size_) return bad("tensor " + t.name + " runs past the end of the file");
+        if (t.offset > blob || nb > blob - t.offset) return bad("tensor " + t.name + " runs past the end of the file");
     }
     return true;
 }

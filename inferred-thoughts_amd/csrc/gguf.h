@@ -17,7 +17,15 @@ struct Tensor {
     std::vector<uint64_t> dims;  // ggml order: dims[0] is the row length
     uint32_t ty = 0;
     uint64_t offset = 0;  // relative to the data blob
-    uint64_t n_elems() const {
+    // the product of the dims; false when it does not fit 64 bits (a corrupt or hostile file)
+    bool n_elems_checked(uint64_t* out) const {
+        uint64_t n = 1;
+        for (auto d : dims)
+            if (__builtin_mul_overflow(n, d, &n)) return false;
+        *out = n;
+        return true;
+    }
+    uint64_t n_elems() const {  // of a tensor File::open has accepted
         uint64_t n = 1;
         for (auto d : dims) n *= d;
         return n;
@@ -52,5 +60,7 @@ class File {
 // bytes of `n` elements of a ggml type; 0 when unsupported or not whole blocks
 // (src/gguf/types.rs:143-210)
 uint64_t type_bytes(uint32_t ty, uint64_t n);
+// the same with the multiplication checked: false when the byte count does not fit 64 bits
+bool type_bytes_checked(uint32_t ty, uint64_t n, uint64_t* out);
 
 }  // namespace itg

@@ -681,9 +681,9 @@ __global__ __launch_bounds__(256) void attend_merge_wide_k(const float* __restri
     }
 }
 
-void attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hipStream_t s) {
-    if (attend_prefill(a, out, s)) return;
-    attend_split_gated(a, n_split, scratch, out, nullptr, 0, s);
+bool attend_split(const AttnArgs& a, int n_split, float* scratch, float* out, hipStream_t s) {
+    if (attend_prefill(a, out, s)) return true;
+    return attend_split_gated(a, n_split, scratch, out, nullptr, 0, s);
 }
 
 // queries at or below this count take the tile kernel (chunk TILE); larger batches the
@@ -710,22 +710,24 @@ bool attend_tile_prep_ok(const AttnArgs& a, const TilePrepP& pr) {
     return a.kv_dim % 4 == 0;
 }
 
-static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
+static bool attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
                               const float* gate, int gate_stride, hipStream_t s);
 
-void attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* out, const float* gate,
+bool attend_split_gated(const AttnArgs& a, int n_split, float* scratch, float* out, const float* gate,
                         int gate_stride, hipStream_t s) {
-    attend_split_impl(a, nullptr, n_split, scratch, out, gate, gate_stride, s);
+    return attend_split_impl(a, nullptr, n_split, scratch, out, gate, gate_stride, s);
 }
 
-void attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
+bool attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
                              const float* gate, int gate_stride, hipStream_t s) {
-    attend_split_impl(a, &pr, n_split, scratch, out, gate, gate_stride, s);
+    return attend_split_impl(a, &pr, n_split, scratch, out, gate, gate_stride, s);
 }
 
-static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
+// false: nothing was launched and `out` is untouched (a group size the kernels do not take, or the tile kernel's
+// LDS size could not be set); the caller records the error
+static bool attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_split, float* scratch, float* out,
                               const float* gate, int gate_stride, hipStream_t s) {
-    if (a.n_q <= 0) return;
+    if (a.n_q <= 0) return true;
     const int G = a.n_head / a.n_head_kv;
     dim3 grid(a.n_q * a.n_head_kv, n_split), block(256);
     const bool tile = tile_path(a.n_q, a.head_dim, G);
@@ -738,7 +740,7 @@ static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_sp
             const void* fn = prep ? (const void*)attend_decode_k<HD, GG, true> : (const void*)attend_decode_k<HD, GG, false>; \
             if (lds > 64 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { \
                 (void)hipGetLastError();                                                                         \
-                return;                                                                                          \
+                return false;                                                                                    \
             }                                                                                                    \
             sized[prep ? 1 : 0] = true;                                                                          \
         }                                                                                                        \
@@ -751,7 +753,7 @@ static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_sp
         case 2: IT_TILE(HD, 2); break; \
         case 4: IT_TILE(HD, 4); break; \
         case 8: IT_TILE(HD, 8); break; \
-        default: return;               \
+        default: return false;         \
     }
         if (a.head_dim == 64) { IT_TILE_G(64) }
         else if (a.head_dim == 128) { IT_TILE_G(128) }
@@ -765,17 +767,18 @@ static void attend_split_impl(const AttnArgs& a, const TilePrepP* prep, int n_sp
             case 2: hipLaunchKernelGGL(attend_split_k<2>, grid, block, lds, s, a, n_split, scratch); break;
             case 4: hipLaunchKernelGGL(attend_split_k<4>, grid, block, lds, s, a, n_split, scratch); break;
             case 8: hipLaunchKernelGGL(attend_split_k<8>, grid, block, lds, s, a, n_split, scratch); break;
-            default: return;  // the caller falls back to the exact kernel for other group sizes
+            default: return false;  // the caller takes the exact kernel for other group sizes
         }
     }
     if (tile && n_split <= MERGE_MAX_SPLIT && a.head_dim % 32 == 0) {
         hipLaunchKernelGGL(attend_merge_wide_k, dim3(a.n_q * a.n_head, a.head_dim / 32), dim3(256), 0, s, scratch, n_split,
                            a.head_dim, out, gate, gate_stride);
-        return;
+        return true;
     }
     hipLaunchKernelGGL(attend_merge_k, dim3(a.n_q * a.n_head), dim3(4 * a.head_dim),
                        (size_t)(n_split + 4 * a.head_dim) * sizeof(float), s, scratch, n_split, a.head_dim, out, gate,
                        gate_stride, a.n_q, a.n_head, tile ? 1 : CHUNK, a.n_pos, a.n_pos_dyn);  // the few-query kernel spreads the keys over every split
+    return true;
 }
 
 }  // namespace itk

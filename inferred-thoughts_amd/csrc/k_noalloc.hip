@@ -97,7 +97,8 @@ extern "C" int it_hip_attend_noalloc(const it_attn* a, float* out, uint64_t out_
     if (e != hipSuccess) return fail(err, err_len, 3, "attend_noalloc: hipGetSymbolAddress(scratch)", hipGetErrorString(e));
     itk::AttnArgs args{a->q, a->k, a->v, (int)n_q, (int)a->kv_dim, (int)a->n_pos, (int)a->head_dim,
                        (int)a->n_head, (int)a->n_head_kv, a->scale, nullptr};
-    itk::attend_split_gated(args, n_split, part, out, nullptr, 0, (hipStream_t)stream);
+    if (!itk::attend_split_gated(args, n_split, part, out, nullptr, 0, (hipStream_t)stream))
+        return fail(err, err_len, 3, "attend_noalloc: the split-K kernels could not be launched");
     e = hipGetLastError();
     if (e != hipSuccess) return fail(err, err_len, 3, "attend_noalloc: kernel launch", hipGetErrorString(e));
     return 0;

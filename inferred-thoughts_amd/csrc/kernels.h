@@ -147,7 +147,7 @@ struct AttnArgs {
 void attend_exact(const AttnArgs& a, float* scratch, float* out, hipStream_t s);
 // split-K flash decoding; scratch: n_q*n_head*n_split*(head_dim+2) floats.
 int attend_split_count(int n_pos_max, int n_q, int head_dim, int group);
-void attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);
+bool attend_split(const AttnArgs& a, int n_split_max, float* scratch, float* out, hipStream_t s);  // false: not launched
 // more than 16 queries, fast mode: one pass over the keys on the f16 matrix cores; false when the shape is not taken
 bool attend_prefill(const AttnArgs& a, float* out, hipStream_t s);
 bool attend_prefill_takes(const AttnArgs& a, const float* out);
@@ -163,10 +163,10 @@ struct TilePrepP {
     uint16_t *k_slab, *v_slab;
 };
 bool attend_tile_prep_ok(const AttnArgs& a, const TilePrepP& pr);
-void attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
+bool attend_split_gated_prep(const AttnArgs& a, const TilePrepP& pr, int n_split, float* scratch, float* out,
                              const float* gate, int gate_stride, hipStream_t s);
 // the same with the merge multiplying by sigmoid(gate[head * gate_stride + i]) (n_q == 1)
-void attend_split_gated(const AttnArgs& a, int n_split_max, float* scratch, float* out, const float* gate,
+bool attend_split_gated(const AttnArgs& a, int n_split_max, float* scratch, float* out, const float* gate,
                         int gate_stride, hipStream_t s);
 
 }  // namespace itk

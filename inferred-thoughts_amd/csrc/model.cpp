@@ -242,8 +242,12 @@ struct it_model {
 // (src/model/qwen35.rs:572-583, 653-673).
 struct HostBuf {
     std::vector<float> v;
-    void fit(uint64_t n) {
-        if (v.size() < n) v.resize(n, 0.0f);
+    // Growing moves the buffer: the backend's mirror and quantized copy are keyed on the OLD address and would
+    // otherwise leak, or be inherited by whatever the allocator places there next.
+    void fit(uint64_t n, it_hip* be) {
+        if (v.size() >= n) return;
+        if (!v.empty() && n > v.capacity()) it_hip_release(be, v.data());
+        v.resize(n, 0.0f);
     }
     float* p() { return v.data(); }
 };
@@ -282,18 +286,18 @@ constexpr uint64_t MOE_CHUNK = 512;  // src/model/qwen35.rs:650: the reference's
 
 void fit(it_engine* e, uint64_t n) {
     const Dims& d = e->m->d;
-    e->x.fit(n * d.n_embd); e->normed.fit(n * d.n_embd); e->mixed.fit(n * d.n_embd); e->ffn_out.fit(n * d.n_embd);
-    e->qg.fit(n * d.q_gate()); e->q.fit(n * d.q_dim()); e->g.fit(n * d.q_dim());
-    e->k.fit(n * d.kv_dim()); e->v.fit(n * d.kv_dim()); e->attn.fit(n * d.q_dim());
-    e->qkv.fit(n * d.conv_dim()); e->z.fit(n * d.value_dim()); e->alpha.fit(n * d.dt_rank); e->beta.fit(n * d.dt_rank);
-    e->convo.fit(n * d.conv_dim()); e->q_part.fit(n * d.key_dim()); e->k_part.fit(n * d.key_dim());
-    e->v_part.fit(n * d.value_dim()); e->core.fit(n * d.value_dim());
+    e->x.fit(n * d.n_embd, e->be); e->normed.fit(n * d.n_embd, e->be); e->mixed.fit(n * d.n_embd, e->be); e->ffn_out.fit(n * d.n_embd, e->be);
+    e->qg.fit(n * d.q_gate(), e->be); e->q.fit(n * d.q_dim(), e->be); e->g.fit(n * d.q_dim(), e->be);
+    e->k.fit(n * d.kv_dim(), e->be); e->v.fit(n * d.kv_dim(), e->be); e->attn.fit(n * d.q_dim(), e->be);
+    e->qkv.fit(n * d.conv_dim(), e->be); e->z.fit(n * d.value_dim(), e->be); e->alpha.fit(n * d.dt_rank, e->be); e->beta.fit(n * d.dt_rank, e->be);
+    e->convo.fit(n * d.conv_dim(), e->be); e->q_part.fit(n * d.key_dim(), e->be); e->k_part.fit(n * d.key_dim(), e->be);
+    e->v_part.fit(n * d.value_dim(), e->be); e->core.fit(n * d.value_dim(), e->be);
     uint64_t nt = n < e->moe_chunk ? n : e->moe_chunk;
     uint64_t ff = d.expert_ff > d.shared_ff ? d.expert_ff : d.shared_ff;
-    e->router.fit(nt * d.n_expert); e->e_gate.fit(nt * ff); e->e_up.fit(nt * ff); e->e_out.fit(nt * d.n_embd);
-    e->e_in.fit(nt * d.n_embd); e->g_all.fit(nt * d.n_used * d.expert_ff); e->u_all.fit(nt * d.n_used * d.expert_ff);
-    e->o_all.fit(nt * d.n_used * d.n_embd); e->shexp_logit.fit(nt);
-    e->last.fit(d.n_embd); e->final_norm.fit(d.n_embd); e->logits.fit(d.n_vocab);
+    e->router.fit(nt * d.n_expert, e->be); e->e_gate.fit(nt * ff, e->be); e->e_up.fit(nt * ff, e->be); e->e_out.fit(nt * d.n_embd, e->be);
+    e->e_in.fit(nt * d.n_embd, e->be); e->g_all.fit(nt * d.n_used * d.expert_ff, e->be); e->u_all.fit(nt * d.n_used * d.expert_ff, e->be);
+    e->o_all.fit(nt * d.n_used * d.n_embd, e->be); e->shexp_logit.fit(nt, e->be);
+    e->last.fit(d.n_embd, e->be); e->final_norm.fit(d.n_embd, e->be); e->logits.fit(d.n_vocab, e->be);
 }
 
 void moe_batch(it_engine* e, const Block& b, uint64_t at, uint64_t n, uint64_t total) {

@@ -100,7 +100,8 @@ it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
 it_engine_v_slab it_synth_write_gguf it_hip_attend_noalloc it_hip_reserve_for_weights it_hip_reserve_for_kv
 it_hip_set_prefetch it_hip_set_model_path it_hip_set_map_base it_hip_expert_coverage it_hip_replace_experts_by_counts
-it_hip_expert_counts""".split()
+it_hip_expert_counts it_hip_mean_streams it_hip_mul_rows it_hip_silu it_hip_sigmoid it_hip_mul_streams it_hip_row_dot
+it_hip_signed_sqrt_sigmoid it_hip_dilated_conv it_hip_qsa_pool it_hip_qsa_select it_hip_attend_sparse""".split()
 
 _lib = None
 
@@ -183,6 +184,17 @@ def lib() -> C.CDLL:
         "it_hip_expert_coverage": (C.c_int, [vp, vp, vp]),
         "it_hip_replace_experts_by_counts": (C.c_int64, [vp]),
         "it_hip_expert_counts": (u64, [vp, vp, vp, u64]),
+        "it_hip_mean_streams": (None, [vp, vp, u64, u64, u64, f32, vp, u64]),
+        "it_hip_mul_rows": (None, [vp, vp, u64, vp, u64]),
+        "it_hip_silu": (None, [vp, vp, u64]),
+        "it_hip_sigmoid": (None, [vp, vp, u64]),
+        "it_hip_mul_streams": (None, [vp, vp, u64, vp, u64, vp, u64, u64]),
+        "it_hip_row_dot": (None, [vp, vp, u64, vp, u64, u64, vp, u64]),
+        "it_hip_signed_sqrt_sigmoid": (None, [vp, vp, u64]),
+        "it_hip_dilated_conv": (None, [vp, vp, u64, vp, u64, vp, u64, u64, u64, vp, u64]),
+        "it_hip_qsa_pool": (None, [vp, vp, u64, vp, u64, vp]),
+        "it_hip_qsa_select": (None, [vp, vp, u64, vp, u64, vp, vp, u64, vp, u64]),
+        "it_hip_attend_sparse": (None, [vp, vp, vp, u64, vp, vp, u64]),
         "it_hip_clock_pick": (C.c_int64, [vp, vp, u64, vp]),
         "it_hip_argmax": (u32, [vp, vp, u64]),
         "it_hip_sync": (None, [vp]),

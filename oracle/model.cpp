@@ -183,15 +183,23 @@ struct Gguf {
         uint64_t align = u.count("general.alignment") ? u["general.alignment"] : 32;
         size_t pos = (size_t)(c.p - base);
         data_start = (pos + align - 1) / align * align;
+        if (data_start > size) {
+            err = "data blob starts past the end of the file";
+            return false;
+        }
         for (auto& kv : tensors) {
             uint64_t n = 1;
-            for (auto d : kv.second.dims) n *= d;
+            for (auto d : kv.second.dims)
+                if (__builtin_mul_overflow(n, d, &n) || n > (1ull << 56)) {
+                    err = "tensor element count overflows: " + kv.first;
+                    return false;
+                }
             uint64_t bytes = orc_type_bytes(kv.second.ty, n);
             if (bytes == 0 && n != 0) {
                 err = "unsupported tensor type in " + kv.first;
                 return false;
             }
-            if (data_start + kv.second.offset + bytes > size) {
+            if (kv.second.offset > size - data_start || bytes > size - data_start - kv.second.offset) {
                 err = "tensor past end of file: " + kv.first;
                 return false;
             }

@@ -100,3 +100,29 @@ def test_refusals():
     be.matmul_experts(ih.experts(wb, ih.Q8_0, n_in, n_out, n_expert), route, x, np.zeros(2 * n_out, np.float32))
     assert "holds 3" in (be.take_error() or "")
     be.end_pass(); be.close()
+
+
+def test_qwen4exp_only_methods_are_refused_not_run():
+    """The trait methods only the qwen4exp architecture calls (src/ops/mod.rs:705-966) are exported, launch nothing
+    and leave their name in the sticky error."""
+    import inferred_hip as ih
+    be = ih.Hip()
+    L, h = be.L, be.h
+    x = np.ones(8, np.float32); p = x.ctypes.data
+    calls = [("mean_streams", lambda: L.it_hip_mean_streams(h, p, 8, 2, 4, 0.5, p, 4)),
+             ("mul_rows", lambda: L.it_hip_mul_rows(h, p, 8, p, 4)), ("silu", lambda: L.it_hip_silu(h, p, 8)),
+             ("sigmoid", lambda: L.it_hip_sigmoid(h, p, 8)),
+             ("mul_streams", lambda: L.it_hip_mul_streams(h, p, 8, p, 4, p, 2, 2)),
+             ("row_dot", lambda: L.it_hip_row_dot(h, p, 8, p, 8, 4, p, 2)),
+             ("signed_sqrt_sigmoid", lambda: L.it_hip_signed_sqrt_sigmoid(h, p, 8)),
+             ("dilated_conv", lambda: L.it_hip_dilated_conv(h, p, 4, p, 8, p, 8, 2, 1, p, 8)),
+             ("qsa_pool", lambda: L.it_hip_qsa_pool(h, p, 8, p, 8, None)),
+             ("qsa_select", lambda: L.it_hip_qsa_select(h, p, 8, p, 8, None, p, 8, p, 8)),
+             ("attend_sparse", lambda: L.it_hip_attend_sparse(h, None, p, 8, None, p, 8))]
+    before = be.launch_count()
+    for name, call in calls:
+        call()
+        err = be.take_error() or ""
+        assert err.startswith(name + ":") and "qwen4exp-only" in err, (name, err)
+    assert be.launch_count() == before and np.array_equal(x, np.ones(8, np.float32))
+    be.close()

@@ -144,14 +144,15 @@ def test_attention_block(pair):
     slabs = [dict(k=k0.copy(), v=v0.copy()) for _ in range(2)]
     sc = float(1.0 / np.sqrt(np.float32(HD)))
 
-    def block(ops, i, b, s, pos):
+    def block(ops, i, b, s, pos, rope_pos=None):
+        rope_pos = pos if rope_pos is None else rope_pos
         W = lambda t: t[i]
         ops.rms_norm(b["x"], norm_w, EPS, b["normed"])
         ops.matmul(W(wq), b["normed"], b["qg"])
         ops.gather_chunks(b["qg"], HD, 2 * HD, 0, b["q"]); ops.gather_chunks(b["qg"], HD, 2 * HD, HD, b["g"])
         ops.matmul(W(wk), b["normed"], b["k"]); ops.matmul(W(wv), b["normed"], b["v"])
         ops.rms_norm_heads(b["q"], qn, HD, EPS); ops.rms_norm_heads(b["k"], kn, HD, EPS)
-        ops.rope_neox(b["q"], pos, HD, NROT, NH, THETA); ops.rope_neox(b["k"], pos, HD, NROT, NKV, THETA)
+        ops.rope_neox(b["q"], rope_pos, HD, NROT, NH, THETA); ops.rope_neox(b["k"], rope_pos, HD, NROT, NKV, THETA)
         ops.kv_write(s["k"], pos * kd, b["k"]); ops.kv_write(s["v"], pos * kd, b["v"])
         ops.attend(b["q"], s["k"], s["v"], kd, pos + 1, HD, NH, NKV, sc, b["attn"])
         ops.sigmoid_mul(b["attn"], b["g"])
@@ -186,6 +187,19 @@ def test_attention_block(pair):
             assert np.array_equal(a[:POS0 * kd], b[:POS0 * kd]) and not a[(pos + 1) * kd:].any()  # only new rows moved
             assert close(a[POS0 * kd:(pos + 1) * kd], b[POS0 * kd:(pos + 1) * kd], 2e-3), (p, t)   # one f16 step
     fused_graph_ran(hip, 3)      # q/k/v projections, attention with norm + rope + cache write folded in, out-proj
+    # The fused kernel takes ONE position for the rotation, the cache row and the context length; the seam passes
+    # them separately.  A pass whose rotation position differs from its cache row (same op sequence, so the graph's
+    # signature still matches) must not be replayed with the graph's single position: it runs op by op.
+    pos = POS0 + PASSES
+    x0 = rng(399).standard_normal(ND).astype(np.float32)
+    B[0]["x"][:] = x0; B[1]["x"][:] = x0
+    hip.begin_pass(1); hip.host_wrote(B[0]["x"]); block(hip, 0, B[0], slabs[0], pos, rope_pos=pos + 7); hip.end_pass()
+    hip.host_needs(B[0]["x"]); hip.host_needs(B[0]["attn"]); hip.read_kv(slabs[0]["k"]); hip.raise_if_error()
+    block(orc, 1, B[1], slabs[1], pos, rope_pos=pos + 7)
+    assert hip.graph_stats()["aborts"] == 1
+    assert close(B[0]["attn"], B[1]["attn"]), worst(B[0]["attn"], B[1]["attn"])
+    a = slabs[0]["k"].view(np.float16).astype(np.float32); b = slabs[1]["k"].view(np.float16).astype(np.float32)
+    assert close(a[pos * kd:(pos + 1) * kd], b[pos * kd:(pos + 1) * kd], 2e-3)
 
 
 # --------------------------------------------------------------------------------------------- routed FFN

@@ -120,3 +120,51 @@ def test_oracle_greedy_run_is_reproducible(tiny_gguf):
     a, _ = ob.Engine(m, 128).generate(prompt_ids(), 64)
     b, _ = ob.Engine(m, 128).generate(prompt_ids(), 64)
     assert len(a) == 64 and np.array_equal(a, b) and len(set(a.tolist())) > 8
+
+
+def _gguf_with_one_tensor(path, dims, ty, offset, extra_kv=b"", n_kv=1, pad_data=4096):
+    """A minimal GGUF v3 file: the architecture key (plus raw extra key/value bytes) and one tensor entry whose
+    dims, type and offset the caller chooses, followed by pad_data bytes of data."""
+    import struct
+
+    def s(b):
+        return struct.pack("<Q", len(b)) + b
+    out = bytearray(b"GGUF" + struct.pack("<Iqq", 3, 1, n_kv))
+    out += s(b"general.architecture") + struct.pack("<I", 8) + s(b"qwen35moe") + extra_kv
+    out += s(b"token_embd.weight") + struct.pack("<I", len(dims)) + struct.pack(f"<{len(dims)}q", *dims)
+    out += struct.pack("<IQ", ty, offset & (2 ** 64 - 1))
+    out += b"\0" * ((-len(out)) % 32) + b"\0" * pad_data
+    path.write_bytes(bytes(out))
+    return path
+
+
+def test_reader_checks_file_supplied_sizes_without_wrapping(tmp_path):
+    """Sizes read from the file (dims, offsets, array lengths) are combined with checked arithmetic: a product or
+    sum that wraps round 64 bits must not pass the bounds test (a tensor pointer outside the mapping would follow)."""
+    import struct
+    import inferred_hip as ih
+    cases = {
+        # 2^33 x 2^33 F32 elements: the product wraps to 0 elements
+        "dims": (_gguf_with_one_tensor(tmp_path / "dims.gguf", [1 << 33, 1 << 33], 0, 0), "overflows"),
+        # 2^62 F32 elements: the byte count wraps
+        "bytes": (_gguf_with_one_tensor(tmp_path / "bytes.gguf", [1 << 62], 0, 0), "overflows"),
+        # an offset just below 2^64: data_start + offset + size wraps to a small number
+        "offset": (_gguf_with_one_tensor(tmp_path / "offset.gguf", [64], 0, -64), "past the end"),
+        # an honest tensor that simply does not fit
+        "long": (_gguf_with_one_tensor(tmp_path / "long.gguf", [1 << 20], 0, 0), "past the end"),
+        # a u8 array whose length times its width wraps / exceeds the file
+        "array": (_gguf_with_one_tensor(tmp_path / "array.gguf", [64], 0, 0, n_kv=2,
+                                        extra_kv=struct.pack("<Q", 1) + b"k" + struct.pack("<IIQ", 9, 10, 1 << 62)),
+                  "overflows"),
+        "i32 array": (_gguf_with_one_tensor(tmp_path / "i32.gguf", [64], 0, 0, n_kv=2,
+                                            extra_kv=struct.pack("<Q", 1) + b"k" + struct.pack("<IIQ", 9, 5, 1 << 61)),
+                      "longer than the file"),
+    }
+    for name, (path, want) in cases.items():
+        with pytest.raises(RuntimeError) as e:
+            ih.Model(path)
+        assert want in str(e.value), (name, str(e.value))
+    from oracle import binding as ob
+    for name in ("dims", "bytes", "offset", "long"):
+        with pytest.raises(RuntimeError):
+            ob.Model(cases[name][0])
