@@ -27,12 +27,27 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0    # dense int8 MFMA, published
 FP32_MFMA_PEAK_TFLOPS = 157.3
-# HBM bytes per launch (fetched + written) of each kernel family, averaged over the full model's per-layer launches,
-# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by a 256 MiB copy
-# (profiles/decode_kernels_hbm_traffic_pmc.txt holds the commands and the per-kernel readings)
-PMC_TRAFFIC_BYTES = {"fused_gemv (norm + quantize + dense GEMVs)": 12_190_000, "moe_glu (expert gate+up)": 14_400_000,
-                     "matmul_experts (expert down)": 7_430_000, "gdn_rows (l2 norm + delta rule)": 4_400_000,
-                     "lm_head (norm + GEMV)": 331_660_000}
+# Per kernel family of the decode graph, from the committed rocprofv3 summary of this same workload
+# (profiles/decode_config5_families.txt: its "@" lines; the file says which commands made it): launches per token,
+# average duration in the replayed graph (--kernel-trace), HBM bytes fetched and written per launch (--pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by a 256 MiB copy).
+FAMILY_PROFILE = ROOT / "profiles" / "decode_config5_families.txt"
+
+
+def family_profile():
+    out = {}
+    try:
+        for line in FAMILY_PROFILE.read_text().splitlines():
+            if not line.startswith("@ "):
+                continue
+            f = [t.strip() for t in line[2:].split("|")]
+            if len(f) != 5 or f[0] == "family":
+                continue
+            out[f[0]] = {"launches_per_token": float(f[1]), "rocprof_avg_us": float(f[2]), "fetched": float(f[3]),
+                         "written": float(f[4])}
+    except OSError:
+        pass
+    return out
 
 
 def model_path(args):
@@ -117,6 +132,9 @@ def main():
                     help="stop after the timed decode stretch (no per-kernel events, no second prefill, no CPU leg): the "
                          "run to put under rocprofv3 --kernel-trace, whose last steps x graph-kernels records are then "
                          "the replayed decode graph and nothing else")
+    ap.add_argument("--no-exact-check", action="store_true",
+                    help="skip the exact-mode run of the same model (512-token prompt + 32 greedy ids) that the fast "
+                         "mode's ids are compared with")
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -276,6 +294,7 @@ def main():
     tok_bytes = w_bytes + state_bytes + kv_bytes
     whole = tok_bytes * tok_s / 1e9
 
+    headline = args.layers == 48 and args.prompt == 5700 and not args.router_f32 and not args.exact
     rows.sort(key=lambda r: -r["ms"])
     timed = [r for r in rows if r["bytes"]]
     dom = timed[0] if timed else None
@@ -285,11 +304,41 @@ def main():
     roofline = None
     if dom:
         ach = (dom["bytes"] / 1e9) / (dom["ms"] / 1e3)
+        per_launch = dom["bytes"] // dom["launches"]
+        prof = family_profile().get(dom["name"]) if headline else None
         roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                    "traffic": PMC_TRAFFIC_BYTES.get(dom["name"]) if args.layers == 48 else None,
+                    "traffic": int(prof["fetched"] + prof["written"]) if prof else None,
                     "avg_launch_us": round(1e3 * dom["ms"] / dom["launches"], 2),
-                    "bytes_per_launch": dom["bytes"] // dom["launches"]}
+                    "bytes_per_launch": per_launch,
+                    # the same fraction with the launch duration rocprofv3 reports for this family inside the replayed
+                    # graph (no event pair around the launch), from the committed summary
+                    "rocprof_avg_launch_us": prof["rocprof_avg_us"] if prof else None,
+                    "frac_rocprof": round(per_launch / (prof["rocprof_avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if prof else None,
+                    "profile": str(FAMILY_PROFILE.relative_to(ROOT)) if prof else None}
+
+    # the two arithmetic modes on this very model: a 512-token prompt and 32 greedy ids each.  Exact mode reproduces
+    # the CPU path bit for bit (the parity tests); fast mode differs in the last bits, and on random weights, whose
+    # logits are nearly tied, a last-bit difference soon picks another token, after which the runs are unrelated.
+    mode_check = None
+    if not args.exact and not args.no_exact_check:
+        n_p, n_g = min(512, args.prompt), 32
+        eng.reset()
+        lf = eng.prefill(prompt[:n_p])
+        ids_fast = np.asarray(eng.decode_greedy(n_g))
+        be_x = ih.Hip(exact=True)
+        eng_x = ih.Engine(model, be_x, args.ctx, args.max_batch)
+        lx = eng_x.prefill(prompt[:n_p])
+        ids_exact = np.asarray(eng_x.decode_greedy(n_g))
+        err = be_x.take_error() or be.take_error()
+        if err:
+            raise SystemExit(f"device error in the mode check: {err}")
+        same = ids_fast == ids_exact
+        mode_check = {"prompt": int(n_p), "ids": int(n_g), "ids_equal": int(same.sum()),
+                      "equal_prefix": int(np.argmin(same)) if not same.all() else int(n_g),
+                      "prefill_logits_max_abs_diff": float(np.abs(lf - lx).max()),
+                      "prefill_logits_max_abs": float(np.abs(lx).max())}
+        eng_x.close(); be_x.close()
 
     cpu = None
     c1 = None
@@ -322,7 +371,8 @@ def main():
                                f"VARIANT / reduced check run: {args.layers} layers, prompt {args.prompt}, "
                                f"router {'F32' if args.router_f32 else 'Q8_0'}",
                    "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "prefill_batch": args.max_batch, "decode_pos": int(pos0),
-                   "experts": "512 top-10 + shared, NVFP4", "dense": "Q8_0 (router and ssm_alpha/beta Q8_0)",
+                   "experts": "512 routed experts top-10, NVFP4 with per-expert second scales; one shared expert, Q8_0",
+                   "dense": "Q8_0 (attention, GDN, LM head; router, shared-gate logit and ssm_alpha/beta Q8_0 too)",
                    "mode": "exact" if args.exact else "fast", "batch": 1},
         "prefill_tok_s": round(args.prompt / t_prefill, 1),
         "prefill_kernels": prefill_kernels,
@@ -337,6 +387,7 @@ def main():
         "config1": c1,
         "setup_s": {"synth": round(t_synth, 1), "upload_repack": round(t_upload, 1)},
         "graph": graph_stats, "seam_ops_per_token": launches_per_token,
+        "exact_vs_fast": mode_check,
     }
     print(json.dumps(line), flush=True)
     eng.close(); model.close(); be.close()

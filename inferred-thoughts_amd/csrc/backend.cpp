@@ -252,28 +252,33 @@ float* it_hip::act_inout(const float* host, size_t len) {
     return d;
 }
 
+bool it_hip::act_q_reserve(Act& a, size_t len) {
+    if (a.q_cap >= len) return true;
+    need_eager("a quantized-activation buffer has to grow");
+    if (a.q_scales) {
+        check(hipStreamSynchronize(stream), "sync before quant free");
+        quant_bytes -= a.q_cap / 32 * 4 + a.q_cap;
+        (void)hipFree(a.q_scales);
+        (void)hipFree(a.q_quants);
+        a.q_scales = nullptr;
+        a.q_quants = nullptr;
+        a.q_cap = 0;
+    }
+    if (!check(hipMalloc((void**)&a.q_scales, (len / 32 + 1) * sizeof(float)), "hipMalloc(q8 scales)") ||
+        !check(hipMalloc((void**)&a.q_quants, len + 32), "hipMalloc(q8 quants)"))
+        return false;
+    a.q_cap = len;
+    quant_bytes += len / 32 * 4 + len;
+    a.q_valid = false;
+    return true;
+}
+
 bool it_hip::act_quantized(const float* host, size_t len, const float** scales, const int8_t** quants,
                            float** dev_x) {
     float* x = act_in(host, len);
     if (!x) return false;
     Act& a = acts[host];
-    if (a.q_cap < len) {
-        need_eager("a quantized-activation buffer has to grow");
-        if (a.q_scales) {
-            check(hipStreamSynchronize(stream), "sync before quant free");
-            quant_bytes -= a.q_cap / 32 * 4 + a.q_cap;
-            (void)hipFree(a.q_scales);
-            (void)hipFree(a.q_quants);
-            a.q_scales = nullptr;
-            a.q_quants = nullptr;
-        }
-        if (!check(hipMalloc((void**)&a.q_scales, (len / 32 + 1) * sizeof(float)), "hipMalloc(q8 scales)") ||
-            !check(hipMalloc((void**)&a.q_quants, len + 32), "hipMalloc(q8 quants)"))
-            return false;
-        a.q_cap = len;
-        quant_bytes += len / 32 * 4 + len;
-        a.q_valid = false;
-    }
+    if (!act_q_reserve(a, len)) return false;
     if (!a.q_valid || a.q_len != len) {
         float* qs = a.q_scales;
         int8_t* qq = a.q_quants;
@@ -927,10 +932,23 @@ void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w,
     if (out == x) be->acts[x].q_valid = false;
     int64_t rows = (int64_t)(x_len / w_len);
     int nd = (int)w_len, exact = be->exact;
+    // A batch's normed rows go to products with quantized weights next (qwen35.rs:1006-1093): their Q8_0 form is
+    // written by the same launch.  Single-token passes keep the two ops apart for the pass fuser.
+    float* qs = nullptr;
+    int8_t* qq = nullptr;
+    if (rows > 1 && be->mode == it_hip::Mode::Eager && nd % 32 == 0) {
+        it_hip::Act& a = be->acts[out];
+        if (be->act_q_reserve(a, out_len)) {
+            qs = a.q_scales;
+            qq = a.q_quants;
+            a.q_valid = true;
+            a.q_len = out_len;
+        }
+    }
     it_hip::OpRec rec;
     rec.id = OP_RMS; rec.p[0] = dx; rec.p[1] = dw; rec.p[2] = dout; rec.i[0] = rows; rec.i[1] = nd; rec.f[0] = eps;
     be->submit(it_hip::FAM_NORM, x_len * 8, sig_of(OP_RMS, dx, dw, eps, dout, rows, nd), rec,
-               [=](hipStream_t s) { rms_norm(dx, dw, eps, dout, rows, nd, exact, s); });
+               [=](hipStream_t s) { rms_norm(dx, dw, eps, dout, rows, nd, exact, s, qs, qq); });
 }
 
 void it_hip_rms_norm_heads(it_hip* be, float* x, uint64_t x_len, const float* w, uint64_t w_len,
@@ -1371,7 +1389,7 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
-                   expert_count(ids, np, counts, tally, s);
+                   expert_count(ids, np, v.n_expert, counts, nullptr, tally, s);
                    if (f16_shape && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
@@ -1428,8 +1446,7 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
                sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
                [=](hipStream_t s) {
-                   expert_count(ids, np, cg, tally, s);
-                   expert_count(ids, np, cu, tally, s);
+                   expert_count(ids, np, g.n_expert, cg, cu, tally, s);
                    if (f16_shape && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))

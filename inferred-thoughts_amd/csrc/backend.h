@@ -78,6 +78,7 @@ struct it_hip {
     float* act_inout(const float* host, size_t len);  // read then written in place
     bool act_quantized(const float* host, size_t len, const float** scales, const int8_t** quants,
                        float** dev_x);
+    bool act_q_reserve(Act& a, size_t len);  // room for the Q8_0 form of `len` floats
 
     // ---- constants (f32 vectors uploaded once: norm weights, conv taps, ssm_a, dt_bias)
     struct Const {

@@ -32,9 +32,62 @@ __global__ __launch_bounds__(THREADS) void rms_norm_k(const float* __restrict__ 
     for (int i = threadIdx.x; i < nd; i += THREADS) o[i] = lds[i] * scale * w[i];
 }
 
+// The same rows, four outputs per lane, with the Q8_0 form of every output row written beside it (naive.rs:652-675,
+// the arithmetic of quantize_q8_0_k: eight neighbouring lanes hold one 32-element block).  What the next op, a
+// product with quantized weights, would otherwise compute in a launch of its own; values and quants are bit for bit
+// those of the two separate kernels.  nd a multiple of 32.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void rms_norm_q8_k(const float* __restrict__ x, const float* __restrict__ w,
+                                                         float eps, float* __restrict__ out, int nd, int exact,
+                                                         float* __restrict__ q_scales, int8_t* __restrict__ q_quants) {
+    extern __shared__ float lds[];
+    __shared__ double red[THREADS / 64 + 1];
+    const float* row = x + (int64_t)blockIdx.x * nd;
+    float* o = out + (int64_t)blockIdx.x * nd;
+    for (int i = threadIdx.x; i < nd / 4; i += THREADS) ((float4*)lds)[i] = ((const float4*)row)[i];
+    __syncthreads();
+    double sum = block_sumsq<THREADS>(lds, nd, exact, red);
+    float mean = (float)(sum / (double)nd);
+    float scale = 1.0f / sqrtf(mean + eps);
+    const int64_t blk0 = (int64_t)blockIdx.x * (nd / 32);
+    for (int i0 = 0; i0 < nd / 4; i0 += THREADS) {      // uniform trip count: the lane moves below need every lane
+        const int i = i0 + threadIdx.x;
+        const bool live = i < nd / 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            const float4 a = ((const float4*)lds)[i], ww = ((const float4*)w)[i];
+            v = make_float4(a.x * scale * ww.x, a.y * scale * ww.y, a.z * scale * ww.z, a.w * scale * ww.w);
+            ((float4*)o)[i] = v;
+        }
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        if (!live) continue;
+        const float d = amax / 127.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const float r[4] = {roundf(v.x * id), roundf(v.y * id), roundf(v.z * id), roundf(v.w * id)};
+        uint32_t packed = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float c = fminf(fmaxf(r[k], -128.0f), 127.0f);
+            const int q = (r[k] != r[k]) ? 0 : (int)c;
+            packed |= ((uint32_t)(q & 0xff)) << (8 * k);
+        }
+        *(uint32_t*)(q_quants + (int64_t)blockIdx.x * nd + (int64_t)i * 4) = packed;
+        if ((i & 7) == 0) q_scales[blk0 + (i >> 3)] = it_f16_to_f32(it_f32_to_f16(d));
+    }
+}
+
 void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
-              hipStream_t s) {
+              hipStream_t s, float* q_scales, int8_t* q_quants) {
     if (n_rows <= 0) return;
+    auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (q_scales && q_quants && nd % 32 == 0 && al(x) && al(w) && al(out)) {
+        hipLaunchKernelGGL(rms_norm_q8_k<256>, dim3((unsigned)n_rows), dim3(256), nd * sizeof(float), s, x, w, eps, out, nd,
+                           exact, q_scales, q_quants);
+        return;
+    }
     hipLaunchKernelGGL(rms_norm_k<256>, dim3((unsigned)n_rows), dim3(256), nd * sizeof(float), s, x, w, eps, out,
                        nd, exact);
 }

@@ -4,6 +4,8 @@
 // ascending scan that takes a new best only on a strict '>' (ties to the lower id),
 // then the picked probabilities summed in pick order and divided by
 // max(sum, 6.103515625e-5).  moe_finish follows src/ops/mod.rs:1134-1171.
+#include <algorithm>
+
 #include "it_device.h"
 #include "kernels.h"
 
@@ -106,16 +108,46 @@ __global__ __launch_bounds__(256) void route_topk_wave_k(const float* __restrict
     }
 }
 
-__global__ void expert_count_k(const int32_t* __restrict__ ids, int n_picks, uint32_t* __restrict__ counts,
-                               unsigned long long* __restrict__ tally) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n_picks) atomicAdd(counts + ids[i], 1u);
-    if (i == 0) atomicAdd(tally, (unsigned long long)n_picks);
+// A block counts its slice of the picks in LDS and adds the bins it touched to the global counters: a few hundred
+// global atomics for a prefill batch's tens of thousands of picks.  counts_b: a second tensor read with the same
+// picks (the up matrices beside the gate matrices), or null.
+constexpr int COUNT_BINS = 2048;
+__global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict__ ids, int n_picks, int n_expert,
+                                                      uint32_t* __restrict__ counts_a, uint32_t* __restrict__ counts_b,
+                                                      unsigned long long* __restrict__ tally) {
+    __shared__ unsigned bins[COUNT_BINS];
+    const bool local = n_expert <= COUNT_BINS;
+    if (local)
+        for (int e = threadIdx.x; e < n_expert; e += 256) bins[e] = 0;
+    __syncthreads();
+    const int per = (n_picks + gridDim.x - 1) / gridDim.x;
+    const int lo = blockIdx.x * per, hi = min(n_picks, lo + per);
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const int e = ids[i];
+        if (local) {
+            atomicAdd(&bins[e], 1u);
+        } else {
+            atomicAdd(counts_a + e, 1u);
+            if (counts_b) atomicAdd(counts_b + e, 1u);
+        }
+    }
+    __syncthreads();
+    if (local)
+        for (int e = threadIdx.x; e < n_expert; e += 256) {
+            const unsigned c = bins[e];
+            if (c) {
+                atomicAdd(counts_a + e, c);
+                if (counts_b) atomicAdd(counts_b + e, c);
+            }
+        }
+    if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(tally, (unsigned long long)n_picks * (counts_b ? 2 : 1));
 }
 
-void expert_count(const int32_t* ids, int n_picks, uint32_t* counts, unsigned long long* tally, hipStream_t s) {
-    if (n_picks <= 0 || !counts || !tally) return;
-    hipLaunchKernelGGL(expert_count_k, dim3((n_picks + 255) / 256), dim3(256), 0, s, ids, n_picks, counts, tally);
+void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
+                  unsigned long long* tally, hipStream_t s) {
+    if (n_picks <= 0 || !counts_a || !tally) return;
+    const int blocks = std::max(1, std::min(64, (n_picks + 1023) / 1024));
+    hipLaunchKernelGGL(expert_count_k, dim3(blocks), dim3(256), 0, s, ids, n_picks, n_expert, counts_a, counts_b, tally);
 }
 
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,

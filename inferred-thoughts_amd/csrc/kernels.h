@@ -78,9 +78,11 @@ void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids,
              int x_mode, const float* act_scales, const int8_t* act_quants, float* out, hipStream_t s);
 
 // ---- expert read counters -------------------------------------------------------
-// counts[ids[i]] += 1 for every pick and tally[0] += n_picks: the device-side read counters of the expert cache
-// (reads served from device memory; tally[1], reads served from a host tier, stays 0 when every expert is resident)
-void expert_count(const int32_t* ids, int n_picks, uint32_t* counts, unsigned long long* tally, hipStream_t s);
+// counts_a[ids[i]] += 1 (and counts_b, when given: a second tensor read with the same picks) for every pick, and
+// tally[0] += the reads counted: the device-side read counters of the expert cache (reads served from device memory;
+// tally[1], reads served from a host tier, stays 0 when every expert is resident)
+void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
+                  unsigned long long* tally, hipStream_t s);
 
 // ---- router ----------------------------------------------------------------------
 void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);
@@ -90,8 +92,10 @@ void moe_finish(float* out, int64_t at, int n, const float* rows, const float* w
                 const float* shared, const float* logit, int64_t logit_at, int exact, hipStream_t s);
 
 // ---- norms and elementwise ------------------------------------------------------
+// q_scales / q_quants (optional, nd a multiple of 32): the Q8_0 form of `out` is written as well, bit for bit what
+// quantize_q8_0 gives on it
 void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
-              hipStream_t s);
+              hipStream_t s, float* q_scales = nullptr, int8_t* q_quants = nullptr);
 void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int exact,
                     hipStream_t s);
 void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s);

@@ -17,7 +17,8 @@ F32, F16, Q8_0, BF16, NVFP4 = 0, 1, 8, 30, 40
 EXACT, NO_GRAPH, NO_FUSE = 1, 2, 4
 
 _HERE = Path(__file__).resolve().parent
-LIB_PATH = _HERE / "libinferred_hip.so"
+# INFERRED_HIP_LIB names another build of the library (comparing two builds on one machine)
+LIB_PATH = Path(os.environ.get("INFERRED_HIP_LIB") or _HERE / "libinferred_hip.so")
 CSRC = _HERE.parent / "csrc"
 
 c_u64, c_u32, c_f32 = C.c_uint64, C.c_uint32, C.c_float

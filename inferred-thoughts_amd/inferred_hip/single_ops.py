@@ -123,6 +123,70 @@ def expert_ffn(ih, be, seed=0, tokens=(1, 8, 64, 512), n_expert=512, n_used=10, 
     return out
 
 
+def expert_ffn_fused_decode(ih, seed=0, n_expert=512, n_used=10, nd=2048, ff=512, reps=16):
+    """Config 2's one-token point through the path a decode pass takes: the routed FFN issued as the model loop issues
+    it (norm, router + shared-gate logit, softmax, top-k, experts' gate/up, down, shared expert, combine, residual)
+    inside a single-token pass, which the backend fuses into three launches (router GEMV; gate/up with the in-kernel
+    top-10; down + combine + residual) and replays as a graph.  Timed like the other points: the fused launches
+    issued one by one between HIP events.  Bytes: ten routed experts + the shared one + the router matrix."""
+    from inferred_hip import F32  # noqa: F401  (the package is the caller's)
+    r = np.random.default_rng(seed + 3)
+    be = ih.Hip(exact=False)
+    try:
+        def q8(n_out, n_in, gain):
+            w = (r.standard_normal((n_out, n_in)) * (gain / np.sqrt(n_in))).astype(np.float32).reshape(-1, 32)
+            d = np.abs(w).max(1) / 127.0
+            q = np.where(d[:, None] > 0, np.rint(w / np.maximum(d, 1e-30)[:, None]), 0).astype(np.int8)
+            blk = np.zeros((w.shape[0], 34), np.uint8)
+            blk[:, :2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+            blk[:, 2:] = q.view(np.uint8)
+            return blk.reshape(-1)
+        gate, up, down = _nvfp4(r, n_expert * ff, nd), _nvfp4(r, n_expert * ff, nd), _nvfp4(r, n_expert * nd, ff)
+        scales = [(r.random(n_expert).astype(np.float32) * 0.01 + 0.002) for _ in range(3)]
+        eg = ih.experts(gate, ih.NVFP4, nd, ff, n_expert, scales[0])
+        eu = ih.experts(up, ih.NVFP4, nd, ff, n_expert, scales[1])
+        ed = ih.experts(down, ih.NVFP4, ff, nd, n_expert, scales[2])
+        router_b, logit_b = q8(n_expert, nd, 3.0), q8(1, nd, 1.0)
+        sg_b, su_b, sd_b = q8(ff, nd, 1.5), q8(ff, nd, 1.5), q8(nd, ff, 2.0)
+        wr, wl = ih.weights(router_b, ih.Q8_0, nd, n_expert), ih.weights(logit_b, ih.Q8_0, nd, 1)
+        wg, wu, wd = ih.weights(sg_b, ih.Q8_0, nd, ff), ih.weights(su_b, ih.Q8_0, nd, ff), ih.weights(sd_b, ih.Q8_0, ff, nd)
+        norm_w = np.ones(nd, np.float32)
+        z = lambda n: np.zeros(n, np.float32)
+        x, normed, e_in, router, logit = z(nd), z(nd), z(nd), z(n_expert), z(1)
+        g_all, u_all, o_all, e_gate, e_up, e_out, ffn = z(n_used * ff), z(n_used * ff), z(n_used * nd), z(ff), z(ff), z(nd), z(nd)
+        xs = [r.standard_normal(nd).astype(np.float32) for _ in range(reps + 3)]
+
+        def once(i):
+            x[:] = xs[i]
+            be.begin_pass(1); be.host_wrote(x)
+            be.rms_norm(x, norm_w, 1e-6, normed)
+            be.gather_chunks(normed, nd, nd, 0, e_in)
+            be.matmul_pair(wr, wl, e_in, router, logit)
+            be.softmax(router, n_expert)
+            route = be.route(router, n_expert, n_used)
+            be.moe_glu(eg, eu, route, e_in, g_all, u_all)
+            be.matmul_experts(ed, route, g_all, o_all)
+            be.matmul(wg, e_in, e_gate); be.matmul(wu, e_in, e_up)
+            be.silu_mul(e_gate, e_up)
+            be.matmul(wd, e_gate, e_out)
+            be.moe_finish(ffn, 0, nd, o_all, route, e_out, logit, 0)
+            be.add_assign(x, ffn)
+            be.end_pass()
+
+        for i in range(3):
+            once(reps + i)       # eager, eager, captured
+        be.sync()
+        st = be.graph_stats()
+        ms, launches, _ = _timed(be, once, reps)
+        expert_bytes = 3 * ff * nd // 64 * 36
+        bytes_ = n_used * expert_bytes + 3 * ff * nd // 32 * 34 + (n_expert + 1) * nd // 32 * 34 + 2 * nd * 4
+        return _line(bytes_, ms, launches, fused_launches=st["graph_kernels"], experts_touched=n_used,
+                     note="the decode path: router GEMV, gate/up with the in-kernel top-10, down + combine; "
+                          "Q8_0 router and shared expert as in the headline model")
+    finally:
+        be.close()
+
+
 def attention_decode(ih, be, seed=0, contexts=(1024, 8192, 32000), n_head=16, n_head_kv=2, hd=256):
     r = np.random.default_rng(seed + 1)
     kv_dim = n_head_kv * hd
@@ -202,6 +266,7 @@ def run(ih, seed=0, exact=False):
         return {"timing": "sum of per-launch HIP-event durations of one call sequence (each launch carries about "
                           "2 us of event overhead); operands rotated over copies so that they come from HBM",
                 "expert_ffn_nvfp4_512x10": expert_ffn(ih, be, seed),
+                "expert_ffn_nvfp4_512x10_one_token_fused": None if exact else expert_ffn_fused_decode(ih, seed),
                 "attention_decode_16q_2kv_hd256": attention_decode(ih, be, seed),
                 "gated_delta_net_16k_32v_128": delta_net(ih, be, seed)}
     finally:
