@@ -1018,6 +1018,13 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     bool one_expert = false, grouped = false;
     // (from 513 tokens on: a call costs 55-80 us for the grouping, the f16 split and a latency-bound handful of
     // tiles, which the GEMVs reach at about 512 tokens)
+    // A dense NVFP4 matrix over 128 .. 512 tokens: eight or sixteen tokens per pass over the rows (k_moe_rows.hip) instead
+    // of one GEMV per token (32 against 70 us for the shared expert's 2048 x 512 at 512 tokens; below 128 tokens the
+    // GEMVs, which fill the chip with one block row per token, are as fast).
+    ExpertsView rv{};
+    rv.q = v.q; rv.scales = v.scales; rv.q_stride = 0; rv.s_stride = 0; rv.fmt = v.fmt; rv.n_in = v.n_in; rv.n_out = v.n_out;
+    rv.n_expert = 1; rv.scale2 = nullptr; rv.counts = nullptr;
+    const bool rows_dense = !exact && v.fmt == W_NVFP4 && n >= 128 && n <= 512 && itk::expert_rows_takes(rv, nullptr, aq);
     if (!exact && v.fmt == W_NVFP4 && n > 512) {
         ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
         ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr; ev.counts = nullptr;
@@ -1034,6 +1041,7 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
                sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout), rec,
                [=](hipStream_t s) {
+                   if (rows_dense && expert_rows(rv, nullptr, nullptr, nt, 1, 0, as, aq, dout, 1.0f, nullptr, 0, false, s)) return;
                    if (one_expert && experts_gemm_f16(ev, nullptr, zids, nt, 1, 0, as, aq, dout, work, work_ints, fwork,
                                                       fwork_bytes, grouped, s))
                        return;
@@ -1345,6 +1353,20 @@ static bool host_ids_in_range(it_hip* be, const it_route* r, uint64_t n_expert, 
 // the tiles win from about 3.5 pairs per expert on (a batch of 128 tokens at top-10 still takes 653 us per pair
 // against 772 us tiled; at 256 tokens it is 1,180 against 848).
 static bool expert_tiles_pay(uint64_t picks, uint64_t n_expert) { return picks >= 32 && 2 * picks >= 7 * n_expert; }
+// Fast mode between the per-pair GEMVs and the wide matrix-core tiles, measured on the 512-expert top-10 FFN (hidden
+// 2048, inter 512): from 1.25 pairs per expert on, grouping the pairs by expert beats one GEMV per pair; NVFP4 then
+// runs 16-pair tiles on the f16 matrix cores (k_gemm_f16s.hip) up to 18 pairs per expert, where the 128-pair tiles
+// take over; what that kernel does not take (Q8_0, odd shapes) streams each expert's rows once for all its pairs
+// (k_moe_rows.hip) until the int8 tiles pay.
+static bool expert_grouping_pays(const it_hip* be, uint64_t picks, uint64_t n_expert) {
+    return !be->exact && picks >= 32 && 4 * picks >= 5 * n_expert;
+}
+static bool expert_skinny_pay(const it_hip* be, uint64_t picks, uint64_t n_expert) {
+    return expert_grouping_pays(be, picks, n_expert) && picks < 18 * n_expert;
+}
+static bool expert_rows_pay(const it_hip* be, uint64_t picks, uint64_t n_expert) {
+    return expert_grouping_pays(be, picks, n_expert) && !expert_tiles_pay(picks, n_expert);
+}
 
 void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* route, const float* x,
                            uint64_t x_len, float* out, uint64_t out_len) {
@@ -1370,16 +1392,21 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
     size_t work_ints = 0;
-    int32_t* work = expert_tiles_pay(picks, w->n_expert) ? be->moe_work_for(picks, w->n_expert, &work_ints) : nullptr;
+    const bool skinny_pay = expert_skinny_pay(be, picks, w->n_expert) && v.fmt == itk::W_NVFP4;
+    const bool rows_pay = !skinny_pay && expert_rows_pay(be, picks, w->n_expert);
+    int32_t* work = skinny_pay || rows_pay || expert_tiles_pay(picks, w->n_expert) ? be->moe_work_for(picks, w->n_expert, &work_ints) : nullptr;
+    const bool rows_shape = rows_pay && work && itk::expert_rows_takes(v, nullptr, aq);
     void* fwork = nullptr;
     size_t fwork_bytes = 0;
-    if (!be->exact && work && v.fmt == itk::W_NVFP4) {
+    if (!be->exact && work && !rows_shape && v.fmt == itk::W_NVFP4) {
         fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)w->n_in);
         fwork = be->moe_f16_for(fwork_bytes);
     }
-    // the tile size the launch below will group for: 128 pairs for the f16 kernel, 16 for the int8 one
-    const bool f16_shape = fwork && itk::experts_f16_takes(v, nullptr, np, aq, dout);
-    const bool grouped = work && be->group_cached(np, (int)w->n_expert, f16_shape ? 128 : 16);
+    const bool skinny_shape = skinny_pay && fwork && itk::experts_f16s_takes(v, nullptr, np, aq, dout);
+    // the tile size the launch below will group for: 8 or 16 pairs for the row kernel, 128 for the wide f16 kernel,
+    // 16 for the skinny f16 kernel and the int8 one
+    const bool f16_shape = !skinny_shape && fwork && itk::experts_f16_takes(v, nullptr, np, aq, dout);
+    const bool grouped = work && be->group_cached(np, (int)w->n_expert, rows_shape ? itk::expert_rows_tile(np, (int)w->n_expert, v.n_in) : f16_shape ? 128 : 16);
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
@@ -1390,6 +1417,9 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
                sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
                    expert_count(ids, np, v.n_expert, counts, nullptr, tally, s);
+                   if (skinny_shape && experts_gemm_f16s(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
+                       return;
+                   if (rows_shape && expert_rows(v, nullptr, ids, np, nu, xm, as, aq, dout, 1.0f, work, work_ints, grouped, s)) return;
                    if (f16_shape && experts_gemm_f16(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))
@@ -1426,15 +1456,19 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     if (!dout) return;
     int np = (int)picks, nu = (int)n_used, xm = x_mode_of(rows, picks);
     size_t work_ints = 0;
-    int32_t* work = expert_tiles_pay(picks, gate->n_expert) ? be->moe_work_for(picks, gate->n_expert, &work_ints) : nullptr;
+    const bool skinny_pay = expert_skinny_pay(be, picks, gate->n_expert) && g.fmt == itk::W_NVFP4;
+    const bool rows_pay = !skinny_pay && expert_rows_pay(be, picks, gate->n_expert);
+    int32_t* work = skinny_pay || rows_pay || expert_tiles_pay(picks, gate->n_expert) ? be->moe_work_for(picks, gate->n_expert, &work_ints) : nullptr;
+    const bool rows_shape = rows_pay && work && itk::expert_rows_takes(g, &u, aq);
     void* fwork = nullptr;
     size_t fwork_bytes = 0;
-    if (!be->exact && work && g.fmt == itk::W_NVFP4) {
+    if (!be->exact && work && !rows_shape && g.fmt == itk::W_NVFP4) {
         fwork_bytes = itk::experts_f16_work_bytes((int)rows, (int)gate->n_in);
         fwork = be->moe_f16_for(fwork_bytes);
     }
-    const bool f16_shape = fwork && itk::experts_f16_takes(g, &u, np, aq, dout);
-    const bool grouped = work && be->group_cached(np, (int)gate->n_expert, f16_shape ? 128 : 16);
+    const bool skinny_shape = skinny_pay && fwork && itk::experts_f16s_takes(g, &u, np, aq, dout);
+    const bool f16_shape = !skinny_shape && fwork && itk::experts_f16_takes(g, &u, np, aq, dout);
+    const bool grouped = work && be->group_cached(np, (int)gate->n_expert, rows_shape ? itk::expert_rows_tile(np, (int)gate->n_expert, g.n_in) : f16_shape ? 128 : 16);
     it_hip::OpRec rec;
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
@@ -1447,6 +1481,9 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
                       as, aq, dout), rec,
                [=](hipStream_t s) {
                    expert_count(ids, np, g.n_expert, cg, cu, tally, s);
+                   if (skinny_shape && experts_gemm_f16s(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
+                       return;
+                   if (rows_shape && expert_rows(g, &u, ids, np, nu, xm, as, aq, dout, 1.0f, work, work_ints, grouped, s)) return;
                    if (f16_shape && experts_gemm_f16(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (!experts_gemm(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, grouped && !f16_shape, s))

@@ -46,6 +46,35 @@ IT_DEV void unit_nvfp4(const uint4 w, uint32_t sc2, const uint4 a0, const uint4 
     *tB = (dy * dB) * (float)sb;
 }
 
+// ------------------------------------------------------------------ E2M1 nibbles -> f16
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+// four nibbles (one per byte, 0..15) -> four f16 weights (two dwords), scaled by the sub-block scale
+IT_DEV void fp4x4_to_f16x4(uint32_t v, h2 scale, h2* a, h2* b) {
+    // f16 high bytes of 128 x the doubled e2m1 magnitudes 0 1 2 3 4 6 8 12 (the low bytes are zero): the 128 pays
+    // for the 2^-8 the scale carries (see expand) and the halving that goes with the doubled magnitudes
+    const uint32_t mag = __builtin_amdgcn_perm(0x66646260u, 0x5e5c5800u, v & 0x07070707u);
+    const uint32_t hb = mag | ((v & 0x08080808u) << 4);
+    const uint32_t d0 = __builtin_amdgcn_perm(hb, hb, 0x010c000cu);   // bytes 0, hb.0, 0, hb.1
+    const uint32_t d1 = __builtin_amdgcn_perm(hb, hb, 0x030c020cu);   // bytes 0, hb.2, 0, hb.3
+    *a = __builtin_bit_cast(h2, d0) * scale;
+    *b = __builtin_bit_cast(h2, d1) * scale;
+}
+
+
+// operands of the f16 expert tile kernels (k_gemm_f16.hip, k_gemm_f16s.hip)
+struct ExpertsF16P {
+    const uint8_t *q, *s, *q2, *s2;
+    int64_t q_stride, s_stride;
+    const float *scale2, *scale2_up;
+    const uint16_t *xh, *xl;
+    const float* rscale;
+    float* out;
+    int n_in, n_out, x_mode, n_used;
+    const int32_t* n_tiles;
+    const int4* tiles;
+    const int32_t* order;
+};
+
 // Serial ascending fold of T per-block terms from a 16-byte aligned LDS row: the loads are
 // issued four float4 at a time so the chain of adds never waits on LDS latency.
 IT_DEV float fold_terms(const float* tr, int T) {

@@ -404,7 +404,8 @@ __global__ __launch_bounds__(GT) void experts_gemm_k(ExpertsGemmP p) {
 }  // namespace
 
 size_t experts_group_work_ints(int n_picks, int n_expert) {
-    return 16 + (size_t)(n_expert + n_picks / 16 + 2) * 4 + (size_t)n_picks;
+    // sized for the smallest tiles any kernel groups for (eight pairs)
+    return 16 + (size_t)(n_expert + n_picks / 8 + 2) * 4 + (size_t)n_picks;
 }
 
 bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,

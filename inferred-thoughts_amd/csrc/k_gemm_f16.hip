@@ -25,6 +25,7 @@
 // l / 32, for both A (weight rows) and B (tokens); it receives D for token l % 32 and weight
 // rows 8 * (i / 4) + 4 * (l / 32) + i % 4, i = 0..15.
 #include "it_device.h"
+#include "it_dot.h"
 #include "kernels.h"
 
 // Phase stamps for tuning: a build with -DIT_STAMPS records the 100 MHz wall clock of one block's first
@@ -46,7 +47,6 @@ __device__ int it_gemm_stamp_tile, it_gemm_stamp_slab;
 namespace itk {
 namespace {
 
-typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int FK = 64;          // k per slab
@@ -90,30 +90,6 @@ __global__ __launch_bounds__(256) void acts_split_f16_k(const int8_t* __restrict
     }
 }
 
-// four nibbles (one per byte, 0..15) -> four f16 weights (two dwords), scaled by the sub-block scale
-__device__ __forceinline__ void fp4x4_to_f16x4(uint32_t v, h2 scale, h2* a, h2* b) {
-    // f16 high bytes of 128 x the doubled e2m1 magnitudes 0 1 2 3 4 6 8 12 (the low bytes are zero): the 128 pays
-    // for the 2^-8 the scale carries (see expand) and the halving that goes with the doubled magnitudes
-    const uint32_t mag = __builtin_amdgcn_perm(0x66646260u, 0x5e5c5800u, v & 0x07070707u);
-    const uint32_t hb = mag | ((v & 0x08080808u) << 4);
-    const uint32_t d0 = __builtin_amdgcn_perm(hb, hb, 0x010c000cu);   // bytes 0, hb.0, 0, hb.1
-    const uint32_t d1 = __builtin_amdgcn_perm(hb, hb, 0x030c020cu);   // bytes 0, hb.2, 0, hb.3
-    *a = __builtin_bit_cast(h2, d0) * scale;
-    *b = __builtin_bit_cast(h2, d1) * scale;
-}
-
-struct ExpertsF16P {
-    const uint8_t *q, *s, *q2, *s2;
-    int64_t q_stride, s_stride;
-    const float *scale2, *scale2_up;
-    const uint16_t *xh, *xl;
-    const float* rscale;
-    float* out;
-    int n_in, n_out, x_mode, n_used;
-    const int32_t* n_tiles;
-    const int4* tiles;
-    const int32_t* order;
-};
 
 template <bool GLU, int T>
 __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int4 td, uint16_t* Bh, uint16_t* Bl,

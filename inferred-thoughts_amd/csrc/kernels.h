@@ -70,6 +70,20 @@ bool experts_f16_takes(const ExpertsView& w, const ExpertsView* up, int n_picks,
 bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
                       int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
                       size_t work_ints, void* fwork, size_t fwork_bytes, bool grouped, hipStream_t s);
+// NVFP4 experts with few pairs per expert in fast mode (k_gemm_f16s.hip): tiles of 16 pairs on MFMA 16x16x32 f16, no LDS;
+// the grouping has the layout of experts_gemm's (tiles of 16 pairs).  Scratch as for experts_gemm_f16.
+bool experts_f16s_takes(const ExpertsView& w, const ExpertsView* up, int n_picks, const int8_t* act_quants, const float* out);
+bool experts_gemm_f16s(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used,
+                       int x_mode, const float* act_scales, const int8_t* act_quants, float* out, int32_t* work,
+                       size_t work_ints, void* fwork, size_t fwork_bytes, bool grouped, hipStream_t s);
+// Small batches in fast mode (k_moe_rows.hip): pairs sorted by expert in tiles of 8 or 16, every weight row of a tile's
+// expert streamed once and multiplied with all its pairs by integer dots.  ids null: one dense matrix (strides
+// ignored), tile t = tokens 8 t .. 8 t + 7.  False: nothing launched (shape, alignment or scratch do not fit).
+bool expert_rows_takes(const ExpertsView& w, const ExpertsView* up, const int8_t* act_quants);
+int expert_rows_tile(int n_picks, int n_expert, int n_in);   // pairs per tile the launch groups for
+bool expert_rows(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
+                 const float* act_scales, const int8_t* act_quants, float* out, float out_scale, int32_t* work,
+                 size_t work_ints, bool grouped, hipStream_t s);
 bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* ids, int n_picks, int n_used, int x_mode,
                   const float* act_scales, const int8_t* act_quants, float* out, int32_t* work, size_t work_ints,
                   bool grouped, hipStream_t s);
