@@ -50,6 +50,110 @@ def family_profile():
     return out
 
 
+def summarize_profile(root_dir):
+    """The text kept under profiles/ for the decode graph, from three rocprofv3 runs of `bench.py --decode-only` whose
+    output directories sit under `root_dir`: trace/ (--kernel-trace), pmc_FETCH_SIZE/ and pmc_WRITE_SIZE/ (--pmc, with
+    --copy-ref, whose 256 MiB device copy calibrates the counters).  Needs no GPU.  Prints the per-kernel table of the
+    last 48 replayed tokens (count, average duration, average gap before the launch), the "@" lines that
+    family_profile() reads, and one GDN layer, one attention layer and the output head node by node."""
+    import collections
+    import csv
+    import glob
+    import re
+    steps = 48
+
+    def short(n):
+        n = n.replace("itk::(anonymous namespace)::", "").replace("itk::", "").replace("void ", "")
+        return re.sub(r"\(.*", "", n)
+
+    def grid_of(r):
+        if "Grid_Size" in r:
+            return int(r["Grid_Size"])
+        return int(r["Grid_Size_X"]) * int(r.get("Grid_Size_Y", 1) or 1) * int(r.get("Grid_Size_Z", 1) or 1)
+
+    def family(name, grid):
+        n = short(name)
+        if n.startswith("fused_gemv_fast_k"):
+            return "lm_head (norm + GEMV)" if grid >= 400000 else "fused_gemv (norm + quantize + dense GEMVs)"
+        if n.startswith("moe_glu_fast_k"):
+            return "moe_glu (expert gate+up)"
+        if n.startswith("moe_down_fast_k"):
+            return "matmul_experts (expert down)"
+        if n.startswith("gdn_rows_fast_k"):
+            return "gdn_rows (l2 norm + delta rule)"
+        if n.startswith("attend_decode_k") or n.startswith("attend_merge"):
+            return "attend"
+        if n.startswith("argmax"):
+            return "other"
+        return None
+
+    trace = glob.glob(f"{root_dir}/trace/**/*kernel_trace.csv", recursive=True)[0]
+    rows = []
+    for r in csv.DictReader(open(trace)):
+        if not r["Kernel_Name"].startswith("__amd_rocclr"):
+            rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"], grid_of(r)))
+    rows.sort()
+    # whole tokens: from just after one output-head launch to the next; the last `steps` of them
+    heads = [i for i, r in enumerate(rows) if family(r[2], r[3]) == "lm_head (norm + GEMV)"]
+    tail = rows[heads[-steps - 1] + 1:heads[-1] + 1]
+    nodes = len(tail) // steps
+    fam = collections.defaultdict(lambda: [0, 0.0])
+    kern = collections.defaultdict(lambda: [0, 0.0, 0.0])
+    gaps = 0.0
+    for i, (s0, e0, n, g) in enumerate(tail):
+        d = (e0 - s0) / 1e3
+        fam[family(n, g)][0] += 1
+        fam[family(n, g)][1] += d
+        k = kern[(short(n), g)]
+        k[0] += 1
+        k[1] += d
+        if i:
+            k[2] += (s0 - tail[i - 1][1]) / 1e3
+            gaps += (s0 - tail[i - 1][1]) / 1e3
+    span = (tail[-1][1] - tail[0][0]) / 1e3
+    print(f"kernel trace: the last {steps} replayed decode tokens, {nodes} graph kernels each")
+    print(f"per token: {sum(v[1] for v in fam.values()) / steps:.1f} us inside kernels + {gaps / steps:.1f} us between them "
+          f"= {span / steps:.1f} us from first start to last end (under the profiler)")
+    print(f"{'kernel':50s} {'grid threads':>12s} {'per token':>9s} {'avg us':>8s} {'avg gap before us':>17s} {'us/token':>9s}")
+    for (n, g), (c, d, gap) in sorted(kern.items(), key=lambda kv: -kv[1][1]):
+        print(f"{n[:50]:50s} {g:12d} {c / steps:9.2f} {d / c:8.2f} {gap / c:17.2f} {d / steps:9.1f}")
+    res, scale = {}, {}
+    for c in ("FETCH_SIZE", "WRITE_SIZE"):
+        f = glob.glob(f"{root_dir}/pmc_{c}/**/*counter_collection.csv", recursive=True)[0]
+        acc = collections.defaultdict(lambda: [0, 0.0])
+        copies = []
+        for r in csv.DictReader(open(f)):
+            if r["Counter_Name"] != c:
+                continue
+            if r["Kernel_Name"].startswith("__amd_rocclr_copyBuffer") and float(r["Counter_Value"]) > 50000:
+                copies.append(float(r["Counter_Value"]))
+            k = family(r["Kernel_Name"], grid_of(r))
+            if k:
+                acc[k][0] += 1
+                acc[k][1] += float(r["Counter_Value"])
+        res[c] = acc
+        scale[c] = 262144.0 / (sum(copies) / len(copies)) if copies else float("nan")
+        print(f"{c}: a 256 MiB device copy reads {sum(copies) / max(len(copies), 1):.0f} per dispatch over {len(copies)} "
+              f"copies -> x {scale[c]:.3f} to KiB")
+    print("\n@ family | launches per token | rocprofv3 avg duration us | fetched bytes per launch | written bytes per launch")
+    for k in sorted((k for k in fam if k), key=lambda k: -fam[k][1]):
+        c, d = fam[k]
+        fb, wb = res["FETCH_SIZE"].get(k, [0, 0.0]), res["WRITE_SIZE"].get(k, [0, 0.0])
+        print(f"@ {k} | {c / steps:.2f} | {d / c:.3f} | {fb[1] / max(fb[0], 1) * scale['FETCH_SIZE'] * 1024:.0f} | "
+              f"{wb[1] / max(wb[0], 1) * scale['WRITE_SIZE'] * 1024:.0f}")
+    # the last token: its third GDN layer, the attention layer after it and the output head, node by node
+    last = tail[-nodes:]
+    glu = [i for i, r in enumerate(last) if short(r[2]).startswith("moe_down_fast_k")]
+    cut = last[glu[1] + 1:glu[3] + 1] + last[glu[-1] + 1:] if len(glu) >= 4 else last
+    print("\nlast replayed token, layers 2 (GDN) and 3 (attention) and the output head, node by node: start offset us, "
+          "duration us, gap before us, kernel, grid threads")
+    t0, prev = last[0][0], None
+    for s0, e0, n, g in cut:
+        gap = "" if prev is None else f"{(s0 - prev) / 1e3:6.2f}"
+        print(f"{(s0 - t0) / 1e3:9.2f} {(e0 - s0) / 1e3:7.2f} {gap:>6s}  {short(n)[:70]} {g}")
+        prev = e0
+
+
 def model_path(args):
     base = Path("/dev/shm") if Path("/dev/shm").is_dir() and os.access("/dev/shm", os.W_OK) else Path("/tmp")
     return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}{'_f32router' if args.router_f32 else ''}.gguf"
@@ -138,7 +242,13 @@ def main():
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--summarize-profile", metavar="DIR",
+                    help="no run: print the profiles/ summary of the rocprofv3 outputs under DIR (trace/, pmc_FETCH_SIZE/, "
+                         "pmc_WRITE_SIZE/ of --decode-only runs) and exit")
     args = ap.parse_args()
+    if args.summarize_profile:
+        summarize_profile(args.summarize_profile)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no collective: experts, layers or heads "
               "would shard across GPUs, none of which is built); run with --gpus 1", file=sys.stderr)
