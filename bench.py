@@ -242,6 +242,10 @@ def main():
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--expert-slots", type=int, default=0,
+                    help="variant run: fix the expert pool's device tier at this many expert matrices; the rest of the pool "
+                         "goes to pinned host memory that the kernels read in place (with --decode-only: prints the tier's "
+                         "counters, exchanges experts by the counts of the timed stretch and times a second stretch)")
     ap.add_argument("--summarize-profile", metavar="DIR",
                     help="no run: print the profiles/ summary of the rocprofv3 outputs under DIR (trace/, pmc_FETCH_SIZE/, "
                          "pmc_WRITE_SIZE/ of --decode-only runs) and exit")
@@ -280,6 +284,8 @@ def main():
         single = single_ops.run(ih, seed=args.seed, exact=args.exact)
         print(f"[bench] single-op configurations in {time.time() - t_s:.1f}s", file=sys.stderr, flush=True)
     be = ih.Hip(exact=args.exact)
+    if args.expert_slots:
+        be.set_expert_slots(args.expert_slots)
     model = ih.Model(path)
     eng = ih.Engine(model, be, args.ctx, args.max_batch)
     rng = np.random.default_rng(args.seed)
@@ -314,9 +320,28 @@ def main():
         err = be.take_error()
         if err:
             raise SystemExit(f"device error: {err}")
-        print(json.dumps({"metric": "decode tok/s (decode-only run for a kernel trace)", "value": round(tok_s, 2),
-                          "unit": "tok/s", "steps": args.steps, "warmup": args.warmup,
-                          "ms_per_step": round(1e3 * dt / args.steps, 4), "graph": graph_stats}), flush=True)
+        line = {"metric": "decode tok/s (decode-only run for a kernel trace)", "value": round(tok_s, 2),
+                "unit": "tok/s", "steps": args.steps, "warmup": args.warmup,
+                "ms_per_step": round(1e3 * dt / args.steps, 4), "graph": graph_stats}
+        if args.expert_slots:
+            # the pool's two tiers: where the reads of the run so far were served from, then the same stretch again
+            # after the busy host-tier experts have changed places with idle device-tier ones
+            st = be.expert_stats()
+            t4 = time.perf_counter()
+            moved = be.replace_experts_by_counts()
+            t_move = time.perf_counter() - t4
+            t5 = time.perf_counter()
+            eng.decode_greedy(args.steps)
+            be.sync()
+            dt2 = time.perf_counter() - t5
+            st2 = be.expert_stats()
+            line["expert_tiers"] = {
+                "device_slots": int(st.slots), "host_slots": int(st.host_slots), "slot_bytes": int(st.slot_bytes),
+                "reads": int(st.lookups), "reads_from_device_memory": int(st.hits),
+                "exchanged_by_counts": int(moved), "exchange_s": round(t_move, 3),
+                "tok_s_after_exchange": round(args.steps / dt2, 2),
+                "reads_after": int(st2.lookups - st.lookups), "from_device_memory_after": int(st2.hits - st.hits)}
+        print(json.dumps(line), flush=True)
         eng.close(); model.close(); be.close()
         if not args.keep:
             try:

@@ -85,7 +85,9 @@ typedef struct {
     uint64_t slots, resident_bytes, weight_bytes, kv_bytes, quant_bytes, pool_bytes;
 } it_tier_counters;
 
-/* struct ExpertStats, src/ops/cuda/experts.rs:210-315 (the all-resident subset) */
+/* struct ExpertStats, src/ops/cuda/experts.rs:210-315 (the fields of the device and pinned-host tiers): hits = reads
+ * served from device memory, lookups - hits = reads that crossed the bus, host_slots = experts in the host tier,
+ * evictions = experts moved out of device memory by replace_experts_by_counts, fetched = 0 (no third tier) */
 typedef struct {
     uint64_t slots, slot_bytes, resident, pool, host_slots, evictions, fetched, lookups, hits;
     uint32_t oversubscribed, _pad;
@@ -216,16 +218,22 @@ size_t it_hip_config_report(it_hip*, char* buf, size_t buf_len);
 uint64_t it_hip_setup_cost(it_hip*, char* label, size_t label_len);
 void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x, uint64_t x_len, uint64_t k);
 
-/* ---- expert cache API, all-resident tier (src/ops/cuda/ops/placement.rs:15-363) ----
- * 288 GB of device memory hold every expert of the models this backend serves, so the cache is one tier: each expert
- * matrix of a pooled tensor takes a slot at first sight of its tensor and is never evicted.  The slab keeps the
+/* ---- expert cache API (src/ops/cuda/ops/placement.rs:15-363, src/ops/cuda/experts.rs:34-62) ----
+ * 288 GB of device memory hold every expert of the models this backend is measured on, so the cache normally is one
+ * tier: each expert matrix of a pooled tensor takes a device slot at first sight of its tensor.  The slab keeps the
  * reference's shape: one uniform slot size (the bytes of one expert matrix; a tensor of another size is refused,
  * experts.rs:890-901), a capacity in slots fixed when the first pooled tensor arrives (set_expert_slots, else
  * set_expert_budget, else free device memory minus the reserves), and per-expert read counters on the device that
- * the expert kernels write.  A pool larger than the capacity is refused with a sticky error: the pinned-host and SSD
- * tiers are not part of this backend. */
+ * the expert kernels write.
+ * A pool larger than the capacity spills into a second tier, as in the reference: the experts that do not fit live in
+ * page-locked host memory mapped into the device's address space (up to set_expert_host_budget bytes), every pooled
+ * tensor is then read through a device table of per-expert addresses, and a kernel dereferences an expert wherever it
+ * lies, so a miss is slow (it crosses the bus) but never blocks and never changes a value.  Placement is first touch
+ * wins device memory; replace_experts_by_counts exchanges busy host-tier experts with idle device-tier ones.  A pool
+ * that outgrows both tiers is refused with a sticky error: experts fetched from the model file (the reference's third
+ * tier) are not part of this backend. */
 void it_hip_set_expert_budget(it_hip*, uint64_t bytes);      /* placement.rs:178 */
-void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes); /* placement.rs:322; kept and reported, no host tier */
+void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes); /* placement.rs:322; 0 = 64 GiB */
 void it_hip_set_expert_slots(it_hip*, uint64_t n);           /* placement.rs:157; 0 = by budget */
 void it_hip_set_expert_pool(it_hip*, uint64_t n);            /* sizes the read counters, experts.rs:424-438 */
 void it_hip_reserve_for_weights(it_hip*, uint64_t dense_bytes); /* placement.rs:203 */
@@ -238,8 +246,8 @@ void it_hip_expert_stats(it_hip*, it_expert_stats* out);
 /* share of all expert reads taken by the busiest slab-many matrices, and the reads counted (placement.rs:347,
  * experts.rs:861-873); 0 = ok, 1 = no pooled tensor yet */
 int it_hip_expert_coverage(it_hip*, double* fraction, uint64_t* total_reads);
-/* re-place the pool by the reads counted so far; returns the experts moved (always 0 here), -1 on a device error
- * (placement.rs:113) */
+/* re-place the pool by the reads counted so far: busy host-tier experts change places with idle device-tier ones;
+ * returns the experts moved into device memory (0 with the whole pool there), -1 on a device error (placement.rs:113) */
 int64_t it_hip_replace_experts_by_counts(it_hip*);
 /* extension: the per-expert read counts of one tensor (keyed on its data pointer), expert order; returns entries */
 uint64_t it_hip_expert_counts(it_hip*, const uint8_t* tensor_data, uint32_t* out, uint64_t cap);

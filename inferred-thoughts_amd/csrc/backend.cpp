@@ -437,12 +437,12 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
             fail(std::string(who) + ": expert tensor length is not n_expert matrices of its shape");
             return false;
         }
-        if (expert_resident && expert_slot_bytes != one) {
+        if (expert_slot_bytes && expert_slot_bytes != one) {
             fail(std::string(who) + ": expert matrix is " + std::to_string(one) + " bytes but the slab's slot is " +
                  std::to_string(expert_slot_bytes) + "; the pool is not uniform, which this arena assumes");
             return false;
         }
-        if (!expert_resident) {
+        if (!expert_slot_bytes) {
             // sized at the first pooled tensor, from what is free then (placement.rs:294-312, 423-453)
             expert_slot_bytes = one;
             size_t fr = 0, tot = 0;
@@ -450,20 +450,27 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
             const uint64_t by_budget = expert_budget ? expert_budget : (fr > expert_reserve ? fr - expert_reserve : 0);
             expert_slots_cap = expert_slots_req ? expert_slots_req : by_budget / one;
         }
-        if (expert_resident + w->n_expert > expert_slots_cap) {
-            fail(std::string(who) + ": the expert pool needs " + std::to_string(expert_resident + w->n_expert) +
-                 " slots of " + std::to_string(one) + " bytes but the device tier holds " + std::to_string(expert_slots_cap) +
-                 "; tiers beyond device memory (pinned host, SSD) are not part of this backend");
-            return false;
-        }
         if (!expert_counters_reserve(expert_counted + w->n_expert)) return false;
     }
-    const Resident* r = resident(w->data, w->len, w->ty, w->n_in, w->n_out * w->n_expert, who);
-    if (!r) return false;
+    if (fresh && expert_resident + w->n_expert > expert_slots_cap) {
+        // The pool outgrows the device tier: the experts that still fit take device slots, the rest go to pinned host
+        // memory, and from here on every pooled tensor is read through its placement table.
+        const uint64_t free_slots = expert_slots_cap > expert_resident ? expert_slots_cap - expert_resident : 0;
+        if (!place_two_tier(w, std::min<uint64_t>(free_slots, w->n_expert), who)) return false;
+    } else {
+        const Resident* r = resident(w->data, w->len, w->ty, w->n_in, w->n_out * w->n_expert, who);
+        if (!r) return false;
+        if (fresh) {
+            expert_resident += w->n_expert;
+            Resident& nr = weights[w->data];
+            nr.n_expert = w->n_expert;
+            nr.q_stride = nr.q_bytes / w->n_expert;
+            nr.s_stride = nr.s_bytes / w->n_expert;
+            if (pool_tabled && !table_for(nr)) return false;
+        }
+    }
     if (fresh) {
-        // all-resident tier: every expert of the tensor is placed at first sight
-        expert_resident += w->n_expert;
-        if (expert_pool < expert_resident) expert_pool = expert_resident;
+        if (expert_pool < expert_resident + expert_host_entries) expert_pool = expert_resident + expert_host_entries;
         weights[w->data].counter_base = (int64_t)expert_counted;
         expert_counted += w->n_expert;
     }
@@ -491,7 +498,202 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
     }
     out->scale2 = (w->scale && w->scale_len) ? rw->scale2 : nullptr;
     out->counts = rw->counter_base >= 0 ? expert_counts + rw->counter_base : nullptr;
+    out->q_tab = rw->q_tab;
+    out->s_tab = rw->s_tab;
+    out->tier = rw->tier;
     return true;
+}
+
+// ------------------------------------------------------------------ two-tier placement
+// src/ops/cuda/experts.rs:34-62: an expert lives in a device slot or in a page-locked host block that the device
+// addresses directly, so a kernel dereferences it either way and a miss is slow, never blocking.  Placement is first
+// touch wins device memory; replace_by_counts() later exchanges busy host experts with idle device ones.
+static constexpr uint64_t DEFAULT_EXPERT_HOST_BUDGET = 64ull << 30;
+
+bool it_hip::table_upload(Resident& r) {
+    const size_t n = r.n_expert;
+    if (!r.q_tab) {
+        if (!check(hipMalloc((void**)&r.q_tab, n * sizeof(void*)), "hipMalloc(expert table)") ||
+            !check(hipMalloc((void**)&r.s_tab, n * sizeof(void*)), "hipMalloc(expert table)") ||
+            !check(hipMalloc((void**)&r.tier, n), "hipMalloc(expert tiers)"))
+            return false;
+    }
+    return check(hipMemcpy(r.q_tab, r.h_q.data(), n * sizeof(void*), hipMemcpyHostToDevice), "upload expert table") &&
+           check(hipMemcpy(r.s_tab, r.h_s.data(), n * sizeof(void*), hipMemcpyHostToDevice), "upload expert table") &&
+           check(hipMemcpy(r.tier, r.h_tier.data(), n, hipMemcpyHostToDevice), "upload expert tiers");
+}
+
+bool it_hip::table_for(Resident& r) {
+    if (r.q_tab || !r.n_expert) return true;
+    need_eager("an expert tensor gets a placement table");
+    drop_graph();   // a captured graph reads this tensor at its stride
+    check(hipStreamSynchronize(stream), "sync before an expert table is made");
+    r.h_q.resize(r.n_expert);
+    r.h_s.resize(r.n_expert);
+    r.h_tier.assign(r.n_expert, 0);
+    for (uint64_t e = 0; e < r.n_expert; e++) {
+        r.h_q[e] = (const uint8_t*)r.q + e * r.q_stride;
+        r.h_s[e] = (const uint8_t*)r.scales + e * r.s_stride;
+    }
+    return table_upload(r);
+}
+
+bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who) {
+    const uint64_t n = w->n_expert, n_host = n - n_dev;
+    const uint64_t raw_one = type_row_bytes(w->ty, w->n_in) * w->n_out;
+    const bool q8 = w->ty == IT_Q8_0;
+    const uint64_t q_stride = q8 ? w->n_out * w->n_in : w->n_out * (w->n_in / 2);
+    const uint64_t s_stride = q8 ? w->n_out * (w->n_in / 32) * 2 : w->n_out * (w->n_in / 16);
+    const uint64_t budget = expert_host_budget ? expert_host_budget : DEFAULT_EXPERT_HOST_BUDGET;
+    if (expert_host_bytes + n_host * (q_stride + s_stride) > budget) {
+        fail(std::string(who) + ": the expert pool needs " + std::to_string(expert_resident + expert_host_entries + n) +
+             " slots but the device tier holds " + std::to_string(expert_slots_cap) + " and the pinned host tier's budget of " +
+             std::to_string(budget) + " bytes is used up; a tier behind it (experts fetched from the model file) is not part of this backend");
+        return false;
+    }
+    need_eager("an expert tensor is placed in two tiers");
+    drop_graph();
+    check(hipStreamSynchronize(stream), "sync before two-tier placement");
+    uint64_t t0 = now_us();
+    // every tensor placed so far is read through a table from now on
+    if (!pool_tabled) {
+        pool_tabled = true;
+        for (auto& kv : weights)
+            if (kv.second.counter_base >= 0 && !table_for(kv.second)) return false;
+    }
+    Resident r;
+    r.fmt = (int)w->ty;
+    r.n_in = w->n_in;
+    r.rows = w->n_out * n;
+    r.ident = weight_ident(w->data, w->len);
+    r.n_expert = n;
+    r.q_stride = q_stride;
+    r.s_stride = s_stride;
+    r.q_bytes = n_dev * q_stride;
+    r.s_bytes = n_dev * s_stride;
+    if (n_dev && (!check(hipMalloc(&r.q, r.q_bytes), "hipMalloc(expert quants)") ||
+                  !check(hipMalloc(&r.scales, r.s_bytes), "hipMalloc(expert scales)")))
+        return false;
+    uint8_t *dq_host = nullptr, *ds_host = nullptr;   // the pinned blocks as the device addresses them
+    if (n_host) {
+        if (!check(hipHostMalloc(&r.host_q, n_host * q_stride, hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc(expert host tier)") ||
+            !check(hipHostMalloc(&r.host_s, n_host * s_stride, hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc(expert host tier)") ||
+            !check(hipHostGetDevicePointer((void**)&dq_host, r.host_q, 0), "hipHostGetDevicePointer") ||
+            !check(hipHostGetDevicePointer((void**)&ds_host, r.host_s, 0), "hipHostGetDevicePointer"))
+            return false;
+    }
+    // upload and repack a few experts at a time through device staging, then move each to its place
+    const uint64_t chunk = std::min<uint64_t>(8, n);
+    void *raw = nullptr, *tq = nullptr, *ts = nullptr;
+    if (!check(hipMalloc(&raw, chunk * raw_one), "hipMalloc(expert staging)") ||
+        !check(hipMalloc(&tq, chunk * q_stride), "hipMalloc(expert staging)") ||
+        !check(hipMalloc(&ts, chunk * s_stride), "hipMalloc(expert staging)"))
+        return false;
+    bool ok = true;
+    for (uint64_t e0 = 0; e0 < n && ok; e0 += chunk) {
+        const uint64_t m = std::min(chunk, n - e0);
+        ok = ok && check(hipMemcpyAsync(raw, w->data + e0 * raw_one, m * raw_one, hipMemcpyHostToDevice, stream), "upload experts");
+        if (q8) repack_q8_0((const uint8_t*)raw, (int8_t*)tq, (uint16_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
+        else repack_nvfp4((const uint8_t*)raw, (uint8_t*)tq, (uint8_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
+        for (uint64_t k = 0; k < m && ok; k++) {
+            const uint64_t e = e0 + k;
+            const uint8_t* fq = (const uint8_t*)tq + k * q_stride;
+            const uint8_t* fs = (const uint8_t*)ts + k * s_stride;
+            if (e < n_dev) {
+                ok = check(hipMemcpyAsync((uint8_t*)r.q + e * q_stride, fq, q_stride, hipMemcpyDeviceToDevice, stream), "place expert") &&
+                     check(hipMemcpyAsync((uint8_t*)r.scales + e * s_stride, fs, s_stride, hipMemcpyDeviceToDevice, stream), "place expert");
+            } else {
+                ok = check(hipMemcpyAsync((uint8_t*)r.host_q + (e - n_dev) * q_stride, fq, q_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier") &&
+                     check(hipMemcpyAsync((uint8_t*)r.host_s + (e - n_dev) * s_stride, fs, s_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier");
+            }
+        }
+        ok = ok && check(hipStreamSynchronize(stream), "place experts");
+    }
+    (void)hipFree(raw);
+    (void)hipFree(tq);
+    (void)hipFree(ts);
+    if (!ok) return false;
+    h2d++;
+    h2d_bytes += w->len;
+    r.h_q.resize(n);
+    r.h_s.resize(n);
+    r.h_tier.resize(n);
+    for (uint64_t e = 0; e < n; e++) {
+        const bool dev = e < n_dev;
+        r.h_q[e] = dev ? (const uint8_t*)r.q + e * q_stride : dq_host + (e - n_dev) * q_stride;
+        r.h_s[e] = dev ? (const uint8_t*)r.scales + e * s_stride : ds_host + (e - n_dev) * s_stride;
+        r.h_tier[e] = dev ? 0 : 1;
+    }
+    if (!table_upload(r)) return false;
+    weight_bytes += r.q_bytes + r.s_bytes;
+    expert_resident += n_dev;
+    expert_host_entries += n_host;
+    expert_host_bytes += n_host * (q_stride + s_stride);
+    setup_us += now_us() - t0;
+    weights.emplace(w->data, std::move(r));
+    return true;
+}
+
+// Exchange busy host-tier experts with idle device-tier ones until every device expert has been read at least as often
+// as every host one (replace_experts_by_counts, placement.rs:113-128; the counts are kept).  Returns the exchanges.
+int64_t it_hip::replace_by_counts() {
+    std::vector<uint32_t> counts;
+    uint64_t tally[2];
+    if (!expert_counters_read(&counts, tally)) return -1;
+    if (!pool_tabled || !expert_host_entries) return 0;
+    struct Entry { Resident* r; uint32_t e; uint32_t count; };
+    std::vector<Entry> dev, host;
+    for (auto& kv : weights) {
+        Resident& r = kv.second;
+        if (r.counter_base < 0 || !r.q_tab) continue;
+        for (uint64_t e = 0; e < r.n_expert; e++) {
+            Entry en{&r, (uint32_t)e, counts[(size_t)r.counter_base + e]};
+            (r.h_tier[e] ? host : dev).push_back(en);
+        }
+    }
+    // idle device experts first, busy host experts first; ties by placement order so that the outcome is repeatable
+    std::stable_sort(dev.begin(), dev.end(), [](const Entry& a, const Entry& b) {
+        return a.count != b.count ? a.count < b.count : (a.r->counter_base + a.e) < (b.r->counter_base + b.e);
+    });
+    std::stable_sort(host.begin(), host.end(), [](const Entry& a, const Entry& b) {
+        return a.count != b.count ? a.count > b.count : (a.r->counter_base + a.e) < (b.r->counter_base + b.e);
+    });
+    size_t pairs = 0;
+    while (pairs < dev.size() && pairs < host.size() && host[pairs].count > dev[pairs].count) pairs++;
+    if (!pairs) return 0;
+    need_eager("experts move between tiers");
+    if (!check(hipStreamSynchronize(stream), "sync before experts move")) return -1;
+    const uint64_t qs = dev[0].r->q_stride, ss = dev[0].r->s_stride;
+    void *tq = nullptr, *ts = nullptr;
+    if (!check(hipMalloc(&tq, qs), "hipMalloc(expert exchange)") || !check(hipMalloc(&ts, ss), "hipMalloc(expert exchange)")) return -1;
+    bool ok = true;
+    std::vector<Resident*> touched;
+    for (size_t k = 0; k < pairs && ok; k++) {
+        Entry &d = dev[k], &h = host[k];
+        uint8_t* slot_q = const_cast<uint8_t*>(d.r->h_q[d.e]);
+        uint8_t* slot_s = const_cast<uint8_t*>(d.r->h_s[d.e]);
+        uint8_t* blk_q = const_cast<uint8_t*>(h.r->h_q[h.e]);   // device-visible addresses of the pinned block
+        uint8_t* blk_s = const_cast<uint8_t*>(h.r->h_s[h.e]);
+        ok = check(hipMemcpyAsync(tq, slot_q, qs, hipMemcpyDeviceToDevice, stream), "exchange experts") &&
+             check(hipMemcpyAsync(ts, slot_s, ss, hipMemcpyDeviceToDevice, stream), "exchange experts") &&
+             check(hipMemcpyAsync(slot_q, blk_q, qs, hipMemcpyDefault, stream), "exchange experts") &&
+             check(hipMemcpyAsync(slot_s, blk_s, ss, hipMemcpyDefault, stream), "exchange experts") &&
+             check(hipMemcpyAsync(blk_q, tq, qs, hipMemcpyDefault, stream), "exchange experts") &&
+             check(hipMemcpyAsync(blk_s, ts, ss, hipMemcpyDefault, stream), "exchange experts");
+        d.r->h_q[d.e] = blk_q; d.r->h_s[d.e] = blk_s; d.r->h_tier[d.e] = 1;
+        h.r->h_q[h.e] = slot_q; h.r->h_s[h.e] = slot_s; h.r->h_tier[h.e] = 0;
+        touched.push_back(d.r);
+        touched.push_back(h.r);
+    }
+    ok = ok && check(hipStreamSynchronize(stream), "exchange experts");
+    (void)hipFree(tq);
+    (void)hipFree(ts);
+    std::sort(touched.begin(), touched.end());
+    touched.erase(std::unique(touched.begin(), touched.end()), touched.end());
+    for (Resident* r : touched) ok = ok && table_upload(*r);
+    if (!ok) return -1;
+    expert_swaps += pairs;
+    return (int64_t)pairs;
 }
 
 // the device read counters hold at least `entries` (tensor, expert) entries; existing counts survive a growth
@@ -789,6 +991,11 @@ void it_hip::drop_all() {
         if (kv.second.q) (void)hipFree(kv.second.q);
         if (kv.second.scales) (void)hipFree(kv.second.scales);
         if (kv.second.scale2) (void)hipFree(kv.second.scale2);
+        if (kv.second.q_tab) (void)hipFree((void*)kv.second.q_tab);
+        if (kv.second.s_tab) (void)hipFree((void*)kv.second.s_tab);
+        if (kv.second.tier) (void)hipFree(kv.second.tier);
+        if (kv.second.host_q) (void)hipHostFree(kv.second.host_q);
+        if (kv.second.host_s) (void)hipHostFree(kv.second.host_s);
     }
     weights.clear();
     for (auto& kv : slabs)
@@ -800,6 +1007,8 @@ void it_hip::drop_all() {
     expert_slot_bytes = 0;
     expert_slots_cap = 0;
     expert_counted = 0;
+    expert_host_entries = expert_host_bytes = expert_swaps = 0;
+    pool_tabled = false;
     if (expert_counts) (void)hipMemset(expert_counts, 0, expert_counts_cap * sizeof(uint32_t));
     if (expert_tally) (void)hipMemset(expert_tally, 0, 2 * sizeof(unsigned long long));
 }
@@ -1410,13 +1619,13 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     it_hip::OpRec rec;
     rec.id = OP_EXPERTS; rec.p[0] = v.q; rec.p[1] = v.scales; rec.p[2] = v.scale2; rec.p[3] = ids; rec.p[4] = as; rec.p[5] = aq;
     rec.p[6] = dout; rec.i[0] = v.fmt; rec.i[1] = v.n_in; rec.i[2] = v.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
-    rec.i[6] = v.q_stride; rec.i[7] = v.s_stride; rec.p[7] = v.counts;
+    rec.i[6] = v.q_stride; rec.i[7] = v.s_stride; rec.p[7] = v.counts; rec.i[8] = v.q_tab ? 1 : 0;
     unsigned long long* tally = be->expert_tally;
     uint32_t* counts = v.counts;
     be->submit(it_hip::FAM_MOE_DOWN, picks * (w->len / w->n_expert) + x_len + out_len * 4,
-               sig_of(OP_EXPERTS, v.q, v.scales, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
+               sig_of(OP_EXPERTS, v.q, v.scales, (const void*)v.q_tab, v.fmt, v.n_in, v.n_out, v.scale2, ids, np, nu, xm, as, aq, dout), rec,
                [=](hipStream_t s) {
-                   expert_count(ids, np, v.n_expert, counts, nullptr, tally, s);
+                   expert_count(ids, np, v.n_expert, counts, nullptr, tally, s, v.tier, nullptr);
                    if (skinny_shape && experts_gemm_f16s(v, nullptr, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (rows_shape && expert_rows(v, nullptr, ids, np, nu, xm, as, aq, dout, 1.0f, work, work_ints, grouped, s)) return;
@@ -1473,14 +1682,14 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     rec.id = OP_GLU; rec.p[0] = g.q; rec.p[1] = g.scales; rec.p[2] = u.q; rec.p[3] = u.scales; rec.p[4] = g.scale2;
     rec.p[5] = u.scale2; rec.p[6] = ids; rec.p[7] = as; rec.p[8] = aq; rec.p[9] = dout;
     rec.i[0] = g.fmt; rec.i[1] = g.n_in; rec.i[2] = g.n_out; rec.i[3] = np; rec.i[4] = nu; rec.i[5] = xm;
-    rec.i[6] = g.q_stride; rec.i[7] = g.s_stride; rec.p[10] = g.counts; rec.p[11] = u.counts;
+    rec.i[6] = g.q_stride; rec.i[7] = g.s_stride; rec.p[10] = g.counts; rec.p[11] = u.counts; rec.i[8] = (g.q_tab || u.q_tab) ? 1 : 0;
     unsigned long long* tally = be->expert_tally;
     uint32_t *cg = g.counts, *cu = u.counts;
     be->submit(it_hip::FAM_MOE_GLU, 2 * picks * (gate->len / gate->n_expert) + x_len + out_len * 4,
-               sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
+               sig_of(OP_GLU, g.q, g.scales, u.q, u.scales, (const void*)g.q_tab, (const void*)u.q_tab, g.fmt, g.n_in, g.n_out, g.scale2, u.scale2, ids, np, nu, xm,
                       as, aq, dout), rec,
                [=](hipStream_t s) {
-                   expert_count(ids, np, g.n_expert, cg, cu, tally, s);
+                   expert_count(ids, np, g.n_expert, cg, cu, tally, s, g.tier, u.tier);
                    if (skinny_shape && experts_gemm_f16s(g, &u, ids, np, nu, xm, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
                        return;
                    if (rows_shape && expert_rows(g, &u, ids, np, nu, xm, as, aq, dout, 1.0f, work, work_ints, grouped, s)) return;
@@ -1741,20 +1950,24 @@ int it_hip_tier_counters(it_hip* be, it_tier_counters* out) {
     out->pool_bytes = be->attn_scratch_cap * 4;
     out->resident_bytes = be->weight_bytes + be->kv_bytes + be->quant_bytes + be->mirror_bytes +
                           be->const_bytes + out->pool_bytes;
-    out->oversubscribed = be->expert_resident > be->expert_slots_cap;
+    out->oversubscribed = be->pool_tabled;
     return 1;
 }
 
 size_t it_hip_config_report(it_hip* be, char* buf, size_t buf_len) {
     int n = snprintf(buf, buf_len,
-                     "backend=hip gfx950\nreductions=%s\ndecode graph=%s\nattention=%s\nexpert tier=all-resident\n"
-                     "expert slots=%llu of %llu bytes (%s)\nexpert host budget=%llu (no host tier)\nexpert prefetch=%s (nothing to fetch)\n"
+                     "backend=hip gfx950\nreductions=%s\ndecode graph=%s\nattention=%s\nexpert tier=%s\n"
+                     "expert slots=%llu of %llu bytes (%s)\nexpert host tier=%llu experts, %llu bytes of a budget of %llu\n"
+                     "expert prefetch=%s (no tier to fetch from: a host-tier expert is read in place)\n"
                      "model path=%s\n",
                      be->exact ? "serial (CPU order)" : "tree / split-K", be->allow_graph ? "on" : "off",
                      be->exact ? "exact" : "split-K flash decoding (128-position chunks)",
+                     be->pool_tabled ? "device memory + pinned host, read through placement tables" : "all-resident",
                      (unsigned long long)be->expert_slots_cap, (unsigned long long)be->expert_slot_bytes,
                      be->expert_slots_req ? "fixed" : be->expert_budget ? "by budget" : "by free device memory",
-                     (unsigned long long)be->expert_host_budget, be->expert_prefetch ? "on" : "off",
+                     (unsigned long long)be->expert_host_entries, (unsigned long long)be->expert_host_bytes,
+                     (unsigned long long)(be->expert_host_budget ? be->expert_host_budget : DEFAULT_EXPERT_HOST_BUDGET),
+                     be->expert_prefetch ? "on" : "off",
                      be->model_path.empty() ? "(not set)" : be->model_path.c_str());
     return n < 0 ? 0 : (size_t)n;
 }
@@ -1764,14 +1977,14 @@ uint64_t it_hip_setup_cost(it_hip* be, char* label, size_t label_len) {
     return be->setup_us;
 }
 void it_hip_prefetch_hint(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, uint64_t k) {
-    (void)be; (void)w; (void)x; (void)x_len; (void)k;  // every expert is resident: nothing to fetch
+    (void)be; (void)w; (void)x; (void)x_len; (void)k;  // every expert is addressable where it lies: nothing to fetch
 }
 
 // Cap the expert slab, in bytes; 0 restores sizing from free device memory (placement.rs:178-189).  Like the
 // reference's, read once: when the first pooled tensor sizes the slab.
 void it_hip_set_expert_budget(it_hip* be, uint64_t bytes) { be->expert_budget = bytes; }
-// The pinned-host tier behind the slab (placement.rs:322-326).  This backend has no host tier: the value is kept and
-// reported, and a pool that does not fit the device tier is refused instead of spilling.
+// The pinned-host tier behind the slab (placement.rs:322-326): experts that do not fit the device tier go to page-locked
+// host memory up to this many bytes (0 = the default of 64 GiB); a pool that outgrows both is refused.
 void it_hip_set_expert_host_budget(it_hip* be, uint64_t bytes) { be->expert_host_budget = bytes; }
 // Fix the slab at n slots whatever the budget says; 0 restores sizing by budget (placement.rs:157-159)
 void it_hip_set_expert_slots(it_hip* be, uint64_t n) { be->expert_slots_req = n; }
@@ -1804,8 +2017,9 @@ void it_hip_expert_stats(it_hip* be, it_expert_stats* out) {
     out->pool = be->expert_pool;
     out->lookups = tally[0] + tally[1];
     out->hits = tally[0];
-    out->host_slots = 0;
-    out->oversubscribed = be->expert_resident > be->expert_slots_cap;
+    out->host_slots = be->expert_host_entries;
+    out->evictions = be->expert_swaps;
+    out->oversubscribed = be->pool_tabled;
 }
 
 // What fraction of all expert reads the busiest slab-many matrices took, and the reads counted
@@ -1825,13 +2039,10 @@ int it_hip_expert_coverage(it_hip* be, double* fraction, uint64_t* total_reads) 
     return 0;
 }
 
-// Re-place the pool by the reads counted so far (placement.rs:113-128): with every expert in device memory no host
-// expert can be busier than a resident one, so nothing moves.  Returns the experts moved, or -1 on a device error.
-int64_t it_hip_replace_experts_by_counts(it_hip* be) {
-    uint64_t tally[2];
-    if (!be->expert_counters_read(nullptr, tally)) return -1;
-    return 0;
-}
+// Re-place the pool by the reads counted so far (placement.rs:113-128): busy experts of the pinned host tier change
+// places with idle ones of the device tier; with every expert in device memory nothing moves.  Returns the experts
+// moved into device memory, or -1 on a device error.
+int64_t it_hip_replace_experts_by_counts(it_hip* be) { return be->replace_by_counts(); }
 
 // per-expert read counts of one tensor, in expert order (the rows of `counts` the gather wrote for it); returns the
 // number of entries written, 0 when the tensor has not been seen

@@ -99,7 +99,24 @@ struct it_hip {
         float* scale2 = nullptr;  // experts' per-expert second scale
         int64_t counter_base = -1;  // first of this tensor's entries in expert_counts (expert tensors only)
         uint64_t ident = 0;         // length and a sample of the host bytes: another file mapped at the same address differs
+        // Two-tier placement of an expert tensor (src/ops/cuda/experts.rs:34-52): once the pool outgrows its device tier
+        // every pooled tensor is read through a table of per-expert addresses, each a device slot or a block of pinned
+        // host memory mapped into the device's address space.  Host copies of the tables beside the device arrays.
+        uint64_t n_expert = 0, q_stride = 0, s_stride = 0;
+        const uint8_t** q_tab = nullptr;
+        const uint8_t** s_tab = nullptr;
+        uint8_t* tier = nullptr;                 // device: 0 = device memory, 1 = pinned host
+        std::vector<const uint8_t*> h_q, h_s;
+        std::vector<uint8_t> h_tier;
+        void* host_q = nullptr;                  // pinned blocks of the experts first placed in the host tier
+        void* host_s = nullptr;
     };
+    bool place_two_tier(const it_experts* w, uint64_t n_dev, const char* who);
+    bool table_for(Resident& r);                 // an identity table for a tensor that sits in device memory whole
+    bool table_upload(Resident& r);
+    int64_t replace_by_counts();
+    uint64_t expert_host_entries = 0, expert_host_bytes = 0, expert_swaps = 0;
+    bool pool_tabled = false;                    // some pooled tensor did not fit the device tier
     std::unordered_map<const void*, Resident> weights;
     const Resident* resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in, uint64_t rows,
                              const char* who);

@@ -396,6 +396,8 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
     const Op &q3 = o[i + 13], &sdm = o[i + 14], &fin = o[i + 15], &add = o[i + 16];
     int64_t nd = rms.i[1];
     if (rms.i[0] != 1) return false;
+    // experts placed through a table (a pool larger than its device tier) are read by the unfused kernels only
+    if (glu.i[8] || ex.i[8]) return false;
     if (ga.p[0] != rms.p[2] || ga.i[0] != nd || ga.i[2] != 0 || ga.i[3] != nd) return false;
     const void* x = ga.p[1];
     if (q1.p[0] != x || q1.i[0] != nd || ml.i[2] != 1) return false;

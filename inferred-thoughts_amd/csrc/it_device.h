@@ -28,6 +28,11 @@ IT_DEV void it_count_expert_reads(const int32_t* ids, int n_used, uint32_t* cg, 
     if (t == 0) atomicAdd(tally, (unsigned long long)((cg ? 1 : 0) + (cu ? 1 : 0) + (cd ? 1 : 0)) * n_used);
 }
 
+// expert e's bytes: through the placement table when the pool has one, else at its stride from the tensor's base
+IT_DEV const uint8_t* it_expert_at(const uint8_t* base, const uint8_t* const* tab, int64_t e, int64_t stride) {
+    return tab ? tab[e] : base + e * stride;
+}
+
 IT_DEV float it_f16_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 IT_DEV uint16_t it_f32_to_f16(float f) { return __half_as_ushort(__float2half_rn(f)); }
 IT_DEV float it_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }

@@ -64,6 +64,7 @@ IT_DEV void fp4x4_to_f16x4(uint32_t v, h2 scale, h2* a, h2* b) {
 // operands of the f16 expert tile kernels (k_gemm_f16.hip, k_gemm_f16s.hip)
 struct ExpertsF16P {
     const uint8_t *q, *s, *q2, *s2;
+    const uint8_t* const *q_tab, *const *s_tab, *const *q2_tab, *const *s2_tab;  // expert placement tables or null
     int64_t q_stride, s_stride;
     const float *scale2, *scale2_up;
     const uint16_t *xh, *xl;

@@ -232,6 +232,7 @@ __global__ __launch_bounds__(1024) void moe_group_k(const int32_t* __restrict__ 
 
 struct ExpertsGemmP {
     const uint8_t *q, *s, *q2, *s2;
+    const uint8_t* const *q_tab, *const *s_tab, *const *q2_tab, *const *s2_tab;  // expert placement tables or null
     int64_t q_stride, s_stride;
     const float *scale2, *scale2_up;
     const float* act_scales;
@@ -272,8 +273,8 @@ __global__ __launch_bounds__(GT) void experts_gemm_k(ExpertsGemmP p) {
         xrow_s[tid] = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
     }
     __syncthreads();
-    const uint8_t* wq[2] = {p.q + e * p.q_stride, GLU ? p.q2 + e * p.q_stride : nullptr};
-    const uint8_t* ws[2] = {p.s + e * p.s_stride, GLU ? p.s2 + e * p.s_stride : nullptr};
+    const uint8_t* wq[2] = {it_expert_at(p.q, p.q_tab, e, p.q_stride), GLU ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : nullptr};
+    const uint8_t* ws[2] = {it_expert_at(p.s, p.s_tab, e, p.s_stride), GLU ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : nullptr};
 
     uint4 ra[NM][2], rb;
     float rsa[NM][2], rsb;
@@ -428,6 +429,10 @@ bool experts_gemm(const ExpertsView& w, const ExpertsView* up, const int32_t* id
     p.s2 = up ? (const uint8_t*)up->scales : nullptr;
     p.q_stride = w.q_stride;
     p.s_stride = w.s_stride;
+    p.q_tab = w.q_tab;
+    p.s_tab = w.s_tab;
+    p.q2_tab = up ? up->q_tab : nullptr;
+    p.s2_tab = up ? up->s_tab : nullptr;
     p.scale2 = w.scale2;
     p.scale2_up = up ? up->scale2 : nullptr;
     p.act_scales = act_scales;

@@ -106,8 +106,10 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     const int rows_per_block = GLU ? 128 : 256;
     const int rb0 = blockIdx.y * rows_per_block + (GLU ? 32 : 64) * wave;
     const int rbase[2] = {rb0, GLU ? rb0 : rb0 + 32};
-    const uint8_t* wq[2] = {p.q + e * p.q_stride, GLU ? p.q2 + e * p.q_stride : p.q + e * p.q_stride};
-    const uint8_t* ws[2] = {p.s + e * p.s_stride, GLU ? p.s2 + e * p.s_stride : p.s + e * p.s_stride};
+    const uint8_t* wq0 = it_expert_at(p.q, p.q_tab, e, p.q_stride);
+    const uint8_t* ws0 = it_expert_at(p.s, p.s_tab, e, p.s_stride);
+    const uint8_t* wq[2] = {wq0, GLU ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : wq0};
+    const uint8_t* ws[2] = {ws0, GLU ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : ws0};
     // this wave's row segments in the block's weight buffer: GLU [set][wave][row], else [wave][set][row]
     const int myseg[2] = {GLU ? 32 * wave + r : 64 * wave + r, GLU ? 128 + 32 * wave + r : 64 * wave + 32 + r};
     // the segments this thread loads (four rows, one 16-byte piece of each row's 128 nibble bytes) and, for the
@@ -411,6 +413,10 @@ bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t
     p.s2 = up ? (const uint8_t*)up->scales : nullptr;
     p.q_stride = w.q_stride;
     p.s_stride = w.s_stride;
+    p.q_tab = w.q_tab;
+    p.s_tab = w.s_tab;
+    p.q2_tab = up ? up->q_tab : nullptr;
+    p.s2_tab = up ? up->s_tab : nullptr;
     p.scale2 = w.scale2;
     p.scale2_up = up ? up->scale2 : nullptr;
     p.xh = xh;

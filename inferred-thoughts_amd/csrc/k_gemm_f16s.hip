@@ -123,8 +123,8 @@ __global__ __launch_bounds__(256) void experts_f16s_k(ExpertsF16P p, int gpw) {
     const int xrow = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
     const uint16_t* bh = p.xh + (int64_t)xrow * n_in + 32 * kg;
     const uint16_t* bl = p.xl + (int64_t)xrow * n_in + 32 * kg;
-    const uint8_t* wq = (z ? p.q2 : p.q) + e * p.q_stride;
-    const uint8_t* ws = (z ? p.s2 : p.s) + e * p.s_stride;
+    const uint8_t* wq = z ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : it_expert_at(p.q, p.q_tab, e, p.q_stride);
+    const uint8_t* ws = z ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : it_expert_at(p.s, p.s_tab, e, p.s_stride);
 
     v4f acc[SK_G];
 #pragma unroll
@@ -258,6 +258,10 @@ bool experts_gemm_f16s(const ExpertsView& w, const ExpertsView* up, const int32_
     p.s2 = up ? (const uint8_t*)up->scales : nullptr;
     p.q_stride = w.q_stride;
     p.s_stride = w.s_stride;
+    p.q_tab = w.q_tab;
+    p.s_tab = w.s_tab;
+    p.q2_tab = up ? up->q_tab : nullptr;
+    p.s2_tab = up ? up->s_tab : nullptr;
     p.scale2 = w.scale2;
     p.scale2_up = up ? up->scale2 : nullptr;
     p.xh = xh;

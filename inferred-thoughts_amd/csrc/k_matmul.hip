@@ -63,6 +63,7 @@ struct GemvP {
     const uint8_t *q, *s;     // weights (gate when GLU)
     const uint8_t *q2, *s2;   // up weights when GLU
     int64_t q_stride, s_stride;  // bytes per expert (0 for a dense matrix)
+    const uint8_t* const *q_tab, *const *s_tab, *const *q2_tab, *const *s2_tab;  // expert placement tables or null
     const int32_t* ids;       // expert id per y, or null
     const float *scale2, *scale2_up;  // per-expert second scales or null
     const float* act_scales;  // [x_rows][n_in/32]
@@ -93,10 +94,10 @@ __global__ __launch_bounds__(64 * GEMV_WAVES) void gemv_k(GemvP p) {
     const int nrows = min(R, p.n_out - row0);
 
     int64_t e = p.ids ? (int64_t)p.ids[y] : 0;
-    const uint8_t* wq = p.q + e * p.q_stride;
-    const uint8_t* ws = p.s + e * p.s_stride;
-    const uint8_t* wq2 = GLU ? p.q2 + e * p.q_stride : nullptr;
-    const uint8_t* ws2 = GLU ? p.s2 + e * p.s_stride : nullptr;
+    const uint8_t* wq = it_expert_at(p.q, p.q_tab, e, p.q_stride);
+    const uint8_t* ws = it_expert_at(p.s, p.s_tab, e, p.s_stride);
+    const uint8_t* wq2 = GLU ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : nullptr;
+    const uint8_t* ws2 = GLU ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : nullptr;
     int xr = p.x_mode == 0 ? y : (p.x_mode == 1 ? y / p.n_used : 0);
     const int8_t* aq = p.act_quants + (int64_t)xr * p.n_in;
     const float* as = p.act_scales + (int64_t)xr * U;
@@ -357,6 +358,8 @@ static GemvP experts_params(const ExpertsView& w, const int32_t* ids, int n_used
     p.q_stride = w.q_stride;
     p.s_stride = w.s_stride;
     p.ids = ids;
+    p.q_tab = w.q_tab;
+    p.s_tab = w.s_tab;
     p.scale2 = w.scale2;
     p.act_scales = act_scales;
     p.act_quants = act_quants;
@@ -383,6 +386,8 @@ void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids,
     GemvP p = experts_params(gate, ids, n_used, x_mode, act_scales, act_quants, out);
     p.q2 = (const uint8_t*)up.q;
     p.s2 = (const uint8_t*)up.scales;
+    p.q2_tab = up.q_tab;
+    p.s2_tab = up.s_tab;
     p.scale2_up = up.scale2;
     if (gate.fmt == W_Q8_0) launch_gemv<W_Q8_0, true>(p, n_picks, s);
     else launch_gemv<W_NVFP4, true>(p, n_picks, s);

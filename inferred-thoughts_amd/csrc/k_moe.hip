@@ -114,8 +114,11 @@ __global__ __launch_bounds__(256) void route_topk_wave_k(const float* __restrict
 constexpr int COUNT_BINS = 2048;
 __global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict__ ids, int n_picks, int n_expert,
                                                       uint32_t* __restrict__ counts_a, uint32_t* __restrict__ counts_b,
-                                                      unsigned long long* __restrict__ tally) {
+                                                      unsigned long long* __restrict__ tally,
+                                                      const uint8_t* __restrict__ tier_a, const uint8_t* __restrict__ tier_b) {
     __shared__ unsigned bins[COUNT_BINS];
+    __shared__ unsigned host_reads;
+    if (threadIdx.x == 0) host_reads = 0;
     const bool local = n_expert <= COUNT_BINS;
     if (local)
         for (int e = threadIdx.x; e < n_expert; e += 256) bins[e] = 0;
@@ -129,6 +132,8 @@ __global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict_
         } else {
             atomicAdd(counts_a + e, 1u);
             if (counts_b) atomicAdd(counts_b + e, 1u);
+            const unsigned h = (tier_a && tier_a[e] ? 1u : 0u) + (counts_b && tier_b && tier_b[e] ? 1u : 0u);
+            if (h) atomicAdd(&host_reads, h);
         }
     }
     __syncthreads();
@@ -138,16 +143,28 @@ __global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict_
             if (c) {
                 atomicAdd(counts_a + e, c);
                 if (counts_b) atomicAdd(counts_b + e, c);
+                const unsigned h = (tier_a && tier_a[e] ? c : 0u) + (counts_b && tier_b && tier_b[e] ? c : 0u);
+                if (h) atomicAdd(&host_reads, h);
             }
         }
-    if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(tally, (unsigned long long)n_picks * (counts_b ? 2 : 1));
+    __syncthreads();
+    // tally[0]: reads served from device memory, tally[1]: reads that crossed the bus to the pinned host tier
+    if (threadIdx.x == 0) {
+        const unsigned long long h = host_reads;
+        if (h) atomicAdd(tally + 1, h);
+        const unsigned long long all = blockIdx.x == 0 ? (unsigned long long)n_picks * (counts_b ? 2 : 1) : 0ull;
+        // block 0 books every read as a device read; each block takes its host reads back out (unsigned wrap-around
+        // of the running sum is harmless: the total is exact once every block has added)
+        atomicAdd(tally, all - h);
+    }
 }
 
 void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
-                  unsigned long long* tally, hipStream_t s) {
+                  unsigned long long* tally, hipStream_t s, const uint8_t* tier_a, const uint8_t* tier_b) {
     if (n_picks <= 0 || !counts_a || !tally) return;
     const int blocks = std::max(1, std::min(64, (n_picks + 1023) / 1024));
-    hipLaunchKernelGGL(expert_count_k, dim3(blocks), dim3(256), 0, s, ids, n_picks, n_expert, counts_a, counts_b, tally);
+    hipLaunchKernelGGL(expert_count_k, dim3(blocks), dim3(256), 0, s, ids, n_picks, n_expert, counts_a, counts_b, tally,
+                       tier_a, tier_b);
 }
 
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,

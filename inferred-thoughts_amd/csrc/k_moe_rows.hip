@@ -30,6 +30,7 @@ namespace {
 
 struct ExpertRowsP {
     const uint8_t *q, *s, *q2, *s2;
+    const uint8_t* const *q_tab, *const *s_tab, *const *q2_tab, *const *s2_tab;  // expert placement tables or null
     int64_t q_stride, s_stride;
     const float *scale2, *scale2_up;
     const float* act_scales;
@@ -125,10 +126,10 @@ __global__ __launch_bounds__(256) void expert_rows_k(ExpertRowsP p) {
     constexpr int RPI = 64 / L;          // rows per wave instruction
     const int sub = lane / L, ul = lane % L;
     const int upl = U / L;               // units per lane and row
-    const uint8_t* wq = p.q + e * p.q_stride;
-    const uint8_t* ws = p.s + e * p.s_stride;
-    const uint8_t* wq2 = GLU ? p.q2 + e * p.q_stride : nullptr;
-    const uint8_t* ws2 = GLU ? p.s2 + e * p.s_stride : nullptr;
+    const uint8_t* wq = it_expert_at(p.q, p.q_tab, e, p.q_stride);
+    const uint8_t* ws = it_expert_at(p.s, p.s_tab, e, p.s_stride);
+    const uint8_t* wq2 = GLU ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : nullptr;
+    const uint8_t* ws2 = GLU ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : nullptr;
     const int row_lo = blockIdx.x * RB, row_hi = min(row_lo + RB, p.n_out);
     // rows row_lo + RPI * (wave + 4 i) + sub; a row past the end repeats the last one and is not stored.
     // A step is one unit of one row: steps i * upl .. i * upl + upl - 1 walk row i's units L apart.
@@ -295,6 +296,10 @@ bool expert_rows(const ExpertsView& w, const ExpertsView* up, const int32_t* ids
     p.s2 = up ? (const uint8_t*)up->scales : nullptr;
     p.q_stride = ids ? w.q_stride : 0;
     p.s_stride = ids ? w.s_stride : 0;
+    p.q_tab = ids ? w.q_tab : nullptr;
+    p.s_tab = ids ? w.s_tab : nullptr;
+    p.q2_tab = ids && up ? up->q_tab : nullptr;
+    p.s2_tab = ids && up ? up->s_tab : nullptr;
     p.scale2 = w.scale2;
     p.scale2_up = up ? up->scale2 : nullptr;
     p.act_scales = act_scales;

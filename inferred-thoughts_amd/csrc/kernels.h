@@ -46,6 +46,12 @@ struct ExpertsView {
     int fmt, n_in, n_out, n_expert;
     const float* scale2;  // per-expert second scale or null
     uint32_t* counts;     // this tensor's per-expert read counters (device), or null
+    // Two-tier placement (device arrays of n_expert entries, or null when every expert sits in device memory at its
+    // stride): where expert e's quants and scales are, in a device slot or in pinned host memory that the device
+    // reads across the bus, and which of the two (0 device, 1 host) for the read tallies.
+    const uint8_t* const* q_tab;
+    const uint8_t* const* s_tab;
+    const uint8_t* tier;
 };
 // One matmul per pick.  x rows: mode 0 = one row per pick, 1 = one row per token
 // (pick i reads row i / n_used), 2 = a single shared row.
@@ -96,7 +102,7 @@ void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids,
 // tally[0] += the reads counted: the device-side read counters of the expert cache (reads served from device memory;
 // tally[1], reads served from a host tier, stays 0 when every expert is resident)
 void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
-                  unsigned long long* tally, hipStream_t s);
+                  unsigned long long* tally, hipStream_t s, const uint8_t* tier_a = nullptr, const uint8_t* tier_b = nullptr);
 
 // ---- router ----------------------------------------------------------------------
 void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);

@@ -1,4 +1,4 @@
-"""The expert cache API as an all-resident tier (/root/reference src/ops/cuda/ops/placement.rs:15-363,
+"""The expert cache API with every expert in device memory (/root/reference src/ops/cuda/ops/placement.rs:15-363,
 src/ops/cuda/experts.rs:210-315, 424-438, 890-901): device-side read counters, slab sizing, refusals."""
 import numpy as np
 import pytest
@@ -86,20 +86,26 @@ def test_refusals():
     be.matmul_experts(ih.experts(wb2, ih.Q8_0, n_in, 2 * n_out, n_expert), route, x, np.zeros(4 * n_out, np.float32))
     assert "not uniform" in (be.take_error() or "")
     be.end_pass(); be.close()
-    # a slab fixed at fewer slots than the pool needs: refused, not spilled (no host tier in this backend)
+    # a slab fixed at fewer slots than the pool needs spills into the pinned host tier (tests/test_gpu_expert_tiers.py);
+    # with that tier's budget used up as well the tensor is refused: no tier behind it
     be = ih.Hip()
     be.set_expert_slots(n_expert - 1)
+    be.set_expert_host_budget(1)
     be.begin_pass(1)
     be.matmul_experts(ih.experts(wb, ih.Q8_0, n_in, n_out, n_expert), route, x, np.zeros(2 * n_out, np.float32))
-    assert "tiers beyond device memory" in (be.take_error() or "")
+    err = be.take_error() or ""
+    assert "pinned host tier's budget" in err and "holds 7" in err
     be.end_pass(); be.close()
-    # a budget in bytes sizes the slab the same way
+    # a budget in bytes sizes the slab the same way: three slots, five experts in the host tier
     be = ih.Hip()
     be.set_expert_budget(3 * n_out * n_in // 32 * 34)
     be.begin_pass(1)
     be.matmul_experts(ih.experts(wb, ih.Q8_0, n_in, n_out, n_expert), route, x, np.zeros(2 * n_out, np.float32))
-    assert "holds 3" in (be.take_error() or "")
-    be.end_pass(); be.close()
+    be.end_pass()
+    assert be.take_error() is None
+    st = be.expert_stats()
+    assert st.slots == 3 and st.resident == 3 and st.host_slots == 5 and st.oversubscribed == 1
+    be.close()
 
 
 def test_qwen4exp_only_methods_are_refused_not_run():
