@@ -291,11 +291,11 @@ struct it_hip {
     uint64_t launches = 0, h2d = 0, d2h = 0, h2d_bytes = 0, d2h_bytes = 0;
     uint64_t weight_bytes = 0, kv_bytes = 0, quant_bytes = 0, mirror_bytes = 0, const_bytes = 0;
     uint64_t setup_us = 0;
-    // ---- expert cache, all-resident tier (src/ops/cuda/ops/placement.rs, experts.rs)
-    // Every expert matrix of a pooled tensor is placed in device memory at first sight of the tensor.  The slab has
-    // one uniform slot size (the bytes of one expert matrix in the file); its capacity in slots comes from
-    // set_expert_slots, else set_expert_budget, else free device memory minus the reserves, and a pool that does not
-    // fit is refused (the pinned-host and SSD tiers are not part of this backend).  Reads are counted on the device.
+    // ---- expert cache (src/ops/cuda/ops/placement.rs, experts.rs)
+    // Every expert matrix of a pooled tensor is placed at first sight of the tensor: in device memory while slots are
+    // left, else in pinned host memory (place_two_tier).  The slab has one uniform slot size (the bytes of one expert
+    // matrix in the file); its capacity in slots comes from set_expert_slots, else set_expert_budget, else free
+    // device memory minus the reserves.  Reads are counted on the device.
     uint64_t expert_resident = 0, expert_slot_bytes = 0, expert_pool = 0, expert_slots_cap = 0;
     uint64_t expert_budget = 0, expert_host_budget = 0, expert_slots_req = 0, expert_reserve = 1ull << 30;
     bool expert_prefetch = true;
