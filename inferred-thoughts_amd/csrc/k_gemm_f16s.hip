@@ -221,6 +221,114 @@ __global__ __launch_bounds__(256) void experts_f16s_k(ExpertsF16P p, int gpw) {
     }
 }
 
+
+// The same products with the k range split over the waves of a block.  Above, a wave walks one 128-byte column of its
+// rows chunk after chunk, so every DRAM page is opened once per chunk and the stream stops at 3.5 TB/s.  Here the KW
+// waves of a row set take one 256-wide chunk EACH (n_in = 256 KW, KW = 1, 2, 4 or 8) and walk the same row groups
+// together: the block reads whole rows at a time, a wave's B operands are loaded once for the whole kernel, and both
+// matrices of the gate/up pair share them.  The price is a reduction of the KW partial sums of every 16 x 16 tile
+// through LDS: a batch of four tiles per wave (two row groups of gate and up, or four of one matrix), one barrier per
+// batch, two LDS buffers in turn.
+template <bool GLU, int KW>
+__global__ __launch_bounds__(512) void experts_f16k_k(ExpertsF16P p, int batches_per_block) {
+    constexpr int NM = GLU ? 2 : 1;
+    constexpr int GB = 4 / NM;        // row groups per batch
+    constexpr int RS = 8 / KW;        // row sets per block
+    __shared__ float4 red[2][8][4][64];   // [buffer][wave][tile of the batch][lane]
+    const int tile = blockIdx.x;
+    if (tile >= *p.n_tiles) return;
+    const int4 td = p.tiles[tile];
+    const int64_t e = td.x;
+    const int cnt = td.z;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kw = wave % KW, rs = wave / KW;
+    const int r16 = lane & 15, kg = lane >> 4;
+    const int n_in = p.n_in, n_groups = (p.n_out + 15) / 16;
+    const int pair = p.order[td.y + min(r16, cnt - 1)];
+    const int xrow = p.x_mode == 0 ? pair : (p.x_mode == 1 ? pair / p.n_used : 0);
+    const uint8_t* wq[2] = {it_expert_at(p.q, p.q_tab, e, p.q_stride), GLU ? it_expert_at(p.q2, p.q2_tab, e, p.q_stride) : nullptr};
+    const uint8_t* ws[2] = {it_expert_at(p.s, p.s_tab, e, p.s_stride), GLU ? it_expert_at(p.s2, p.s2_tab, e, p.s_stride) : nullptr};
+
+    // step st = batch i, group slot j, matrix z of this wave: i = st / 4, (j, z) = st % 4
+    const int n_steps = batches_per_block * 4;
+    auto group_of = [&](int st) { return ((blockIdx.y * batches_per_block + st / 4) * RS + rs) * GB + (st % 4) / NM; };
+    auto load_step = [&](int st) __attribute__((always_inline)) -> RawW {
+        RawW o;
+        const int z = GLU ? st & 1 : 0;
+        const int64_t row = min(group_of(st) * 16 + r16, p.n_out - 1);
+        const int u = 8 * kw + kg;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            o.nib[h] = *(const uint4*)(wq[z] + row * (n_in >> 1) + (u + 4 * h) * 16);
+            o.sc[h] = *(const uint16_t*)(ws[z] + row * (n_in >> 4) + (u + 4 * h) * 2);
+        }
+        return o;
+    };
+    RawW q0 = load_step(0), q1 = load_step(1);
+    // this wave's B operands: chunk kw of the tile's 16 pairs, for the whole kernel
+    h8 fh[8], fl[8];
+    {
+        const uint16_t* bh = p.xh + (int64_t)xrow * n_in + kw * SK_KC + 32 * kg;
+        const uint16_t* bl = p.xl + (int64_t)xrow * n_in + kw * SK_KC + 32 * kg;
+#pragma unroll
+        for (int n = 0; n < 8; n++) {
+            fh[n] = __builtin_bit_cast(h8, *(const uint4*)(bh + 128 * (n >> 2) + 8 * (n & 3)));
+            fl[n] = __builtin_bit_cast(h8, *(const uint4*)(bl + 128 * (n >> 2) + 8 * (n & 3)));
+        }
+    }
+    const float rsc = p.rscale[xrow];
+    const float e2a = p.scale2 ? p.scale2[e] : 1.0f;
+    const float e2b = GLU ? (p.scale2_up ? p.scale2_up[e] : 1.0f) : e2a;
+
+    for (int i = 0; i < batches_per_block; i++) {
+        const int buf = i & 1;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int st = 4 * i + t;
+            RawW nx = q0;
+            if (st + 2 < n_steps) nx = load_step(st + 2);
+            v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int n = 0; n < 8; n++) {
+                const h8 a = expand_frag(q0.nib[n >> 2], q0.sc[n >> 2], n & 3);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fh[n], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fl[n], acc, 0, 0, 0);
+            }
+            red[buf][wave][t][lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            q0 = q1;
+            q1 = nx;
+        }
+        __syncthreads();
+        // group slot j of the batch is finished by the wave kw == j % KW of its row set: the KW partial sums of its
+        // tile (of both tiles for the gate/up pair), the epilogue and the store
+#pragma unroll
+        for (int j = 0; j < GB; j++) {
+            if (j % KW != kw) continue;
+            const int g = group_of(4 * i + j * NM);
+            const int row = g * 16 + 4 * kg;
+            if (g >= n_groups || row >= p.n_out || r16 >= cnt) continue;
+            float sum[NM][4];
+#pragma unroll
+            for (int z = 0; z < NM; z++) {
+                sum[z][0] = sum[z][1] = sum[z][2] = sum[z][3] = 0.0f;
+#pragma unroll
+                for (int k = 0; k < KW; k++) {
+                    const float4 v = red[buf][rs * KW + k][j * NM + z][lane];
+                    sum[z][0] += v.x; sum[z][1] += v.y; sum[z][2] += v.z; sum[z][3] += v.w;
+                }
+            }
+            float o[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (GLU) o[q] = fx_silu(sum[0][q] * rsc * e2a) * (sum[NM - 1][q] * rsc * e2b);
+                else o[q] = sum[0][q] * rsc * e2a;
+            }
+            *(float4*)(p.out + (int64_t)pair * p.n_out + row) = make_float4(o[0], o[1], o[2], o[3]);
+        }
+    }
+}
+
 }  // namespace
 
 bool experts_f16s_takes(const ExpertsView& w, const ExpertsView* up, int n_picks, const int8_t* act_quants, const float* out) {
@@ -275,9 +383,27 @@ bool experts_gemm_f16s(const ExpertsView& w, const ExpertsView* up, const int32_
     p.n_tiles = n_tiles;
     p.tiles = tiles;
     p.order = order;
-    // row groups per wave: as many as keep about three blocks per CU in flight
     const int groups = (w.n_out + 15) / 16;
     const int likely_tiles = std::min(n_picks, w.n_expert) + n_picks / SK_PAIRS;
+    const int n_chunk = w.n_in / SK_KC;
+    if (n_chunk == 1 || n_chunk == 2 || n_chunk == 4 || n_chunk == 8) {
+        // k split over the waves: a batch is 4 / NM row groups per row set, 8 / n_chunk row sets per block; 8 batches
+        // per block while that leaves about 1,024 blocks (16 or 32 batches measured 10 % slower, 4 the same)
+        const int per_batch = (up ? 2 : 4) * (8 / n_chunk);
+        const int batches = (groups + per_batch - 1) / per_batch;
+        int bpb = std::min(batches, 8);
+        while (bpb > 1 && (int64_t)likely_tiles * ((batches + bpb - 1) / bpb) < 1024) bpb >>= 1;
+        const dim3 grid(std::min(n_picks, max_tiles), (batches + bpb - 1) / bpb);
+#define IT_F16K(G, K) hipLaunchKernelGGL((experts_f16k_k<G, K>), grid, dim3(512), 0, s, p, bpb)
+        if (up) {
+            if (n_chunk == 8) IT_F16K(true, 8); else if (n_chunk == 4) IT_F16K(true, 4); else if (n_chunk == 2) IT_F16K(true, 2); else IT_F16K(true, 1);
+        } else {
+            if (n_chunk == 8) IT_F16K(false, 8); else if (n_chunk == 4) IT_F16K(false, 4); else if (n_chunk == 2) IT_F16K(false, 2); else IT_F16K(false, 1);
+        }
+#undef IT_F16K
+        return true;
+    }
+    // other row lengths: every wave walks the whole k range of its own rows
     int gpw = SK_G;
     const int wpb = up ? 2 : 4;   // shares of a block's row groups (the gate/up pair puts two waves on each)
     while (gpw > 1 && (int64_t)likely_tiles * ((groups + wpb * gpw - 1) / (wpb * gpw)) < 2048) gpw >>= 1;
