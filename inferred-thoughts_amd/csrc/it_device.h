@@ -28,9 +28,16 @@ IT_DEV void it_count_expert_reads(const int32_t* ids, int n_used, uint32_t* cg, 
     if (t == 0) atomicAdd(tally, (unsigned long long)((cg ? 1 : 0) + (cu ? 1 : 0) + (cd ? 1 : 0)) * n_used);
 }
 
-// expert e's bytes: through the placement table when the pool has one, else at its stride from the tensor's base
+// Expert e's bytes: through the placement table when the pool has one, else at its stride from the tensor's base.  A
+// pointer read from the table is device-visible memory (a device slot or mapped pinned host memory), never LDS or
+// scratch: saying so keeps the loads through it global loads, whose completion the hardware counts in order (behind a
+// generic pointer every load becomes a flat load, and a wait for one of those waits for all of them).
+typedef __attribute__((address_space(1))) const uint8_t* it_global_bytes;
 IT_DEV const uint8_t* it_expert_at(const uint8_t* base, const uint8_t* const* tab, int64_t e, int64_t stride) {
-    return tab ? tab[e] : base + e * stride;
+    // (the table is read as an array of global pointers: a generic -> global -> generic round trip of the loaded
+    // value would be folded away again)
+    if (tab) return (const uint8_t*)((const it_global_bytes*)tab)[e];
+    return base + e * stride;
 }
 
 IT_DEV float it_f16_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }

@@ -253,28 +253,37 @@ __global__ __launch_bounds__(512) void experts_f16k_k(ExpertsF16P p, int batches
     // step st = batch i, group slot j, matrix z of this wave: i = st / 4, (j, z) = st % 4
     const int n_steps = batches_per_block * 4;
     auto group_of = [&](int st) { return ((blockIdx.y * batches_per_block + st / 4) * RS + rs) * GB + (st % 4) / NM; };
-    auto load_step = [&](int st) __attribute__((always_inline)) -> RawW {
+    // (the matrix z is passed as a constant of the unrolled code: a pointer picked by a run-time index stops being a
+    // global pointer for the compiler, and its loads become flat loads that every wait has to drain)
+    auto load_step = [&](int st, int z) __attribute__((always_inline)) -> RawW {
         RawW o;
-        const int z = GLU ? st & 1 : 0;
         const int64_t row = min(group_of(st) * 16 + r16, p.n_out - 1);
-        const int u = 8 * kw + kg;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            o.nib[h] = *(const uint4*)(wq[z] + row * (n_in >> 1) + (u + 4 * h) * 16);
-            o.sc[h] = *(const uint16_t*)(ws[z] + row * (n_in >> 4) + (u + 4 * h) * 2);
-        }
+        // units 2 kg and 2 kg + 1 of the chunk: the four lanes of a row read its 128-byte line between them, and a
+        // lane's four scale bytes are one load (two-byte loads, eight bytes per row, cost a quarter of the stream's time)
+        const int u = 8 * kw + 2 * kg;
+        o.nib[0] = *(const uint4*)(wq[z] + row * (n_in >> 1) + u * 16);
+        o.nib[1] = *(const uint4*)(wq[z] + row * (n_in >> 1) + u * 16 + 16);
+        o.sc[0] = *(const uint32_t*)(ws[z] + row * (n_in >> 4) + u * 2);   // unit 2 kg in the low half, 2 kg + 1 above
+        o.sc[1] = 0;
         return o;
     };
-    RawW q0 = load_step(0), q1 = load_step(1);
+    // Four register sets, one per step of a batch: step t computes from set t while the load of step t + 3 goes
+    // straight into set (t + 3) % 4.  No set is ever copied (a copy of a load's destination waits for the load) and
+    // the load is unconditional (past the end it repeats the last step), so the compiler's wait before a step counts
+    // exactly the loads issued after the ones it needs.
+    RawW q[4];
+    q[0] = load_step(0, 0);
+    q[1] = load_step(1, GLU ? 1 : 0);
+    q[2] = load_step(2, 0);
     // this wave's B operands: chunk kw of the tile's 16 pairs, for the whole kernel
     h8 fh[8], fl[8];
     {
-        const uint16_t* bh = p.xh + (int64_t)xrow * n_in + kw * SK_KC + 32 * kg;
-        const uint16_t* bl = p.xl + (int64_t)xrow * n_in + kw * SK_KC + 32 * kg;
+        const uint16_t* bh = p.xh + (int64_t)xrow * n_in + kw * SK_KC + 64 * kg;
+        const uint16_t* bl = p.xl + (int64_t)xrow * n_in + kw * SK_KC + 64 * kg;
 #pragma unroll
         for (int n = 0; n < 8; n++) {
-            fh[n] = __builtin_bit_cast(h8, *(const uint4*)(bh + 128 * (n >> 2) + 8 * (n & 3)));
-            fl[n] = __builtin_bit_cast(h8, *(const uint4*)(bl + 128 * (n >> 2) + 8 * (n & 3)));
+            fh[n] = __builtin_bit_cast(h8, *(const uint4*)(bh + 8 * n));
+            fl[n] = __builtin_bit_cast(h8, *(const uint4*)(bl + 8 * n));
         }
     }
     const float rsc = p.rscale[xrow];
@@ -286,18 +295,16 @@ __global__ __launch_bounds__(512) void experts_f16k_k(ExpertsF16P p, int batches
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const int st = 4 * i + t;
-            RawW nx = q0;
-            if (st + 2 < n_steps) nx = load_step(st + 2);
+            q[(t + 3) & 3] = load_step(min(st + 3, n_steps - 1), GLU ? (t + 3) & 1 : 0);
+            __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the step they overlap
             v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int n = 0; n < 8; n++) {
-                const h8 a = expand_frag(q0.nib[n >> 2], q0.sc[n >> 2], n & 3);
+                const h8 a = expand_frag(q[t].nib[n >> 2], n < 4 ? q[t].sc[0] : q[t].sc[0] >> 16, n & 3);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fh[n], acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fl[n], acc, 0, 0, 0);
             }
             red[buf][wave][t][lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-            q0 = q1;
-            q1 = nx;
         }
         __syncthreads();
         // group slot j of the batch is finished by the wave kw == j % KW of its row set: the KW partial sums of its
