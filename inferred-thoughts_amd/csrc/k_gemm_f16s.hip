@@ -271,10 +271,13 @@ __global__ __launch_bounds__(512) void experts_f16k_k(ExpertsF16P p, int batches
     // straight into set (t + 3) % 4.  No set is ever copied (a copy of a load's destination waits for the load) and
     // the load is unconditional (past the end it repeats the last step), so the compiler's wait before a step counts
     // exactly the loads issued after the ones it needs.
-    RawW q[4];
+    constexpr int QD = GLU ? 2 : 4;
+    RawW q[QD];
     q[0] = load_step(0, 0);
-    q[1] = load_step(1, GLU ? 1 : 0);
-    q[2] = load_step(2, 0);
+    if (QD == 4) {
+        q[1] = load_step(1, GLU ? 1 : 0);
+        q[2] = load_step(2, 0);
+    }
     // this wave's B operands: chunk kw of the tile's 16 pairs, for the whole kernel
     h8 fh[8], fl[8];
     {
@@ -295,12 +298,12 @@ __global__ __launch_bounds__(512) void experts_f16k_k(ExpertsF16P p, int batches
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const int st = 4 * i + t;
-            q[(t + 3) & 3] = load_step(min(st + 3, n_steps - 1), GLU ? (t + 3) & 1 : 0);
+            q[(t + QD - 1) % QD] = load_step(min(st + QD - 1, n_steps - 1), GLU ? (t + QD - 1) & 1 : 0);
             __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the step they overlap
             v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int n = 0; n < 8; n++) {
-                const h8 a = expand_frag(q[t].nib[n >> 2], n < 4 ? q[t].sc[0] : q[t].sc[0] >> 16, n & 3);
+                const h8 a = expand_frag(q[t % QD].nib[n >> 2], n < 4 ? q[t % QD].sc[0] : q[t % QD].sc[0] >> 16, n & 3);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fh[n], acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, fl[n], acc, 0, 0, 0);
             }
