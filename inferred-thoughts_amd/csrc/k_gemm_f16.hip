@@ -121,14 +121,16 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
         const int seg = (tid >> 3) + 64 * i;
         const int z = GLU ? seg >> 7 : 0;
         const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? seg & 127 : seg), p.n_out - 1);
-        wload[i] = wq[z] + row * (n_in >> 1) + piece * 16;
+        // (picked by a conditional, not by an index into the array: a pointer that went through an indexed array is a
+        // generic pointer to the compiler, and loads through it are flat loads that every LDS wait has to drain)
+        wload[i] = (z ? wq[1] : wq[0]) + row * (n_in >> 1) + piece * 16;
     }
     const uint8_t* sload;
     {
         const int st = tid & 255;
         const int z = GLU ? st >> 7 : 0;
         const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? st & 127 : st), p.n_out - 1);
-        sload = ws[z] + row * (n_in >> 4);
+        sload = (z ? ws[1] : ws[0]) + row * (n_in >> 4);
     }
 
     // Software pipeline.  Weights come in super-slabs of 256 k: every thread loads full 128-byte lines of

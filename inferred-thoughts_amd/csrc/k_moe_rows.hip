@@ -145,9 +145,8 @@ __global__ __launch_bounds__(256) void expert_rows_k(ExpertRowsP p) {
         if (GLU) o.b = load_raw<FMT>(wq2, ws2, r, n_in, U, u);
         return o;
     };
-    // the first two steps' weights are on their way while the activations are staged
+    // the first step's weights are on their way while the activations are staged
     Both q0 = load_step(0), q1 = q0;
-    if (n_steps > 1) q1 = load_step(1);
 
     uint8_t* xq = lds_raw;                                   // [RP][2][U][16]
     float* xs = (float*)(lds_raw + (size_t)RP * n_in);        // [RP][U]
@@ -210,14 +209,17 @@ __global__ __launch_bounds__(256) void expert_rows_k(ExpertRowsP p) {
             }
         }
     };
+    // Two register sets in turn: while a step computes from one, the next step's load goes straight into the other.
+    // No set is copied (a copy of a load's destination waits for the load), the load is unconditional (past the end it
+    // repeats the last step) and pinned ahead of the step it overlaps, so the wait before a step counts exactly the
+    // loads issued after the ones it needs.
     for (int st = 0; st < n_steps; st += 2) {
-        Both n0 = q0, n1 = q1;
-        if (st + 2 < n_steps) n0 = load_step(st + 2);
-        if (st + 3 < n_steps) n1 = load_step(st + 3);
+        q1 = load_step(min(st + 1, n_steps - 1));
+        __builtin_amdgcn_sched_barrier(0);
         step(st, q0);
+        q0 = load_step(min(st + 2, n_steps - 1));
+        __builtin_amdgcn_sched_barrier(0);
         if (st + 1 < n_steps) step(st + 1, q1);
-        q0 = n0;
-        q1 = n1;
     }
     __syncthreads();
     const float e2a = p.scale2 ? p.scale2[e] : 1.0f;
