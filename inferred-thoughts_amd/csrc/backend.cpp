@@ -1227,14 +1227,27 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     bool one_expert = false, grouped = false;
     // (from 513 tokens on: a call costs 55-80 us for the grouping, the f16 split and a latency-bound handful of
     // tiles, which the GEMVs reach at about 512 tokens)
-    // A dense NVFP4 matrix over 128 .. 512 tokens: eight or sixteen tokens per pass over the rows (k_moe_rows.hip) instead
-    // of one GEMV per token (32 against 70 us for the shared expert's 2048 x 512 at 512 tokens; below 128 tokens the
-    // GEMVs, which fill the chip with one block row per token, are as fast).
+    // A dense NVFP4 matrix over 128 .. 512 tokens whose shape the 16-pair tiles do not take: eight or sixteen tokens per
+    // pass over the rows (k_moe_rows.hip) instead of one GEMV per token (32 against 70 us for 2048 x 512 at 512 tokens;
+    // below 128 tokens the GEMVs, which fill the chip with one block row per token, are as fast).
     ExpertsView rv{};
     rv.q = v.q; rv.scales = v.scales; rv.q_stride = 0; rv.s_stride = 0; rv.fmt = v.fmt; rv.n_in = v.n_in; rv.n_out = v.n_out;
     rv.n_expert = 1; rv.scale2 = nullptr; rv.counts = nullptr;
-    const bool rows_dense = !exact && v.fmt == W_NVFP4 && n >= 128 && n <= 512 && itk::expert_rows_takes(rv, nullptr, aq);
-    if (!exact && v.fmt == W_NVFP4 && n > 512) {
+    // 128 .. 1,024 tokens: as a batch of ONE expert on the 16-pair tiles (2048 x 512 over 1,024 tokens: 34 against 68 us
+    // on the 128-pair tiles, whose handful of blocks is latency-bound there; 16 against 19 us of GEMVs at 128 tokens)
+    bool skinny_dense = false;
+    if (!exact && v.fmt == W_NVFP4 && n >= 128 && n <= 1024) {
+        ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
+        ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr; ev.counts = nullptr;
+        zids = be->zero_ids_for(n);
+        work = be->moe_work_for(n, 1, &work_ints);
+        fwork_bytes = itk::experts_f16_work_bytes(nt, v.n_in);
+        fwork = be->moe_f16_for(fwork_bytes);
+        skinny_dense = zids && work && fwork && itk::experts_f16s_takes(ev, nullptr, nt, aq, dout);
+        if (skinny_dense) grouped = be->group_cached(nt, 1, 16);
+    }
+    const bool rows_dense = !skinny_dense && !exact && v.fmt == W_NVFP4 && n >= 128 && n <= 512 && itk::expert_rows_takes(rv, nullptr, aq);
+    if (!skinny_dense && !exact && v.fmt == W_NVFP4 && n > 512) {   // the 128-pair tiles (82 against 736 us at 5,700 tokens)
         ev.q = v.q; ev.scales = v.scales; ev.q_stride = 0; ev.s_stride = 0;
         ev.fmt = v.fmt; ev.n_in = v.n_in; ev.n_out = v.n_out; ev.n_expert = 1; ev.scale2 = nullptr; ev.counts = nullptr;
         zids = be->zero_ids_for(n);
@@ -1250,6 +1263,8 @@ static void matmul_impl(it_hip* be, const it_weights* w, const float* x, uint64_
     be->submit(it_hip::FAM_MATMUL, w->len + n * w->n_in + n * w->n_out * 4,
                sig_of(OP_MATMUL, v.q, v.scales, v.fmt, v.n_in, v.n_out, dx, as, aq, nt, dout), rec,
                [=](hipStream_t s) {
+                   if (skinny_dense && experts_gemm_f16s(ev, nullptr, zids, nt, 1, 0, as, aq, dout, work, work_ints, fwork, fwork_bytes, grouped, s))
+                       return;
                    if (rows_dense && expert_rows(rv, nullptr, nullptr, nt, 1, 0, as, aq, dout, 1.0f, nullptr, 0, false, s)) return;
                    if (one_expert && experts_gemm_f16(ev, nullptr, zids, nt, 1, 0, as, aq, dout, work, work_ints, fwork,
                                                       fwork_bytes, grouped, s))
