@@ -1579,14 +1579,14 @@ static bool host_ids_in_range(it_hip* be, const it_route* r, uint64_t n_expert, 
 static bool expert_tiles_pay(uint64_t picks, uint64_t n_expert) { return picks >= 32 && 2 * picks >= 7 * n_expert; }
 // Fast mode between the per-pair GEMVs and the wide matrix-core tiles, measured on the 512-expert top-10 FFN (hidden
 // 2048, inter 512): from 1.25 pairs per expert on, grouping the pairs by expert beats one GEMV per pair; NVFP4 then
-// runs 16-pair tiles on the f16 matrix cores (k_gemm_f16s.hip) up to 18 pairs per expert, where the 128-pair tiles
-// take over; what that kernel does not take (Q8_0, odd shapes) streams each expert's rows once for all its pairs
+// runs 16-pair tiles on the f16 matrix cores (k_gemm_f16s.hip) up to 48 pairs per expert (2,048 tokens: 961 against
+// 1,017 us for the whole FFN; 4,096 tokens: 1,571 against 1,447), where the 128-pair tiles take over; what that kernel does not take (Q8_0, odd shapes) streams each expert's rows once for all its pairs
 // (k_moe_rows.hip) until the int8 tiles pay.
 static bool expert_grouping_pays(const it_hip* be, uint64_t picks, uint64_t n_expert) {
     return !be->exact && picks >= 32 && 4 * picks >= 5 * n_expert;
 }
 static bool expert_skinny_pay(const it_hip* be, uint64_t picks, uint64_t n_expert) {
-    return expert_grouping_pays(be, picks, n_expert) && picks < 18 * n_expert;
+    return expert_grouping_pays(be, picks, n_expert) && picks < 48 * n_expert;
 }
 static bool expert_rows_pay(const it_hip* be, uint64_t picks, uint64_t n_expert) {
     return expert_grouping_pays(be, picks, n_expert) && !expert_tiles_pay(picks, n_expert);

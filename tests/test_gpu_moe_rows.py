@@ -1,7 +1,7 @@
 """Expert matmuls of a small batch in fast mode against the CPU oracle, through the C ABI.
 
 From 1.25 pairs per expert on, fast mode sorts the (token, pick) pairs by expert.  NVFP4 experts then run tiles of 16
-pairs on the f16 matrix cores (k_gemm_f16s.hip: weights exact in f16, activations as an f16 hi + lo pair) up to 18 pairs
+pairs on the f16 matrix cores (k_gemm_f16s.hip: weights exact in f16, activations as an f16 hi + lo pair) up to 48 pairs
 per expert; Q8_0 experts, and shapes that kernel does not take, stream every touched expert's rows once and multiply by
 the integer dots of the CPU path (k_moe_rows.hip) until the int8 tiles pay.  Only the f32 summation order (and the 2^-22
 of the split) differs from the oracle, so the bound is 2e-5 of the row's largest output, fifty times tighter than the
@@ -62,7 +62,8 @@ def make(r, orc, fmt, rows, n_in):
     (20, 32, 4, 1024, 100),       # a ragged row count (100 rows); 32 lanes per row
     (24, 16, 2, 4096, 64),        # rows of 128 units (two passes of 64 lanes), 3 pairs per expert
     (33, 8, 1, 4096, 64),         # top-1
-    (100, 64, 10, 256, 2048),     # 15.6 pairs per expert, below the switch to the 128-pair tiles
+    (100, 64, 10, 256, 2048),     # 15.6 pairs per expert
+    (150, 32, 10, 512, 256),      # 47 pairs per expert on average (94 on the busy half): just below the switch to the 128-pair tiles
 ])
 def test_expert_rows_glu_and_down(hip, orc, fmt_name, n_tok, n_expert, n_used, nd, ff):
     import inferred_hip as ih
