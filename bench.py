@@ -461,6 +461,13 @@ def main():
         eng.reset()
         lf = eng.prefill(prompt[:n_p])
         ids_fast = np.asarray(eng.decode_greedy(n_g))
+        # control: fast mode against ITSELF with the prompt cut into other passes (200 + 200 + rest), which moves the
+        # chunk boundaries of the delta rule and the attention kernel's tiles, i.e. last bits only
+        eng.reset()
+        lc = None
+        for at in range(0, n_p, 200):
+            lc = eng.forward(prompt[at:min(at + 200, n_p)])
+        ids_ctl = np.asarray(eng.decode_greedy(n_g))
         be_x = ih.Hip(exact=True)
         eng_x = ih.Engine(model, be_x, args.ctx, args.max_batch)
         lx = eng_x.prefill(prompt[:n_p])
@@ -469,10 +476,21 @@ def main():
         if err:
             raise SystemExit(f"device error in the mode check: {err}")
         same = ids_fast == ids_exact
+        lf64, lx64 = np.asarray(lf, np.float64), np.asarray(lx, np.float64)
+        top_x, top_f = np.argsort(-lx64)[:10], np.argsort(-lf64)[:10]
         mode_check = {"prompt": int(n_p), "ids": int(n_g), "ids_equal": int(same.sum()),
                       "equal_prefix": int(np.argmin(same)) if not same.all() else int(n_g),
                       "prefill_logits_max_abs_diff": float(np.abs(lf - lx).max()),
-                      "prefill_logits_max_abs": float(np.abs(lx).max())}
+                      "prefill_logits_max_abs": float(np.abs(lx).max()),
+                      # how alike the two distributions over the 151,936 tokens are after 512 tokens of prefill
+                      "prefill_logits_correlation": round(float(np.corrcoef(lf64, lx64)[0, 1]), 4),
+                      "exact_top1_rank_in_fast": int(np.where(np.argsort(-lf64) == top_x[0])[0][0]),
+                      "top10_overlap": int(len(set(top_x.tolist()) & set(top_f.tolist()))),
+                      "exact_top1_margin": float(lx64[top_x[0]] - lx64[top_x[1]]),
+                      "control_fast_vs_fast_other_passes": {
+                          "ids_equal": int((ids_ctl == ids_fast).sum()),
+                          "prefill_logits_max_abs_diff": float(np.abs(np.asarray(lc) - np.asarray(lf)).max()),
+                          "prefill_logits_correlation": round(float(np.corrcoef(np.asarray(lc, np.float64), lf64)[0, 1]), 4)}}
         eng_x.close(); be_x.close()
 
     cpu = None
