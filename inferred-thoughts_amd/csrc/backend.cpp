@@ -571,24 +571,31 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
     r.s_stride = s_stride;
     r.q_bytes = n_dev * q_stride;
     r.s_bytes = n_dev * s_stride;
+    void *raw = nullptr, *tq = nullptr, *ts = nullptr;
+    auto give_up = [&]() {   // a failed placement leaves nothing behind
+        for (void* d : {r.q, r.scales, raw, tq, ts, (void*)r.q_tab, (void*)r.s_tab, (void*)r.tier})
+            if (d) (void)hipFree(d);
+        if (r.host_q) (void)hipHostFree(r.host_q);
+        if (r.host_s) (void)hipHostFree(r.host_s);
+        return false;
+    };
     if (n_dev && (!check(hipMalloc(&r.q, r.q_bytes), "hipMalloc(expert quants)") ||
                   !check(hipMalloc(&r.scales, r.s_bytes), "hipMalloc(expert scales)")))
-        return false;
+        return give_up();
     uint8_t *dq_host = nullptr, *ds_host = nullptr;   // the pinned blocks as the device addresses them
     if (n_host) {
         if (!check(hipHostMalloc(&r.host_q, n_host * q_stride, hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc(expert host tier)") ||
             !check(hipHostMalloc(&r.host_s, n_host * s_stride, hipHostMallocMapped | hipHostMallocPortable), "hipHostMalloc(expert host tier)") ||
             !check(hipHostGetDevicePointer((void**)&dq_host, r.host_q, 0), "hipHostGetDevicePointer") ||
             !check(hipHostGetDevicePointer((void**)&ds_host, r.host_s, 0), "hipHostGetDevicePointer"))
-            return false;
+            return give_up();
     }
     // upload and repack a few experts at a time through device staging, then move each to its place
     const uint64_t chunk = std::min<uint64_t>(8, n);
-    void *raw = nullptr, *tq = nullptr, *ts = nullptr;
     if (!check(hipMalloc(&raw, chunk * raw_one), "hipMalloc(expert staging)") ||
         !check(hipMalloc(&tq, chunk * q_stride), "hipMalloc(expert staging)") ||
         !check(hipMalloc(&ts, chunk * s_stride), "hipMalloc(expert staging)"))
-        return false;
+        return give_up();
     bool ok = true;
     for (uint64_t e0 = 0; e0 < n && ok; e0 += chunk) {
         const uint64_t m = std::min(chunk, n - e0);
@@ -609,10 +616,11 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
         }
         ok = ok && check(hipStreamSynchronize(stream), "place experts");
     }
+    if (!ok) return give_up();
     (void)hipFree(raw);
     (void)hipFree(tq);
     (void)hipFree(ts);
-    if (!ok) return false;
+    raw = tq = ts = nullptr;
     h2d++;
     h2d_bytes += w->len;
     r.h_q.resize(n);
@@ -624,7 +632,7 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
         r.h_s[e] = dev ? (const uint8_t*)r.scales + e * s_stride : ds_host + (e - n_dev) * s_stride;
         r.h_tier[e] = dev ? 0 : 1;
     }
-    if (!table_upload(r)) return false;
+    if (!table_upload(r)) return give_up();
     weight_bytes += r.q_bytes + r.s_bytes;
     expert_resident += n_dev;
     expert_host_entries += n_host;

@@ -150,12 +150,9 @@ __global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict_
     __syncthreads();
     // tally[0]: reads served from device memory, tally[1]: reads that crossed the bus to the pinned host tier
     if (threadIdx.x == 0) {
-        const unsigned long long h = host_reads;
+        const unsigned long long mine = (unsigned long long)max(hi - lo, 0) * (counts_b ? 2 : 1), h = host_reads;
         if (h) atomicAdd(tally + 1, h);
-        const unsigned long long all = blockIdx.x == 0 ? (unsigned long long)n_picks * (counts_b ? 2 : 1) : 0ull;
-        // block 0 books every read as a device read; each block takes its host reads back out (unsigned wrap-around
-        // of the running sum is harmless: the total is exact once every block has added)
-        atomicAdd(tally, all - h);
+        if (mine > h) atomicAdd(tally, mine - h);
     }
 }
 
