@@ -229,7 +229,8 @@ void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x
  * page-locked host memory mapped into the device's address space (up to set_expert_host_budget bytes), every pooled
  * tensor is then read through a device table of per-expert addresses, and a kernel dereferences an expert wherever it
  * lies, so a miss is slow (it crosses the bus) but never blocks and never changes a value.  Placement is first touch
- * wins device memory; replace_experts_by_counts exchanges busy host-tier experts with idle device-tier ones.  A pool
+ * wins device memory; every 64 tokens, at a pass boundary, a bounded number of busy host-tier experts change places
+ * with idle device-tier ones (placement.rs:33-80), and replace_experts_by_counts runs that exchange to completion.  A pool
  * that outgrows both tiers is refused with a sticky error: experts fetched from the model file (the reference's third
  * tier) are not part of this backend. */
 void it_hip_set_expert_budget(it_hip*, uint64_t bytes);      /* placement.rs:178 */

@@ -644,7 +644,20 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
 
 // Exchange busy host-tier experts with idle device-tier ones until every device expert has been read at least as often
 // as every host one (replace_experts_by_counts, placement.rs:113-128; the counts are kept).  Returns the exchanges.
-int64_t it_hip::replace_by_counts() {
+// Between passes, never inside one (placement.rs:21-80): every 64 tokens of evidence the busiest host-tier experts
+// change places with the idlest device-tier ones, 200 exchanges per 64 tokens and 2,000 per boundary at most, so that a
+// boundary cannot turn into a visible stall.  The tables are ordinary device memory: a recorded graph reads the new
+// addresses at its next replay, with no re-record.  Stops by itself once no host expert is busier than a device one.
+void it_hip::migrate_at_boundary(uint64_t n_tokens) {
+    if (!pool_tabled || !expert_host_entries) return;
+    tokens_since_migration += n_tokens;
+    if (tokens_since_migration < 64) return;
+    const uint64_t budget = std::min<uint64_t>(200 * (tokens_since_migration / 64), 2000);
+    tokens_since_migration = 0;
+    (void)replace_by_counts(budget);
+}
+
+int64_t it_hip::replace_by_counts(uint64_t budget) {
     std::vector<uint32_t> counts;
     uint64_t tally[2];
     if (!expert_counters_read(&counts, tally)) return -1;
@@ -667,7 +680,7 @@ int64_t it_hip::replace_by_counts() {
         return a.count != b.count ? a.count > b.count : (a.r->counter_base + a.e) < (b.r->counter_base + b.e);
     });
     size_t pairs = 0;
-    while (pairs < dev.size() && pairs < host.size() && host[pairs].count > dev[pairs].count) pairs++;
+    while (pairs < dev.size() && pairs < host.size() && pairs < budget && host[pairs].count > dev[pairs].count) pairs++;
     if (!pairs) return 0;
     need_eager("experts move between tiers");
     if (!check(hipStreamSynchronize(stream), "sync before experts move")) return -1;
@@ -1015,7 +1028,7 @@ void it_hip::drop_all() {
     expert_slot_bytes = 0;
     expert_slots_cap = 0;
     expert_counted = 0;
-    expert_host_entries = expert_host_bytes = expert_swaps = 0;
+    expert_host_entries = expert_host_bytes = expert_swaps = tokens_since_migration = 0;
     pool_tabled = false;
     if (expert_counts) (void)hipMemset(expert_counts, 0, expert_counts_cap * sizeof(uint32_t));
     if (expert_tally) (void)hipMemset(expert_tally, 0, 2 * sizeof(unsigned long long));
@@ -1871,7 +1884,12 @@ void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
 }
 
 void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
-    if (be->in_pass) be->finish_pass();
+    if (be->in_pass) {
+        be->finish_pass();
+        be->in_pass = false;
+    }
+    be->mode = it_hip::Mode::Eager;
+    be->migrate_at_boundary(n_tokens);
     be->in_pass = true;
     be->pass_tokens = n_tokens;
     be->pass_signature.clear();

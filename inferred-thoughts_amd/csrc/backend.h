@@ -114,8 +114,9 @@ struct it_hip {
     bool place_two_tier(const it_experts* w, uint64_t n_dev, const char* who);
     bool table_for(Resident& r);                 // an identity table for a tensor that sits in device memory whole
     bool table_upload(Resident& r);
-    int64_t replace_by_counts();
-    uint64_t expert_host_entries = 0, expert_host_bytes = 0, expert_swaps = 0;
+    int64_t replace_by_counts(uint64_t budget = ~0ull);
+    void migrate_at_boundary(uint64_t n_tokens);   // bounded exchange every 64 tokens of evidence (placement.rs:33-80)
+    uint64_t expert_host_entries = 0, expert_host_bytes = 0, expert_swaps = 0, tokens_since_migration = 0;
     bool pool_tabled = false;                    // some pooled tensor did not fit the device tier
     std::unordered_map<const void*, Resident> weights;
     const Resident* resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in, uint64_t rows,

@@ -58,7 +58,9 @@ def test_mid_model_is_identical_with_two_thirds_of_the_pool_in_host_memory(mid_g
     assert st.pool == 384 and st.fetched == 0
     assert st.lookups == ref[4].lookups                     # the same reads, wherever they were served from
     assert 0 < st.hits < st.lookups and tc.host_reads == st.lookups - st.hits
-    assert two[3] > 0 and st.evictions == two[3]            # busy host experts changed places with idle device ones
+    # busy host experts changed places with idle device ones: by themselves at the pass boundaries (every 64 tokens of
+    # evidence, a bounded number) and then to completion by the explicit call
+    assert st.evictions > two[3] > 0
     assert ref[3] == 0 and ref[4].oversubscribed == 0 and ref[4].host_slots == 0
     assert "pinned host" in two[6] and "all-resident" in ref[6]
     if exact:
@@ -68,7 +70,7 @@ def test_mid_model_is_identical_with_two_thirds_of_the_pool_in_host_memory(mid_g
         for a, b in zip(ref[0], fused[0]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert np.array_equal(ref[1], fused[1]) and np.array_equal(ref[2], fused[2])
-        assert fused[7]["replays"] >= 2 * n_new - 6 and fused[3] > 0
+        assert fused[7]["replays"] >= 2 * n_new - 6 and fused[4].evictions > 0
 
 
 def test_tiny_q8_0_model_through_the_row_kernel_and_the_int8_tiles(tiny_gguf):
@@ -80,7 +82,7 @@ def test_tiny_q8_0_model_through_the_row_kernel_and_the_int8_tiles(tiny_gguf):
         for a, b in zip(ref[0], two[0]):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert np.array_equal(ref[1], two[1]) and np.array_equal(ref[2], two[2])
-        assert two[4].host_slots == 192 - 64 and two[3] > 0
+        assert two[4].host_slots == 192 - 64 and two[4].evictions > 0
 
 
 def test_exchange_by_counts_moves_the_busy_experts_in():
