@@ -242,6 +242,11 @@ def main():
     ap.add_argument("--copy-ref", action="store_true",
                     help="also run one 256 MiB device-to-device torch copy: the kernel of known traffic that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--single-ops-only", action="store_true",
+                    help="no model: run the single-op configurations (expert FFN sweep, decode attention, Gated DeltaNet) and "
+                         "print their JSON (for rocprofv3 traces of those kernels)")
+    ap.add_argument("--ffn-tokens", type=str, default="",
+                    help="with --single-ops-only: only the expert FFN, at these token counts (comma-separated)")
     ap.add_argument("--expert-slots", type=int, default=0,
                     help="variant run: fix the expert pool's device tier at this many expert matrices; the rest of the pool "
                          "goes to pinned host memory that the kernels read in place (with --decode-only: prints the tier's "
@@ -259,6 +264,11 @@ def main():
         sys.exit(2)
 
     import inferred_hip as ih
+    if args.single_ops_only:
+        from inferred_hip import single_ops
+        ffn = [int(t) for t in args.ffn_tokens.split(",") if t]
+        print(json.dumps({"single_op": single_ops.run(ih, seed=args.seed, exact=args.exact, ffn_tokens=ffn)}), flush=True)
+        return
     import torch
 
     t0 = time.time()

@@ -259,10 +259,13 @@ def delta_net(ih, be, seed=0, n_k=16, n_v=32, dk=128, dv=128, kernel=4, prefill=
     return out
 
 
-def run(ih, seed=0, exact=False):
-    """All three workloads on a backend of their own (no pass recording: every op launches as it is called)."""
+def run(ih, seed=0, exact=False, ffn_tokens=None):
+    """All three workloads on a backend of their own (no pass recording: every op launches as it is called).
+    ffn_tokens: only the expert FFN, at these token counts (for a kernel trace of one point of the sweep)."""
     be = ih.Hip(exact=exact, graph=False, fuse=False)
     try:
+        if ffn_tokens:
+            return {"expert_ffn_nvfp4_512x10": expert_ffn(ih, be, seed, tokens=tuple(ffn_tokens))}
         return {"timing": "sum of per-launch HIP-event durations of one call sequence (each launch carries about "
                           "2 us of event overhead); operands rotated over copies so that they come from HBM",
                 "expert_ffn_nvfp4_512x10": expert_ffn(ih, be, seed),
