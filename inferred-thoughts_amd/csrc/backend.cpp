@@ -470,9 +470,11 @@ bool it_hip::experts_view(const it_experts* w, const char* who, ExpertsView* out
         }
     }
     if (fresh) {
-        if (expert_pool < expert_resident + expert_host_entries) expert_pool = expert_resident + expert_host_entries;
+        const uint64_t placed = expert_resident + expert_host_entries + expert_cold_entries;
+        if (expert_pool < placed) expert_pool = placed;
         weights[w->data].counter_base = (int64_t)expert_counted;
         expert_counted += w->n_expert;
+        cold_ring_changed();
     }
     Resident* rw = &weights[w->data];
     if (w->scale && w->scale_len && !rw->scale2) {
@@ -539,18 +541,16 @@ bool it_hip::table_for(Resident& r) {
 }
 
 bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who) {
-    const uint64_t n = w->n_expert, n_host = n - n_dev;
+    const uint64_t n = w->n_expert;
     const uint64_t raw_one = type_row_bytes(w->ty, w->n_in) * w->n_out;
     const bool q8 = w->ty == IT_Q8_0;
     const uint64_t q_stride = q8 ? w->n_out * w->n_in : w->n_out * (w->n_in / 2);
     const uint64_t s_stride = q8 ? w->n_out * (w->n_in / 32) * 2 : w->n_out * (w->n_in / 16);
     const uint64_t budget = expert_host_budget ? expert_host_budget : DEFAULT_EXPERT_HOST_BUDGET;
-    if (expert_host_bytes + n_host * (q_stride + s_stride) > budget) {
-        fail(std::string(who) + ": the expert pool needs " + std::to_string(expert_resident + expert_host_entries + n) +
-             " slots but the device tier holds " + std::to_string(expert_slots_cap) + " and the pinned host tier's budget of " +
-             std::to_string(budget) + " bytes is used up; a tier behind it (experts fetched from the model file) is not part of this backend");
-        return false;
-    }
+    // what the pinned tier still takes; the rest of the tensor is cold: no copy is made, the entries point at the
+    // sentinel, and a pick is fetched from the file when a layer asks for it (experts.rs:969-980)
+    const uint64_t room = budget > expert_host_bytes ? (budget - expert_host_bytes) / (q_stride + s_stride) : 0;
+    const uint64_t n_host = std::min<uint64_t>(n - n_dev, room), n_cold = n - n_dev - n_host, n_placed = n_dev + n_host;
     need_eager("an expert tensor is placed in two tiers");
     drop_graph();
     check(hipStreamSynchronize(stream), "sync before two-tier placement");
@@ -561,6 +561,8 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
         for (auto& kv : weights)
             if (kv.second.counter_base >= 0 && !table_for(kv.second)) return false;
     }
+    const uint8_t *cold_q = nullptr, *cold_s = nullptr;
+    if (n_cold && !cold_sentinel(&cold_q, &cold_s, q_stride, s_stride)) return false;
     Resident r;
     r.fmt = (int)w->ty;
     r.n_in = w->n_in;
@@ -590,31 +592,34 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
             !check(hipHostGetDevicePointer((void**)&ds_host, r.host_s, 0), "hipHostGetDevicePointer"))
             return give_up();
     }
-    // upload and repack a few experts at a time through device staging, then move each to its place
-    const uint64_t chunk = std::min<uint64_t>(8, n);
-    if (!check(hipMalloc(&raw, chunk * raw_one), "hipMalloc(expert staging)") ||
-        !check(hipMalloc(&tq, chunk * q_stride), "hipMalloc(expert staging)") ||
-        !check(hipMalloc(&ts, chunk * s_stride), "hipMalloc(expert staging)"))
-        return give_up();
+    // upload and repack a few experts at a time through device staging, then move each to its place; the bytes of a
+    // cold expert are not touched
     bool ok = true;
-    for (uint64_t e0 = 0; e0 < n && ok; e0 += chunk) {
-        const uint64_t m = std::min(chunk, n - e0);
-        ok = ok && check(hipMemcpyAsync(raw, w->data + e0 * raw_one, m * raw_one, hipMemcpyHostToDevice, stream), "upload experts");
-        if (q8) repack_q8_0((const uint8_t*)raw, (int8_t*)tq, (uint16_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
-        else repack_nvfp4((const uint8_t*)raw, (uint8_t*)tq, (uint8_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
-        for (uint64_t k = 0; k < m && ok; k++) {
-            const uint64_t e = e0 + k;
-            const uint8_t* fq = (const uint8_t*)tq + k * q_stride;
-            const uint8_t* fs = (const uint8_t*)ts + k * s_stride;
-            if (e < n_dev) {
-                ok = check(hipMemcpyAsync((uint8_t*)r.q + e * q_stride, fq, q_stride, hipMemcpyDeviceToDevice, stream), "place expert") &&
-                     check(hipMemcpyAsync((uint8_t*)r.scales + e * s_stride, fs, s_stride, hipMemcpyDeviceToDevice, stream), "place expert");
-            } else {
-                ok = check(hipMemcpyAsync((uint8_t*)r.host_q + (e - n_dev) * q_stride, fq, q_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier") &&
-                     check(hipMemcpyAsync((uint8_t*)r.host_s + (e - n_dev) * s_stride, fs, s_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier");
+    if (n_placed) {
+        const uint64_t chunk = std::min<uint64_t>(8, n_placed);
+        if (!check(hipMalloc(&raw, chunk * raw_one), "hipMalloc(expert staging)") ||
+            !check(hipMalloc(&tq, chunk * q_stride), "hipMalloc(expert staging)") ||
+            !check(hipMalloc(&ts, chunk * s_stride), "hipMalloc(expert staging)"))
+            return give_up();
+        for (uint64_t e0 = 0; e0 < n_placed && ok; e0 += chunk) {
+            const uint64_t m = std::min(chunk, n_placed - e0);
+            ok = ok && check(hipMemcpyAsync(raw, w->data + e0 * raw_one, m * raw_one, hipMemcpyHostToDevice, stream), "upload experts");
+            if (q8) repack_q8_0((const uint8_t*)raw, (int8_t*)tq, (uint16_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
+            else repack_nvfp4((const uint8_t*)raw, (uint8_t*)tq, (uint8_t*)ts, (int64_t)(m * w->n_out), (int)w->n_in, stream);
+            for (uint64_t k = 0; k < m && ok; k++) {
+                const uint64_t e = e0 + k;
+                const uint8_t* fq = (const uint8_t*)tq + k * q_stride;
+                const uint8_t* fs = (const uint8_t*)ts + k * s_stride;
+                if (e < n_dev) {
+                    ok = check(hipMemcpyAsync((uint8_t*)r.q + e * q_stride, fq, q_stride, hipMemcpyDeviceToDevice, stream), "place expert") &&
+                         check(hipMemcpyAsync((uint8_t*)r.scales + e * s_stride, fs, s_stride, hipMemcpyDeviceToDevice, stream), "place expert");
+                } else {
+                    ok = check(hipMemcpyAsync((uint8_t*)r.host_q + (e - n_dev) * q_stride, fq, q_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier") &&
+                         check(hipMemcpyAsync((uint8_t*)r.host_s + (e - n_dev) * s_stride, fs, s_stride, hipMemcpyDeviceToHost, stream), "place expert in the host tier");
+                }
             }
+            ok = ok && check(hipStreamSynchronize(stream), "place experts");
         }
-        ok = ok && check(hipStreamSynchronize(stream), "place experts");
     }
     if (!ok) return give_up();
     (void)hipFree(raw);
@@ -622,23 +627,26 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
     (void)hipFree(ts);
     raw = tq = ts = nullptr;
     h2d++;
-    h2d_bytes += w->len;
+    h2d_bytes += n_placed * raw_one;
     r.h_q.resize(n);
     r.h_s.resize(n);
     r.h_tier.resize(n);
     for (uint64_t e = 0; e < n; e++) {
-        const bool dev = e < n_dev;
-        r.h_q[e] = dev ? (const uint8_t*)r.q + e * q_stride : dq_host + (e - n_dev) * q_stride;
-        r.h_s[e] = dev ? (const uint8_t*)r.scales + e * s_stride : ds_host + (e - n_dev) * s_stride;
-        r.h_tier[e] = dev ? 0 : 1;
+        const bool dev = e < n_dev, pinned = !dev && e < n_placed;
+        r.h_q[e] = dev ? (const uint8_t*)r.q + e * q_stride : pinned ? dq_host + (e - n_dev) * q_stride : cold_q;
+        r.h_s[e] = dev ? (const uint8_t*)r.scales + e * s_stride : pinned ? ds_host + (e - n_dev) * s_stride : cold_s;
+        r.h_tier[e] = dev ? 0 : pinned ? 1 : 2;
     }
     if (!table_upload(r)) return give_up();
     weight_bytes += r.q_bytes + r.s_bytes;
     expert_resident += n_dev;
     expert_host_entries += n_host;
     expert_host_bytes += n_host * (q_stride + s_stride);
+    expert_cold_entries += n_cold;
+    expert_cold_at_load += n_cold;
     setup_us += now_us() - t0;
     weights.emplace(w->data, std::move(r));
+    (void)who;
     return true;
 }
 
@@ -649,7 +657,7 @@ bool it_hip::place_two_tier(const it_experts* w, uint64_t n_dev, const char* who
 // boundary cannot turn into a visible stall.  The tables are ordinary device memory: a recorded graph reads the new
 // addresses at its next replay, with no re-record.  Stops by itself once no host expert is busier than a device one.
 void it_hip::migrate_at_boundary(uint64_t n_tokens) {
-    if (!pool_tabled || !expert_host_entries) return;
+    if (!pool_tabled || !expert_host_entries || expert_cold_entries) return;
     tokens_since_migration += n_tokens;
     if (tokens_since_migration < 64) return;
     const uint64_t budget = std::min<uint64_t>(200 * (tokens_since_migration / 64), 2000);
@@ -661,7 +669,8 @@ int64_t it_hip::replace_by_counts(uint64_t budget) {
     std::vector<uint32_t> counts;
     uint64_t tally[2];
     if (!expert_counters_read(&counts, tally)) return -1;
-    if (!pool_tabled || !expert_host_entries) return 0;
+    // with cold experts every slot change is the fetch path's (leases, heat): migration is paused (experts.rs:1857-1870)
+    if (!pool_tabled || !expert_host_entries || expert_cold_entries) return 0;
     struct Entry { Resident* r; uint32_t e; uint32_t count; };
     std::vector<Entry> dev, host;
     for (auto& kv : weights) {
@@ -997,6 +1006,7 @@ it_hip::Span::~Span() {
 void it_hip::drop_all() {
     need_eager("mirrors are dropped");
     drop_graph();
+    cold_drop();
     prev_signature.clear();
     if (stream) (void)hipStreamSynchronize(stream);
     for (auto& kv : acts) {
@@ -1029,6 +1039,9 @@ void it_hip::drop_all() {
     expert_slots_cap = 0;
     expert_counted = 0;
     expert_host_entries = expert_host_bytes = expert_swaps = tokens_since_migration = 0;
+    expert_cold_entries = expert_cold_at_load = expert_fetched = expert_fetch_bytes = expert_cold_evictions = 0;
+    fetch_read_us = fetch_upload_us = fetch_writes_us = picks_wait_us = picks_copy_us = 0;
+    prefetch_reads = prefetch_used = prefetch_wasted = 0;
     pool_tabled = false;
     if (expert_counts) (void)hipMemset(expert_counts, 0, expert_counts_cap * sizeof(uint32_t));
     if (expert_tally) (void)hipMemset(expert_tally, 0, 2 * sizeof(unsigned long long));
@@ -1579,6 +1592,7 @@ void it_hip_route(it_hip* be, float* probs, uint64_t probs_len, uint64_t n_exper
     be->route_n_used = n_used;
     be->route_n_tok = n_tok;
     be->route_gen++;
+    be->cold_clear_lease();   // a new routing decision: the last one's experts may be evicted again
 }
 
 static int x_mode_of(uint64_t rows, uint64_t picks) { return rows == picks ? 0 : (rows > 1 ? 1 : 2); }
@@ -1630,6 +1644,10 @@ void it_hip_matmul_experts(it_hip* be, const it_experts* w, const it_route* rout
     REQUIRE(out_len == picks * w->n_out, "matmul_experts: out.len() must be picks * n_out");
     if (picks == 0) return;
     REQUIRE(picks <= 65535, "matmul_experts: more than 65535 picks in one call");
+    if (be->expert_cold_entries) {
+        const uint8_t* keys[1] = {w->data};
+        if (!be->cold_resolve(keys, 1, route, false)) return;
+    }
     const float* as;
     const int8_t* aq;
     if (!be->act_quantized(x, x_len, &as, &aq, nullptr)) return;
@@ -1694,6 +1712,10 @@ void it_hip_moe_glu(it_hip* be, const it_experts* gate, const it_experts* up, co
     REQUIRE(out_len == picks * gate->n_out, "moe_glu: out.len() must be picks * n_out");
     if (picks == 0) return;
     REQUIRE(picks <= 65535, "moe_glu: more than 65535 picks in one call");
+    if (be->expert_cold_entries) {
+        const uint8_t* keys[2] = {gate->data, up->data};
+        if (!be->cold_resolve(keys, 2, route, true)) return;
+    }
     const float* as;
     const int8_t* aq;
     if (!be->act_quantized(x, x_len, &as, &aq, nullptr)) return;
@@ -1899,7 +1921,8 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
     be->replay_cursor = 0;
     be->mode = it_hip::Mode::Eager;
     be->profile_pass = false;
-    if (n_tokens == 1 && be->allow_graph && !be->mid_pass_read && !be->has_error) {
+    // cold experts are resolved from the picks inside the pass, which a graph cannot replay (experts.rs:91-93)
+    if (n_tokens == 1 && be->allow_graph && !be->mid_pass_read && !be->has_error && !be->expert_cold_entries) {
         if (be->graph.valid) {
             // while profiling, the pass is recorded like a replay and its fused launches are
             // then issued one by one between timing events instead of as the graph
@@ -1991,7 +2014,16 @@ int it_hip_tier_counters(it_hip* be, it_tier_counters* out) {
     out->pool_bytes = be->attn_scratch_cap * 4;
     out->resident_bytes = be->weight_bytes + be->kv_bytes + be->quant_bytes + be->mirror_bytes +
                           be->const_bytes + out->pool_bytes;
-    out->oversubscribed = be->pool_tabled;
+    out->oversubscribed = be->expert_cold_entries ? 1 : 0;
+    out->fetched = be->expert_fetched;
+    out->fetch_bytes = be->expert_fetch_bytes;
+    out->read_us = be->fetch_read_us;
+    out->upload_us = be->fetch_upload_us;
+    out->writes_us = be->fetch_writes_us;
+    out->picks_wait_us = be->picks_wait_us;
+    out->picks_copy_us = be->picks_copy_us;
+    out->prefetch_reads = be->prefetch_reads;
+    out->prefetch_used = be->prefetch_used;
     return 1;
 }
 
@@ -1999,15 +2031,20 @@ size_t it_hip_config_report(it_hip* be, char* buf, size_t buf_len) {
     int n = snprintf(buf, buf_len,
                      "backend=hip gfx950\nreductions=%s\ndecode graph=%s\nattention=%s\nexpert tier=%s\n"
                      "expert slots=%llu of %llu bytes (%s)\nexpert host tier=%llu experts, %llu bytes of a budget of %llu\n"
-                     "expert prefetch=%s (no tier to fetch from: a host-tier expert is read in place)\n"
+                     "expert cold tier=%llu experts (fetched on demand from %s)\n"
+                     "expert prefetch=%s (acts on cold experts only: a host-tier expert is read in place)\n"
                      "model path=%s\n",
                      be->exact ? "serial (CPU order)" : "tree / split-K", be->allow_graph ? "on" : "off",
                      be->exact ? "exact" : "split-K flash decoding (128-position chunks)",
-                     be->pool_tabled ? "device memory + pinned host, read through placement tables" : "all-resident",
+                     be->expert_cold_entries ? "device memory + pinned host + cold (fetched on demand), read through placement tables"
+                     : be->pool_tabled     ? "device memory + pinned host, read through placement tables"
+                                           : "all-resident",
                      (unsigned long long)be->expert_slots_cap, (unsigned long long)be->expert_slot_bytes,
                      be->expert_slots_req ? "fixed" : be->expert_budget ? "by budget" : "by free device memory",
                      (unsigned long long)be->expert_host_entries, (unsigned long long)be->expert_host_bytes,
                      (unsigned long long)(be->expert_host_budget ? be->expert_host_budget : DEFAULT_EXPERT_HOST_BUDGET),
+                     (unsigned long long)be->expert_cold_entries,
+                     !be->model_path.empty() && be->map_base ? "the model file" : "the tensors' mapping",
                      be->expert_prefetch ? "on" : "off",
                      be->model_path.empty() ? "(not set)" : be->model_path.c_str());
     return n < 0 ? 0 : (size_t)n;
@@ -2017,8 +2054,9 @@ uint64_t it_hip_setup_cost(it_hip* be, char* label, size_t label_len) {
     if (label && label_len) snprintf(label, label_len, "weight upload and repack");
     return be->setup_us;
 }
+// src/ops/mod.rs:915-924: acts only while some expert is cold; with every expert addressable there is nothing to read ahead
 void it_hip_prefetch_hint(it_hip* be, const it_weights* w, const float* x, uint64_t x_len, uint64_t k) {
-    (void)be; (void)w; (void)x; (void)x_len; (void)k;  // every expert is addressable where it lies: nothing to fetch
+    be->cold_hint(w, x, x_len, k);
 }
 
 // Cap the expert slab, in bytes; 0 restores sizing from free device memory (placement.rs:178-189).  Like the
@@ -2059,8 +2097,9 @@ void it_hip_expert_stats(it_hip* be, it_expert_stats* out) {
     out->lookups = tally[0] + tally[1];
     out->hits = tally[0];
     out->host_slots = be->expert_host_entries;
-    out->evictions = be->expert_swaps;
-    out->oversubscribed = be->pool_tabled;
+    out->evictions = be->expert_swaps + be->expert_cold_evictions;
+    out->fetched = be->expert_fetched;
+    out->oversubscribed = be->expert_cold_entries ? 1 : 0;
 }
 
 // What fraction of all expert reads the busiest slab-many matrices took, and the reads counted

@@ -105,11 +105,12 @@ struct it_hip {
         uint64_t n_expert = 0, q_stride = 0, s_stride = 0;
         const uint8_t** q_tab = nullptr;
         const uint8_t** s_tab = nullptr;
-        uint8_t* tier = nullptr;                 // device: 0 = device memory, 1 = pinned host
+        uint8_t* tier = nullptr;                 // device: 0 = device memory, 1 = pinned host, 2 = cold (no copy held)
         std::vector<const uint8_t*> h_q, h_s;
         std::vector<uint8_t> h_tier;
         void* host_q = nullptr;                  // pinned blocks of the experts first placed in the host tier
         void* host_s = nullptr;
+        std::vector<int32_t> slot_at;            // per expert: its slot in the cold tier's ring of device slots, or -1
     };
     bool place_two_tier(const it_experts* w, uint64_t n_dev, const char* who);
     bool table_for(Resident& r);                 // an identity table for a tensor that sits in device memory whole
@@ -118,6 +119,22 @@ struct it_hip {
     void migrate_at_boundary(uint64_t n_tokens);   // bounded exchange every 64 tokens of evidence (placement.rs:33-80)
     uint64_t expert_host_entries = 0, expert_host_bytes = 0, expert_swaps = 0, tokens_since_migration = 0;
     bool pool_tabled = false;                    // some pooled tensor did not fit the device tier
+    // The third tier (src/ops/cuda/experts.rs:67-93): experts that found room in neither tier are cold.  A cold
+    // expert's table entry points at a zeroed sentinel; before an expert kernel runs, the picks are read back, every
+    // cold pick is fetched from the model file (or its mapping) into a device slot taken from an expert the layer did
+    // not pick (GCLOCK with leases), and the tables are patched.  State and code in expert_cold.cpp.
+    struct ColdTier;
+    ColdTier* cold = nullptr;
+    uint64_t expert_cold_entries = 0, expert_cold_at_load = 0, expert_fetched = 0, expert_fetch_bytes = 0;
+    uint64_t expert_cold_evictions = 0, fetch_read_us = 0, fetch_upload_us = 0, fetch_writes_us = 0;
+    uint64_t picks_wait_us = 0, picks_copy_us = 0, prefetch_reads = 0, prefetch_used = 0, prefetch_wasted = 0;
+    bool cold_sentinel(const uint8_t** q, const uint8_t** s, uint64_t q_stride, uint64_t s_stride);
+    // make every expert that `route` picks from these tensors readable (fetching the cold ones) and lease them
+    bool cold_resolve(const uint8_t* const* tensor_keys, int n_tensors, const it_route* route, bool opens_layer);
+    void cold_clear_lease();
+    void cold_ring_changed();                    // a pooled tensor was placed: the ring of device slots is rebuilt
+    void cold_hint(const it_weights* next_router, const float* x, uint64_t x_len, uint64_t k);
+    void cold_drop();
     std::unordered_map<const void*, Resident> weights;
     const Resident* resident(const uint8_t* data, uint64_t len, uint32_t ty, uint64_t n_in, uint64_t rows,
                              const char* who);

@@ -46,6 +46,7 @@ class File {
     bool get_string(const std::string& key, std::string* out) const;
     const std::vector<int32_t>* get_i32_array(const std::string& key) const;
     size_t size() const { return size_; }
+    const uint8_t* base() const { return base_; }   // where the file is mapped
     const std::vector<Tensor>& tensors() const { return tensors_; }
 
   private:

@@ -156,6 +156,22 @@ __global__ __launch_bounds__(256) void expert_count_k(const int32_t* __restrict_
     }
 }
 
+// Placement-table entries of experts that changed tier (a cold expert fetched into a slot, its victim pointed at the
+// sentinel): one thread per entry, ordered on the stream between the kernels that read the old and the new placement.
+__global__ void expert_patch_k(const ExpertPatch* __restrict__ patches, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const ExpertPatch p = patches[i];
+    *p.q_at = p.q;
+    *p.s_at = p.s;
+    *p.tier_at = (uint8_t)p.tier;
+}
+
+void expert_patch(const ExpertPatch* patches, int n, hipStream_t s) {
+    if (n <= 0) return;
+    hipLaunchKernelGGL(expert_patch_k, dim3((n + 63) / 64), dim3(64), 0, s, patches, n);
+}
+
 void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
                   unsigned long long* tally, hipStream_t s, const uint8_t* tier_a, const uint8_t* tier_b) {
     if (n_picks <= 0 || !counts_a || !tally) return;

@@ -104,6 +104,17 @@ void moe_glu(const ExpertsView& gate, const ExpertsView& up, const int32_t* ids,
 void expert_count(const int32_t* ids, int n_picks, int n_expert, uint32_t* counts_a, uint32_t* counts_b,
                   unsigned long long* tally, hipStream_t s, const uint8_t* tier_a = nullptr, const uint8_t* tier_b = nullptr);
 
+// one entry of a tensor's placement table changes: the expert's quants, scales and tier byte (written by one thread)
+struct ExpertPatch {
+    const uint8_t** q_at;
+    const uint8_t** s_at;
+    uint8_t* tier_at;
+    const uint8_t* q;
+    const uint8_t* s;
+    uint32_t tier, pad;
+};
+void expert_patch(const ExpertPatch* patches, int n, hipStream_t s);
+
 // ---- router ----------------------------------------------------------------------
 void softmax_rows(float* x, int64_t n_rows, int row, int exact, hipStream_t s);
 void route_topk(const float* probs, int n_tok, int n_expert, int n_used, int32_t* ids, float* weights,

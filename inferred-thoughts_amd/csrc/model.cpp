@@ -60,6 +60,7 @@ struct Block {
 
 struct it_model {
     itg::File file;
+    std::string path;
     Dims d;
     it_weights tok_embd{}, output{};
     bool has_output_scale = false;
@@ -141,7 +142,8 @@ struct it_model {
         return true;
     }
 
-    bool load(const std::string& path) {
+    bool load(const std::string& path_in) {
+        path = path_in;
         if (!file.open(path, &err)) return false;
         std::string arch;
         if (!file.get_string("general.architecture", &arch)) return fail("missing general.architecture");
@@ -282,6 +284,7 @@ struct it_engine {
 };
 
 namespace {
+constexpr uint64_t PREFETCH_K = 10;  // src/model/qwen4exp.rs:45: how many of the next router's picks a hint guesses
 constexpr uint64_t MOE_CHUNK = 512;  // src/model/qwen35.rs:650: the reference's routed-FFN sub-batch; a larger engine batch raises it (it_engine_new)
 
 void fit(it_engine* e, uint64_t n) {
@@ -300,7 +303,10 @@ void fit(it_engine* e, uint64_t n) {
     e->last.fit(d.n_embd, e->be); e->final_norm.fit(d.n_embd, e->be); e->logits.fit(d.n_vocab, e->be);
 }
 
-void moe_batch(it_engine* e, const Block& b, uint64_t at, uint64_t n, uint64_t total) {
+// next_router: the router of the next layer, for a single-token pass.  The reference's qwen35 loop does not hint; its
+// qwen4exp loop does (src/model/qwen4exp.rs:1885-1896), between the routing decision and the expert products, and the
+// hint changes no value.  The backend acts on it only while part of the expert pool is cold.
+void moe_batch(it_engine* e, const Block& b, uint64_t at, uint64_t n, uint64_t total, const it_weights* next_router) {
     const Dims& d = e->m->d;
     it_hip* be = e->be;
     uint64_t nd = d.n_embd;
@@ -310,6 +316,7 @@ void moe_batch(it_engine* e, const Block& b, uint64_t at, uint64_t n, uint64_t t
     it_hip_softmax(be, e->router.p(), n * d.n_expert, d.n_expert);
     it_route route;
     it_hip_route(be, e->router.p(), n * d.n_expert, d.n_expert, d.n_used, &route);
+    if (total == 1 && next_router) it_hip_prefetch_hint(be, next_router, x, nd, PREFETCH_K);
     uint64_t pairs = n * d.n_used, ff = pairs * d.expert_ff;
     it_hip_moe_glu(be, &b.gate, &b.up, &route, x, n * nd, e->g_all.p(), ff, e->u_all.p(), ff);
     it_hip_matmul_experts(be, &b.down, &route, e->g_all.p(), ff, e->o_all.p(), pairs * nd);
@@ -425,7 +432,7 @@ int forward(it_engine* e, const uint32_t* tokens, uint64_t n, uint64_t start, bo
         it_hip_rms_norm(be, e->x.p(), n * nd, b.ffn_norm.data(), nd, d.eps, e->normed.p(), n * nd);
         for (uint64_t t = 0; t < n;) {
             uint64_t take = e->moe_chunk < n - t ? e->moe_chunk : n - t;
-            moe_batch(e, b, t * nd, take, n);
+            moe_batch(e, b, t * nd, take, n, il + 1 < d.layers() ? &m->blocks[il + 1].router : nullptr);
             t += take;
         }
         e->tr("ffn_moe_out", il, e->ffn_out, n * nd);
@@ -529,6 +536,9 @@ it_engine* it_engine_new(it_model* m, it_hip* be, uint64_t n_ctx, uint64_t max_b
         else dense += b.wq.len + b.wk.len + b.wv.len + b.wo.len;
         dense += b.router.len + b.sh_gate.len + b.sh_up.len + b.sh_down.len + b.sh_gate_inp.len;
     }
+    // where the experts' bytes can be read from when they are not kept anywhere else (src/main.rs:559-560)
+    it_hip_set_model_path(be, m->path.c_str());
+    it_hip_set_map_base(be, (uint64_t)(uintptr_t)m->file.base());
     it_hip_reserve_for_weights(be, dense);
     it_hip_set_expert_pool(be, d.layers() * 3 * d.n_expert);
     e->kv_reserved = 2 * m->n_kv_layer * n_ctx * d.kv_dim() * sizeof(uint16_t) +

@@ -87,15 +87,17 @@ def test_refusals():
     assert "not uniform" in (be.take_error() or "")
     be.end_pass(); be.close()
     # a slab fixed at fewer slots than the pool needs spills into the pinned host tier (tests/test_gpu_expert_tiers.py);
-    # with that tier's budget used up as well the tensor is refused: no tier behind it
+    # with that tier's budget used up as well the rest is cold and fetched when picked (tests/test_gpu_expert_cold.py)
     be = ih.Hip()
     be.set_expert_slots(n_expert - 1)
     be.set_expert_host_budget(1)
     be.begin_pass(1)
     be.matmul_experts(ih.experts(wb, ih.Q8_0, n_in, n_out, n_expert), route, x, np.zeros(2 * n_out, np.float32))
-    err = be.take_error() or ""
-    assert "pinned host tier's budget" in err and "holds 7" in err
-    be.end_pass(); be.close()
+    be.end_pass()
+    assert be.take_error() is None
+    st = be.expert_stats()
+    assert st.slots == 7 and st.resident == 7 and st.host_slots == 0 and st.oversubscribed == 1 and st.fetched == 0
+    be.close()
     # a budget in bytes sizes the slab the same way: three slots, five experts in the host tier
     be = ih.Hip()
     be.set_expert_budget(3 * n_out * n_in // 32 * 34)
@@ -104,7 +106,7 @@ def test_refusals():
     be.end_pass()
     assert be.take_error() is None
     st = be.expert_stats()
-    assert st.slots == 3 and st.resident == 3 and st.host_slots == 5 and st.oversubscribed == 1
+    assert st.slots == 3 and st.resident == 3 and st.host_slots == 5 and st.oversubscribed == 0   # nothing is cold
     be.close()
 
 
