@@ -251,6 +251,11 @@ def main():
                     help="variant run: fix the expert pool's device tier at this many expert matrices; the rest of the pool "
                          "goes to pinned host memory that the kernels read in place (with --decode-only: prints the tier's "
                          "counters, exchanges experts by the counts of the timed stretch and times a second stretch)")
+    ap.add_argument("--expert-host-slots", type=int, default=-1,
+                    help="with --expert-slots: cap the pinned host tier at this many expert matrices; what fits neither tier "
+                         "is cold and fetched from the model file when a layer picks it (0 = no host tier)")
+    ap.add_argument("--no-prefetch", action="store_true",
+                    help="with a cold tier: do not read the next layer's likely experts ahead (set_prefetch off)")
     ap.add_argument("--summarize-profile", metavar="DIR",
                     help="no run: print the profiles/ summary of the rocprofv3 outputs under DIR (trace/, pmc_FETCH_SIZE/, "
                          "pmc_WRITE_SIZE/ of --decode-only runs) and exit")
@@ -296,6 +301,11 @@ def main():
     be = ih.Hip(exact=args.exact)
     if args.expert_slots:
         be.set_expert_slots(args.expert_slots)
+        if args.expert_host_slots >= 0:
+            # one repacked expert matrix takes its file bytes (NVFP4: 9 bytes per 16 weights, Q8_0: 34 per 32)
+            one = cfg.expert_ff * cfg.n_embd * (9 if cfg.expert_type == ih.NVFP4 else 17) // 16
+            be.set_expert_host_budget(max(1, args.expert_host_slots * one))
+        be.set_prefetch(not args.no_prefetch)
     model = ih.Model(path)
     eng = ih.Engine(model, be, args.ctx, args.max_batch)
     rng = np.random.default_rng(args.seed)
@@ -351,6 +361,15 @@ def main():
                 "exchanged_by_counts": int(moved), "exchange_s": round(t_move, 3),
                 "tok_s_after_exchange": round(args.steps / dt2, 2),
                 "reads_after": int(st2.lookups - st.lookups), "from_device_memory_after": int(st2.hits - st.hits)}
+            if st2.oversubscribed:
+                tc = be.tier_counters()
+                line["expert_tiers"]["cold"] = {
+                    "cold_experts": int(st.pool - st.slots - st.host_slots), "fetched": int(tc.fetched),
+                    "fetched_in_second_stretch": int(st2.fetched - st.fetched), "fetch_mb": round(tc.fetch_bytes / 1e6, 1),
+                    "file_read_ms": round(tc.read_us / 1e3, 1), "upload_issue_ms": round(tc.upload_us / 1e3, 1),
+                    "table_writes_ms": round(tc.writes_us / 1e3, 1), "picks_wait_ms": round(tc.picks_wait_us / 1e3, 1),
+                    "picks_copy_ms": round(tc.picks_copy_us / 1e3, 1), "prefetch_reads": int(tc.prefetch_reads),
+                    "prefetch_used": int(tc.prefetch_used), "prefetch": not args.no_prefetch}
         print(json.dumps(line), flush=True)
         eng.close(); model.close(); be.close()
         if not args.keep:

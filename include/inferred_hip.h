@@ -85,9 +85,10 @@ typedef struct {
     uint64_t slots, resident_bytes, weight_bytes, kv_bytes, quant_bytes, pool_bytes;
 } it_tier_counters;
 
-/* struct ExpertStats, src/ops/cuda/experts.rs:210-315 (the fields of the device and pinned-host tiers): hits = reads
- * served from device memory, lookups - hits = reads that crossed the bus, host_slots = experts in the host tier,
- * evictions = experts moved out of device memory by replace_experts_by_counts, fetched = 0 (no third tier) */
+/* struct ExpertStats, src/ops/cuda/experts.rs:210-315: hits = reads served from device memory, lookups - hits = reads
+ * that crossed the bus to the pinned host tier, host_slots = experts in that tier, fetched = cold experts brought into
+ * device memory from the model file, evictions = experts that left device memory (exchanged by counts, or displaced
+ * by a fetched one), oversubscribed = some expert is cold (both tiers filled before the pool did) */
 typedef struct {
     uint64_t slots, slot_bytes, resident, pool, host_slots, evictions, fetched, lookups, hits;
     uint32_t oversubscribed, _pad;
@@ -230,9 +231,13 @@ void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x
  * tensor is then read through a device table of per-expert addresses, and a kernel dereferences an expert wherever it
  * lies, so a miss is slow (it crosses the bus) but never blocks and never changes a value.  Placement is first touch
  * wins device memory; every 64 tokens, at a pass boundary, a bounded number of busy host-tier experts change places
- * with idle device-tier ones (placement.rs:33-80), and replace_experts_by_counts runs that exchange to completion.  A pool
- * that outgrows both tiers is refused with a sticky error: experts fetched from the model file (the reference's third
- * tier) are not part of this backend. */
+ * with idle device-tier ones (placement.rs:33-80), and replace_experts_by_counts runs that exchange to completion.
+ * A pool that outgrows both tiers has cold experts (experts.rs:67-93): no copy of them is held; before an expert kernel
+ * runs the picks are read back (such passes run eagerly, never from a graph; the exchange by counts is paused), and
+ * each cold pick is fetched from the model file (set_model_path + set_map_base; else from the tensor's mapping) into a
+ * device slot taken by GCLOCK from an expert the routing decision did not pick.  The device tier must hold one
+ * decision's picks of a layer's three tensors, else the call is refused with a sticky error.  prefetch_hint (the next
+ * layer's router on this layer's input) starts reading the next layer's likely cold experts while this one computes. */
 void it_hip_set_expert_budget(it_hip*, uint64_t bytes);      /* placement.rs:178 */
 void it_hip_set_expert_host_budget(it_hip*, uint64_t bytes); /* placement.rs:322; 0 = 64 GiB */
 void it_hip_set_expert_slots(it_hip*, uint64_t n);           /* placement.rs:157; 0 = by budget */
