@@ -156,7 +156,8 @@ def summarize_profile(root_dir):
 
 def model_path(args):
     base = Path("/dev/shm") if Path("/dev/shm").is_dir() and os.access("/dev/shm", os.W_OK) else Path("/tmp")
-    return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}{'_f32router' if args.router_f32 else ''}.gguf"
+    tag = ("_f32router" if args.router_f32 else "") + ("_nvfp4shared" if args.shared_nvfp4 else "")
+    return base / f"inferred_hip_bench_L{args.layers}_s{args.seed}{tag}.gguf"
 
 
 def config1(ih, ob, seed, tmp_dir):
@@ -222,6 +223,10 @@ def main():
     ap.add_argument("--router-f32", action="store_true",
                     help="router, shared-expert gate and ssm alpha / beta matrices in F32 (as real files keep them) "
                          "instead of the baseline's Q8_0: a variant, not the baseline workload")
+    ap.add_argument("--shared-nvfp4", action="store_true",
+                    help="the shared expert's three matrices in NVFP4 with a second scale each (as an NVFP4 file of this "
+                         "model stores them) instead of the baseline's Q8_0: a variant; with --router-f32 it is the "
+                         "layout of a real file")
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--max-batch", type=int, default=8192,
                     help="tokens per prefill pass; the default takes the 5,700-token prompt through each layer in one "
@@ -281,6 +286,8 @@ def main():
     cfg = ih.big_config(seed=args.seed, n_layer=args.layers, n_threads=min(16, os.cpu_count() or 8))
     if args.router_f32:
         cfg.router_type = ih.ROUTER_F32
+    if args.shared_nvfp4:
+        cfg.shared_type = ih.NVFP4
     if not path.exists():
         ih.synth_write_gguf(path, cfg)
     t_synth = time.time() - t0
@@ -458,7 +465,7 @@ def main():
     tok_bytes = w_bytes + state_bytes + kv_bytes
     whole = tok_bytes * tok_s / 1e9
 
-    headline = args.layers == 48 and args.prompt == 5700 and not args.router_f32 and not args.exact
+    headline = args.layers == 48 and args.prompt == 5700 and not args.router_f32 and not args.shared_nvfp4 and not args.exact
     rows.sort(key=lambda r: -r["ms"])
     timed = [r for r in rows if r["bytes"]]
     dom = timed[0] if timed else None
@@ -549,11 +556,13 @@ def main():
         "vs_baseline": None, "dtype": "int8 dot / f32 accumulate (NVFP4 + Q8_0 weights, Q8_0 activations)",
         "data": "synthetic",
         "config": {"workload": "config 5: full 35B-A3B-shaped model, greedy decode after a 5,700-token prefill at ctx 8192"
-                               if args.layers == 48 and args.prompt == 5700 and not args.router_f32 else
+                               if args.layers == 48 and args.prompt == 5700 and not args.router_f32 and not args.shared_nvfp4 else
                                f"VARIANT / reduced check run: {args.layers} layers, prompt {args.prompt}, "
-                               f"router {'F32' if args.router_f32 else 'Q8_0'}",
+                               f"router {'F32' if args.router_f32 else 'Q8_0'}, shared expert "
+                               f"{'NVFP4 with second scales' if args.shared_nvfp4 else 'Q8_0'}",
                    "layers": args.layers, "prompt": args.prompt, "ctx": args.ctx, "prefill_batch": args.max_batch, "decode_pos": int(pos0),
-                   "experts": "512 routed experts top-10, NVFP4 with per-expert second scales; one shared expert, Q8_0",
+                   "experts": "512 routed experts top-10, NVFP4 with per-expert second scales; one shared expert, " +
+                              ("NVFP4 with a second scale per matrix" if args.shared_nvfp4 else "Q8_0"),
                    "dense": "Q8_0 (attention, GDN, LM head; router, shared-gate logit and ssm_alpha/beta Q8_0 too)",
                    "mode": "exact" if args.exact else "fast", "batch": 1},
         "prefill_tok_s": round(args.prompt / t_prefill, 1),

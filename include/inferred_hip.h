@@ -384,7 +384,8 @@ typedef struct {
     uint32_t expert_type; /* IT_Q8_0 or IT_NVFP4 */
     uint32_t router_type; /* router, shared-gate and ssm alpha/beta matrices: 0 = as dense_type, IT_Q8_0, or
                              IT_SYNTH_ROUTER_F32 for F32 (what real files keep them in; IT_F32 itself is 0) */
-    uint32_t _pad;
+    uint32_t shared_type; /* the shared expert's matrices: 0 = as dense_type; IT_NVFP4 = NVFP4 with a second, per-tensor
+                             scale each (ffn_*_shexp.scale), which is how an NVFP4 file of this model stores them */
     uint64_t seed;
     float weight_std; /* N(0, std) for Q8_0 matrices */
     uint32_t n_threads;

@@ -1471,7 +1471,7 @@ void it_hip_scale(it_hip* be, float* buf, uint64_t len, float sv) {
     if (!d) return;
     int64_t n = (int64_t)len;
     it_hip::OpRec rec;
-    rec.id = OP_SCALE;
+    rec.id = OP_SCALE; rec.p[0] = d; rec.i[0] = n; rec.f[0] = sv;
     be->submit(it_hip::FAM_OTHER, len * 8, sig_of(OP_SCALE, d, sv, n), rec, [=](hipStream_t s) { scale(d, sv, n, s); });
 }
 

@@ -377,23 +377,55 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     return true;
 }
 
-// routed FFN: 17 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
+// routed FFN: 17 to 20 ops -> fused_gemv (norm + router + shared gate logit) + moe_glu_fused + moe_down_fused
 bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long long* tally) {
     // With a quantized router the activation is quantized before the router matmul; with an unquantized one
     // (F32 in real files) the first reader of the quantized form is the expert gate/up product, after the route.
-    const bool q_first = pl.ids(i, {OP_RMS, OP_GATHER, OP_QUANT, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_GLU, OP_QUANT,
-                                    OP_EXPERTS, OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW});
-    const bool q_late = !q_first && !exact &&
-                        pl.ids(i, {OP_RMS, OP_GATHER, OP_MATMUL, OP_MATMUL, OP_SOFTMAX, OP_ROUTE, OP_QUANT, OP_GLU, OP_QUANT,
-                                   OP_EXPERTS, OP_MATMUL, OP_MATMUL, OP_EW, OP_QUANT, OP_MATMUL, OP_FINISH, OP_EW});
-    if (!q_first && !q_late) return false;
+    // An NVFP4 file carries a second, per-tensor scale for each of the shared expert's matrices
+    // (src/model/qwen35.rs:1669-1682): up to two SCALE ops follow the shared gate / up products and one the
+    // shared down product.  The walk below takes the fixed ops in order and those three where they are present.
     auto& o = pl.ops;
-    const Op &rms = o[i], &ga = o[i + 1];
-    const Op &q1 = q_first ? o[i + 2] : o[i + 6];
-    const Op &mr = q_first ? o[i + 3] : o[i + 2], &ml = q_first ? o[i + 4] : o[i + 3];
-    const Op &sm = q_first ? o[i + 5] : o[i + 4], &rt = q_first ? o[i + 6] : o[i + 5];
-    const Op &glu = o[i + 7], &q2 = o[i + 8], &ex = o[i + 9], &sgm = o[i + 10], &sum_ = o[i + 11], &sil = o[i + 12];
-    const Op &q3 = o[i + 13], &sdm = o[i + 14], &fin = o[i + 15], &add = o[i + 16];
+    size_t k = i;
+    auto take = [&](int id) -> const Op* { return k < o.size() && o[k].id == id ? &o[k++] : nullptr; };
+    const Op *rms_p = take(OP_RMS), *ga_p = take(OP_GATHER);
+    if (!rms_p || !ga_p) return false;
+    const Op* q1_p = take(OP_QUANT);
+    const bool q_first = q1_p != nullptr;
+    if (!q_first && exact) return false;
+    const Op *mr_p = take(OP_MATMUL), *ml_p = take(OP_MATMUL), *sm_p = take(OP_SOFTMAX), *rt_p = take(OP_ROUTE);
+    if (!mr_p || !ml_p || !sm_p || !rt_p) return false;
+    if (!q_first && !(q1_p = take(OP_QUANT))) return false;
+    const Op *glu_p = take(OP_GLU), *q2_p = take(OP_QUANT), *ex_p = take(OP_EXPERTS), *sgm_p = take(OP_MATMUL), *sum_p = take(OP_MATMUL);
+    if (!glu_p || !q2_p || !ex_p || !sgm_p || !sum_p) return false;
+    float sh_scale[3] = {1.0f, 1.0f, 1.0f};   // gate, up, down
+    bool has_up = false, has_gate = false;
+    while (k < o.size() && o[k].id == OP_SCALE) {   // the up product is scaled first, then the gate product
+        const Op& sc = o[k];
+        if (!has_up && !has_gate && sc.p[0] == sum_p->p[5] && sc.i[0] == sum_p->i[2]) {
+            sh_scale[1] = sc.f[0];
+            has_up = true;
+        } else if (!has_gate && sc.p[0] == sgm_p->p[5] && sc.i[0] == sgm_p->i[2]) {
+            sh_scale[0] = sc.f[0];
+            has_gate = true;
+        } else {
+            return false;
+        }
+        k++;
+    }
+    const Op *sil_p = take(OP_EW), *q3_p = take(OP_QUANT), *sdm_p = take(OP_MATMUL);
+    if (!sil_p || !q3_p || !sdm_p) return false;
+    if (k < o.size() && o[k].id == OP_SCALE) {
+        const Op& sc = o[k];
+        if (sc.p[0] != sdm_p->p[5] || sc.i[0] != sdm_p->i[2]) return false;
+        sh_scale[2] = sc.f[0];
+        k++;
+    }
+    const Op *fin_p = take(OP_FINISH), *add_p = take(OP_EW);
+    if (!fin_p || !add_p) return false;
+    const size_t n_ops = k - i;
+    const Op &rms = *rms_p, &ga = *ga_p, &q1 = *q1_p, &mr = *mr_p, &ml = *ml_p, &sm = *sm_p, &rt = *rt_p;
+    const Op &glu = *glu_p, &q2 = *q2_p, &ex = *ex_p, &sgm = *sgm_p, &sum_ = *sum_p, &sil = *sil_p;
+    const Op &q3 = *q3_p, &sdm = *sdm_p, &fin = *fin_p, &add = *add_p;
     int64_t nd = rms.i[1];
     if (rms.i[0] != 1) return false;
     // experts placed through a table (a pool larger than its device tier) are read by the unfused kernels only
@@ -470,6 +502,8 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
     g.sh_us = (const uint8_t*)sum_.p[1];
     g.sh_fmt = (int)sgm.i[0];
     g.sh_n_out = (int)sff;
+    g.sh_gscale = sh_scale[0];
+    g.sh_uscale = sh_scale[1];
     g.out = (float*)g_all;
     g.sh_out = (float*)e_gate;
     g.route_ids = (const int32_t*)rt.p[1];
@@ -496,6 +530,7 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
     d.sh_s = (const uint8_t*)sdm.p[1];
     d.sh_fmt = (int)sdm.i[0];
     d.sh_n_in = (int)sff;
+    d.sh_dscale = sh_scale[2];
     d.route_ids = (const int32_t*)rt.p[1];
     d.route_w = (const float*)rt.p[2];
     d.logit = (const float*)ml.p[5];
@@ -505,7 +540,7 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
     d.counts_down = (uint32_t*)ex.p[7];
     d.tally = tally;
 
-    pl.take(i, 17);
+    pl.take(i, n_ops);
     const uint64_t glu_b = 2 * rows_bytes(g.fmt, (uint64_t)nu * ff, nd) + 2 * rows_bytes(g.sh_fmt, sff, nd) + (uint64_t)nd * 4 +
                            (uint64_t)(nu * ff + sff) * 4;
     const uint64_t down_b = rows_bytes(d.fmt, (uint64_t)nu * nd, ff) + rows_bytes(d.sh_fmt, nd, sff) +

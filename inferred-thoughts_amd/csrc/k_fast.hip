@@ -717,7 +717,7 @@ __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
                                   p.out + (int64_t)y * p.n_out, lane, tg, tu, false);
         } else {
             const int row0 = (g - routed_groups) * gg.s_rg;
-            glu_job<SF, SCPL, SL>(p.sh_gq, p.sh_gs, p.sh_uq, p.sh_us, n_in, p.sh_n_out, row0, 1.0f, 1.0f, xq, xs,
+            glu_job<SF, SCPL, SL>(p.sh_gq, p.sh_gs, p.sh_uq, p.sh_us, n_in, p.sh_n_out, row0, p.sh_gscale, p.sh_uscale, xq, xs,
                                   p.sh_out, lane, sg, su, loaded);
         }
         loaded = false;
@@ -834,7 +834,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     if (quarter == 3) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
     const float x_old = (!quarter && sub == L - 1 && live) ? p.x[row] : 0.0f;
     if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
-    const float gate = fx_sigmoid(p.logit[0]);
+    const float gate = fx_sigmoid(p.logit[0]) * p.sh_dscale;
     IT_STAMP(1);
 
 #pragma unroll

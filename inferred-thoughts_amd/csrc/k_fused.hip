@@ -648,6 +648,9 @@ __global__ __launch_bounds__(256) void moe_glu_fused_k(MoeGluP p) {
             if (!shared) {
                 if (p.gscale2) ag *= p.gscale2[e];
                 if (p.uscale2) au *= p.uscale2[e];
+            } else {   // a scale of 1 (no scale tensor) leaves the bits as they are
+                au *= p.sh_uscale;
+                ag *= p.sh_gscale;
             }
             out[row0 + lane] = it_silu(ag) * au;
         }
@@ -744,6 +747,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_k(MoeDownP p) {
             const int y = lane / nrows, r = lane - y * nrows;
             dot = fold_terms(terms + ((size_t)y * R + r) * tstride, y < NU ? T : shT);
             if (y < NU && p.scale2) dot *= p.scale2[p.route_ids[y]];
+            if (y == NU) dot *= p.sh_dscale;
         }
         wave_lds_sync();
         if (lane < pairs) {

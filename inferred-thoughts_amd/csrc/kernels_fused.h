@@ -55,6 +55,9 @@ struct MoeGluP {
     int fmt, n_in, n_out, n_expert, n_used, exact, rows_per_wave;
     const uint8_t *sh_gq, *sh_gs, *sh_uq, *sh_us;
     int sh_fmt, sh_n_out;
+    // the shared expert's per-tensor second scales (ffn_gate_shexp.scale, ffn_up_shexp.scale of an NVFP4 file;
+    // src/model/qwen35.rs:1669-1676: up is scaled, then gate, then silu(gate) * up); 1 when the file has none
+    float sh_gscale, sh_uscale;
     float* out;            // [n_used][n_out]
     float* sh_out;         // [sh_n_out]
     const int32_t* route_ids;  // [n_used], chosen by the router kernel (when logits is null)
@@ -75,6 +78,7 @@ struct MoeDownP {
     int fmt, n_in, n_out, n_used, rows_per_wave, exact;
     const uint8_t *sh_q, *sh_s;
     int sh_fmt, sh_n_in;
+    float sh_dscale;        // ffn_down_shexp.scale (qwen35.rs:1680-1682: applied to the product, before the gate); 1 when absent
     const int32_t* route_ids;
     const float* route_w;
     const float* logit;     // shared expert gate logit

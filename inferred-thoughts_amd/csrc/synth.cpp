@@ -93,6 +93,7 @@ extern "C" int it_synth_write_gguf(const char* path, const it_synth_config* c, c
     if (c->n_embd % 64 || c->expert_ff % 64 || c->shared_ff % 64 || c->head_dim % 32)
         return bad("n_embd, expert_ff, shared_ff must be multiples of 64 and head_dim of 32");
     if (c->expert_type != IT_Q8_0 && c->expert_type != IT_NVFP4) return bad("expert_type must be Q8_0 or NVFP4");
+    if (c->shared_type != 0 && c->shared_type != IT_NVFP4) return bad("shared_type must be 0 (as the dense matrices) or NVFP4");
     const uint64_t nd = c->n_embd, dk = c->ssm_d_state, nv = c->ssm_dt_rank, nk = c->ssm_n_group;
     const uint64_t d_inner = dk * nv, key_dim = dk * nk, conv_dim = 2 * key_dim + d_inner;
     const uint64_t qd = c->head_dim * c->n_head, kvd = c->head_dim * c->n_head_kv;
@@ -138,9 +139,18 @@ extern "C" int it_synth_write_gguf(const char* path, const it_synth_config* c, c
             add(nm("ffn_up_exps.scale"), {c->n_expert}, IT_F32, 5);
             add(nm("ffn_down_exps.scale"), {c->n_expert}, IT_F32, 5);
         }
-        add(nm("ffn_gate_shexp.weight"), {nd, c->shared_ff}, D, 0);
-        add(nm("ffn_up_shexp.weight"), {nd, c->shared_ff}, D, 0);
-        add(nm("ffn_down_shexp.weight"), {c->shared_ff, nd}, D, 0);
+        if (c->shared_type == IT_NVFP4) {
+            add(nm("ffn_gate_shexp.weight"), {nd, c->shared_ff}, IT_NVFP4, 4);
+            add(nm("ffn_up_shexp.weight"), {nd, c->shared_ff}, IT_NVFP4, 4);
+            add(nm("ffn_down_shexp.weight"), {c->shared_ff, nd}, IT_NVFP4, 4);
+            add(nm("ffn_gate_shexp.scale"), {1}, IT_F32, 5);
+            add(nm("ffn_up_shexp.scale"), {1}, IT_F32, 5);
+            add(nm("ffn_down_shexp.scale"), {1}, IT_F32, 5);
+        } else {
+            add(nm("ffn_gate_shexp.weight"), {nd, c->shared_ff}, D, 0);
+            add(nm("ffn_up_shexp.weight"), {nd, c->shared_ff}, D, 0);
+            add(nm("ffn_down_shexp.weight"), {c->shared_ff, nd}, D, 0);
+        }
         add(nm("ffn_gate_inp_shexp.weight"), {nd}, R, 0);
     }
     const uint64_t align = 32;

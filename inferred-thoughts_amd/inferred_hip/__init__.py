@@ -81,7 +81,7 @@ class SynthConfig(C.Structure):
                                       "n_expert", "n_expert_used", "expert_ff", "shared_ff", "ssm_d_conv",
                                       "ssm_d_state", "ssm_n_group", "ssm_dt_rank", "full_attention_interval")] + \
                [("rope_theta", c_f32), ("rms_eps", c_f32), ("dense_type", c_u32), ("expert_type", c_u32),
-                ("router_type", c_u32), ("_pad", c_u32), ("seed", c_u64), ("weight_std", c_f32),
+                ("router_type", c_u32), ("shared_type", c_u32), ("seed", c_u64), ("weight_std", c_f32),
                 ("n_threads", c_u32)]
 
 

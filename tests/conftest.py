@@ -53,3 +53,24 @@ def tiny_nvfp4_gguf(tmp_path_factory):
     p = tmp_path_factory.mktemp("models") / "tiny_nvfp4.gguf"
     ih.synth_write_gguf(str(p), ih.tiny_config(seed=1, expert_type=ih.NVFP4))
     return p
+
+
+@pytest.fixture(scope="session")
+def tiny_real_layout_gguf(tmp_path_factory):
+    """The tiny shape laid out as an NVFP4 file of this model is: NVFP4 experts with per-expert scales, an NVFP4 shared
+    expert with a second scale per matrix (ffn_*_shexp.scale), and the router, shared-expert gate and ssm alpha / beta
+    in F32."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "tiny_real_layout.gguf"
+    ih.synth_write_gguf(str(p), ih.tiny_config(seed=4, expert_type=ih.NVFP4, shared_type=ih.NVFP4, router_type=ih.ROUTER_F32))
+    return p
+
+
+@pytest.fixture(scope="session")
+def tiny_nvfp4_shared_gguf(tmp_path_factory):
+    """The tiny shape with NVFP4 experts and an NVFP4 shared expert with second scales, Q8_0 router (so that exact mode
+    fuses the routed FFN of a single-token pass as well)."""
+    import inferred_hip as ih
+    p = tmp_path_factory.mktemp("models") / "tiny_nvfp4_shared.gguf"
+    ih.synth_write_gguf(str(p), ih.tiny_config(seed=5, expert_type=ih.NVFP4, shared_type=ih.NVFP4))
+    return p

@@ -203,7 +203,10 @@ def test_attention_block(pair):
 
 
 # --------------------------------------------------------------------------------------------- routed FFN
-def test_ffn_block_512_experts(pair):
+@pytest.mark.parametrize("shared", ["q8_0", "nvfp4_scaled"])
+def test_ffn_block_512_experts(pair, shared):
+    """shared = nvfp4_scaled: the shared expert as an NVFP4 file stores it, three NVFP4 matrices with a second scale
+    each, applied by SCALE ops after the products (qwen35.rs:1669-1682); the fused kernels take the scales as scalars."""
     hip, orc, ih = pair.hip, pair.orc, pair.ih
     NE, NU, FF, SFF = 512, 10, 512, 512
     r = rng(103)
@@ -214,7 +217,13 @@ def test_ffn_block_512_experts(pair):
     gate = pair.e(nvfp4_rows(r, NE * FF, ND), ih.NVFP4, ND, FF, NE, g_s)
     up = pair.e(nvfp4_rows(r, NE * FF, ND), ih.NVFP4, ND, FF, NE, u_s)
     down = pair.e(nvfp4_rows(r, NE * ND, FF), ih.NVFP4, FF, ND, NE, d_s)
-    sg, su, sd = pair.q8(r, SFF, ND, 1.5), pair.q8(r, SFF, ND, 1.5), pair.q8(r, ND, SFF, 2.0)
+    if shared == "q8_0":
+        sg, su, sd = pair.q8(r, SFF, ND, 1.5), pair.q8(r, SFF, ND, 1.5), pair.q8(r, ND, SFF, 2.0)
+        s_g = s_u = s_d = None
+    else:
+        sg, su = pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF), pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF)
+        sd = pair.w(nvfp4_rows(r, ND, SFF), ih.NVFP4, SFF, ND)
+        s_g, s_u, s_d = float(0.7 / 54.0), float(1.3 / 54.0), float(1.1 / 27.0)
     norm_w = (0.5 + r.random(ND)).astype(np.float32)
     B = bufs(x=ND, normed=ND, e_in=ND, router=NE, logit=1, g_all=NU * FF, u_all=NU * FF, o_all=NU * ND, e_gate=SFF,
              e_up=SFF, e_out=ND, ffn_out=ND)
@@ -234,8 +243,12 @@ def test_ffn_block_512_experts(pair):
             ops.moe_glu(W(gate), W(up), ids, NU, b["e_in"], b["g_all"], b["u_all"])
             ops.matmul_experts(W(down), ids, NU, b["g_all"], b["o_all"])
         ops.matmul(W(sg), b["e_in"], b["e_gate"]); ops.matmul(W(su), b["e_in"], b["e_up"])
+        if s_u is not None:
+            ops.scale(b["e_up"], s_u); ops.scale(b["e_gate"], s_g)
         ops.silu_mul(b["e_gate"], b["e_up"])
         ops.matmul(W(sd), b["e_gate"], b["e_out"])
+        if s_d is not None:
+            ops.scale(b["e_out"], s_d)
         if is_hip:
             ops.moe_finish(b["ffn_out"], 0, ND, b["o_all"], route, b["e_out"], b["logit"], 0)
         else:
@@ -262,6 +275,8 @@ def test_ffn_block_512_experts(pair):
         o_all = np.zeros(NU * ND, np.float32); e_out = np.zeros(ND, np.float32); ffn = np.zeros(ND, np.float32)
         orc.matmul_experts(down[1], ids, NU, B[0]["g_all"], o_all)
         orc.matmul(sd[1], B[0]["e_gate"], e_out)
+        if s_d is not None:
+            orc.scale(e_out, s_d)
         orc.moe_finish(ffn, 0, ND, o_all, w, NU, e_out, B[1]["logit"], 0)
         got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
         assert np.abs(want).max() > 0.3

@@ -25,7 +25,8 @@ def prompt_ids(n=32, vocab=4096, seed=0):
     return np.random.default_rng(seed).integers(0, vocab, n).astype(np.uint32)
 
 
-@pytest.mark.parametrize("which", ["tiny_gguf", "tiny_nvfp4_gguf", "mid_gguf", "tiny_f32_router_gguf"])
+@pytest.mark.parametrize("which", ["tiny_gguf", "tiny_nvfp4_gguf", "mid_gguf", "tiny_f32_router_gguf",
+                                   "tiny_nvfp4_shared_gguf", "tiny_real_layout_gguf"])
 def test_greedy_tokens_bit_identical(hip, request, which):
     import inferred_hip as ih
     from oracle import binding as ob
@@ -138,12 +139,13 @@ def _rel(a, b):
     return float(np.abs(a - b).max()) / max(1.0, float(np.abs(b).max()))
 
 
-def test_float_router_is_fused_in_fast_mode(tiny_nvfp4_gguf, tiny_f32_router_gguf):
+def test_float_router_is_fused_in_fast_mode(tiny_nvfp4_gguf, tiny_f32_router_gguf, tiny_real_layout_gguf):
     """F32 router / shared-gate / ssm alpha, beta matrices (what real files hold) go into the same fused launches
-    as quantized ones in fast mode: the decode graph has the same number of kernels."""
+    as quantized ones in fast mode, and so does an NVFP4 shared expert whose second scales arrive as SCALE ops: the
+    decode graph has the same number of kernels."""
     import inferred_hip as ih
     counts = []
-    for path in (tiny_nvfp4_gguf, tiny_f32_router_gguf):
+    for path in (tiny_nvfp4_gguf, tiny_f32_router_gguf, tiny_real_layout_gguf):
         be = ih.Hip(exact=False)
         hm = ih.Model(path); e = ih.Engine(hm, be, 64)
         e.generate(prompt_ids(8), 12)
@@ -152,11 +154,11 @@ def test_float_router_is_fused_in_fast_mode(tiny_nvfp4_gguf, tiny_f32_router_ggu
         assert st["captures"] == 1 and st["replays"] >= 6 and st["aborts"] == 0
         counts.append(st["graph_kernels"])
         e.close(); hm.close(); be.close()
-    assert counts[0] == counts[1], counts
+    assert counts[0] == counts[1] == counts[2], counts
 
 
 @pytest.mark.parametrize("which,n_prompt,vocab", [("tiny_gguf", 48, 4096), ("tiny_nvfp4_gguf", 33, 4096),
-                                                  ("tiny_f32_router_gguf", 40, 4096)])
+                                                  ("tiny_f32_router_gguf", 40, 4096), ("tiny_real_layout_gguf", 36, 4096)])
 def test_fast_mode_stays_within_tolerance(request, which, n_prompt, vocab):
     """Fast mode (wave-order sums, split-K attention, lane-split delta rule, fused fast GEMVs) on whole models.
 
