@@ -244,8 +244,35 @@ IT_DEV int fast_mat_index(const FusedGemvP& p, int g) {
     return mi;
 }
 
+// row fr of the unquantized matrices (they follow the n_mats quantized ones in p.m): its matrix and its row there
+// (an index, not a pointer: the address of a kernel argument would move the whole argument block to scratch memory)
+IT_DEV int frow_locate(const FusedGemvP& p, int fr, int* j) {
+    int k = p.n_mats;
+    while (k + 1 < p.n_mats + p.n_fmats && fr >= p.m[k].n_out) {
+        fr -= p.m[k].n_out;
+        k++;
+    }
+    *j = fr;
+    return k;
+}
+// issues the loads of an F32 row's chunks (16 bytes per lane per 256 weights); false when the row is not F32
+constexpr int FC = 8;
+// (with the row shared by `split` waves, wave `part` of them takes the chunks c = part, part + split, ...)
+IT_DEV bool frow_fetch(const FusedGemvP& p, int fr, int n_in, int lane, float4 fw[FC], int split, int part) {
+    int j;
+    const FusedMat& m = p.m[frow_locate(p, fr, &j)];
+    if (m.fmt != W_F32) return false;
+    const float* row = (const float*)m.q + (int64_t)j * n_in;
+#pragma unroll
+    for (int c = 0; c < FC; c++)
+        if (c * 256 < n_in && c % split == part) fw[c] = *(const float4*)(row + c * 256 + lane * 4);
+    return true;
+}
+
 // ONE: one step per group (a matrix of few rows spreads over more blocks, i.e. more CUs pull its weights)
-template <int FMT, int CPL, int L, bool ONE = false>
+// FM: the launch has unquantized matrices as well (a kernel of its own, so that the registers their rows are held in
+// are not charged to the launches without them)
+template <int FMT, int CPL, int L, bool ONE = false, bool FM = false>
 __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     constexpr int P = 64 / L;
     constexpr int RB = ONE || CPL >= 4 ? 1 : 4 / CPL;  // steps per group: four chunk loads per lane in flight
@@ -278,10 +305,19 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     };
     // the first group's weights start moving before the activation prologue runs
     if (g < p.total_groups) fetch(g);
+    const bool f32_regs = FM && n_in % 256 == 0 && n_in <= FC * 256;
+    float4 fw[FM ? FC : 1];
+    bool f_loaded = false;
+    const int fsplit = FM ? p.fsplit : 1;                       // 1, 2 or 4 waves a row; more than 1 only with f32_regs
+    const int fpart = wave % fsplit, frows_blk = FW / fsplit;  // rows a block takes per trip
+    if constexpr (FM) {
+        const int fr0 = blockIdx.x * frows_blk + wave / fsplit;
+        if (f32_regs && fr0 < p.total_frows) f_loaded = frow_fetch(p, fr0, n_in, lane, fw, fsplit, fpart);
+    }
 
     const bool first = blockIdx.x == 0;
     stage_activation<FT>(p.x, n_in, p.mode, p.norm_w, p.gate, p.head_dim, p.eps, first ? p.x_copy : nullptr,
-                         first ? p.x_copy2 : nullptr, xq, xs, red, p.n_fmats ? xf : nullptr);
+                         first ? p.x_copy2 : nullptr, xq, xs, red, FM ? xf : nullptr);
     XChunks<FMT, CPL> x;
     load_x<FMT, CPL, L>(x, xq, xs, sub);
 
@@ -330,31 +366,66 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
     }
 
     // unquantized matrices (the router and ssm alpha / beta of real files are F32): one wave per row, the row sum
-    // split over the lanes
-    for (int fr = blockIdx.x * FW + wave; fr < p.total_frows; fr += gstride) {
-        int k = p.n_mats, j = fr;
-        while (k + 1 < p.n_mats + p.n_fmats && j >= p.m[k].n_out) {
-            j -= p.m[k].n_out;
-            k++;
-        }
-        const FusedMat& m = p.m[k];
-        const int esz = m.fmt == W_F32 ? 4 : 2;
-        const uint8_t* row = m.q + (int64_t)j * n_in * esz;
+    // split over the lanes.  An F32 row of up to 2,048 weights is held in registers: all of its loads are in flight
+    // at once, the first row's since before the prologue and the next row's while this one is reduced.
+    if constexpr (!FM) return;
+    const int fstride = gridDim.x * frows_blk;
+    // every wave of a block makes the same number of trips (the partial sums of a shared row meet behind a barrier)
+    for (int base = blockIdx.x * frows_blk; base < p.total_frows; base += fstride) {
+        const int fr = base + wave / fsplit;
+        const bool live = fr < p.total_frows;
+        float* outp = nullptr;
         float acc = 0.0f;
-        for (int i = lane * 4; i < n_in; i += 256) {
-            float4 wv;
-            if (m.fmt == W_F32) {
-                wv = *(const float4*)(row + (int64_t)i * 4);
-            } else {
-                const uint2 h = *(const uint2*)(row + (int64_t)i * 2);
-                wv = m.fmt == W_F16 ? make_float4(it_f16_to_f32(h.x & 0xffffu), it_f16_to_f32(h.x >> 16), it_f16_to_f32(h.y & 0xffffu), it_f16_to_f32(h.y >> 16))
-                                    : make_float4(it_bf16_to_f32(h.x & 0xffffu), it_bf16_to_f32(h.x >> 16), it_bf16_to_f32(h.y & 0xffffu), it_bf16_to_f32(h.y >> 16));
+        if (live) {
+            int j;
+            const FusedMat& m = p.m[frow_locate(p, fr, &j)];
+            outp = m.out + j;
+            if (f32_regs && m.fmt == W_F32) {
+                if (!f_loaded) frow_fetch(p, fr, n_in, lane, fw, fsplit, fpart);
+                f_loaded = false;
+                float4 cur[FC];
+#pragma unroll
+                for (int c = 0; c < FC; c++) cur[c] = fw[c];
+                const int nxt = fr + fstride;
+                if (nxt < p.total_frows) f_loaded = frow_fetch(p, nxt, n_in, lane, fw, fsplit, fpart);
+#pragma unroll
+                for (int c = 0; c < FC; c++) {
+                    if (c * 256 >= n_in) break;
+                    if (c % fsplit != fpart) continue;
+                    const float4 xv = *(const float4*)(xf + c * 256 + lane * 4);
+                    acc = fmaf(cur[c].x, xv.x, fmaf(cur[c].y, xv.y, fmaf(cur[c].z, xv.z, fmaf(cur[c].w, xv.w, acc))));
+                }
+            } else if (fpart == 0) {   // other element types and row lengths: one wave walks the row
+                const int esz = m.fmt == W_F32 ? 4 : 2;
+                const uint8_t* row = m.q + (int64_t)j * n_in * esz;
+                for (int i = lane * 4; i < n_in; i += 256) {
+                    float4 wv;
+                    if (m.fmt == W_F32) {
+                        wv = *(const float4*)(row + (int64_t)i * 4);
+                    } else {
+                        const uint2 h = *(const uint2*)(row + (int64_t)i * 2);
+                        wv = m.fmt == W_F16 ? make_float4(it_f16_to_f32(h.x & 0xffffu), it_f16_to_f32(h.x >> 16), it_f16_to_f32(h.y & 0xffffu), it_f16_to_f32(h.y >> 16))
+                                            : make_float4(it_bf16_to_f32(h.x & 0xffffu), it_bf16_to_f32(h.x >> 16), it_bf16_to_f32(h.y & 0xffffu), it_bf16_to_f32(h.y >> 16));
+                    }
+                    const float4 xv = *(const float4*)(xf + i);
+                    acc = fmaf(wv.x, xv.x, fmaf(wv.y, xv.y, fmaf(wv.z, xv.z, fmaf(wv.w, xv.w, acc))));
+                }
             }
-            const float4 xv = *(const float4*)(xf + i);
-            acc = fmaf(wv.x, xv.x, fmaf(wv.y, xv.y, fmaf(wv.z, xv.z, fmaf(wv.w, xv.w, acc))));
         }
         acc = reduce_lanes<64>(acc);
-        if (lane == 63) m.out[j] = acc;
+        if (fsplit == 1) {
+            if (live && lane == 63) *outp = acc;
+        } else {
+            float* fsum = (float*)red;   // the prologue is done with it; FW doubles hold FW floats
+            if (lane == 63) fsum[wave] = acc;
+            __syncthreads();
+            if (live && fpart == 0 && lane == 63) {
+                float v = fsum[wave];
+                for (int k = 1; k < fsplit; k++) v += fsum[wave + k];
+                *outp = v;
+            }
+            __syncthreads();
+        }
     }
 }
 
@@ -418,7 +489,17 @@ static bool fused_gemv_fast_prepare(FusedGemvP& p, Geo* geo, int* fmt_out, int* 
     }
     p.total_groups = groups;
     p.rows_per_wave = RG;
-    int blocks = (max(groups, p.total_frows) + FW - 1) / FW;
+    // a launch of unquantized rows only (the F32 router of a real file: 513 rows of 8 KB) would sit on 65 CUs with a
+    // wave per row; two waves a row use 129 (431 against 427 tok/s for the model with such a router; four waves a
+    // row, 257 CUs, give the gain back to the barrier: 426)
+    p.fsplit = 1;
+    if (nq == 0 && p.n_in % 256 == 0 && p.n_in <= FC * 256) {
+        bool all_f32 = true;
+        for (int i = 0; i < nf; i++) all_f32 = all_f32 && fm[i].fmt == W_F32;
+        const int chunks = p.n_in / 256;
+        while (all_f32 && p.fsplit < 2 && chunks % (2 * p.fsplit) == 0 && (p.total_frows * p.fsplit + FW - 1) / FW < 200) p.fsplit *= 2;
+    }
+    int blocks = (max(groups, p.total_frows * p.fsplit) + FW - 1) / FW;
     // Whole multiples of the CU count, so that every CU carries the same number of blocks: four per CU for a matrix
     // that loops (the LM head), two per CU for one that would need between two and four (the GDN in-projection's 772
     // blocks, three on some CUs and four on others, ran 0.03 ms per token slower than 512 that loop once or twice;
@@ -449,10 +530,13 @@ bool fused_gemv_fast(FusedGemvP p, hipStream_t s) {
     int fmt, blocks;
     if (!fused_gemv_fast_prepare(p, &g, &fmt, &blocks)) return false;
     const bool one = p.rows_per_wave == 64 / g.l && g.cpl < 4;
-#define IT_LAUNCH(F, C, LL)                                                                          \
-    do {                                                                                             \
-        if (one) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, true>), dim3(blocks), dim3(FT), 0, s, p); \
-        else hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL>), dim3(blocks), dim3(FT), 0, s, p);      \
+    const bool fm = p.n_fmats > 0;
+#define IT_LAUNCH(F, C, LL)                                                                                            \
+    do {                                                                                                               \
+        if (one && fm) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, true, true>), dim3(blocks), dim3(FT), 0, s, p);  \
+        else if (one) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, true, false>), dim3(blocks), dim3(FT), 0, s, p);  \
+        else if (fm) hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, false, true>), dim3(blocks), dim3(FT), 0, s, p);   \
+        else hipLaunchKernelGGL((fused_gemv_fast_k<F, C, LL, false, false>), dim3(blocks), dim3(FT), 0, s, p);          \
     } while (0)
     if (fmt == W_Q8_0) {
         if (g.l == 64 && g.cpl == 1) IT_LAUNCH(W_Q8_0, 1, 64);

@@ -25,6 +25,7 @@ struct FusedGemvP {
     // fast kernels only: the launcher moves unquantized (F32 / F16 / BF16) matrices behind the quantized ones;
     // m[n_mats .. n_mats + n_fmats) are those, total_frows rows in all (epi 0 only)
     int n_fmats, total_frows;
+    int fsplit;   // waves that share one unquantized row (1 or 2; the kernel also takes 4): a launch of few such rows and nothing else spreads over more CUs
     float* conv_state;    // epi 1
     const float* conv_w;
     // optional: matrix 0 is the router; the last block to finish picks the experts
