@@ -1314,6 +1314,27 @@ void it_hip_matmul(it_hip* be, const it_weights* w, const float* x, uint64_t x_l
 
 void it_hip_matmul_pair(it_hip* be, const it_weights* a, const it_weights* b, const float* x, uint64_t x_len,
                         float* out_a, uint64_t out_a_len, float* out_b, uint64_t out_b_len) {
+    // A batch against two unquantized matrices (the F32 router with the shared-gate logit, ssm alpha with beta, of a
+    // real file): one launch reads the activations once for both.  Single-token passes keep two ops for the fuser.
+    const bool floats = a && b && a->data && b->data && (a->ty == IT_F32 || a->ty == IT_F16 || a->ty == IT_BF16) && a->ty == b->ty;
+    if (!be->exact && floats && a->n_in == b->n_in && a->n_in && x_len % a->n_in == 0 && x_len / a->n_in > 16 &&
+        x_len / a->n_in <= 65535 && out_a_len == x_len / a->n_in * a->n_out && out_b_len == x_len / a->n_in * b->n_out) {
+        WView va, vb;
+        if (!be->weights_view(a, "matmul_pair(a)", &va) || !be->weights_view(b, "matmul_pair(b)", &vb)) return;
+        const float* dx = be->act_in(x, x_len);
+        float* da = be->act_out(out_a, out_a_len);
+        float* db = be->act_out(out_b, out_b_len);
+        if (!dx || !da || !db) return;
+        const int nt = (int)(x_len / a->n_in);
+        if ((reinterpret_cast<uintptr_t>(va.q) & 15) == 0 && (reinterpret_cast<uintptr_t>(vb.q) & 15) == 0 && va.n_in % 16 == 0) {
+            it_hip::OpRec rec;
+            rec.id = OP_MATMUL;
+            be->submit(it_hip::FAM_MATMUL, a->len + b->len + x_len * 4 + (out_a_len + out_b_len) * 4,
+                       sig_of(OP_MATMUL, va.q, vb.q, va.fmt, va.n_in, va.n_out, vb.n_out, dx, nt, da, db), rec,
+                       [=](hipStream_t s) { float_matmul_pair(va, vb, dx, nt, da, db, s); });
+            return;
+        }
+    }
     matmul_impl(be, a, x, x_len, out_a, out_a_len, "matmul_pair(a)");
     matmul_impl(be, b, x, x_len, out_b, out_b_len, "matmul_pair(b)");
 }

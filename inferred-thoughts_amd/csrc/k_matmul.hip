@@ -243,33 +243,54 @@ __global__ __launch_bounds__(256) void float_gemv_fast_k(const uint8_t* __restri
     }
 }
 
-// More tokens: a block owns 64 weight rows x 64 tokens, stages 16-wide k slabs of both operands in LDS and every
-// thread keeps a 4 x 4 tile of sums.
+// Two matrices read with the same activations (matmul_pair: router + shared-gate logit, ssm alpha + beta) as one
+// launch: rows 0 .. n0 are matrix 0's, the next n1 matrix 1's, each with its own output.  n1 = 0: one matrix.
+struct FloatMats {
+    const uint8_t *w0, *w1;
+    float *out0, *out1;
+    int n0, n1;
+};
 template <int FMT>
-__global__ __launch_bounds__(256) void float_gemm_fast_k(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                                         float* __restrict__ out, int n_in, int n_out, int n_tok,
+IT_DEV const uint8_t* float_row(const FloatMats& m, int j, int n_in) {
+    constexpr int ESZ = FMT == W_F32 ? 4 : 2;
+    const int last = m.n0 + m.n1 - 1;
+    j = j < last ? j : last;
+    return j < m.n0 ? m.w0 + (int64_t)j * n_in * ESZ : m.w1 + (int64_t)(j - m.n0) * n_in * ESZ;
+}
+IT_DEV void float_store(const FloatMats& m, int t, int j, float v) {
+    if (j < m.n0) m.out0[(int64_t)t * m.n0 + j] = v;
+    else if (j < m.n0 + m.n1) m.out1[(int64_t)t * m.n1 + (j - m.n0)] = v;
+}
+
+// More tokens: a block owns 64 weight rows x 64 tokens, stages 16-wide k slabs of both operands in LDS (the next
+// slab's loads in flight while this one is multiplied) and every thread keeps a 4 x 4 tile of sums.
+template <int FMT>
+__global__ __launch_bounds__(256) void float_gemm_fast_k(FloatMats m, const float* __restrict__ x, int n_in, int n_tok,
                                                          float out_scale) {
     constexpr int KS = 16;
     __shared__ float Ws[KS][64 + 4], Xs[KS][64 + 4];
     const int tid = threadIdx.x, tr = tid & 15, tc = tid >> 4;   // rows 4 tr .. + 3, tokens 4 tc .. + 3
     const int row0 = blockIdx.x * 64, tok0 = blockIdx.y * 64;
     const int lr = tid >> 2, lk = (tid & 3) * 4;                 // staging: row (or token) lr, k lk .. + 3
-    const int64_t wrow = min(row0 + lr, n_out - 1);
     const int64_t xrow = min(tok0 + lr, n_tok - 1);
-    const uint8_t* wp = w + wrow * n_in * (FMT == W_F32 ? 4 : 2);
+    const uint8_t* wp = float_row<FMT>(m, row0 + lr, n_in);
     const float* xp = x + xrow * n_in;
     float acc[4][4];
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
         for (int b = 0; b < 4; b++) acc[a][b] = 0.0f;
+    float4 wv = load_w4<FMT>(wp, lk);
+    float4 xv = *(const float4*)(xp + lk);
     for (int k0 = 0; k0 < n_in; k0 += KS) {
-        const float4 wv = load_w4<FMT>(wp, k0 + lk);
-        const float4 xv = *(const float4*)(xp + k0 + lk);
         __syncthreads();
         Ws[lk][lr] = wv.x; Ws[lk + 1][lr] = wv.y; Ws[lk + 2][lr] = wv.z; Ws[lk + 3][lr] = wv.w;
         Xs[lk][lr] = xv.x; Xs[lk + 1][lr] = xv.y; Xs[lk + 2][lr] = xv.z; Xs[lk + 3][lr] = xv.w;
         __syncthreads();
+        if (k0 + KS < n_in) {
+            wv = load_w4<FMT>(wp, k0 + KS + lk);
+            xv = *(const float4*)(xp + k0 + KS + lk);
+        }
 #pragma unroll
         for (int k = 0; k < KS; k++) {
             const float4 a = *(const float4*)&Ws[k][4 * tr];
@@ -286,11 +307,86 @@ __global__ __launch_bounds__(256) void float_gemm_fast_k(const uint8_t* __restri
         const int t = tok0 + 4 * tc + ib;
         if (t >= n_tok) continue;
 #pragma unroll
-        for (int ia = 0; ia < 4; ia++) {
-            const int j = row0 + 4 * tr + ia;
-            if (j < n_out) out[(int64_t)t * n_out + j] = out_scale != 1.0f ? acc[ia][ib] * out_scale : acc[ia][ib];
+        for (int ia = 0; ia < 4; ia++) float_store(m, t, row0 + 4 * tr + ia, out_scale != 1.0f ? acc[ia][ib] * out_scale : acc[ia][ib]);
+    }
+}
+
+// A long batch against a matrix of many rows (the F32 router of a real file over a prefill pass): 128 rows x 128
+// tokens per block and an 8 x 8 tile of sums per thread, i.e. a quarter of the LDS bytes per multiply-add of the
+// 4 x 4 form.  Every sum runs over k in the same order as there.
+template <int FMT>
+__global__ __launch_bounds__(256) void float_gemm_wide_k(FloatMats m, const float* __restrict__ x, int n_in, int n_tok,
+                                                         float out_scale) {
+    constexpr int KS = 16, TILE = 128;
+    __shared__ __align__(16) float Ws[KS][TILE + 4], Xs[KS][TILE + 4];
+    const int tid = threadIdx.x, tr = tid & 15, tc = tid >> 4;   // rows 4 tr .. + 3 and 64 + 4 tr .. + 3; tokens likewise by tc
+    const int row0 = blockIdx.x * TILE, tok0 = blockIdx.y * TILE;
+    const int lr = tid >> 2, lk = (tid & 3) * 4;                 // staging: rows (tokens) lr and lr + 64, k lk .. + 3
+    const uint8_t* wp[2];
+    const float* xp[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        wp[h] = float_row<FMT>(m, row0 + lr + 64 * h, n_in);
+        xp[h] = x + (int64_t)min(tok0 + lr + 64 * h, n_tok - 1) * n_in;
+    }
+    float acc[8][8];
+#pragma unroll
+    for (int a = 0; a < 8; a++)
+#pragma unroll
+        for (int b = 0; b < 8; b++) acc[a][b] = 0.0f;
+    float4 wv[2], xv[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        wv[h] = load_w4<FMT>(wp[h], lk);
+        xv[h] = *(const float4*)(xp[h] + lk);
+    }
+    for (int k0 = 0; k0 < n_in; k0 += KS) {
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int c = lr + 64 * h;
+            Ws[lk][c] = wv[h].x; Ws[lk + 1][c] = wv[h].y; Ws[lk + 2][c] = wv[h].z; Ws[lk + 3][c] = wv[h].w;
+            Xs[lk][c] = xv[h].x; Xs[lk + 1][c] = xv[h].y; Xs[lk + 2][c] = xv[h].z; Xs[lk + 3][c] = xv[h].w;
+        }
+        __syncthreads();
+        if (k0 + KS < n_in) {   // the next slab's loads fly while this one is multiplied
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                wv[h] = load_w4<FMT>(wp[h], k0 + KS + lk);
+                xv[h] = *(const float4*)(xp[h] + k0 + KS + lk);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < KS; k++) {
+            const float4 a0 = *(const float4*)&Ws[k][4 * tr], a1 = *(const float4*)&Ws[k][64 + 4 * tr];
+            const float4 b0 = *(const float4*)&Xs[k][4 * tc], b1 = *(const float4*)&Xs[k][64 + 4 * tc];
+            const float av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const float bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int ia = 0; ia < 8; ia++)
+#pragma unroll
+                for (int ib = 0; ib < 8; ib++) acc[ia][ib] = fmaf(av[ia], bv[ib], acc[ia][ib]);
         }
     }
+#pragma unroll
+    for (int ib = 0; ib < 8; ib++) {
+        const int t = tok0 + (ib < 4 ? 4 * tc + ib : 64 + 4 * tc + ib - 4);
+        if (t >= n_tok) continue;
+#pragma unroll
+        for (int ia = 0; ia < 8; ia++) {
+            const int j = row0 + (ia < 4 ? 4 * tr + ia : 64 + 4 * tr + ia - 4);
+            float_store(m, t, j, out_scale != 1.0f ? acc[ia][ib] * out_scale : acc[ia][ib]);
+        }
+    }
+}
+
+template <int FMT>
+static void float_gemm_launch(const FloatMats& m, const float* x, int n_in, int n_tok, float out_scale, hipStream_t s) {
+    const int rows = m.n0 + m.n1;
+    if (n_tok >= 1024 && rows >= 256)
+        hipLaunchKernelGGL(float_gemm_wide_k<FMT>, dim3((rows + 127) / 128, (n_tok + 127) / 128), dim3(256), 0, s, m, x, n_in, n_tok, out_scale);
+    else
+        hipLaunchKernelGGL(float_gemm_fast_k<FMT>, dim3((rows + 63) / 64, (n_tok + 63) / 64), dim3(256), 0, s, m, x, n_in, n_tok, out_scale);
 }
 
 template <int FMT>
@@ -298,8 +394,7 @@ static bool float_matmul_fast(const WView& w, const float* x, int n_tok, float* 
     if (w.n_in % 16 || (reinterpret_cast<uintptr_t>(w.q) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return false;
     const uint8_t* wp = (const uint8_t*)w.q;
     if (n_tok > 16) {
-        hipLaunchKernelGGL(float_gemm_fast_k<FMT>, dim3((w.n_out + 63) / 64, (n_tok + 63) / 64), dim3(256), 0, s, wp, x, out,
-                           w.n_in, w.n_out, n_tok, out_scale);
+        float_gemm_launch<FMT>(FloatMats{wp, nullptr, out, nullptr, w.n_out, 0}, x, w.n_in, n_tok, out_scale, s);
         return true;
     }
     for (int t0 = 0; t0 < n_tok; t0 += 8) {
@@ -310,6 +405,18 @@ static bool float_matmul_fast(const WView& w, const float* x, int n_tok, float* 
             hipLaunchKernelGGL((float_gemv_fast_k<FMT, 8>), dim3((w.n_out + 3) / 4), dim3(256), 0, s, wp, x, out, w.n_in, w.n_out,
                                n_tok, t0, out_scale);
     }
+    return true;
+}
+
+// matmul_pair over a batch with two unquantized matrices of one element type (fast mode): one launch for both
+bool float_matmul_pair(const WView& a, const WView& b, const float* x, int n_tok, float* out_a, float* out_b, hipStream_t s) {
+    if (a.fmt != b.fmt || a.n_in != b.n_in || n_tok <= 16 || a.n_in % 16 || a.n_out <= 0 || b.n_out <= 0) return false;
+    if (a.fmt != W_F32 && a.fmt != W_F16 && a.fmt != W_BF16) return false;
+    if ((reinterpret_cast<uintptr_t>(a.q) & 15) || (reinterpret_cast<uintptr_t>(b.q) & 15) || (reinterpret_cast<uintptr_t>(x) & 15)) return false;
+    const FloatMats m{(const uint8_t*)a.q, (const uint8_t*)b.q, out_a, out_b, a.n_out, b.n_out};
+    if (a.fmt == W_F32) float_gemm_launch<W_F32>(m, x, a.n_in, n_tok, 1.0f, s);
+    else if (a.fmt == W_F16) float_gemm_launch<W_F16>(m, x, a.n_in, n_tok, 1.0f, s);
+    else float_gemm_launch<W_BF16>(m, x, a.n_in, n_tok, 1.0f, s);
     return true;
 }
 

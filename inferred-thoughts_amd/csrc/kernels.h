@@ -23,6 +23,8 @@ struct WView {
 };
 
 // repack kernels: file layout -> device layout
+// two unquantized matrices of one element type over the same batch of activations, one launch (fast mode, > 16 tokens)
+bool float_matmul_pair(const WView& a, const WView& b, const float* x, int n_tok, float* out_a, float* out_b, hipStream_t s);
 void repack_q8_0(const uint8_t* raw, int8_t* q, uint16_t* scales, int64_t n_rows, int n_in, hipStream_t s);
 void repack_nvfp4(const uint8_t* raw, uint8_t* nib, uint8_t* scales, int64_t n_rows, int n_in, hipStream_t s);
 

@@ -225,10 +225,10 @@ def test_nvfp4_tiles_keep_subnormal_and_extreme_scales(hip, orc):
 
 
 # unquantized weights (the router and ssm alpha / beta of real files are F32): wave-split row sums for up to 16
-# tokens, LDS-tiled products for more
+# tokens, LDS-tiled products for more (64 x 64 tiles; 128 x 128 for 1,024 tokens and 256 rows on: the router over a prefill pass)
 @pytest.mark.parametrize("ty", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("n_in,n_out,n", [(2048, 512, 1), (2048, 32, 1), (2048, 1, 5), (512, 16, 16), (2048, 512, 100),
-                                          (512, 70, 17), (2048, 33, 300)])
+                                          (512, 70, 17), (2048, 33, 300), (2048, 513, 1100), (512, 300, 1024)])
 def test_matmul_float_types_fast(hip, orc, ty, n_in, n_out, n):
     import inferred_hip as ih
     from oracle import binding as ob
@@ -249,6 +249,30 @@ def test_matmul_float_types_fast(hip, orc, ty, n_in, n_out, n):
     hip.raise_if_error()
     assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(np.abs(b), np.sqrt(n_in))), np.abs(a - b).max()
     assert np.abs(a - b).max() <= 2e-4 * np.sqrt(n_in)     # f32 rounding of a different sum order, no more
+
+
+@pytest.mark.parametrize("n_in,n_a,n_b,n", [(2048, 513, 1, 1100), (2048, 32, 32, 300), (512, 70, 3, 17), (2048, 513, 1, 16)])
+def test_matmul_pair_float_batch(hip, orc, n_in, n_a, n_b, n):
+    """Two F32 matrices read with one batch of activations (the router with the shared-gate logit, ssm alpha with beta,
+    of a real file during prefill): above 16 tokens one launch serves both; rows of the second matrix follow the
+    first's inside the tiles, each matrix keeps its own output."""
+    import inferred_hip as ih
+    from oracle import binding as ob
+    fresh(hip)
+    hip.begin_pass(n)
+    r = rng(43)
+    wa = r.standard_normal((n_a, n_in)).astype(np.float32).view(np.uint8).reshape(-1).copy()
+    wb = r.standard_normal((n_b, n_in)).astype(np.float32).view(np.uint8).reshape(-1).copy()
+    x = r.standard_normal(n * n_in).astype(np.float32)
+    oa, ob_ = np.zeros(n * n_a, np.float32), np.zeros(n * n_b, np.float32)
+    ra, rb = np.zeros_like(oa), np.zeros_like(ob_)
+    hip.matmul_pair(ih.weights(wa, ih.F32, n_in, n_a), ih.weights(wb, ih.F32, n_in, n_b), x, oa, ob_)
+    hip.host_needs(oa); hip.host_needs(ob_)
+    orc.matmul(ob.weights(wa, ih.F32, n_in, n_a), x, ra)
+    orc.matmul(ob.weights(wb, ih.F32, n_in, n_b), x, rb)
+    hip.raise_if_error()
+    for got, want in ((oa, ra), (ob_, rb)):
+        assert np.abs(got - want).max() <= 2e-4 * np.sqrt(n_in)
 
 
 @pytest.mark.parametrize("n,nd", [(1, 2048), (33, 2048), (3, 512)])
