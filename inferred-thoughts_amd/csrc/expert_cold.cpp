@@ -84,10 +84,6 @@ class ReadPool {
             close(fd);
         }
     }
-    bool from_file() {
-        std::lock_guard<std::mutex> g(m_);
-        return fd_ >= 0;
-    }
     void submit(const Job& j) {
         {
             std::lock_guard<std::mutex> g(m_);
@@ -267,7 +263,7 @@ bool it_hip::cold_sentinel(const uint8_t** q, const uint8_t** s, uint64_t q_stri
 
 namespace {
 
-// everything a resolve needs beyond the tier's state, so that the steps below stay free functions of (backend, tier)
+// a cold pick: its tensor (the placement record and the host address of its bytes) and the expert
 struct Want {
     it_hip::Resident* r;
     const uint8_t* key;
