@@ -233,7 +233,7 @@ void it_hip_prefetch_hint(it_hip*, const it_weights* next_router, const float* x
  * wins device memory; every 64 tokens, at a pass boundary, a bounded number of busy host-tier experts change places
  * with idle device-tier ones (placement.rs:33-80), and replace_experts_by_counts runs that exchange to completion.
  * A pool that outgrows both tiers has cold experts (experts.rs:67-93): no copy of them is held; before an expert kernel
- * runs the picks are read back (such passes run eagerly, never from a graph; the exchange by counts is paused), and
+ * runs the picks are read back (such passes never run from a graph; the exchange by counts is paused), and
  * each cold pick is fetched from the model file (set_model_path + set_map_base; else from the tensor's mapping) into a
  * device slot taken by GCLOCK from an expert the routing decision did not pick.  The device tier must hold one
  * decision's picks of a layer's three tensors, else the call is refused with a sticky error.  prefetch_hint (the next

@@ -91,9 +91,25 @@ void it_hip::drop_graph() {
     stable_passes = 0;
 }
 
+// what a deferred pass has recorded so far goes to the stream, fused; the pass stays deferred
+void it_hip::flush_deferred() {
+    for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
+    precopies.clear();
+    dyn_upload();
+    if (pending.empty()) return;
+    auto todo = std::move(pending);
+    pending.clear();
+    run_fused(todo);
+    check(hipGetLastError(), "kernel launch");
+}
+
 void it_hip::need_eager(const char* why) {
     if (mode == Mode::Eager) return;
     (void)why;
+    if (mode == Mode::Deferred) {
+        flush_deferred();
+        return;
+    }
     drop_graph();
     graph_aborts++;
     mode = Mode::Eager;
@@ -107,6 +123,12 @@ void it_hip::need_eager(const char* why) {
 }
 
 void it_hip::finish_pass() {
+    if (mode == Mode::Deferred) {
+        flush_deferred();
+        mode = Mode::Eager;
+        stable_passes = 0;
+        return;
+    }
     if (mode == Mode::Eager) {
         if (pass_tokens == 1 && allow_graph && !mid_pass_read && !prof_on) {
             stable_passes = (pass_signature == prev_signature && !pass_signature.empty()) ? stable_passes + 1 : 0;
@@ -1952,6 +1974,8 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
         } else if (be->stable_passes >= 1 && !be->prof_on) {
             be->mode = it_hip::Mode::Capture;
         }
+    } else if (n_tokens == 1 && be->expert_cold_entries && be->fuse_enabled && !be->has_error) {
+        be->mode = it_hip::Mode::Deferred;   // picks are read back inside the pass: fused launches, no graph
     }
     for (auto& kv : be->acts) {
         kv.second.dev_current = false;

@@ -213,7 +213,11 @@ struct it_hip {
         std::vector<std::array<int, 4>> attn_slots;
     };
     Graph graph;
-    enum class Mode { Eager, Capture, Replay } mode = Mode::Eager;
+    // Deferred: a single-token pass whose ops are recorded like a captured pass's and issued as fused launches whenever
+    // something needs them on the stream (a cold expert's resolve reads the picks back, a host read, the pass's end):
+    // the fusion of the decode path without its graph, for passes a graph cannot hold.
+    enum class Mode { Eager, Capture, Replay, Deferred } mode = Mode::Eager;
+    void flush_deferred();
     std::vector<uint64_t> pass_signature, prev_signature;
     int stable_passes = 0;      // consecutive eager decode passes with the same op sequence
     size_t replay_cursor = 0;
@@ -274,6 +278,7 @@ struct it_hip {
         rec.run = f;
         pending.push_back(std::move(rec));
         pass_signature.push_back(sig);
+        if (mode == Mode::Deferred) return;
         if (mode == Mode::Capture) {
             // queued: the whole pass is fused and captured at end_pass
         } else if (replay_cursor >= graph.signature.size() || graph.signature[replay_cursor] != sig) {

@@ -4,7 +4,7 @@
 // make_resident :1418-1540, start_prefetch :1196-1280, evict_unleased and clock_pick :2112-2233; the caller's side in
 // src/ops/cuda/ops/moe.rs:820-1060).  A cold expert has no copy anywhere but the model file; its table entry points at
 // a zeroed sentinel.  Before an expert kernel of an oversubscribed pool is launched the picks are read back (a host
-// decision inside the pass, so such passes run eagerly, never from a graph), every pick is leased, and each cold pick
+// decision inside the pass, so such passes never run from a graph), every pick is leased, and each cold pick
 // is fetched into a device slot taken from an expert the layer did not pick: GCLOCK over a ring of all device slots,
 // heat 0..3, an arrival entering at 1.  The victim's entry is pointed at the sentinel, the fetched expert's at the
 // slot.  All of it is ordered on the launch stream: the copies into a slot, the repack and the table patches are
@@ -291,7 +291,6 @@ void it_hip::cold_hint(const it_weights* w, const float* x, uint64_t x_len, uint
 
 bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route* route, bool opens_layer) {
     if (!expert_cold_entries) return true;
-    need_eager("cold experts are resolved");
     if (!cold) cold = new ColdTier();
     ColdTier& c = *cold;
     Resident* first = &weights[keys[0]];
@@ -307,6 +306,7 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
     } else {
         const size_t n = (size_t)(route_n_used * route_n_tok);
         if (c.picks_gen != route_gen || c.picks.size() != n) {
+            need_eager("the picks are read back");   // the route kernel itself may still be waiting in a recorded pass
             uint64_t t0 = clock_us();
             if (!check(hipStreamSynchronize(stream), "sync before the picks are read back")) return false;
             uint64_t t1 = clock_us();
@@ -330,6 +330,7 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
     c.hint_ids.clear();
     if (c.hint_pending && opens_layer) {
         c.hint_pending = false;
+        need_eager("the hint's logits are read back");
         auto a = acts.find(c.hint_logits.data());
         if (c.hint_gen == route_gen && a != acts.end() && a->second.dev && a->second.dev_current) {
             std::vector<float> host(c.hint_n);
@@ -412,6 +413,8 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
         }
     }
     if (want.empty() && c.hint_ids.empty()) return true;
+    // slots change hands on the stream: everything recorded so far must be ahead of that
+    need_eager("cold experts are fetched");
     c.leased.assign(c.ring.size(), 0);
     for (size_t i = 0; i < c.ring.size(); i++)
         if (c.ring[i].owner && c.lease.count((uint64_t)c.ring[i].owner->counter_base + c.ring[i].e)) c.leased[i] = 1;

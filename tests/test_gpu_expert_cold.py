@@ -60,7 +60,8 @@ def test_mid_model_is_identical_with_cold_experts(mid_gguf, exact):
     assert tc.fetched == st.fetched and tc.fetch_bytes == st.fetched * 512 * 2048 // 32 * 18   # file bytes: 18 per 32
     assert st.lookups == ref[2].lookups                                  # the same reads, wherever they were served
     assert tc.picks_copy_us > 0 and tc.read_us > 0
-    assert cold[5]["replays"] == 0                                       # picks are read back mid-pass: no graph
+    assert cold[5]["replays"] == 0 and cold[5]["captures"] == 0          # picks are read back mid-pass: no graph ...
+    assert cold[5]["graph_kernels"] > 0                                  # ... but single-token passes are issued as fused launches
     assert cold[6] == 0                                                  # migration by counts is paused
     assert "cold" in cold[4] and "the model file" in cold[4]
     # the lookahead read ahead of the layers during decode, and some of its guesses were used
