@@ -104,6 +104,7 @@ void it_hip::flush_deferred() {
 }
 
 void it_hip::need_eager(const char* why) {
+    if (!held.empty()) release_held();   // whatever follows (a copy, a free, a wait) must find the stream complete
     if (mode == Mode::Eager) return;
     (void)why;
     if (mode == Mode::Deferred) {
@@ -123,6 +124,7 @@ void it_hip::need_eager(const char* why) {
 }
 
 void it_hip::finish_pass() {
+    if (!held.empty()) release_held();
     if (mode == Mode::Deferred) {
         flush_deferred();
         mode = Mode::Eager;
@@ -250,7 +252,8 @@ float* it_hip::act_in(const float* host, size_t len) {
     if (!a->dev_current) {
         if (mode != Mode::Eager) {
             precopies.push_back(PreCopy{a->dev, host, len * sizeof(float)});
-        } else if (!check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream),
+        } else if ((held.empty() || (release_held(), true)) &&
+                   !check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream),
                           "upload activation")) {
             return nullptr;
         }
@@ -778,6 +781,7 @@ bool it_hip::expert_counters_read(std::vector<uint32_t>* counts, uint64_t tally[
     tally[0] = tally[1] = 0;
     if (counts) counts->assign(expert_counted, 0);
     if (!expert_tally || !expert_counted) return true;
+    if (!held.empty()) release_held();
     if (in_pass) finish_pass();
     if (!check(hipStreamSynchronize(stream), "sync before reading the expert counters")) return false;
     unsigned long long t[2] = {0, 0};
@@ -1935,6 +1939,7 @@ void it_hip_host_wrote(it_hip* be, const float* buf, uint64_t len) {
 void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
     auto it = be->acts.find(buf);
     if (it == be->acts.end() || !it->second.dev_current) return;
+    if (!be->held.empty()) be->release_held();
     if (be->in_pass) {
         // a read inside a pass cannot be served from a graph that has not run yet:
         // graphs are latched off for this backend (src/ops/cuda/ops/mod.rs:565-582)
@@ -2354,7 +2359,10 @@ int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
     return n;
 }
 
-void it_hip_sync(it_hip* be) { be->check(hipStreamSynchronize(be->stream), "sync"); }
+void it_hip_sync(it_hip* be) {
+    if (!be->held.empty()) be->release_held();
+    be->check(hipStreamSynchronize(be->stream), "sync");
+}
 void it_hip_drop_mirrors(it_hip* be) { be->drop_all(); }
 uint64_t it_hip_launch_count(it_hip* be) { return be->launches; }
 

@@ -227,6 +227,8 @@ struct it_hip {
     // arguments (meaning per op, see the OpId table in backend.cpp), and the launch.
     struct OpRec {
         int id = 0;
+        int fam = 0;          // timing family and algorithmic bytes of the launch (kept for ops that are held back)
+        uint64_t bytes = 0;
         const void* p[12] = {};
         int64_t i[10] = {};
         float f[2] = {};
@@ -244,6 +246,11 @@ struct it_hip {
         const void* host;
         size_t bytes;
     };
+    // ops of a batch pass held back because they begin a run that has a one-kernel form (fuser.cpp)
+    std::vector<OpRec> held;
+    int hold_step(const OpRec& rec) const;   // 0: not part of a run, 1: continues it, 2: completes it
+    void release_held();                     // the run broke off: issue what is held op by op, in order
+    void finish_held();                      // the run is complete: one kernel (or op by op when its shape is not taken)
     std::vector<PreCopy> precopies;  // host -> device inputs of a graphed pass, issued before the graph
     int* dyn_dev = nullptr;    // device ints read by position-dependent kernels
     // pinned staging, double-buffered: a pass may fill one while the previous pass's async
@@ -270,6 +277,25 @@ struct it_hip {
         launches++;
         if (mode == Mode::Eager) {
             if (in_pass && pass_tokens == 1) pass_signature.push_back(sig);
+            if (in_pass && pass_tokens > 1 && !exact && fuse_enabled) {
+                // a batch pass in fast mode holds back the ops of two known elementwise runs and issues each run as
+                // one kernel once it is complete (hold_step, fuser.cpp); anything else releases what is held first
+                int st = hold_step(rec);
+                if (!st && !held.empty()) {
+                    release_held();
+                    st = hold_step(rec);
+                }
+                if (st) {
+                    rec.run = f;
+                    rec.fam = fam;
+                    rec.bytes = bytes;
+                    held.push_back(std::move(rec));
+                    if (st == 2) finish_held();
+                    return;
+                }
+            } else if (!held.empty()) {
+                release_held();
+            }
             Span sp(this, fam, bytes);
             f(stream);
             check(hipGetLastError(), "kernel launch");

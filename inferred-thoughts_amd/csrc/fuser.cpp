@@ -559,6 +559,76 @@ bool references(const Op& op, const void* a, const void* b) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------------- batch passes
+// Two runs of elementwise ops of a Gated DeltaNet layer over a batch (src/model/qwen35.rs:1255-1315) have a one-kernel
+// form in fast mode:
+//   CONV, GATHER q, GATHER k, GATHER v, L2 q, L2 k      -> conv_split_l2 (the conv output and the unnormed q, k are
+//                                                          not written: nothing else in the loop reads them)
+//   RMS_HEADS core, EW silu_mul(z, core), QUANT z        -> gated_norm_silu_q8 (core is left unnormed)
+// The ops are held back as they arrive and checked link by link (an op's input must be the run's own buffer).
+int it_hip::hold_step(const OpRec& r) const {
+    const size_t n = held.size();
+    if (n == 0) {
+        if (r.id == OP_CONV && r.i[2] >= 64 && r.i[1] % 128 == 0) return 1;
+        if (r.id == OP_RMS_HEADS && r.i[0] == 128 && r.i[1] >= 256) return 1;
+        return 0;
+    }
+    const OpRec& h0 = held[0];
+    if (h0.id == OP_CONV) {
+        const int64_t nc = h0.i[1], nt = h0.i[2];
+        if (n <= 3) {
+            if (r.id != OP_GATHER || r.p[0] != h0.p[3] || r.i[1] != nc) return 0;
+            const int64_t kdim = n == 1 ? r.i[0] : held[1].i[0];
+            if (kdim <= 0 || kdim % 128 || 2 * kdim >= nc) return 0;
+            const int64_t chunk = n == 3 ? nc - 2 * kdim : kdim, off = (int64_t)(n - 1) * kdim;
+            return r.i[0] == chunk && r.i[2] == off && r.i[3] == nt * chunk ? 1 : 0;
+        }
+        const OpRec& g = held[n - 3];   // n = 4: the q part, n = 5: the k part
+        if (r.id != OP_L2 || r.p[0] != g.p[1] || r.i[0] != 128 || r.i[1] * 128 != nt * held[1].i[0]) return 0;
+        if (n == 5 && r.f[0] != held[4].f[0]) return 0;
+        return n == 5 ? 2 : 1;
+    }
+    if (h0.id == OP_RMS_HEADS) {
+        if (n == 1) return r.id == OP_EW && r.i[0] == 0 && r.p[1] == h0.p[0] && r.i[1] == h0.i[1] * 128 ? 1 : 0;
+        if (n == 2) return r.id == OP_QUANT && r.p[0] == held[1].p[0] && r.i[0] == held[1].i[1] ? 2 : 0;
+    }
+    return 0;
+}
+
+void it_hip::release_held() {
+    auto ops = std::move(held);
+    held.clear();
+    for (auto& op : ops) {
+        Span sp(this, op.fam, op.bytes);
+        op.run(stream);
+    }
+    check(hipGetLastError(), "kernel launch");
+}
+
+void it_hip::finish_held() {
+    bool done = false;
+    uint64_t bytes = 0;
+    for (auto& op : held) bytes += op.bytes;
+    {
+        Span sp(this, held[0].fam, bytes);
+        if (held[0].id == OP_CONV && held.size() == 6) {
+            const OpRec &c = held[0], &gq = held[1], &gk = held[2], &gv = held[3], &l = held[4];
+            done = conv_split_l2((float*)c.p[0], (const float*)c.p[1], (const float*)c.p[2], (int)c.i[0], (int)c.i[1], (int)c.i[2],
+                                 (float*)gq.p[1], (float*)gk.p[1], (float*)gv.p[1], (int)gq.i[0], l.f[0], stream);
+        } else if (held[0].id == OP_RMS_HEADS && held.size() == 3) {
+            const OpRec &n = held[0], &e = held[1], &q = held[2];
+            done = gated_norm_silu_q8((const float*)n.p[0], (const float*)n.p[1], (float*)e.p[0], (float*)q.p[1], (int8_t*)q.p[2],
+                                      n.i[1], n.f[0], stream);
+        }
+    }
+    if (done) {
+        held.clear();
+        check(hipGetLastError(), "kernel launch");
+    } else {
+        release_held();
+    }
+}
+
 void it_hip::run_fused(std::vector<OpRec>& ops) {
     Plan pl(this, ops);
     fused_attn_slots.clear();

@@ -560,6 +560,138 @@ __global__ __launch_bounds__(128) void ssm_conv4_k(float* __restrict__ state, co
     }
 }
 
+// The Gated DeltaNet's input path over a batch in one pass over the data (fast mode): the causal conv + silu of
+// ssm_conv4_k over the q | k | v channels, each part written straight to its own buffer (the three gather_chunks that
+// follow the conv, qwen35.rs:1262-1270) and the q and k heads l2-normalised on the way (head_norm_wave_k's arithmetic:
+// f64 sum of the squares, 1 / max(norm, eps)).  A head is 128 channels: the 32 neighbouring lanes of four channels.
+template <int KEEP>
+__global__ __launch_bounds__(128) void conv_split_l2_k(float* __restrict__ state, const float* __restrict__ x,
+                                                       const float* __restrict__ w, int nc, int n_tok,
+                                                       float* __restrict__ q_out, float* __restrict__ k_out,
+                                                       float* __restrict__ v_out, int kdim, float eps) {
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (c >= nc) return;
+    const int t0 = blockIdx.y * CONV_TOK, t1 = min(n_tok, t0 + CONV_TOK);
+    const int vdim = nc - 2 * kdim;
+    float past[KEEP][4], wt[KEEP + 1][4];
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        if (blockIdx.y == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) past[k][e] = state[(int64_t)(c + e) * KEEP + k];
+        } else {
+            const float4 v = *(const float4*)(x + (int64_t)(t0 - KEEP + k) * nc + c);
+            past[k][0] = v.x; past[k][1] = v.y; past[k][2] = v.z; past[k][3] = v.w;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k <= KEEP; k++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) wt[k][e] = w[(int64_t)(c + e) * (KEEP + 1) + k];
+    float4 xin[CONV_TOK];
+#pragma unroll
+    for (int i = 0; i < CONV_TOK; i++)
+        xin[i] = t0 + i < t1 ? *(const float4*)(x + (int64_t)(t0 + i) * nc + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool normed = c < 2 * kdim;   // the same for the 32 lanes of a head
+    float* const dst = c < kdim ? q_out + c : (normed ? k_out + (c - kdim) : v_out + (c - 2 * kdim));
+    const int dstride = normed ? kdim : vdim;
+#pragma unroll
+    for (int i = 0; i < CONV_TOK; i++) {
+        if (t0 + i >= t1) break;
+        const float xv[4] = {xin[i].x, xin[i].y, xin[i].z, xin[i].w};
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KEEP; k++) sum += past[k][e] * wt[k][e];
+            sum += xv[e] * wt[KEEP][e];
+            o[e] = silu_of<true>(sum);
+#pragma unroll
+            for (int k = 0; k + 1 < KEEP; k++) past[k][e] = past[k + 1][e];
+            past[KEEP - 1][e] = xv[e];
+        }
+        if (normed) {
+            double part = 0.0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) part += (double)(o[e] * o[e]);
+#pragma unroll
+            for (int m = 1; m < 32; m <<= 1) part += __shfl_xor(part, m, 64);
+            const float nrm = sqrtf((float)part);
+            const float scale = 1.0f / fmaxf(nrm, eps);
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = o[e] * scale;
+        }
+        *(float4*)(dst + (int64_t)(t0 + i) * dstride) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+    if (blockIdx.y == 0) {
+#pragma unroll
+        for (int k = 0; k < KEEP; k++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) state[(int64_t)(c + e) * KEEP + k] = x[(int64_t)(n_tok - KEEP + k) * nc + c + e];
+    }
+}
+
+bool conv_split_l2(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* q_out, float* k_out,
+                   float* v_out, int kdim, float eps, hipStream_t s) {
+    if (n_tok < 64 || nc % 128 || kdim <= 0 || kdim % 128 || 2 * kdim >= nc || kernel < 2 || kernel > 5) return false;
+    if (!aligned16(x) || !aligned16(q_out) || !aligned16(k_out) || !aligned16(v_out)) return false;
+    dim3 grid((nc / 4 + 127) / 128, (n_tok + CONV_TOK - 1) / CONV_TOK), block(128);
+    switch (kernel) {
+        case 2: hipLaunchKernelGGL(conv_split_l2_k<1>, grid, block, 0, s, state, x, w, nc, n_tok, q_out, k_out, v_out, kdim, eps); break;
+        case 3: hipLaunchKernelGGL(conv_split_l2_k<2>, grid, block, 0, s, state, x, w, nc, n_tok, q_out, k_out, v_out, kdim, eps); break;
+        case 4: hipLaunchKernelGGL(conv_split_l2_k<3>, grid, block, 0, s, state, x, w, nc, n_tok, q_out, k_out, v_out, kdim, eps); break;
+        default: hipLaunchKernelGGL(conv_split_l2_k<4>, grid, block, 0, s, state, x, w, nc, n_tok, q_out, k_out, v_out, kdim, eps); break;
+    }
+    return true;
+}
+
+// The Gated DeltaNet's output path over a batch in one pass (fast mode): the per-head rms norm of the delta rule's
+// output (head_norm_wave_k<2>), z = silu(z) * normed (silu_mul4_k) and the Q8_0 form of z for the out-projection
+// (quantize_q8_0_k), each with the arithmetic of the kernel it replaces.  A wave per head of 128, two elements a lane;
+// a Q8_0 block is 16 neighbouring lanes.
+__global__ __launch_bounds__(256) void gated_norm_silu_q8_k(const float* __restrict__ core, const float* __restrict__ w,
+                                                            float* __restrict__ z, float* __restrict__ scales,
+                                                            int8_t* __restrict__ quants, int64_t n_heads, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t h = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (h >= n_heads) return;
+    const int64_t at = h * 128 + lane * 2;
+    const float2 v = *(const float2*)(core + at);
+    double part = 0.0;
+    part += (double)(v.x * v.x);
+    part += (double)(v.y * v.y);
+    const double sum = __shfl(wave_sum_f64_tail(part), 63, 64);
+    const float mean = (float)(sum / 128.0);
+    const float scale = 1.0f / sqrtf(mean + eps);
+    const float n0 = v.x * scale * w[lane * 2], n1 = v.y * scale * w[lane * 2 + 1];
+    const float2 g = *(const float2*)(z + at);
+    const float o0 = silu_of<true>(g.x) * n0, o1 = silu_of<true>(g.y) * n1;
+    *(float2*)(z + at) = make_float2(o0, o1);
+    float amax = fmaxf(fabsf(o0), fabsf(o1));
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float r[2] = {roundf(o0 * id), roundf(o1 * id)};
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const float cl = fminf(fmaxf(r[i], -128.0f), 127.0f);
+        const int q = (r[i] != r[i]) ? 0 : (int)cl;
+        packed |= ((uint32_t)(q & 0xff)) << (8 * i);
+    }
+    *(uint16_t*)(quants + at) = (uint16_t)packed;
+    if ((lane & 15) == 0) scales[at >> 5] = it_f16_to_f32(it_f32_to_f16(d));
+}
+
+bool gated_norm_silu_q8(const float* core, const float* w, float* z, float* scales, int8_t* quants, int64_t n_heads, float eps,
+                        hipStream_t s) {
+    if (n_heads < 256 || ((uintptr_t)core & 7) || ((uintptr_t)z & 7) || ((uintptr_t)quants & 1)) return false;
+    hipLaunchKernelGGL(gated_norm_silu_q8_k, dim3((unsigned)((n_heads + 3) / 4)), dim3(256), 0, s, core, w, z, scales, quants, n_heads, eps);
+    return true;
+}
+
 void ssm_conv(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* out, int exact,
               hipStream_t s) {
     if (nc <= 0 || n_tok <= 0) return;

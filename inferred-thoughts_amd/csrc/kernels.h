@@ -23,6 +23,11 @@ struct WView {
 };
 
 // repack kernels: file layout -> device layout
+// batch runs of elementwise ops as one kernel each (fast mode); false: not a case for the fused form
+bool conv_split_l2(float* state, const float* x, const float* w, int kernel, int nc, int n_tok, float* q_out, float* k_out,
+                   float* v_out, int kdim, float eps, hipStream_t s);
+bool gated_norm_silu_q8(const float* core, const float* w, float* z, float* scales, int8_t* quants, int64_t n_heads, float eps,
+                        hipStream_t s);
 // two unquantized matrices of one element type over the same batch of activations, one launch (fast mode, > 16 tokens)
 bool float_matmul_pair(const WView& a, const WView& b, const float* x, int n_tok, float* out_a, float* out_b, hipStream_t s);
 void repack_q8_0(const uint8_t* raw, int8_t* q, uint16_t* scales, int64_t n_rows, int n_in, hipStream_t s);
