@@ -642,9 +642,15 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
             if (match_norm_matmuls(pl, i, exact)) continue;
             if (match_matmul_residual(pl, i, exact)) continue;
         }
-        // a dropped quantization whose output an unfused op still reads is put back
+        // a dropped quantization whose output an unfused op still reads is put back; a deferred pass is issued in
+        // pieces, and a later piece (the expert products after the picks were read back) may read what this one
+        // quantized, so there every quantization is kept
         for (size_t i = 0; i < ops.size(); i++) {
             if (!pl.consumed[i] || ops[i].id != OP_QUANT) continue;
+            if (mode == Mode::Deferred) {
+                pl.consumed[i] = 0;
+                continue;
+            }
             for (size_t k = i + 1; k < ops.size(); k++) {
                 if (pl.consumed[k]) continue;
                 if (ops[k].id == OP_QUANT && ops[k].p[1] == ops[i].p[1]) break;  // re-quantized later
