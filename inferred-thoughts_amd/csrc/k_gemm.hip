@@ -26,7 +26,7 @@ constexpr int LSTR = SLAB + 8;  // LDS row stride in bytes (padded)
 // operands and their block scales into LDS with coalesced 16-byte loads (the next slab's
 // loads are in flight while the current one is multiplied), then every wave runs its 16 rows
 // against all token tiles: one MFMA per (block, tile), four scaled adds per lane after it.
-template <int NT>
+template <int NT, bool FMA = false>
 __global__ __launch_bounds__(GT) void q8_gemm_k(const int8_t* __restrict__ wq, const uint16_t* __restrict__ ws,
                                                 const int8_t* __restrict__ xq, const float* __restrict__ xs,
                                                 float* __restrict__ out, int n_in, int n_out, int n_tok,
@@ -117,7 +117,10 @@ __global__ __launch_bounds__(GT) void q8_gemm_k(const int8_t* __restrict__ wq, c
                 const v4i z = {0, 0, 0, 0};
                 const v4i d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bv, z, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) acc[tt][i] += (float)d[i] * (dw[i] * dx);
+                for (int i = 0; i < 4; i++) {
+                    if (FMA) acc[tt][i] = fmaf((float)d[i], dw[i] * dx, acc[tt][i]);
+                    else acc[tt][i] += (float)d[i] * (dw[i] * dx);
+                }
             }
         }
         if (s + 1 < nslab) stash(buf ^ 1);
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(GT) void q8_gemm_k(const int8_t* __restrict__ wq, c
 }  // namespace
 
 bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, int n_tok, float* out, float out_scale,
-             hipStream_t s) {
+             hipStream_t s, bool fma) {
     if (w.fmt != W_Q8_0 || n_tok < 16 || w.n_in % 32 || w.n_in <= 0 || w.n_out <= 0) return false;
     if ((reinterpret_cast<uintptr_t>(w.q) & 15) || (reinterpret_cast<uintptr_t>(act_quants) & 15)) return false;
     const int tiles = (n_tok + 15) / 16;
@@ -146,8 +149,12 @@ bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, 
     const int8_t* wq = (const int8_t*)w.q;
     const uint16_t* ws = (const uint16_t*)w.scales;
 #define IT_GEMM(NT)                                                                                                  \
-    hipLaunchKernelGGL((q8_gemm_k<NT>), dim3(gx, (tiles + NT - 1) / NT), dim3(GT), 0, s, wq, ws, act_quants, act_scales, \
-                       out, w.n_in, w.n_out, n_tok, out_scale)
+    do {                                                                                                             \
+        if (fma) hipLaunchKernelGGL((q8_gemm_k<NT, true>), dim3(gx, (tiles + NT - 1) / NT), dim3(GT), 0, s, wq, ws, act_quants, act_scales, \
+                                    out, w.n_in, w.n_out, n_tok, out_scale);                                        \
+        else hipLaunchKernelGGL((q8_gemm_k<NT, false>), dim3(gx, (tiles + NT - 1) / NT), dim3(GT), 0, s, wq, ws, act_quants, act_scales, \
+                                out, w.n_in, w.n_out, n_tok, out_scale);                                            \
+    } while (0)
     // 64 tokens per block at most: four blocks fit a CU (38 KB of LDS, 98 VGPRs) and hide each other's LDS and
     // barrier waits; 128 tokens per block (two blocks per CU) measured 20 % slower despite reading the weights half as often
     // ... unless that leaves fewer than two blocks per CU (a short batch, few rows): then narrower blocks, which re-read

@@ -43,8 +43,9 @@ void matmul(const WView& w, const float* x, const float* act_scales, const int8_
 
 // The same product for 16 or more tokens on the int8 matrix cores (Q8_0 weights only): bit-identical
 // to `matmul`.  Returns false without launching when the shape or format is not handled.
+// fma: the scaled block sum is added with one rounding instead of two (fast mode only: not the CPU path's bits)
 bool q8_gemm(const WView& w, const float* act_scales, const int8_t* act_quants, int n_tok, float* out, float out_scale,
-             hipStream_t s);
+             hipStream_t s, bool fma = false);
 
 struct ExpertsView {
     const void* q;       // expert e at q + e*q_stride

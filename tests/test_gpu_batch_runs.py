@@ -103,6 +103,6 @@ def test_gated_norm_silu_and_quantized_product(hip, orc, n, with_matmul):
     if with_matmul:
         # The product, against the oracle's product of the SAME z (the backend's): Q8_0 rounding is a step function, so a
         # z that differs in its last bits moves a few quants by one and the sums with them; given equal inputs the
-        # quantization and the integer dots are the oracle's, bit for bit.
+        # quantization and the integer dots are the oracle's, and only the f32 additions round differently.
         orc.matmul(ob.weights(wo, ih.Q8_0, VD, 256), B[0]["z"], B[1]["out"])
-        assert np.array_equal(B[0]["out"].view(np.uint32), B[1]["out"].view(np.uint32)), worst(B[0]["out"], B[1]["out"])
+        assert close(B[0]["out"], B[1]["out"], 1e-5), worst(B[0]["out"], B[1]["out"])
