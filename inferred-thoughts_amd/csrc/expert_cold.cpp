@@ -27,7 +27,6 @@
 #include <deque>
 #include <mutex>
 #include <thread>
-#include <unordered_set>
 
 #include "backend.h"
 
@@ -168,9 +167,22 @@ struct it_hip::ColdTier {
     uint64_t hand = 0;
     bool ring_valid = false;
     uint64_t q_stride = 0, s_stride = 0;
-    // the current lease: (tensor, expert) entries of the routing decision being computed, as counter indices
-    std::unordered_set<uint64_t> lease;
+    // the current lease: the (tensor, expert) entries of the routing decision being computed; `leased` flags the ring
+    // slots they hold and is kept in step entry by entry (a sweep over the ring per resolve would cost more than the
+    // fetches of a large pool)
+    std::vector<std::pair<Resident*, uint32_t>> lease;
     std::vector<uint32_t> lease_picks;
+    void lease_add(Resident* r, uint32_t e) {
+        lease.emplace_back(r, e);
+        if (ring_valid && r->slot_at.size() > e && r->slot_at[e] >= 0) leased[(size_t)r->slot_at[e]] = 1;
+    }
+    void lease_clear() {
+        if (ring_valid)
+            for (auto& le : lease)
+                if (le.first->slot_at.size() > le.second && le.first->slot_at[le.second] >= 0) leased[(size_t)le.first->slot_at[le.second]] = 0;
+        lease.clear();
+        lease_picks.clear();
+    }
     // the picks of a device route, read back once per decision
     std::vector<int32_t> picks;
     uint64_t picks_gen = ~0ull;
@@ -214,8 +226,7 @@ void it_hip::cold_ring_changed() {
 
 void it_hip::cold_clear_lease() {
     if (!cold) return;
-    cold->lease.clear();
-    cold->lease_picks.clear();
+    cold->lease_clear();
 }
 
 void it_hip::cold_drop() {
@@ -349,7 +360,7 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
 
     // ---- 2. a new routing decision ends the lease of the last one (moe.rs:847-853)
     if (uniq != c.lease_picks) {
-        c.lease.clear();
+        c.lease_clear();
         c.lease_picks = uniq;
     }
 
@@ -389,8 +400,12 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
                 }
         }
         c.heat.assign(c.ring.size(), 0);
+        c.leased.assign(c.ring.size(), 0);
         c.hand = 0;
         c.ring_valid = true;
+        auto held_lease = std::move(c.lease);   // the flags of a lease taken before the ring was (re)built
+        c.lease.clear();
+        for (auto& le : held_lease) c.lease_add(le.first, le.second);
     }
     if (c.ring.empty()) {
         fail("expert pool: cold experts were picked but the device tier has no slot to fetch them into");
@@ -404,7 +419,7 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
         if (it == weights.end() || it->second.counter_base < 0 || it->second.n_expert != n_expert || !it->second.q_tab) continue;
         Resident* r = &it->second;
         for (uint32_t e : uniq) {
-            c.lease.insert((uint64_t)r->counter_base + e);
+            c.lease_add(r, e);
             if (r->h_tier[e] == 2) want.push_back({r, t, e});
             else if (r->h_tier[e] == 0 && r->slot_at[e] >= 0) {
                 uint8_t& h = c.heat[(size_t)r->slot_at[e]];
@@ -415,9 +430,6 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
     if (want.empty() && c.hint_ids.empty()) return true;
     // slots change hands on the stream: everything recorded so far must be ahead of that
     need_eager("cold experts are fetched");
-    c.leased.assign(c.ring.size(), 0);
-    for (size_t i = 0; i < c.ring.size(); i++)
-        if (c.ring[i].owner && c.lease.count((uint64_t)c.ring[i].owner->counter_base + c.ring[i].e)) c.leased[i] = 1;
 
     // ---- 6. staging
     const uint64_t raw_one = expert_slot_bytes;
