@@ -146,6 +146,19 @@ class ReadPool {
     std::string path_;
 };
 
+// it_hip_clock_pick's walk (experts.rs:2215-2233) without its scan for an unleased slot before the walk: heat is at
+// most HEAT_MAX, so a ring with an unleased slot yields it within HEAT_MAX + 1 sweeps, and one sweep more finds none.
+int64_t clock_walk(uint8_t* heat, const uint8_t* leased, uint64_t n, uint64_t* hand) {
+    for (uint64_t step = 0; step < (uint64_t)(HEAT_MAX + 2) * n; step++) {
+        const uint64_t i = *hand % n;
+        *hand = (i + 1) % n;
+        if (leased[i]) continue;
+        if (heat[i] == 0) return (int64_t)i;
+        heat[i]--;
+    }
+    return -1;
+}
+
 int fetch_threads() {
     const char* e = getenv("INFERRED_FETCH_THREADS");   // the reference's switch (experts.rs:556-560)
     int n = e ? atoi(e) : 8;
@@ -470,7 +483,7 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
 
     // one expert's bytes (in staging on the device at `src`) into a slot taken from an unleased expert
     auto place = [&](const Want& w, const uint8_t* dev_raw) -> bool {
-        const int64_t at = it_hip_clock_pick(c.heat.data(), c.leased.data(), c.ring.size(), &c.hand);
+        const int64_t at = clock_walk(c.heat.data(), c.leased.data(), c.ring.size(), &c.hand);
         if (at < 0) {
             fail("expert pool: every one of the " + std::to_string(c.ring.size()) +
                  " device slots holds an expert the layer being resolved picked; the device tier is smaller than one layer's picks");
