@@ -101,6 +101,7 @@ enum {
     IT_HIP_EXACT = 1,    /* every reduction in the CPU path's order (bit-identical results) */
     IT_HIP_NO_GRAPH = 2, /* never capture decode passes into a HIP graph */
     IT_HIP_NO_FUSE = 4,  /* capture decode passes op by op, without the fused kernels */
+    IT_HIP_NO_CHAIN = 8, /* keep every fused decode stage a launch of its own (no persistent kernel over runs of layers) */
 };
 
 /* Cuda::new, src/ops/cuda/mod.rs:757-935.  NULL on failure with a message in err. */
@@ -296,6 +297,10 @@ void it_hip_drop_mirrors(it_hip*);
 uint64_t it_hip_launch_count(it_hip*);
 /* decode graphs: captures, replays, fallbacks to eager, kernel launches in the captured graph */
 void it_hip_graph_stats(it_hip*, uint64_t out[4]);
+/* layer chains (runs of decode layers as one persistent kernel, fast mode; no counterpart in the reference, whose
+ * graph keeps one node per kernel: src/ops/cuda/mod.rs:600-647): chain launches in the last fused pass, layers they
+ * cover, 1 while chains are enabled for this backend, the bound on a hand-off wait in polls */
+void it_hip_chain_stats(it_hip*, uint64_t out[4]);
 /* The caller has zeroed the host copy of every recurrent-state slab (a sequence reset): the device copies are
  * zeroed in place, where forget_state (mod.rs:1360-1419) would upload the zeros again at their next use. */
 void it_hip_zero_state(it_hip*);

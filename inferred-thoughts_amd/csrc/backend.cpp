@@ -6,6 +6,8 @@
 // (/root/reference src/ops/cuda/ops/mod.rs:91-110).
 #include "backend.h"
 
+#include <mutex>
+
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -145,6 +147,8 @@ void it_hip::finish_pass() {
         for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
         precopies.clear();
         hipGraph_t g = nullptr;
+        // a chain's hand-off space is allocated and cleared here: neither is allowed while the stream is capturing
+        if (chain_enabled && fuse_enabled && !exact && (!itk::layer_chain_fits() || !chain_acquire())) chain_enabled = false;
         hipError_t e = hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed);
         if (e == hipSuccess) {
             run_fused(pending);
@@ -162,6 +166,8 @@ void it_hip::finish_pass() {
                 graph.exec = ex;
                 graph.signature = pass_signature;
                 graph.attn_slots = fused_attn_slots;
+                graph.elided = fused_elided;
+                graph.has_chain = chain_launches > 0;
                 graph.valid = true;
                 graph_captures++;
                 stable_passes = 1;
@@ -199,6 +205,8 @@ void it_hip::finish_pass() {
         check(hipGraphLaunch(graph.exec, stream), "hipGraphLaunch");
         graph_launches++;
     }
+    mark_elided(graph.elided);
+    if (graph.has_chain) chain_ran = true;
     pending.clear();
 }
 
@@ -268,8 +276,20 @@ float* it_hip::act_out(const float* host, size_t len) {
     Act* a = act_slot(host, len);
     if (!a) return nullptr;
     a->dev_current = true;
+    a->elided = false;
     a->q_valid = false;
     return a->dev;
+}
+it_hip::Act* it_hip::act_by_dev(const void* dev) {
+    for (auto& kv : acts) {
+        const char* base = (const char*)kv.second.dev;
+        if (base && (const char*)dev >= base && (const char*)dev < base + kv.second.cap * sizeof(float)) return &kv.second;
+    }
+    return nullptr;
+}
+void it_hip::mark_elided(const std::vector<const void*>& devs) {
+    for (const void* d : devs)
+        if (Act* a = act_by_dev(d)) a->elided = true;
 }
 float* it_hip::act_inout(const float* host, size_t len) {
     float* d = act_in(host, len);
@@ -1098,7 +1118,74 @@ it_hip::~it_hip() {
         if (dyn_evt[i]) (void)hipEventDestroy(dyn_evt[i]);
     }
     drop_graph();
+    chain_release();
     if (stream) (void)hipStreamDestroy(stream);
+}
+
+// ------------------------------------------------------------------ layer-chain resources
+namespace {
+std::mutex chain_pool_mu;
+std::vector<it_hip::ChainRes> chain_pool;   // handed back by backends that are gone; never freed
+}  // namespace
+
+bool it_hip::chain_acquire() {
+    if (chain.ll) return true;
+    {
+        std::lock_guard<std::mutex> g(chain_pool_mu);
+        for (size_t i = 0; i < chain_pool.size(); i++) {
+            if (chain_pool[i].device == device) {
+                chain = chain_pool[i];
+                chain_pool.erase(chain_pool.begin() + (long)i);
+                break;
+            }
+        }
+    }
+    if (!chain.ll) {
+        ChainRes r;
+        r.device = device;
+        if (hipExtMallocWithFlags((void**)&r.ll, itk::CHAIN_LL_WORDS * 8, hipDeviceMallocUncached) != hipSuccess ||
+            hipExtMallocWithFlags((void**)&r.abort_flag, 256, hipDeviceMallocUncached) != hipSuccess ||
+            hipMalloc((void**)&r.epoch, 256) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;   // (what was allocated stays allocated: a handful of kilobytes, once)
+        }
+        if (hipMemset(r.ll, 0, itk::CHAIN_LL_WORDS * 8) != hipSuccess || hipMemset(r.abort_flag, 0, 256) != hipSuccess ||
+            hipMemset(r.epoch, 0, 256) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        chain = r;
+    }
+    return true;
+}
+
+void it_hip::chain_release() {
+    if (!chain.ll) return;
+    if (stream) (void)hipStreamSynchronize(stream);
+    (void)hipMemset(chain.abort_flag, 0, 4);
+    std::lock_guard<std::mutex> g(chain_pool_mu);
+    chain_pool.push_back(chain);
+    chain = ChainRes{};
+}
+
+void it_hip::chain_check() {
+    if (!chain_ran || !chain.abort_flag) return;
+    chain_ran = false;
+    unsigned flag = 0;
+    if (hipMemcpy(&flag, chain.abort_flag, 4, hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (!flag) return;
+    // a wait inside a chain ran out of tries: what the pass computed is void.  The chains are switched off for this
+    // backend, the graph that holds them is dropped and the hand-off space starts from zero again.
+    chain_enabled = false;
+    drop_graph();
+    stable_passes = 0;
+    (void)hipMemset(chain.abort_flag, 0, 4);
+    (void)hipMemset(chain.ll, 0, itk::CHAIN_LL_WORDS * 8);
+    fail("layer chain: a hand-off wait inside the persistent decode kernel gave up (the grid was not resident at once, or a "
+         "block stalled); the pass's results are void and the chains are switched off for this backend");
 }
 
 // =================================================================== C ABI
@@ -1126,6 +1213,11 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->exact = (flags & IT_HIP_EXACT) != 0;
     be->allow_graph = (flags & IT_HIP_NO_GRAPH) == 0;
     be->fuse_enabled = (flags & IT_HIP_NO_FUSE) == 0 && getenv("INFERRED_HIP_NO_FUSE") == nullptr;
+    be->chain_enabled = (flags & IT_HIP_NO_CHAIN) == 0 && getenv("INFERRED_HIP_NO_CHAIN") == nullptr;
+    if (const char* sl = getenv("INFERRED_HIP_CHAIN_SPINS")) {
+        const long v = atol(sl);
+        if (v > 0 && v < (1l << 30)) be->chain_spin_limit = (int)v;
+    }
     if ((e = hipStreamCreate(&be->stream)) != hipSuccess) {
         delete be;
         return bad(std::string("hipStreamCreate: ") + hipGetErrorString(e));
@@ -1159,6 +1251,7 @@ int it_hip_take_error(it_hip* be, char* msg, size_t msg_len) {
         // surface asynchronous faults too
         hipError_t e = hipStreamSynchronize(be->stream);
         if (e != hipSuccess) be->fail(std::string("device: ") + hipGetErrorString(e));
+        else be->chain_check();
     }
     if (!be->has_error) return 0;
     if (msg && msg_len) snprintf(msg, msg_len, "%s", be->error.c_str());
@@ -1940,6 +2033,10 @@ void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
     auto it = be->acts.find(buf);
     if (it == be->acts.end() || !it->second.dev_current) return;
     if (!be->held.empty()) be->release_held();
+    if (it->second.elided) {
+        be->fail("host_needs: the op that writes this buffer was folded into a fused kernel that does not write it");
+        return;
+    }
     if (be->in_pass) {
         // a read inside a pass cannot be served from a graph that has not run yet:
         // graphs are latched off for this backend (src/ops/cuda/ops/mod.rs:565-582)
@@ -1949,6 +2046,7 @@ void it_hip_host_needs(it_hip* be, float* buf, uint64_t len) {
     size_t n = len < it->second.cap ? len : it->second.cap;
     if (!be->check(hipMemcpyAsync(buf, it->second.dev, n * sizeof(float), hipMemcpyDeviceToHost, be->stream), "download activation")) return;
     be->check(hipStreamSynchronize(be->stream), "download activation");
+    be->chain_check();
     be->d2h++;
     be->d2h_bytes += n * 4;
 }
@@ -1984,6 +2082,7 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
     }
     for (auto& kv : be->acts) {
         kv.second.dev_current = false;
+        kv.second.elided = false;
         kv.second.q_valid = false;
     }
 }
@@ -2279,6 +2378,7 @@ void it_hip_read_tokens(it_hip* be, uint64_t first_index, uint64_t n, uint32_t* 
         return;
     }
     be->check(hipStreamSynchronize(be->stream), "sync before reading token ids");
+    be->chain_check();
     for (uint64_t i = 0; i < n;) {
         const uint64_t at = (first_index + i) % it_hip::TOK_RING_CAP;
         const uint64_t take = std::min<uint64_t>(n - i, it_hip::TOK_RING_CAP - at);
@@ -2324,6 +2424,13 @@ void it_hip_graph_stats(it_hip* be, uint64_t out[4]) {
     out[3] = be->fused_launches;
 }
 
+void it_hip_chain_stats(it_hip* be, uint64_t out[4]) {
+    out[0] = be->chain_launches;   // persistent-kernel launches in the last fused pass
+    out[1] = be->chain_layers;     // layers they cover
+    out[2] = be->chain_enabled ? 1 : 0;
+    out[3] = (uint64_t)be->chain_spin_limit;
+}
+
 void it_hip_profile_begin(it_hip* be) {
     be->need_eager("profiling");
     be->check(hipStreamSynchronize(be->stream), "sync");
@@ -2337,7 +2444,8 @@ int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
                                                    "matmul_experts (expert down)", "delta_rule", "attend",
                                                    "norms", "router (softmax + top-k)", "other",
                                                    "fused_gemv (norm + quantize + dense GEMVs)", "lm_head (norm + GEMV)",
-                                                   "gdn_rows (l2 norm + delta rule)", "attn_prep (norm + rope + kv write)"};
+                                                   "gdn_rows (l2 norm + delta rule)", "attn_prep (norm + rope + kv write)",
+                                                   "layer_chain (persistent kernel over a run of layers)"};
     be->prof_on = false;
     be->check(hipStreamSynchronize(be->stream), "sync");
     it_profile_row acc[it_hip::FAM_COUNT];
@@ -2362,6 +2470,7 @@ int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
 void it_hip_sync(it_hip* be) {
     if (!be->held.empty()) be->release_held();
     be->check(hipStreamSynchronize(be->stream), "sync");
+    be->chain_check();
 }
 void it_hip_drop_mirrors(it_hip* be) { be->drop_all(); }
 uint64_t it_hip_launch_count(it_hip* be) { return be->launches; }

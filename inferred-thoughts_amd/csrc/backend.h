@@ -64,6 +64,7 @@ struct it_hip {
         float* dev = nullptr;
         size_t cap = 0;  // floats
         bool dev_current = false;
+        bool elided = false;   // the op that writes this buffer was folded into a kernel that does not: the device copy is not its value
         // cached Q8_0 form of the first q_len floats
         float* q_scales = nullptr;
         int8_t* q_quants = nullptr;
@@ -79,6 +80,10 @@ struct it_hip {
     bool act_quantized(const float* host, size_t len, const float** scales, const int8_t** quants,
                        float** dev_x);
     bool act_q_reserve(Act& a, size_t len);  // room for the Q8_0 form of `len` floats
+    Act* act_by_dev(const void* dev);        // the mirror whose device buffer holds `dev`, or null
+    // marks the mirrors at these device addresses as not holding their ops' values (a fused kernel skipped the writes):
+    // a host read of one raises the sticky error instead of returning what the buffer happens to hold
+    void mark_elided(const std::vector<const void*>& devs);
 
     // ---- constants (f32 vectors uploaded once: norm weights, conv taps, ssm_a, dt_bias)
     struct Const {
@@ -211,6 +216,8 @@ struct it_hip {
         // takes ONE position for all four, so a replay is only valid while write row == rope position and the
         // context length == position + 1 (the seam does not tie them together; the model loop does)
         std::vector<std::array<int, 4>> attn_slots;
+        std::vector<const void*> elided;   // device buffers whose ops the graph's fused kernels skip
+        bool has_chain = false;
     };
     Graph graph;
     // Deferred: a single-token pass whose ops are recorded like a captured pass's and issued as fused launches whenever
@@ -240,6 +247,24 @@ struct it_hip {
     uint64_t fused_launches = 0;  // launches in the captured graph after fusion
     void run_fused(std::vector<OpRec>& ops);
     std::vector<std::array<int, 4>> fused_attn_slots;  // filled by run_fused for the pass being captured
+    // ---- layer chains (k_chain.hip): runs of decode layers as one persistent kernel each
+    // hand-off words in uncached device memory, the epoch counter and the abort word; taken from a per-process pool
+    // at the first chain and handed back when the backend goes (uncached memory is never freed once a kernel read it)
+    struct ChainRes {
+        unsigned long long* ll = nullptr;
+        unsigned* epoch = nullptr;
+        unsigned* abort_flag = nullptr;
+        int device = -1;
+    };
+    ChainRes chain;
+    bool chain_enabled = true;
+    bool chain_ran = false;            // a chain has been issued since the abort word was last looked at
+    int chain_spin_limit = 1 << 21;
+    uint64_t chain_launches = 0, chain_layers = 0;   // per fused pass, for the statistics
+    bool chain_acquire();
+    void chain_release();
+    void chain_check();                // after a stream synchronisation: raises the sticky error if a chain gave up
+    std::vector<const void*> fused_elided;   // device buffers the pass being fused no longer writes (filled by run_fused)
     bool attn_positions_agree(const std::vector<std::array<int, 4>>& slots) const;
     struct PreCopy {
         void* dev;
@@ -316,7 +341,7 @@ struct it_hip {
 
     // ---- per-kernel-family timing with HIP events on the launch stream
     enum Family { FAM_MATMUL = 0, FAM_MOE_GLU, FAM_MOE_DOWN, FAM_DELTA, FAM_ATTEND, FAM_NORM, FAM_ROUTER, FAM_OTHER,
-                  FAM_FUSED_GEMV, FAM_LM_HEAD, FAM_GDN_ROWS, FAM_ATTN_PREP, FAM_COUNT };
+                  FAM_FUSED_GEMV, FAM_LM_HEAD, FAM_GDN_ROWS, FAM_ATTN_PREP, FAM_CHAIN, FAM_COUNT };
     struct ProfSpan {
         hipEvent_t a, b;
         int fam;

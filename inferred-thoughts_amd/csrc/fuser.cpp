@@ -19,15 +19,30 @@ struct Plan {
     it_hip* be;
     std::vector<Op>& ops;
     std::vector<char> consumed;
+    // which stage of a layer a fused launch is (0: none of them), with its arguments: the chain pass below rebuilds
+    // runs of them as one persistent kernel
+    enum Stage { ST_NONE = 0, ST_GDN_IN, ST_GDN_CORE, ST_GDN_OUT, ST_ROUTER, ST_GLU, ST_DOWN };
     struct Launch {
         int fam;         // it_hip::Family, for the per-kernel timing
         uint64_t bytes;  // algorithmic bytes of the launch (weights + state it must move once)
         std::function<void(hipStream_t)> fn;
+        int stage = ST_NONE;
+        FusedGemvP gv{};
+        GdnCoreP gc{};
+        MoeGluP mg{};
+        MoeDownP md{};
     };
     std::vector<std::vector<Launch>> at;  // fused launches keyed by position
-    void add(size_t i, int fam, uint64_t bytes, std::function<void(hipStream_t)> fn) {
+    Launch& add(size_t i, int fam, uint64_t bytes, std::function<void(hipStream_t)> fn) {
         at[i].push_back(Launch{fam, bytes, std::move(fn)});
+        return at[i].back();
     }
+    // buffers a block's chain form leaves unwritten, keyed by the block's position
+    struct Skips {
+        size_t pos;
+        std::vector<const void*> bufs;
+    };
+    std::vector<Skips> gdn_skips, ffn_skips;
     Plan(it_hip* b, std::vector<Op>& o) : be(b), ops(o), consumed(o.size(), 0), at(o.size()) {}
     // slot of a position scalar in the pass's device array, -1 when the pointer is not one
     int dyn_index(const void* p) const {
@@ -165,9 +180,23 @@ bool match_gdn(Plan& pl, size_t i, int exact) {
     b.m[0] = mat_of(mo, 2, (float*)rms.p[0]);
 
     pl.take(i, 18);
-    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a) + (uint64_t)cdim * 8 * 4, [=](hipStream_t s) { fused_gemv(a, s); });
-    pl.add(i, it_hip::FAM_GDN_ROWS, (uint64_t)nv * dv * dk * 8 + (uint64_t)(cdim + vdim) * 4, [=](hipStream_t s) { gdn_core(c, dki, s); });
-    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b) + (uint64_t)vdim * 4, [=](hipStream_t s) { fused_gemv(b, s); });
+    {
+        auto& la = pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a) + (uint64_t)cdim * 8 * 4, [=](hipStream_t s) { fused_gemv(a, s); });
+        la.stage = Plan::ST_GDN_IN;
+        la.gv = a;
+    }
+    {
+        auto& lc = pl.add(i, it_hip::FAM_GDN_ROWS, (uint64_t)nv * dv * dk * 8 + (uint64_t)(cdim + vdim) * 4, [=](hipStream_t s) { gdn_core(c, dki, s); });
+        lc.stage = dki == 128 ? Plan::ST_GDN_CORE : Plan::ST_NONE;
+        lc.gc = c;
+    }
+    {
+        auto& lb = pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b) + (uint64_t)vdim * 4, [=](hipStream_t s) { fused_gemv(b, s); });
+        lb.stage = Plan::ST_GDN_OUT;
+        lb.gv = b;
+    }
+    // what the chain form of this block does not write: the normed input, the conv output, silu(z), alpha, beta, the read-out
+    pl.gdn_skips.push_back({i, {normed, cv, z, ma.p[5], mb.p[5], dl.p[8]}});
     return true;
 }
 
@@ -545,10 +574,180 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
                            (uint64_t)(nu * ff + sff) * 4;
     const uint64_t down_b = rows_bytes(d.fmt, (uint64_t)nu * nd, ff) + rows_bytes(d.sh_fmt, nd, sff) +
                             (uint64_t)(nu * ff + sff) * 4 + (uint64_t)nd * 8;
-    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
-    pl.add(i, it_hip::FAM_MOE_GLU, glu_b, [=](hipStream_t s) { moe_glu_fused(g, s); });
-    pl.add(i, it_hip::FAM_MOE_DOWN, down_b, [=](hipStream_t s) { moe_down_fused(d, s); });
+    {
+        auto& la = pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
+        la.stage = Plan::ST_ROUTER;
+        la.gv = a;
+    }
+    {
+        auto& lg = pl.add(i, it_hip::FAM_MOE_GLU, glu_b, [=](hipStream_t s) { moe_glu_fused(g, s); });
+        lg.stage = Plan::ST_GLU;
+        lg.mg = g;
+    }
+    {
+        auto& ld = pl.add(i, it_hip::FAM_MOE_DOWN, down_b, [=](hipStream_t s) { moe_down_fused(d, s); });
+        ld.stage = Plan::ST_DOWN;
+        ld.md = d;
+    }
+    // what the chain form does not write: the normed input and its copy, the logits, the intermediates
+    pl.ffn_skips.push_back({i, {rms.p[2], x, router, ml.p[5], g_all, e_gate}});
     return true;
+}
+
+
+// ---------------------------------------------------------------------------------- layer chains
+// Runs of fused layer stages become one persistent kernel each (k_chain.hip): a Gated DeltaNet block's three launches
+// followed by its routed FFN's three are one layer of a chain; an FFN whose mixer is not a Gated DeltaNet block (an
+// attention layer's) may open a chain.  A run ends at anything else: an unfused op, another fused launch, a layer of
+// another shape, the chain's capacity.
+bool q8(const FusedMat& m, int n_out, int epi) { return m.fmt == W_Q8_0 && m.n_out == n_out && m.epi == epi; }
+bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+bool chain_mixer(const FusedGemvP& a, const GdnCoreP& c, const FusedGemvP& b, ChainMixer* m) {
+    if (a.exact || a.n_in != 2048 || a.mode != 1 || a.n_mats != 4 || a.route_counter) return false;
+    if (!q8(a.m[0], 8192, 1) || !q8(a.m[1], 4096, 3) || !q8(a.m[2], 32, 0) || !q8(a.m[3], 32, 0)) return false;
+    if (c.n_k_heads != 16 || c.n_v_heads != 32 || c.exact) return false;
+    if (b.n_in != 4096 || b.mode != 3 || b.head_dim != 128 || b.n_mats != 1 || !q8(b.m[0], 2048, 2) || b.m[0].out != a.x) return false;
+    if (c.conv != a.m[0].out || c.alpha != a.m[2].out || c.beta != a.m[3].out || b.gate != a.m[1].out || b.x != c.core) return false;
+    for (int i = 0; i < 4; i++)
+        if (!al16(a.m[i].q) || !al16(a.m[i].s)) return false;
+    if (!al16(b.m[0].q) || !al16(b.m[0].s) || !al16(a.norm_w) || !al16(a.conv_w) || !al16(c.state) || !al16(a.x)) return false;
+    m->norm_w = a.norm_w;
+    m->qkv_q = a.m[0].q; m->qkv_s = a.m[0].s;
+    m->z_q = a.m[1].q; m->z_s = a.m[1].s;
+    m->a_q = a.m[2].q; m->a_s = a.m[2].s;
+    m->b_q = a.m[3].q; m->b_s = a.m[3].s;
+    m->conv_state = a.conv_state;
+    m->conv_w = a.conv_w;
+    m->ssm_a = c.ssm_a;
+    m->dt_bias = c.dt_bias;
+    m->state = c.state;
+    m->head_norm_w = b.norm_w;
+    m->o_q = b.m[0].q; m->o_s = b.m[0].s;
+    m->eps_norm = a.eps;
+    m->eps_l2 = c.eps;
+    m->eps_head = b.eps;
+    m->q_scale = c.q_scale;
+    return true;
+}
+
+bool chain_ffn(const FusedGemvP& r, const MoeGluP& g, const MoeDownP& d, ChainFfn* f, int* sh_fmt) {
+    if (r.exact || r.n_in != 2048 || r.mode != 1 || r.n_mats != 2 || r.route_counter || !q8(r.m[0], 512, 0) || !q8(r.m[1], 1, 0)) return false;
+    if (g.exact || g.fmt != W_NVFP4 || g.n_in != 2048 || g.n_out != 512 || g.n_expert != 512 || g.n_used != 10 || g.sh_n_out != 512) return false;
+    if (g.sh_fmt != W_Q8_0 && g.sh_fmt != W_NVFP4) return false;
+    if (!g.logits || g.logits != r.m[0].out || !g.route_ids_out || !g.route_w_out || g.x != r.x_copy2) return false;
+    if (d.exact || d.fmt != W_NVFP4 || d.n_in != 512 || d.n_out != 2048 || d.n_used != 10 || d.sh_fmt != g.sh_fmt || d.sh_n_in != 512) return false;
+    if (d.g_all != g.out || d.g_shared != g.sh_out || d.logit != r.m[1].out || d.x != r.x || d.route_ids != g.route_ids_out || d.route_w != g.route_w_out)
+        return false;
+    const void* ptrs[] = {r.m[0].q, r.m[0].s, r.m[1].q, r.m[1].s, g.gq, g.gs, g.uq, g.us, g.sh_gq, g.sh_gs, g.sh_uq, g.sh_us, d.q, d.s, d.sh_q, d.sh_s, r.norm_w, r.x};
+    for (const void* p : ptrs)
+        if (!p || !al16(p)) return false;
+    if (g.q_stride % 16 || g.s_stride % 16 || d.q_stride % 16 || d.s_stride % 16) return false;
+    f->norm_w = r.norm_w;
+    f->r_q = r.m[0].q; f->r_s = r.m[0].s;
+    f->l_q = r.m[1].q; f->l_s = r.m[1].s;
+    f->sg_q = g.sh_gq; f->sg_s = g.sh_gs; f->su_q = g.sh_uq; f->su_s = g.sh_us;
+    f->sd_q = d.sh_q; f->sd_s = d.sh_s;
+    f->eg_q = g.gq; f->eg_s = g.gs; f->eu_q = g.uq; f->eu_s = g.us; f->ed_q = d.q; f->ed_s = d.s;
+    f->gscale2 = g.gscale2; f->uscale2 = g.uscale2; f->dscale2 = d.scale2;
+    f->gu_q_stride = g.q_stride; f->gu_s_stride = g.s_stride; f->d_q_stride = d.q_stride; f->d_s_stride = d.s_stride;
+    f->sh_gscale = g.sh_gscale; f->sh_uscale = g.sh_uscale; f->sh_dscale = d.sh_dscale;
+    f->eps = r.eps;
+    f->route_ids = g.route_ids_out;
+    f->route_w = g.route_w_out;
+    f->counts_gate = d.counts_gate; f->counts_up = d.counts_up; f->counts_down = d.counts_down;
+    *sh_fmt = g.sh_fmt;
+    return true;
+}
+
+void build_chains(Plan& pl, unsigned long long* tally) {
+    it_hip* be = pl.be;
+    be->chain_launches = be->chain_layers = 0;
+    if (!be->chain_enabled || be->exact || !layer_chain_fits()) return;
+    struct Unit {
+        size_t pos;
+        bool gdn;
+    };
+    ChainP cp{};
+    std::vector<Unit> units;          // the blocks folded into cp so far
+    bool mixer_open = false;          // the last layer of cp has its mixer and still waits for its FFN
+    uint64_t bytes = 0;
+    auto skips_of = [&](const std::vector<Plan::Skips>& v, size_t pos, std::vector<const void*>* out) {
+        for (auto& sk : v)
+            if (sk.pos == pos) out->insert(out->end(), sk.bufs.begin(), sk.bufs.end());
+    };
+    auto emit = [&]() {
+        int n = cp.n_layers;
+        size_t n_units = units.size();
+        if (mixer_open) {   // a mixer without its FFN stays three launches
+            n--;
+            n_units--;
+        }
+        if (n >= 1 && be->chain_acquire()) {
+            cp.n_layers = n;
+            cp.ll = be->chain.ll;
+            cp.epoch = be->chain.epoch;
+            cp.abort_flag = be->chain.abort_flag;
+            cp.tally = tally;
+            cp.spin_limit = be->chain_spin_limit;
+            const ChainP launch = cp;
+            for (size_t u = 0; u < n_units; u++) {
+                pl.at[units[u].pos].clear();
+                skips_of(units[u].gdn ? pl.gdn_skips : pl.ffn_skips, units[u].pos, &be->fused_elided);
+            }
+            pl.add(units[0].pos, it_hip::FAM_CHAIN, bytes, [=](hipStream_t s) {
+                if (!layer_chain(launch, s)) be->fail("layer chain: the persistent kernel could not be launched");
+            });
+            be->chain_launches++;
+            be->chain_layers += (uint64_t)n;
+        }
+        cp = ChainP{};
+        units.clear();
+        mixer_open = false;
+        bytes = 0;
+    };
+    for (size_t i = 0; i < pl.ops.size(); i++) {
+        auto& ls = pl.at[i];
+        const bool is_gdn = ls.size() == 3 && ls[0].stage == Plan::ST_GDN_IN && ls[1].stage == Plan::ST_GDN_CORE && ls[2].stage == Plan::ST_GDN_OUT;
+        const bool is_ffn = ls.size() == 3 && ls[0].stage == Plan::ST_ROUTER && ls[1].stage == Plan::ST_GLU && ls[2].stage == Plan::ST_DOWN;
+        bool taken = false;
+        if (is_gdn) {
+            if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            ChainMixer m{};
+            if (chain_mixer(ls[0].gv, ls[1].gc, ls[2].gv, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
+                cp.layer[cp.n_layers].has_mixer = 1;
+                cp.layer[cp.n_layers].m = m;
+                cp.x = const_cast<float*>(ls[0].gv.x);
+                cp.n_layers++;
+                mixer_open = true;
+                units.push_back({i, true});
+                bytes += ls[0].bytes + ls[1].bytes + ls[2].bytes;
+                taken = true;
+            }
+        } else if (is_ffn) {
+            ChainFfn f{};
+            int sh_fmt = 0;
+            if (!mixer_open && cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            const bool fits = chain_ffn(ls[0].gv, ls[1].mg, ls[2].md, &f, &sh_fmt) && (cp.n_layers == 0 || (cp.x == ls[0].gv.x && (cp.sh_fmt == sh_fmt || (cp.n_layers == 1 && mixer_open))));
+            if (fits) {
+                if (!mixer_open) {
+                    cp.layer[cp.n_layers].has_mixer = 0;
+                    cp.n_layers++;
+                }
+                cp.layer[cp.n_layers - 1].f = f;
+                cp.sh_fmt = sh_fmt;
+                cp.x = const_cast<float*>(ls[0].gv.x);
+                mixer_open = false;
+                units.push_back({i, false});
+                bytes += ls[0].bytes + ls[1].bytes + ls[2].bytes;
+                taken = true;
+            }
+        }
+        if (taken) continue;
+        // anything that runs here ends the run: other fused launches, or an op issued as it is
+        if (!ls.empty() || !pl.consumed[i]) emit();
+    }
+    emit();
 }
 
 bool references(const Op& op, const void* a, const void* b) {
@@ -632,6 +831,8 @@ void it_hip::finish_held() {
 void it_hip::run_fused(std::vector<OpRec>& ops) {
     Plan pl(this, ops);
     fused_attn_slots.clear();
+    fused_elided.clear();
+    chain_launches = chain_layers = 0;
     if (fuse_enabled) {
         for (size_t i = 0; i < ops.size(); i++) {
             if (pl.consumed[i]) continue;
@@ -661,6 +862,7 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
             }
         }
     }
+    if (fuse_enabled && mode != Mode::Deferred) build_chains(pl, expert_tally);
     uint64_t n = 0;
     for (size_t i = 0; i < ops.size(); i++) {
         for (auto& l : pl.at[i]) {

@@ -1,0 +1,639 @@
+// A run of decode layers as one persistent kernel (fast mode).
+//
+// The per-layer chain of a single-token pass is six launches, each needing the whole output vector of the one
+// before (/root/reference src/model/qwen35.rs:1232-1328 the Gated DeltaNet mixer, :1587-1700 the routed FFN), and
+// a dependent launch costs about as much as the few megabytes it streams.  Here the six become stages of one
+// kernel with one block on every compute unit.  A stage's weight rows are fixed per block and wave, so their
+// loads are issued a stage ahead and sit in registers when the stage's input arrives.  The input arrives as
+// 8-byte words {payload, epoch} that the producing blocks store to uncached device memory and the consuming
+// threads poll until the epoch is the current layer's: one trip through memory, no flag, no fence, nothing to
+// clear between uses (an epoch is never reused).  The reference meets the same problem by capturing its decode
+// sequence into one graph (src/ops/cuda/mod.rs:600-647); a graph of dependent kernels still pays every boundary.
+//
+// Stages of a layer (the arithmetic per element is the per-stage fast kernels', k_fast.hip / k_fused.hip):
+//   A  rms_norm + Q8_0 quantization of x; rows of wqkv (+ causal conv, silu), wz (+ silu), alpha, beta
+//   B  l2 norm of q, k; the delta rule on 16 state rows per block; the read-out times silu(z) and the head-norm
+//      weight, with the block's share of the head's sum of squares beside it
+//   C  head-norm scale, quantization, rows of ssm_out, residual
+//   D  rms_norm + quantization; router rows, the shared expert's gate logit, its gate / up rows
+//   E  softmax + top-10 of the logits in every block; 160 blocks take one 32-element block of one pick's gate / up
+//      rows each and publish it quantized; the loads of the down rows go out with them
+//   F  down rows of the ten picks and of the shared expert, combine, residual
+//
+// Every wait is bounded: a poll that runs out of tries sets the abort word, every other wait sees it and the
+// grid drains.  The grid must be resident at once (one block per compute unit), which the launcher checks.
+#include "it_fast.h"
+#include "kernels_fused.h"
+
+namespace itk {
+using namespace fastk;
+namespace {
+
+typedef unsigned long long u64;
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+constexpr int CT = 512, CW = CT / 64, NB = CHAIN_BLOCKS;
+constexpr int D = 2048, NK = 16, NV = 32, DK = 128, KDIM = NK * DK, VDIM = NV * DK, CDIM = 2 * KDIM + VDIM;
+constexpr int NE = 512, NU = 10, FF = 512;
+constexpr int EB = NU * FF / 32;   // blocks that take a 32-element block of a pick's intermediates in stage E
+static_assert(D == 4 * CT && VDIM == 8 * CT && NE == CT && D == 8 * NB && CDIM == 32 * NB && VDIM == 16 * NB && NV * 8 == NB,
+              "the stage geometry below is written for these shapes");
+
+// hand-off regions, in 8-byte words (every start is even: pairs of words are polled with 16-byte loads)
+constexpr int RX = 0;                      // D: the residual stream into a layer
+constexpr int RA = RX + D;                 // [q | k | v] after conv + silu, silu(z), alpha, beta
+constexpr int RA_Z = RA + CDIM, RA_AL = RA_Z + VDIM, RA_BE = RA_AL + NV;
+constexpr int RB = RA_BE + NV;             // VDIM gated read-outs, then NB partial sums of squares
+constexpr int RB_SS = RB + VDIM;
+constexpr int RC = RB_SS + NB;             // D: the residual stream after the mixer
+constexpr int RD = RC + D;                 // NE router logits, the shared expert's gate logit
+constexpr int RS = RD + NE + 2;            // FF shared-expert intermediates
+constexpr int RE = RS + FF;                // NU * FF / 4 packed Q8_0 quads of the routed intermediates, then their scales
+constexpr int RE_SC = RE + NU * FF / 4;
+constexpr int R_END = RE_SC + EB;
+static_assert(R_END <= (int)CHAIN_LL_WORDS, "hand-off space");
+static_assert(!(RA & 1) && !(RA_Z & 1) && !(RB & 1) && !(RB_SS & 1) && !(RC & 1) && !(RD & 1) && !(RS & 1) && !(RE & 1) && !(RE_SC & 1), "");
+
+struct Ctl {
+    unsigned* abort_flag;
+    int spin_limit;
+};
+
+IT_DEV void ll_put(u64* p, uint32_t bits, unsigned e) {
+    __hip_atomic_store(p, ((u64)e << 32) | (u64)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+IT_DEV void ll_putf(u64* p, float v, unsigned e) { ll_put(p, __float_as_uint(v), e); }
+
+// true when the wait must stop: the tries are used up (this thread raises the abort word) or another wait gave up
+IT_DEV bool ll_give_up(int& spins, const Ctl& c) {
+    if (++spins > c.spin_limit) {
+        *(volatile unsigned*)c.abort_flag = 1u;
+        return true;
+    }
+    return (spins & 63) == 0 && *(volatile unsigned*)c.abort_flag != 0u;
+}
+
+// Polls.  A load and its wait are ONE asm statement: the compiler does not know that the destination of an asm
+// load is not ready, so nothing may be schedulable between the two.
+IT_DEV bool ll_wait1(const u64* p, unsigned e, const Ctl& c, uint32_t* out) {
+    int spins = 0;
+    for (;;) {
+        v2u w;
+        asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(w) : "v"(p) : "memory");
+        if (w.y == e) {
+            *out = w.x;
+            return true;
+        }
+        if (ll_give_up(spins, c)) return false;
+    }
+}
+// K pairs of words at a[k] (16-byte aligned); out[2k], out[2k+1] = their payloads.  A pair that is complete is
+// latched; its load is simply repeated while the others are still awaited.
+template <int K>
+IT_DEV bool ll_wait_pairs(const u64* const (&a)[K], unsigned e, const Ctl& c, uint32_t (&out)[2 * K]) {
+    static_assert(K == 1 || K == 2 || K == 4, "");
+    int spins = 0;
+    unsigned done = 0;
+    for (;;) {
+        v4u w[K];
+        if constexpr (K == 4)
+            asm volatile("global_load_dwordx4 %0, %4, off sc0 sc1\n\tglobal_load_dwordx4 %1, %5, off sc0 sc1\n\t"
+                         "global_load_dwordx4 %2, %6, off sc0 sc1\n\tglobal_load_dwordx4 %3, %7, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]) : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]) : "memory");
+        else if constexpr (K == 2)
+            asm volatile("global_load_dwordx4 %0, %2, off sc0 sc1\n\tglobal_load_dwordx4 %1, %3, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+                         : "=&v"(w[0]), "=&v"(w[1]) : "v"(a[0]), "v"(a[1]) : "memory");
+        else
+            asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(w[0]) : "v"(a[0]) : "memory");
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            if (!(done & (1u << k)) && w[k].y == e && w[k].w == e) {
+                out[2 * k] = w[k].x;
+                out[2 * k + 1] = w[k].z;
+                done |= 1u << k;
+            }
+        }
+        if (done == (1u << K) - 1u) return true;
+        if (ll_give_up(spins, c)) return false;
+    }
+}
+
+// the four floats [4 * qi, 4 * qi + 4) of a region
+IT_DEV bool ll_wait_quad(const u64* region, int qi, unsigned e, const Ctl& c, float4* v) {
+    const u64* const a[2] = {region + 4 * qi, region + 4 * qi + 2};
+    uint32_t o[4];
+    if (!ll_wait_pairs<2>(a, e, c, o)) return false;
+    *v = make_float4(__uint_as_float(o[0]), __uint_as_float(o[1]), __uint_as_float(o[2]), __uint_as_float(o[3]));
+    return true;
+}
+
+// The chunks of lane `sub` of one weight row, as load_w of the per-stage kernels, with the lane's part of the address
+// an unsigned 32-bit offset from the row's (wave-uniform or per-lane) base: the loads then take their base from scalar
+// registers and one vector register of offset, instead of a 64-bit vector address each.
+template <int FMT, int CPL, int L>
+IT_DEV void load_row(WChunks<CPL>& t, const uint8_t* q, const uint8_t* s, int n_in, int64_t row, int sub, bool live) {
+    if (!live) {
+#pragma unroll
+        for (int k = 0; k < CPL; k++) {
+            t.w[k] = make_uint4(0, 0, 0, 0);
+            t.sc[k] = 0;
+        }
+        return;
+    }
+    const uint8_t* rp = q + row * (FMT == W_Q8_0 ? n_in : n_in >> 1);
+    const uint8_t* sp = s + row * (n_in >> 5) * 2;
+    const uint32_t sub16 = (uint32_t)sub * 16u;
+#pragma unroll
+    for (int k = 0; k < CPL; k++) {
+        typedef unsigned v4 __attribute__((ext_vector_type(4)));
+        const v4 nt = __builtin_nontemporal_load((const v4*)(rp + (sub16 + (uint32_t)(k * L * 16))));
+        t.w[k] = make_uint4(nt.x, nt.y, nt.z, nt.w);
+        const uint32_t c = (uint32_t)(k * L) + (uint32_t)sub;
+        t.sc[k] = *(const uint16_t*)(sp + (FMT == W_Q8_0 ? (c >> 1) * 2u : c * 2u));
+    }
+}
+
+// ---- stage weights held in registers
+// In-projection: a wave takes four wqkv rows, two wz rows and (wave 0 of the first 64 blocks) one alpha / beta row.
+// The epilogue of row k runs in lane k, which also holds the row's conv window and taps.
+struct AW {
+    WChunks<2> t[7];
+    float4 taps;
+    float past[3];
+};
+IT_DEV int a_row(int k, int b, int wave) {   // row k of the wave in its own matrix
+    return k < 4 ? b + NB * (wave + CW * k) : k < 6 ? b + NB * (wave + CW * (k - 4)) : b < NV ? b : b - NV;
+}
+IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.qkv_q, m.qkv_s, D, a_row(k, b, wave), lane, true);
+#pragma unroll
+    for (int k = 4; k < 6; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.z_q, m.z_s, D, a_row(k, b, wave), lane, true);
+    const bool extra = wave == 0 && b < 2 * NV;
+    load_row<W_Q8_0, 2, 64>(a.t[6], b < NV ? m.a_q : m.b_q, b < NV ? m.a_s : m.b_s, D, a_row(6, b, wave), lane, extra);
+    if (lane < 4) {
+        const int64_t row = b + NB * (wave + CW * lane);
+        a.taps = *(const float4*)(m.conv_w + row * 4);
+        a.past[0] = m.conv_state[row * 3];
+        a.past[1] = m.conv_state[row * 3 + 1];
+        a.past[2] = m.conv_state[row * 3 + 2];
+    }
+}
+
+// rms_norm (naive.rs:633-650) of the 2,048 floats the block's threads hold as quads, then Q8_0 (naive.rs:652-675)
+// into xq / xs.  Two barriers; returns false after the first when the block has to stop.
+IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
+    const double part = wave_sum_f64_tail(quad_sumsq(v));
+    if ((tid & 63) == 63) red[tid >> 6] = part;
+    __syncthreads();
+    if (*dead) return false;
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < CW; i++) sum += red[i];
+    const float mean = (float)(sum / (double)D);
+    const float scale = 1.0f / sqrtf(mean + eps);
+    v.x = v.x * scale * w.x;
+    v.y = v.y * scale * w.y;
+    v.z = v.z * scale * w.z;
+    v.w = v.w * scale * w.w;
+    quant_quad(v, true, tid, xq, xs);
+    __syncthreads();
+    return true;
+}
+
+template <int SF>
+__global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
+    __shared__ __align__(16) int8_t xq[NU * FF + FF];   // the stage's quantized activation (largest: the down stage's)
+    __shared__ __align__(16) float xs[(NU * FF + FF) / 32];
+    __shared__ double red[CW];
+    __shared__ __align__(16) float kq[2 * DK];
+    __shared__ __align__(16) float ssq[NB];
+    __shared__ float sm[64];
+    __shared__ __align__(16) float inter[32];
+    __shared__ RouteLds<CT> route_sh;
+    __shared__ int ids[16];
+    __shared__ __align__(16) float wts[16];
+    __shared__ float coef[16];
+    __shared__ int dead;
+    const int tid0 = threadIdx.x, b0 = blockIdx.x;
+    const Ctl ctl{p.abort_flag, p.spin_limit};
+    const unsigned e0 = *(const volatile unsigned*)p.epoch;
+    if (tid0 == 0) dead = 0;
+    // lane 63 of a wave owns one row of the residual stream: row 8 * block + wave
+    float x_row = (tid0 & 63) == 63 ? p.x[b0 * CW + (tid0 >> 6)] : 0.0f;
+    AW aw;
+    if (p.layer[0].has_mixer) fetch_a(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
+    __syncthreads();
+
+    for (int l = 0; l < p.n_layers; l++) {
+        // The thread's coordinates pass through an empty asm statement once per layer.  Everything addressed from them
+        // (hand-off words, weight rows, LDS slots) is then computed where it is used, a few integer operations, instead
+        // of being hoisted out of the layer loop as loop invariants and held in a hundred registers across it.
+        int tid = tid0, b = b0;
+        asm volatile("" : "+v"(tid), "+s"(b));
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int my_row = b * CW + wave;
+        const ChainLayer& L = p.layer[l];
+        const ChainMixer& m = L.m;
+        const ChainFfn& f = L.f;
+        const unsigned e = e0 + 1 + (unsigned)l;
+        const bool mixer = L.has_mixer != 0;
+
+        // Stage D's rows.  Waves 0, 1: router rows b and NB + b; waves 2, 3: gate and up rows 2 b and 2 b + 1 of the
+        // shared expert; wave 4 of the last block: the shared expert's gate-logit row.  Issued at the head of the stage
+        // before D (small loads issued at the head of a stage are back before its input is).
+        WChunks<2> d0, d1;
+        WChunks<1> n0, n1;
+        const int sh_row = 2 * b + (wave - 2);
+        auto fetch_d = [&]() {
+            const bool r = wave < 2, sh = wave == 2 || wave == 3, lg = wave == 4 && b == NB - 1;
+            if (SF == W_Q8_0) {
+                load_row<W_Q8_0, 2, 64>(d0, r ? f.r_q : sh ? f.sg_q : f.l_q, r ? f.r_s : sh ? f.sg_s : f.l_s, D,
+                                      r ? b + NB * wave : sh ? sh_row : 0, lane, r || sh || lg);
+                load_row<W_Q8_0, 2, 64>(d1, f.su_q, f.su_s, D, sh_row, lane, sh);
+            } else {
+                load_row<W_Q8_0, 2, 64>(d0, r ? f.r_q : f.l_q, r ? f.r_s : f.l_s, D, r ? b + NB * wave : 0, lane, r || lg);
+                load_row<W_NVFP4, 1, 64>(n0, f.sg_q, f.sg_s, D, sh_row, lane, sh);
+                load_row<W_NVFP4, 1, 64>(n1, f.su_q, f.su_s, D, sh_row, lane, sh);
+            }
+        };
+        if (!mixer) fetch_d();
+
+        if (mixer) {
+            // ---------------------------------------------------------------- loads known from the start of the layer
+            const int h = b >> 3, j0 = (b & 7) * 16, kh = h % NK;
+            float* S = m.state + ((int64_t)(h * DK + j0 + (tid >> 5)) * DK + (tid & 31) * 4);
+            const float4 st = *(const float4*)S;
+            const float4 nw = ((const float4*)m.norm_w)[tid];
+            const float ssm_a = m.ssm_a[h], dt_bias = m.dt_bias[h];
+            const float head_w = m.head_norm_w[j0 + (tid >> 5)];
+
+            // ---------------------------------------------------------------- A: in-projection
+            {
+                float4 v;
+                bool ok = true;
+                if (l == 0) v = ((const float4*)p.x)[tid];
+                else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
+                if (!ok) dead = 1;
+                if (!norm_quant(v, nw, m.eps_norm, xq, xs, red, &dead, tid)) break;
+                XChunks<W_Q8_0, 2> x;
+                load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
+                float acc[7];
+#pragma unroll
+                for (int k = 0; k < 7; k++) acc[k] = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
+                // row k's dot goes from lane 63 to lane k, which finishes the row
+                float mine = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 7; k++) {
+                    const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc[k]), 63));
+                    mine = lane == k ? v : mine;
+                }
+                if (lane < 4) {
+                    // causal conv (kernel 4) + silu on channel `row`, state [channel][3] oldest first
+                    const int64_t row = b + NB * (wave + CW * lane);
+                    float sum = 0.0f;
+                    sum += aw.past[0] * aw.taps.x;
+                    sum += aw.past[1] * aw.taps.y;
+                    sum += aw.past[2] * aw.taps.z;
+                    sum += mine * aw.taps.w;
+                    ll_putf(p.ll + RA + row, fx_silu(sum), e);
+                    float* past = m.conv_state + row * 3;
+                    past[0] = aw.past[1];
+                    past[1] = aw.past[2];
+                    past[2] = mine;
+                } else if (lane < 6) {
+                    ll_putf(p.ll + RA_Z + b + NB * (wave + CW * (lane - 4)), fx_silu(mine), e);
+                } else if (lane == 6 && wave == 0 && b < 2 * NV) {
+                    ll_putf(p.ll + RA_AL + b, mine, e);
+                }
+            }
+            // ---------------------------------------------------------------- B: delta rule
+            // (the out-projection's row goes out first: small loads issued at the head of a stage are back before its input is)
+            WChunks<4> wc;
+            load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+            {
+                uint32_t w0 = 0, w1 = 0;
+                bool ok = true;
+                if (tid < 2 * DK) {
+                    ok = ll_wait1(p.ll + (tid < DK ? RA + KDIM + kh * DK + tid : RA + kh * DK + (tid - DK)), e, ctl, &w0);
+                } else if (tid < 2 * DK + 16) {
+                    const int j = h * DK + j0 + (tid - 2 * DK);
+                    ok = ll_wait1(p.ll + RA + 2 * KDIM + j, e, ctl, &w0) && ll_wait1(p.ll + RA_Z + j, e, ctl, &w1);
+                    sm[tid - 2 * DK] = __uint_as_float(w0);
+                    sm[16 + tid - 2 * DK] = __uint_as_float(w1);
+                } else if (tid < 2 * DK + 18) {
+                    ok = ll_wait1(p.ll + (tid == 2 * DK + 16 ? RA_AL : RA_BE) + h, e, ctl, &w0);
+                    sm[32 + tid - (2 * DK + 16)] = __uint_as_float(w0);
+                }
+                if (!ok) dead = 1;
+                // l2 norm of k (threads 0..127) and q (128..255): each vector's sum of squares in its own two waves
+                const float kqv = tid < 2 * DK ? __uint_as_float(w0) : 0.0f;
+                const double part = wave_sum_f64_tail((double)(kqv * kqv));
+                if (lane == 63) red[wave] = part;
+                __syncthreads();
+                if (dead) break;
+                if (tid < 2 * DK) {
+                    const int w2 = tid < DK ? 0 : 2;
+                    const double sum = red[w2] + red[w2 + 1];
+                    kq[tid] = kqv * (1.0f / fmaxf(sqrtf((float)sum), m.eps_l2));
+                }
+                __syncthreads();
+                const float a = sm[32] + dt_bias;
+                const float softplus = a > 20.0f ? a : fx_logf(1.0f + fx_expf(a));
+                const float g = fx_expf(softplus * ssm_a);
+                const float beta = fx_sigmoid(sm[33]);
+                const int j = tid >> 5, seg = tid & 31;
+                const float4 kk = *(const float4*)(kq + seg * 4), qq = *(const float4*)(kq + DK + seg * 4);
+                float row[4] = {st.x, st.y, st.z, st.w};
+                const float kv[4] = {kk.x, kk.y, kk.z, kk.w}, qv[4] = {qq.x, qq.y, qq.z, qq.w};
+                float pred = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    row[i] *= g;
+                    pred += row[i] * kv[i];
+                }
+                pred = group_sum<32>(pred);
+                const float delta = beta * (sm[j] - pred);
+                float o = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    row[i] += kv[i] * delta;
+                    o += row[i] * (qv[i] * m.q_scale);
+                }
+                o = group_sum<32>(o);
+                *(float4*)S = make_float4(row[0], row[1], row[2], row[3]);
+                if (seg == 0) {
+                    // silu(z) * (o * hs * w) with the head's scale hs applied by the reader, which sums the squares
+                    ll_putf(p.ll + RB + h * DK + j0 + j, sm[16 + j] * (o * head_w), e);
+                    sm[40 + j] = o * o;
+                }
+                __syncthreads();
+                if (tid == 0) {
+                    float s = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) s += sm[40 + i];
+                    ll_putf(p.ll + RB_SS + b, s, e);
+                }
+            }
+            // ---------------------------------------------------------------- C: out-projection + residual
+            fetch_d();
+            {
+                const u64* const a4[4] = {p.ll + RB + 4 * tid, p.ll + RB + 4 * tid + 2, p.ll + RB + 4 * (tid + CT), p.ll + RB + 4 * (tid + CT) + 2};
+                uint32_t o[8];
+                bool ok = ll_wait_pairs<4>(a4, e, ctl, o);
+                if (tid < NB / 2) {
+                    const u64* const a1[1] = {p.ll + RB_SS + 2 * tid};
+                    uint32_t s2[2];
+                    ok = ok && ll_wait_pairs<1>(a1, e, ctl, s2);
+                    ssq[2 * tid] = __uint_as_float(s2[0]);
+                    ssq[2 * tid + 1] = __uint_as_float(s2[1]);
+                }
+                if (!ok) dead = 1;
+                __syncthreads();
+                if (dead) break;
+#pragma unroll
+                for (int k = 0; k < 2; k++) {
+                    const int qi = tid + k * CT, head = qi >> 5;
+                    const float4 s0 = *(const float4*)(ssq + head * 8), s1 = *(const float4*)(ssq + head * 8 + 4);
+                    const double sum = (double)s0.x + (double)s0.y + (double)s0.z + (double)s0.w + (double)s1.x + (double)s1.y +
+                                       (double)s1.z + (double)s1.w;
+                    const float hs = 1.0f / sqrtf((float)(sum / (double)DK) + m.eps_head);
+                    const float4 v = make_float4(__uint_as_float(o[4 * k]) * hs, __uint_as_float(o[4 * k + 1]) * hs,
+                                                 __uint_as_float(o[4 * k + 2]) * hs, __uint_as_float(o[4 * k + 3]) * hs);
+                    quant_quad(v, true, qi, xq, xs);
+                }
+                __syncthreads();
+                XChunks<W_Q8_0, 4> x;
+                load_x<W_Q8_0, 4, 64>(x, xq, xs, lane);
+                const float acc = reduce_lanes<64>(dot_chunks<W_Q8_0, 4>(wc, x));
+                if (lane == 63) {
+                    x_row += acc;
+                    ll_putf(p.ll + RC + my_row, x_row, e);
+                }
+            }
+        }
+
+        // -------------------------------------------------------------------- D: router, shared gate logit, shared gate / up
+        XChunks<W_NVFP4, 1> xn;
+        {
+            const float4 nw = ((const float4*)f.norm_w)[tid];
+            float4 v;
+            bool ok = true;
+            if (mixer) ok = ll_wait_quad(p.ll + RC, tid, e, ctl, &v);
+            else if (l == 0) v = ((const float4*)p.x)[tid];
+            else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
+            if (!ok) dead = 1;
+            if (!norm_quant(v, nw, f.eps, xq, xs, red, &dead, tid)) break;
+            XChunks<W_Q8_0, 2> x;
+            load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
+            load_x<W_NVFP4, 1, 64>(xn, xq, xs, lane);
+            if (wave < 2 || (wave == 4 && b == NB - 1)) {
+                const float a = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
+                if (lane == 63) ll_putf(p.ll + RD + (wave < 2 ? b + NB * wave : NE), a, e);
+            } else if (wave < 4) {
+                float ag, au;
+                if (SF == W_Q8_0) {
+                    ag = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
+                    au = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d1, x));
+                } else {
+                    ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(n0, xn));
+                    au = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(n1, xn));
+                }
+                if (lane == 63) {
+                    ag *= f.sh_gscale;
+                    au *= f.sh_uscale;
+                    ll_putf(p.ll + RS + sh_row, fx_silu(ag) * au, e);
+                }
+            }
+        }
+
+        // -------------------------------------------------------------------- E: route, routed gate / up
+        WChunks<1> fd[3];
+        WChunks<1> fsh;   // the shared expert's down row: lanes 32..63 (Q8_0) or 32..47 (NVFP4) beside the last two picks
+        {
+            float lg4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            uint32_t w0 = 0;
+            bool ok = ll_wait1(p.ll + RD + tid, e, ctl, &w0);
+            lg4[0] = __uint_as_float(w0);
+            if (tid == 0) {
+                ok = ok && ll_wait1(p.ll + RD + NE, e, ctl, &w0);
+                sm[34] = __uint_as_float(w0);
+            }
+            if (!ok) dead = 1;
+            __syncthreads();
+            if (dead) break;
+            const float denom = block_route<CT>(lg4, NE, NU, route_sh, ids, wts);
+            // the down rows of this wave's output row: four picks a step over 16 lanes each, the shared row beside the
+            // last two picks
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                const int y = s * 4 + (lane >> 4);
+                const bool routed = y < NU;
+                const int64_t ex = routed ? ids[y] : 0;
+                load_row<W_NVFP4, 1, 16>(fd[s], f.ed_q + ex * f.d_q_stride, f.ed_s + ex * f.d_s_stride, FF, my_row, lane & 15, routed);
+            }
+            if (SF == W_Q8_0) load_row<W_Q8_0, 1, 32>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 31, lane >= 32);
+            else load_row<W_NVFP4, 1, 16>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 15, lane >= 32 && lane < 48);
+            if (tid < NU) {
+                const int ex = ids[tid];
+                const float w = wts[tid] / denom;
+                coef[tid] = w * (f.dscale2 ? f.dscale2[ex] : 1.0f);
+                if (b == 0) {
+                    f.route_ids[tid] = ex;
+                    f.route_w[tid] = w;
+                    if (f.counts_gate) atomicAdd(f.counts_gate + ex, 1u);
+                    if (f.counts_up) atomicAdd(f.counts_up + ex, 1u);
+                    if (f.counts_down) atomicAdd(f.counts_down + ex, 1u);
+                }
+            }
+            if (b == 0 && tid == 0 && p.tally)
+                atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
+            if (b < EB) {
+                const int y = b >> 4, sb = b & 15;
+                const int64_t ex = ids[y];
+                const uint8_t *gq = f.eg_q + ex * f.gu_q_stride, *gs = f.eg_s + ex * f.gu_s_stride;
+                const uint8_t *uq = f.eu_q + ex * f.gu_q_stride, *us = f.eu_s + ex * f.gu_s_stride;
+                WChunks<1> tg[4], tu[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int j = sb * 32 + wave * 4 + i;
+                    load_row<W_NVFP4, 1, 64>(tg[i], gq, gs, D, j, lane, true);
+                    load_row<W_NVFP4, 1, 64>(tu[i], uq, us, D, j, lane, true);
+                }
+                const float scg = f.gscale2 ? f.gscale2[ex] : 1.0f, scu = f.uscale2 ? f.uscale2[ex] : 1.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    float ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tg[i], xn));
+                    float au = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tu[i], xn));
+                    if (lane == 63) {
+                        ag *= scg;
+                        au *= scu;
+                        inter[wave * 4 + i] = fx_silu(ag) * au;
+                    }
+                }
+                __syncthreads();
+                if (tid < 8) {
+                    // Q8_0 of the block's 32 intermediates (naive.rs:652-675), published as four quants a word
+                    const float4 v = *(const float4*)(inter + tid * 4);
+                    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+                    amax = group_max<8>(amax);
+                    const float d = amax / 127.0f;
+                    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+                    const float r[4] = {roundf(v.x * id), roundf(v.y * id), roundf(v.z * id), roundf(v.w * id)};
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float cl = fminf(fmaxf(r[i], -128.0f), 127.0f);
+                        const int q = (r[i] != r[i]) ? 0 : (int)cl;
+                        packed |= ((uint32_t)(q & 0xff)) << (8 * i);
+                    }
+                    ll_put(p.ll + RE + b * 8 + tid, packed, e);
+                    if (tid == 0) ll_putf(p.ll + RE_SC + b, it_f16_to_f32(it_f32_to_f16(d)), e);
+                }
+            }
+        }
+        // the next layer's in-projection rows start moving now: one stage ahead of their use
+        if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer) fetch_a(p.layer[l + 1].m, aw, b, wave, lane);
+
+        // -------------------------------------------------------------------- F: down, combine, residual
+        {
+            // 1,440 words of quantized routed intermediates (pairs tid and tid + 512), the shared ones as quads
+            const int pr1 = tid + CT;
+            const bool two = pr1 < (NU * FF / 4 + EB) / 2, sq = tid < FF / 4;
+            const u64* const a4[4] = {p.ll + RE + 2 * tid, two ? p.ll + RE + 2 * pr1 : p.ll + RE + 2 * tid,
+                                      sq ? p.ll + RS + 4 * tid : p.ll + RE + 2 * tid, sq ? p.ll + RS + 4 * tid + 2 : p.ll + RE + 2 * tid};
+            uint32_t o[8];
+            const bool ok = ll_wait_pairs<4>(a4, e, ctl, o);
+            uint32_t* dst = (uint32_t*)xq;
+            // word i < 1,280 is quad i of the routed quants; the rest are the 160 block scales
+            auto place = [&](int i, uint32_t v) {
+                if (i < NU * FF / 4) dst[i] = v;
+                else xs[i - NU * FF / 4] = __uint_as_float(v);
+            };
+            place(2 * tid, o[0]);
+            place(2 * tid + 1, o[1]);
+            if (two) {
+                place(2 * pr1, o[2]);
+                place(2 * pr1 + 1, o[3]);
+            }
+            if (tid < 2 * 64) {   // whole waves: the quantization's lane exchange needs its eight neighbours
+                const float4 v = make_float4(__uint_as_float(o[4]), __uint_as_float(o[5]), __uint_as_float(o[6]), __uint_as_float(o[7]));
+                quant_quad(v, true, tid, xq + NU * FF, xs + EB);
+            }
+            if (!ok) dead = 1;
+            __syncthreads();
+            if (dead) break;
+            float acc = 0.0f;
+            const int c = lane & 15;
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                const int y = s * 4 + (lane >> 4);
+                if (y < NU) {
+                    const uint4 xa = *(const uint4*)(xq + y * FF + c * 32), xb = *(const uint4*)(xq + y * FF + c * 32 + 16);
+                    float tA, tB;
+                    unit_nvfp4(fd[s].w[0], fd[s].sc[0], xa, xb, xs[y * (FF / 32) + c], &tA, &tB);
+                    float t = 0.0f;
+                    t += tA;
+                    t += tB;
+                    acc += coef[y] * t;
+                }
+            }
+            if (lane >= 32) {
+                const float gate = fx_sigmoid(sm[34]) * f.sh_dscale;
+                const WChunks<1>& ws = fsh;
+                if (SF == W_Q8_0) {
+                    const int c2 = lane - 32;
+                    const uint4 xa = *(const uint4*)(xq + NU * FF + c2 * 16);
+                    int s = 0;
+                    s = dot4(ws.w[0].x, xa.x, s);
+                    s = dot4(ws.w[0].y, xa.y, s);
+                    s = dot4(ws.w[0].z, xa.z, s);
+                    s = dot4(ws.w[0].w, xa.w, s);
+                    acc += gate * ((float)s * (it_f16_to_f32((uint16_t)ws.sc[0]) * xs[EB + (c2 >> 1)]));
+                } else if (lane < 48) {
+                    const uint4 xa = *(const uint4*)(xq + NU * FF + c * 32), xb = *(const uint4*)(xq + NU * FF + c * 32 + 16);
+                    float tA, tB;
+                    unit_nvfp4(ws.w[0], ws.sc[0], xa, xb, xs[EB + c], &tA, &tB);
+                    float t = 0.0f;
+                    t += tA;
+                    t += tB;
+                    acc += gate * t;
+                }
+            }
+            acc = reduce_lanes<64>(acc);
+            if (lane == 63) {
+                x_row += acc;
+                ll_putf(p.ll + RX + my_row, x_row, e + 1);
+                p.x[my_row] = x_row;
+            }
+        }
+    }
+    if (b0 == 0 && tid0 == 0) *p.epoch = e0 + 1u + (unsigned)p.n_layers;
+}
+
+}  // namespace
+
+bool layer_chain_fits() {
+    static const bool fits = [] {
+        int dev = 0, cus = 0, occ = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return false;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < NB) return false;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, layer_chain_k<W_Q8_0>, CT, 0) != hipSuccess || occ < 1) return false;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, layer_chain_k<W_NVFP4>, CT, 0) != hipSuccess || occ < 1) return false;
+        return true;
+    }();
+    return fits;
+}
+
+bool layer_chain(const ChainP& p, hipStream_t s) {
+    if (p.n_layers < 1 || p.n_layers > CHAIN_MAX_LAYERS || !p.ll || !p.epoch || !p.abort_flag || !p.x) return false;
+    if (p.sh_fmt != W_Q8_0 && p.sh_fmt != W_NVFP4) return false;
+    if (!layer_chain_fits()) return false;
+    if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL(layer_chain_k<W_Q8_0>, dim3(NB), dim3(CT), 0, s, p);
+    else hipLaunchKernelGGL(layer_chain_k<W_NVFP4>, dim3(NB), dim3(CT), 0, s, p);
+    return true;
+}
+
+}  // namespace itk

@@ -110,4 +110,60 @@ bool fused_gemv_fast(FusedGemvP p, hipStream_t s);
 bool moe_glu_fast(MoeGluP p, hipStream_t s);
 bool moe_down_fast(MoeDownP p, hipStream_t s);
 
+// ------------------------------------------------------------------ layer chain (k_chain.hip, fast mode)
+// A run of decode layers as ONE persistent kernel, one block per compute unit: the six dependent launches of a
+// Gated DeltaNet layer (in-projection + conv, delta rule, out-projection, router + shared expert gate/up, routed
+// gate/up, down + combine) become six stages inside the kernel.  Between stages every block publishes its outputs
+// as 8-byte {value, epoch} words in uncached device memory and picks up its inputs by polling for the epoch; the
+// weights of a stage are in the block's registers before its inputs arrive.
+// Shapes are fixed (hidden 2048; 16 key / 32 value heads of 128; 512 NVFP4 experts, top 10, 512 rows; a shared
+// expert of 512 rows in Q8_0 or NVFP4; Q8_0 dense matrices); anything else stays on the per-stage launches.
+struct ChainMixer {
+    const float* norm_w;
+    const uint8_t *qkv_q, *qkv_s, *z_q, *z_s, *a_q, *a_s, *b_q, *b_s;
+    float* conv_state;
+    const float* conv_w;
+    const float *ssm_a, *dt_bias;
+    float* state;
+    const float* head_norm_w;
+    const uint8_t *o_q, *o_s;
+    float eps_norm, eps_l2, eps_head, q_scale;
+};
+struct ChainFfn {
+    const float* norm_w;
+    const uint8_t *r_q, *r_s, *l_q, *l_s;       // router rows; the shared expert's gate-logit row
+    const uint8_t *sg_q, *sg_s, *su_q, *su_s;   // shared expert gate / up
+    const uint8_t *sd_q, *sd_s;                 // shared expert down
+    const uint8_t *eg_q, *eg_s, *eu_q, *eu_s, *ed_q, *ed_s;   // routed experts
+    const float *gscale2, *uscale2, *dscale2;
+    int64_t gu_q_stride, gu_s_stride, d_q_stride, d_s_stride;
+    float sh_gscale, sh_uscale, sh_dscale, eps;
+    int32_t* route_ids;     // seam outputs: this layer's picks and their weights
+    float* route_w;
+    uint32_t *counts_gate, *counts_up, *counts_down;   // expert read counters (optional)
+};
+struct ChainLayer {
+    int has_mixer;   // 0: the layer's mixer ran before the chain (an attention layer); the chain starts at its FFN
+    ChainMixer m;
+    ChainFfn f;
+};
+constexpr int CHAIN_MAX_LAYERS = 4;
+constexpr int CHAIN_BLOCKS = 256;
+constexpr size_t CHAIN_LL_WORDS = 24576;   // 8-byte words of hand-off space a chain uses
+struct ChainP {
+    ChainLayer layer[CHAIN_MAX_LAYERS];
+    int n_layers;
+    int sh_fmt;                  // the shared expert's format (W_Q8_0 or W_NVFP4)
+    float* x;                    // residual stream [2048], read at the start and current after every layer
+    unsigned long long* ll;      // CHAIN_LL_WORDS words of uncached device memory, zero before the first chain
+    unsigned* epoch;             // device word: the last epoch any chain has used (starts at 0)
+    unsigned* abort_flag;        // uncached device word: set when a bounded wait gave up (the results are then void)
+    unsigned long long* tally;   // expert read tally (optional)
+    int spin_limit;              // polls a wait may take before it gives up
+};
+// whether this device can hold the chain's grid (one block per compute unit, all resident at once)
+bool layer_chain_fits();
+// false: not launched
+bool layer_chain(const ChainP& p, hipStream_t s);
+
 }  // namespace itk

@@ -14,7 +14,7 @@ from pathlib import Path
 import numpy as np
 
 F32, F16, Q8_0, BF16, NVFP4 = 0, 1, 8, 30, 40
-EXACT, NO_GRAPH, NO_FUSE = 1, 2, 4
+EXACT, NO_GRAPH, NO_FUSE, NO_CHAIN = 1, 2, 4, 8
 
 _HERE = Path(__file__).resolve().parent
 # INFERRED_HIP_LIB names another build of the library (comparing two builds on one machine)
@@ -95,7 +95,7 @@ it_hip_kv_write it_hip_host_wrote it_hip_host_needs it_hip_begin_pass it_hip_end
 it_hip_read_state it_hip_read_kv it_hip_device_report it_hip_reserve_activations it_hip_tier_counters
 it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_budget
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
-it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_hip_zero_state it_hip_mfma_ceiling it_model_open
+it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_hip_chain_stats it_hip_zero_state it_hip_mfma_ceiling it_model_open
 it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_engine_restore it_engine_rewind it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
@@ -205,6 +205,7 @@ def lib() -> C.CDLL:
         "it_hip_drop_mirrors": (None, [vp]),
         "it_hip_launch_count": (u64, [vp]),
         "it_hip_graph_stats": (None, [vp, vp]),
+        "it_hip_chain_stats": (None, [vp, vp]),
         "it_model_open": (vp, [C.c_char_p, C.c_char_p, C.c_size_t]),
         "it_hip_mfma_ceiling": (C.c_int, [vp, C.c_int, C.c_int, vp]),
         "it_hip_zero_state": (None, [vp]),
@@ -279,10 +280,10 @@ def attend_noalloc(q_ptr: int, q_len: int, k_ptr: int, v_ptr: int, kv_len: int, 
 class Hip:
     """One backend instance: `Cuda::new` of the reference, for gfx950."""
 
-    def __init__(self, exact: bool = False, graph: bool = True, device: int = 0, fuse: bool = True):
+    def __init__(self, exact: bool = False, graph: bool = True, device: int = 0, fuse: bool = True, chain: bool = True):
         self.L = lib()
         err = C.create_string_buffer(512)
-        flags = (EXACT if exact else 0) | (0 if graph else NO_GRAPH) | (0 if fuse else NO_FUSE)
+        flags = (EXACT if exact else 0) | (0 if graph else NO_GRAPH) | (0 if fuse else NO_FUSE) | (0 if chain else NO_CHAIN)
         self.h = self.L.it_hip_create(flags, device, err, 512)
         if not self.h:
             raise HipError(err.value.decode())
@@ -451,6 +452,12 @@ class Hip:
         v = (c_u64 * 4)()
         self.L.it_hip_graph_stats(self.h, v)
         return {"captures": int(v[0]), "replays": int(v[1]), "aborts": int(v[2]), "graph_kernels": int(v[3])}
+
+    def chain_stats(self):
+        """Layer chains of the last fused pass: persistent-kernel launches, the layers they cover, enabled, wait bound."""
+        v = (c_u64 * 4)()
+        self.L.it_hip_chain_stats(self.h, v)
+        return {"chains": int(v[0]), "layers": int(v[1]), "enabled": bool(v[2]), "spin_limit": int(v[3])}
 
     MFMA_KINDS = {"int8_16x16x64": 0, "int8_16x16x32": 1, "f16_32x32x16": 2, "f16_16x16x32": 3, "f32_16x16x4": 4}
 

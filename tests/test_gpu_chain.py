@@ -1,0 +1,299 @@
+"""The layer chain (runs of decode layers as ONE persistent kernel, k_chain.hip) against the CPU oracle.
+
+Whole layers of a single-token pass are issued op by op through the C ABI exactly as the host loop issues them
+(/root/reference src/model/qwen35.rs:1232-1328 gated delta net, :1587-1700 routed FFN).  The backend runs the first
+two passes eagerly, captures the third into a HIP graph and replays it; at capture the fuser folds every run of
+(Gated DeltaNet block, routed FFN) layers, optionally opened by an FFN whose mixer is not one, into one persistent
+kernel.  Shapes are config 5's (hidden 2048; 16 key / 32 value heads of 128; 512 NVFP4 experts top-10 of 512 rows +
+a Q8_0 or NVFP4 shared expert).
+
+Compared per pass with the same op sequence composed from the oracle's ops on identical inputs:
+  * the layers' contribution to the residual stream, end to end: |error| <= 2e-3 * max(|value|, rms of the vector).
+    Between the blocks of a layer every activation is quantized to Q8_0, a step function: fast mode's last-bit
+    differences (sums in wave order, exp on the transcendental unit) move a step in roughly every other vector, and
+    one moved step shifts every output of the block by ~2e-4 of the vector's scale, in the oracle as in the kernel, so
+    the bound is against the vector's scale rather than each entry's own size (measured: 1e-6 of the scale when no
+    step moves, 1.4e-5 when one does; tests/test_gpu_fused_fast.py holds each block on its own to 1e-3 per entry
+    by splitting it at the quantization, which a chain cannot be: its intermediates never leave the kernel);
+  * every layer's recurrent state and conv window to 1e-3 per entry;
+  * the routed experts of every layer, exactly (read from the expert cache's device-side read counters);
+and with the per-stage fused kernels (the same arithmetic, six launches a layer) to the same bounds.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from test_gpu_fused_fast import Both, bufs, nvfp4_rows, ND, EPS
+from util import close, rng, worst
+
+pytestmark = pytest.mark.gpu
+
+NK, NV, DK = 16, 32, 128
+KDIM, VDIM = NK * DK, NV * DK
+CDIM = 2 * KDIM + VDIM
+NE, NU, FF, SFF = 512, 10, 512, 512
+PASSES = 5
+
+
+def near(got, want, tol=2e-3):
+    """|got - want| <= tol * max(|want_i|, rms(want)): a bound against the vector's scale."""
+    want = np.asarray(want, np.float64)
+    floor = float(np.sqrt((want ** 2).mean())) if want.size else 0.0
+    return bool(np.all(np.abs(np.asarray(got, np.float64) - want) <= tol * np.maximum(np.abs(want), floor)))
+
+
+def far(got, want):
+    """largest error as a multiple of the bound at tol = 1"""
+    want = np.asarray(want, np.float64)
+    floor = float(np.sqrt((want ** 2).mean())) if want.size else 0.0
+    return float((np.abs(np.asarray(got, np.float64) - want) / np.maximum(np.maximum(np.abs(want), floor), 1e-300)).max())
+
+
+class Layers:
+    """Weights of `n` layers over shared expert tensors (one set of 512 experts serves every layer: 0.9 GB)."""
+
+    def __init__(self, pair, n, shared, seed=7):
+        ih = pair.ih
+        r = rng(seed)
+        self.pair, self.n, self.shared = pair, n, shared
+        g_s = (0.5 + r.random(NE)).astype(np.float32) / 54.0
+        u_s = (0.5 + r.random(NE)).astype(np.float32) / 54.0
+        d_s = (0.5 + r.random(NE)).astype(np.float32) / 108.0
+        self.gate_raw = nvfp4_rows(r, NE * FF, ND)
+        self.gate = pair.e(self.gate_raw, ih.NVFP4, ND, FF, NE, g_s)
+        self.up = pair.e(nvfp4_rows(r, NE * FF, ND), ih.NVFP4, ND, FF, NE, u_s)
+        self.down = pair.e(nvfp4_rows(r, NE * ND, FF), ih.NVFP4, FF, ND, NE, d_s)
+        self.L = []
+        for _ in range(n):
+            d = {}
+            d["wqkv"], d["wz"] = pair.q8(r, CDIM, ND, 2.0), pair.q8(r, VDIM, ND, 2.0)
+            d["wa"], d["wb"], d["wo"] = pair.q8(r, NV, ND, 2.0), pair.q8(r, NV, ND, 2.0), pair.q8(r, ND, VDIM, 1.0)
+            d["norm"] = (0.5 + r.random(ND)).astype(np.float32)
+            d["ssm_norm"] = (0.5 + r.random(DK)).astype(np.float32)
+            d["conv_w"] = (r.standard_normal(CDIM * 4) * 0.5).astype(np.float32)
+            d["ssm_a"] = (-np.exp(r.standard_normal(NV) * 0.5)).astype(np.float32)
+            d["dt"] = (r.standard_normal(NV) * 0.5).astype(np.float32)
+            d["router"], d["sh_inp"] = pair.q8(r, NE, ND, 3.0), pair.q8(r, 1, ND, 1.0)
+            if shared == "q8_0":
+                d["sg"], d["su"], d["sd"] = pair.q8(r, SFF, ND, 1.0), pair.q8(r, SFF, ND, 1.0), pair.q8(r, ND, SFF, 1.0)
+                d["s"] = None
+            else:
+                d["sg"] = pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF)
+                d["su"] = pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF)
+                d["sd"] = pair.w(nvfp4_rows(r, ND, SFF), ih.NVFP4, SFF, ND)
+                d["s"] = (float(0.7 / 54.0), float(1.3 / 54.0), float(1.1 / 27.0))
+            d["ffn_norm"] = (0.5 + r.random(ND)).astype(np.float32)
+            self.L.append(d)
+
+    def buffers(self):
+        """Per backend: one residual stream, per-layer scratch and state."""
+        out = []
+        for _ in range(2):
+            per = {"x": np.zeros(ND, np.float32), "layers": []}
+            for li in range(self.n):
+                b = bufs(normed=ND, qkv=CDIM, z=VDIM, alpha=NV, beta=NV, convo=CDIM, q=KDIM, k=KDIM, v=VDIM, core=VDIM,
+                         mixed=ND, conv_state=CDIM * 3, ssm=NV * DK * DK, fnormed=ND, e_in=ND, router=NE, logit=1,
+                         g_all=NU * FF, u_all=NU * FF, o_all=NU * ND, e_gate=SFF, e_up=SFF, e_out=ND, ffn_out=ND)[0]
+                b["conv_state"][:] = (rng(50 + li).standard_normal(CDIM * 3) * 0.5).astype(np.float32)
+                b["ssm"][:] = (rng(60 + li).standard_normal(NV * DK * DK) * 0.05).astype(np.float32)
+                per["layers"].append(b)
+            out.append(per)
+        return out
+
+    def gdn(self, ops, i, d, b, x):
+        W = lambda t: t[i]
+        ops.rms_norm(x, d["norm"], EPS, b["normed"])
+        ops.matmul(W(d["wqkv"]), b["normed"], b["qkv"]); ops.matmul(W(d["wz"]), b["normed"], b["z"])
+        ops.matmul_pair(W(d["wa"]), W(d["wb"]), b["normed"], b["alpha"], b["beta"])
+        ops.ssm_conv(b["conv_state"], b["qkv"], d["conv_w"], 4, b["convo"])
+        ops.gather_chunks(b["convo"], KDIM, CDIM, 0, b["q"]); ops.gather_chunks(b["convo"], KDIM, CDIM, KDIM, b["k"])
+        ops.gather_chunks(b["convo"], VDIM, CDIM, 2 * KDIM, b["v"])
+        ops.l2_norm_heads(b["q"], DK, EPS); ops.l2_norm_heads(b["k"], DK, EPS)
+        ops.delta_rule(b["q"], b["k"], b["v"], b["alpha"], b["beta"], d["ssm_a"], d["dt"], DK, DK, NK, NV, b["ssm"], b["core"])
+        ops.rms_norm_heads(b["core"], d["ssm_norm"], DK, EPS)
+        ops.silu_mul(b["z"], b["core"])
+        ops.matmul(W(d["wo"]), b["z"], b["mixed"])
+        ops.add_assign(x, b["mixed"])
+
+    def ffn(self, ops, i, d, b, x, is_hip):
+        W = lambda t: t[i]
+        ops.rms_norm(x, d["ffn_norm"], EPS, b["fnormed"])
+        ops.gather_chunks(b["fnormed"], ND, ND, 0, b["e_in"])
+        ops.matmul_pair(W(d["router"]), W(d["sh_inp"]), b["e_in"], b["router"], b["logit"])
+        ops.softmax(b["router"], NE)
+        ids = None
+        if is_hip:
+            route = ops.route(b["router"], NE, NU)
+            ops.moe_glu(W(self.gate), W(self.up), route, b["e_in"], b["g_all"], b["u_all"])
+            ops.matmul_experts(W(self.down), route, b["g_all"], b["o_all"])
+        else:
+            ids, w = ops.route(b["router"], NE, NU)
+            ops.moe_glu(W(self.gate), W(self.up), ids, NU, b["e_in"], b["g_all"], b["u_all"])
+            ops.matmul_experts(W(self.down), ids, NU, b["g_all"], b["o_all"])
+        ops.matmul(W(d["sg"]), b["e_in"], b["e_gate"]); ops.matmul(W(d["su"]), b["e_in"], b["e_up"])
+        if d["s"] is not None:
+            ops.scale(b["e_up"], d["s"][1]); ops.scale(b["e_gate"], d["s"][0])
+        ops.silu_mul(b["e_gate"], b["e_up"])
+        ops.matmul(W(d["sd"]), b["e_gate"], b["e_out"])
+        if d["s"] is not None:
+            ops.scale(b["e_out"], d["s"][2])
+        if is_hip:
+            ops.moe_finish(b["ffn_out"], 0, ND, b["o_all"], route, b["e_out"], b["logit"], 0)
+        else:
+            ops.moe_finish(b["ffn_out"], 0, ND, b["o_all"], w, NU, b["e_out"], b["logit"], 0)
+        ops.add_assign(x, b["ffn_out"])
+        return ids
+
+    def run(self, ops, i, B, is_hip, first_mixer=True):
+        """One pass over the layers; first_mixer False: the first layer contributes its FFN only (as the FFN of a layer
+        whose mixer is an attention block would open a chain)."""
+        picked = []
+        for li, d in enumerate(self.L):
+            if li > 0 or first_mixer:
+                self.gdn(ops, i, d, B["layers"][li], B["x"])
+            picked.append(self.ffn(ops, i, d, B["layers"][li], B["x"], is_hip))
+        return picked
+
+
+def make_pair(chain=True):
+    import inferred_hip as ih
+    from oracle import binding as ob
+    hip = ih.Hip(exact=False, chain=chain)
+    return Both(hip, ob.Oracle(threads=8))
+
+
+def hip_pass(hip, layers, B, x0, first_mixer=True):
+    B["x"][:] = x0
+    hip.begin_pass(1); hip.host_wrote(B["x"]); layers.run(hip, 0, B, True, first_mixer); hip.end_pass()
+    hip.host_needs(B["x"])
+    for li, b in enumerate(B["layers"]):
+        if li > 0 or first_mixer:
+            hip.read_state(b["ssm"]); hip.read_state(b["conv_state"])
+    hip.raise_if_error()
+
+
+@pytest.mark.parametrize("shared,first_mixer", [("q8_0", True), ("nvfp4_scaled", True), ("q8_0", False)])
+def test_layers_as_one_kernel(shared, first_mixer):
+    pair = make_pair()
+    hip, orc = pair.hip, pair.orc
+    try:
+        layers = Layers(pair, 2, shared)
+        B = layers.buffers()
+        counts_before = np.zeros(NE, np.int64)
+        for p in range(PASSES):
+            x0 = rng(700 + p).standard_normal(ND).astype(np.float32)
+            print(f"chain {shared} first_mixer={first_mixer} pass {p}", flush=True)
+            hip_pass(hip, layers, B[0], x0, first_mixer)
+            B[1]["x"][:] = x0
+            picked = layers.run(orc, 1, B[1], False, first_mixer)
+            got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
+            assert np.abs(want).max() > 0.3
+            assert near(got, want), (p, far(got, want))
+            for li in range(2):
+                if li == 0 and not first_mixer:
+                    continue
+                a, b = B[0]["layers"][li], B[1]["layers"][li]
+                assert close(a["ssm"], b["ssm"]), (p, li, worst(a["ssm"], b["ssm"]))
+                assert close(a["conv_state"], b["conv_state"]), (p, li, worst(a["conv_state"], b["conv_state"]))
+            # the picks of both layers, from the device-side read counters of the gate tensor
+            counts = hip.expert_counts(layers.gate_raw, NE).astype(np.int64)
+            want_counts = np.zeros(NE, np.int64)
+            for ids in picked:
+                assert len(set(ids.tolist())) == NU
+                np.add.at(want_counts, ids.astype(np.int64), 1)
+            assert np.array_equal(counts - counts_before, want_counts), (p, np.flatnonzero(counts - counts_before != want_counts))
+            counts_before = counts
+        g, c = hip.graph_stats(), hip.chain_stats()
+        assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] == PASSES - 2, g
+        assert g["graph_kernels"] == 1 and c["chains"] == 1 and c["layers"] == 2 and c["enabled"], (g, c)
+        # what the chain no longer writes is refused to the host instead of handed over stale
+        hip.host_needs(B[0]["layers"][1]["g_all"])
+        err = hip.take_error()
+        assert err is not None and "fused kernel" in err, err
+    finally:
+        err = hip.take_error()
+        hip.close()
+    assert err is None, err
+
+
+def test_chain_against_the_per_stage_kernels():
+    """The same three layers through the chain and through the six launches a layer it replaces."""
+    outs = []
+    for chain in (True, False):
+        pair = make_pair(chain)
+        hip = pair.hip
+        try:
+            layers = Layers(pair, 3, "q8_0", seed=11)
+            B = layers.buffers()[0]
+            xs = []
+            for p in range(PASSES):
+                x0 = rng(900 + p).standard_normal(ND).astype(np.float32)
+                print(f"chain={chain} pass {p}", flush=True)
+                hip_pass(hip, layers, B, x0)
+                xs.append(B["x"].copy())
+            c = hip.chain_stats()
+            assert (c["chains"], c["layers"]) == ((1, 3) if chain else (0, 0)), c
+            assert hip.graph_stats()["graph_kernels"] == (1 if chain else 18)
+            outs.append((xs, [b["ssm"].copy() for b in B["layers"]], [b["conv_state"].copy() for b in B["layers"]],
+                         hip.expert_counts(layers.gate_raw, NE).copy()))
+        finally:
+            err = hip.take_error()
+            hip.close()
+        assert err is None, err
+    (xa, sa, ca, na), (xb, sb, cb, nb) = outs
+    for p in range(PASSES):
+        assert near(xa[p], xb[p]), (p, far(xa[p], xb[p]))
+    for li in range(3):
+        assert close(sa[li], sb[li]), (li, worst(sa[li], sb[li]))
+        assert close(ca[li], cb[li]), (li, worst(ca[li], cb[li]))
+    assert np.array_equal(na, nb)
+
+
+def test_a_wait_that_gives_up_is_an_error_not_a_hang():
+    """With the bound on a hand-off wait forced down to one poll from the host, every block of the chain gives up at
+    its first wait and the kernel drains: the pass's results are void, the sticky error says so, the chains are
+    switched off for the backend, and the next passes run on the per-stage kernels."""
+    os.environ["INFERRED_HIP_CHAIN_SPINS"] = "1"
+    try:
+        pair = make_pair()
+    finally:
+        del os.environ["INFERRED_HIP_CHAIN_SPINS"]
+    hip, orc = pair.hip, pair.orc
+    try:
+        assert hip.chain_stats()["spin_limit"] == 1
+        layers = Layers(pair, 2, "q8_0", seed=13)
+        B = layers.buffers()
+        for p in range(2):          # eager passes
+            hip_pass(hip, layers, B[0], rng(40 + p).standard_normal(ND).astype(np.float32))
+        x0 = rng(42).standard_normal(ND).astype(np.float32)
+        B[0]["x"][:] = x0
+        print("the pass whose chain gives up", flush=True)
+        hip.begin_pass(1); hip.host_wrote(B[0]["x"]); layers.run(hip, 0, B[0], True); hip.end_pass()
+        hip.sync()
+        err = hip.take_error()
+        assert err is not None and "layer chain" in err, err
+        assert not hip.chain_stats()["enabled"]
+        # the backend keeps working without chains: with the oracle's state on both sides again, the next pass agrees
+        # with it, and the passes after that (recorded into a new graph of per-stage kernels) raise nothing
+        for li in range(2):
+            for name in ("ssm", "conv_state"):
+                B[0]["layers"][li][name][:] = B[1]["layers"][li][name]
+        hip.forget_state()          # the host copies are the state again: uploaded at their next use
+        x0 = rng(45).standard_normal(ND).astype(np.float32)
+        print("after the error, pass 0", flush=True)
+        hip_pass(hip, layers, B[0], x0)
+        B[1]["x"][:] = x0
+        layers.run(orc, 1, B[1], False)
+        got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
+        assert near(got, want), far(got, want)
+        for p in range(1, 4):
+            print(f"after the error, pass {p}", flush=True)
+            hip_pass(hip, layers, B[0], rng(45 + p).standard_normal(ND).astype(np.float32))
+            assert np.all(np.isfinite(B[0]["x"]))
+        assert hip.graph_stats()["graph_kernels"] == 12
+        assert hip.chain_stats()["chains"] == 0
+    finally:
+        err = hip.take_error()
+        hip.close()
+    assert err is None, err

@@ -65,7 +65,7 @@ def bufs(**sizes):
 def pair():
     import inferred_hip as ih
     from oracle import binding as ob
-    hip = ih.Hip(exact=False)
+    hip = ih.Hip(exact=False, chain=False)      # the per-stage fused kernels; tests/test_gpu_chain.py covers their chain form
     both = Both(hip, ob.Oracle(threads=8))
     yield both
     err = hip.take_error()
