@@ -55,6 +55,35 @@ constexpr int R_END = RE_SC + EB;
 static_assert(R_END <= (int)CHAIN_LL_WORDS, "hand-off space");
 static_assert(!(RA & 1) && !(RA_Z & 1) && !(RB & 1) && !(RB_SS & 1) && !(RC & 1) && !(RD & 1) && !(RS & 1) && !(RE & 1) && !(RE_SC & 1), "");
 
+// Stage stamps for tuning: a build with -DIT_CHAIN_STAMPS adds up, per stamp point, the 100 MHz wall clock that block
+// 0's first thread spent since its previous point; the library build compiles them away.
+#ifdef IT_CHAIN_STAMPS
+__device__ long long it_chain_stamps[16];
+#define CH_STAMP(i)                                          \
+    do {                                                     \
+        if (b0 == 0 && tid0 == 0) {                          \
+            const long long now = wall_clock64();            \
+            it_chain_stamps[i] += now - tprev;               \
+            tprev = now;                                     \
+        }                                                    \
+    } while (0)
+#else
+#define CH_STAMP(i) \
+    do {            \
+    } while (0)
+#endif
+
+// Where the prefetches sit (tuning switches; the defaults are what measured best).
+#ifndef IT_CHAIN_WC_AT
+#define IT_CHAIN_WC_AT 0      // out-projection row: 0 at the head of stage B, 1 after stage A's input has arrived, 2 after stage A's dots
+#endif
+#ifndef IT_CHAIN_D_AT
+#define IT_CHAIN_D_AT 1       // stage D's rows: 0 at the head of stage C, 1 after stage B's input has arrived
+#endif
+#ifndef IT_CHAIN_A_AT
+#define IT_CHAIN_A_AT 0x034   // next in-projection, a hex digit of fetch_a parts per site: after D's input | after E's publish | after F's input
+#endif
+
 struct Ctl {
     unsigned* abort_flag;
     int spin_limit;
@@ -66,7 +95,11 @@ IT_DEV void ll_put(u64* p, uint32_t bits, unsigned e) {
 IT_DEV void ll_putf(u64* p, float v, unsigned e) { ll_put(p, __float_as_uint(v), e); }
 
 // true when the wait must stop: the tries are used up (this thread raises the abort word) or another wait gave up
+#ifndef IT_CHAIN_SLEEP
+#define IT_CHAIN_SLEEP 0
+#endif
 IT_DEV bool ll_give_up(int& spins, const Ctl& c) {
+    if (IT_CHAIN_SLEEP > 0) __builtin_amdgcn_s_sleep(IT_CHAIN_SLEEP);
     if (++spins > c.spin_limit) {
         *(volatile unsigned*)c.abort_flag = 1u;
         return true;
@@ -76,8 +109,14 @@ IT_DEV bool ll_give_up(int& spins, const Ctl& c) {
 
 // Polls.  A load and its wait are ONE asm statement: the compiler does not know that the destination of an asm
 // load is not ready, so nothing may be schedulable between the two.
+// a short sleep ahead of a wait's first poll: a poll issued the moment the wave arrives nearly always fails, and every
+// failed poll is traffic that the words it waits for queue behind
+#ifndef IT_CHAIN_FIRST_SLEEP
+#define IT_CHAIN_FIRST_SLEEP 8
+#endif
 IT_DEV bool ll_wait1(const u64* p, unsigned e, const Ctl& c, uint32_t* out) {
     int spins = 0;
+    if (IT_CHAIN_FIRST_SLEEP > 0) __builtin_amdgcn_s_sleep(IT_CHAIN_FIRST_SLEEP);
     for (;;) {
         v2u w;
         asm volatile("global_load_dwordx2 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(w) : "v"(p) : "memory");
@@ -95,6 +134,7 @@ IT_DEV bool ll_wait_pairs(const u64* const (&a)[K], unsigned e, const Ctl& c, ui
     static_assert(K == 1 || K == 2 || K == 4, "");
     int spins = 0;
     unsigned done = 0;
+    if (IT_CHAIN_FIRST_SLEEP > 0) __builtin_amdgcn_s_sleep(IT_CHAIN_FIRST_SLEEP);
     for (;;) {
         v4u w[K];
         if constexpr (K == 4)
@@ -165,19 +205,31 @@ struct AW {
 IT_DEV int a_row(int k, int b, int wave) {   // row k of the wave in its own matrix
     return k < 4 ? b + NB * (wave + CW * k) : k < 6 ? b + NB * (wave + CW * (k - 4)) : b < NV ? b : b - NV;
 }
-IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane) {
+// `parts` picks what is fetched: bit 0 the first two wqkv rows and the conv windows, bit 1 the other two wqkv rows,
+// bit 2 the two wz rows and the alpha / beta row.  (A block's 105 KB are issued in pieces, each small enough to have
+// landed when the wave's next poll is due: loads return in the order they were issued, a poll behind a large
+// fetch waits for all of it.)
+IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int parts = 7) {
+    if (parts & 1) {
 #pragma unroll
-    for (int k = 0; k < 4; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.qkv_q, m.qkv_s, D, a_row(k, b, wave), lane, true);
+        for (int k = 0; k < 2; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.qkv_q, m.qkv_s, D, a_row(k, b, wave), lane, true);
+        if (lane < 4) {
+            const int64_t row = b + NB * (wave + CW * lane);
+            a.taps = *(const float4*)(m.conv_w + row * 4);
+            a.past[0] = m.conv_state[row * 3];
+            a.past[1] = m.conv_state[row * 3 + 1];
+            a.past[2] = m.conv_state[row * 3 + 2];
+        }
+    }
+    if (parts & 2) {
 #pragma unroll
-    for (int k = 4; k < 6; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.z_q, m.z_s, D, a_row(k, b, wave), lane, true);
-    const bool extra = wave == 0 && b < 2 * NV;
-    load_row<W_Q8_0, 2, 64>(a.t[6], b < NV ? m.a_q : m.b_q, b < NV ? m.a_s : m.b_s, D, a_row(6, b, wave), lane, extra);
-    if (lane < 4) {
-        const int64_t row = b + NB * (wave + CW * lane);
-        a.taps = *(const float4*)(m.conv_w + row * 4);
-        a.past[0] = m.conv_state[row * 3];
-        a.past[1] = m.conv_state[row * 3 + 1];
-        a.past[2] = m.conv_state[row * 3 + 2];
+        for (int k = 2; k < 4; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.qkv_q, m.qkv_s, D, a_row(k, b, wave), lane, true);
+    }
+    if (parts & 4) {
+#pragma unroll
+        for (int k = 4; k < 6; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.z_q, m.z_s, D, a_row(k, b, wave), lane, true);
+        const bool extra = wave == 0 && b < 2 * NV;
+        load_row<W_Q8_0, 2, 64>(a.t[6], b < NV ? m.a_q : m.b_q, b < NV ? m.a_s : m.b_s, D, a_row(6, b, wave), lane, extra);
     }
 }
 
@@ -226,15 +278,28 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     if (p.layer[0].has_mixer) fetch_a(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
     __syncthreads();
 
+#ifdef IT_CHAIN_STAMPS
+    long long tprev = wall_clock64();
+#endif
     for (int l = 0; l < p.n_layers; l++) {
         // The thread's coordinates pass through an empty asm statement once per layer.  Everything addressed from them
         // (hand-off words, weight rows, LDS slots) is then computed where it is used, a few integer operations, instead
         // of being hoisted out of the layer loop as loop invariants and held in a hundred registers across it.
         int tid = tid0, b = b0;
         asm volatile("" : "+v"(tid), "+s"(b));
-        const int lane = tid & 63;
-        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const int my_row = b * CW + wave;
+        int lane = tid & 63;
+        int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        int my_row = b * CW + wave;
+        // (again before the FFN's stages: what they address is computed there, not held across the mixer's)
+#define CHAIN_RECOORD()                                        \
+        do {                                                   \
+            tid = tid0;                                        \
+            b = b0;                                            \
+            asm volatile("" : "+v"(tid), "+s"(b));             \
+            lane = tid & 63;                                   \
+            wave = __builtin_amdgcn_readfirstlane(tid >> 6);   \
+            my_row = b * CW + wave;                            \
+        } while (0)
         const ChainLayer& L = p.layer[l];
         const ChainMixer& m = L.m;
         const ChainFfn& f = L.f;
@@ -270,6 +335,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             const float ssm_a = m.ssm_a[h], dt_bias = m.dt_bias[h];
             const float head_w = m.head_norm_w[j0 + (tid >> 5)];
 
+            WChunks<4> wc;   // the out-projection's row of this wave
             // ---------------------------------------------------------------- A: in-projection
             {
                 float4 v;
@@ -278,11 +344,14 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
                 if (!ok) dead = 1;
                 if (!norm_quant(v, nw, m.eps_norm, xq, xs, red, &dead, tid)) break;
+                if (IT_CHAIN_WC_AT == 1) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+                CH_STAMP(0);
                 XChunks<W_Q8_0, 2> x;
                 load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
                 float acc[7];
 #pragma unroll
                 for (int k = 0; k < 7; k++) acc[k] = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
+                if (IT_CHAIN_WC_AT == 2) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
                 // row k's dot goes from lane 63 to lane k, which finishes the row
                 float mine = 0.0f;
 #pragma unroll
@@ -310,9 +379,9 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 }
             }
             // ---------------------------------------------------------------- B: delta rule
+            CH_STAMP(1);
             // (the out-projection's row goes out first: small loads issued at the head of a stage are back before its input is)
-            WChunks<4> wc;
-            load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+            if (!IT_CHAIN_WC_AT) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
             {
                 uint32_t w0 = 0, w1 = 0;
                 bool ok = true;
@@ -334,6 +403,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (lane == 63) red[wave] = part;
                 __syncthreads();
                 if (dead) break;
+                CH_STAMP(2);
+                if (IT_CHAIN_D_AT) fetch_d();
                 if (tid < 2 * DK) {
                     const int w2 = tid < DK ? 0 : 2;
                     const double sum = red[w2] + red[w2 + 1];
@@ -378,7 +449,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 }
             }
             // ---------------------------------------------------------------- C: out-projection + residual
-            fetch_d();
+            CH_STAMP(3);
+            if (!IT_CHAIN_D_AT) fetch_d();
             {
                 const u64* const a4[4] = {p.ll + RB + 4 * tid, p.ll + RB + 4 * tid + 2, p.ll + RB + 4 * (tid + CT), p.ll + RB + 4 * (tid + CT) + 2};
                 uint32_t o[8];
@@ -393,6 +465,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (!ok) dead = 1;
                 __syncthreads();
                 if (dead) break;
+                CH_STAMP(4);
 #pragma unroll
                 for (int k = 0; k < 2; k++) {
                     const int qi = tid + k * CT, head = qi >> 5;
@@ -416,6 +489,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         }
 
         // -------------------------------------------------------------------- D: router, shared gate logit, shared gate / up
+        CH_STAMP(5);
         XChunks<W_NVFP4, 1> xn;
         {
             const float4 nw = ((const float4*)f.norm_w)[tid];
@@ -426,6 +500,9 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
             if (!ok) dead = 1;
             if (!norm_quant(v, nw, f.eps, xq, xs, red, &dead, tid)) break;
+            if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer && ((IT_CHAIN_A_AT >> 8) & 15))
+                fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 8) & 15);
+            CH_STAMP(6);
             XChunks<W_Q8_0, 2> x;
             load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
             load_x<W_NVFP4, 1, 64>(xn, xq, xs, lane);
@@ -450,6 +527,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         }
 
         // -------------------------------------------------------------------- E: route, routed gate / up
+        CH_STAMP(7);
+        CHAIN_RECOORD();
         WChunks<1> fd[3];
         WChunks<1> fsh;   // the shared expert's down row: lanes 32..63 (Q8_0) or 32..47 (NVFP4) beside the last two picks
         {
@@ -464,45 +543,27 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             if (!ok) dead = 1;
             __syncthreads();
             if (dead) break;
+            CH_STAMP(8);
             const float denom = block_route<CT>(lg4, NE, NU, route_sh, ids, wts);
-            // the down rows of this wave's output row: four picks a step over 16 lanes each, the shared row beside the
-            // last two picks
-#pragma unroll
-            for (int s = 0; s < 3; s++) {
-                const int y = s * 4 + (lane >> 4);
-                const bool routed = y < NU;
-                const int64_t ex = routed ? ids[y] : 0;
-                load_row<W_NVFP4, 1, 16>(fd[s], f.ed_q + ex * f.d_q_stride, f.ed_s + ex * f.d_s_stride, FF, my_row, lane & 15, routed);
-            }
-            if (SF == W_Q8_0) load_row<W_Q8_0, 1, 32>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 31, lane >= 32);
-            else load_row<W_NVFP4, 1, 16>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 15, lane >= 32 && lane < 48);
-            if (tid < NU) {
-                const int ex = ids[tid];
-                const float w = wts[tid] / denom;
-                coef[tid] = w * (f.dscale2 ? f.dscale2[ex] : 1.0f);
-                if (b == 0) {
-                    f.route_ids[tid] = ex;
-                    f.route_w[tid] = w;
-                    if (f.counts_gate) atomicAdd(f.counts_gate + ex, 1u);
-                    if (f.counts_up) atomicAdd(f.counts_up + ex, 1u);
-                    if (f.counts_down) atomicAdd(f.counts_down + ex, 1u);
-                }
-            }
-            if (b == 0 && tid == 0 && p.tally)
-                atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
+            CH_STAMP(9);
+            const float my_dscale = (tid < NU && f.dscale2) ? f.dscale2[ids[tid]] : 1.0f;   // issued ahead of the rows below
+            // the picks' rows: this block's 32 gate and 32 up rows
+            WChunks<1> tg[4], tu[4];
+            float scg = 1.0f, scu = 1.0f;
             if (b < EB) {
                 const int y = b >> 4, sb = b & 15;
                 const int64_t ex = ids[y];
                 const uint8_t *gq = f.eg_q + ex * f.gu_q_stride, *gs = f.eg_s + ex * f.gu_s_stride;
                 const uint8_t *uq = f.eu_q + ex * f.gu_q_stride, *us = f.eu_s + ex * f.gu_s_stride;
-                WChunks<1> tg[4], tu[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int j = sb * 32 + wave * 4 + i;
                     load_row<W_NVFP4, 1, 64>(tg[i], gq, gs, D, j, lane, true);
                     load_row<W_NVFP4, 1, 64>(tu[i], uq, us, D, j, lane, true);
                 }
-                const float scg = f.gscale2 ? f.gscale2[ex] : 1.0f, scu = f.uscale2 ? f.uscale2[ex] : 1.0f;
+                if (f.gscale2) scg = f.gscale2[ex];
+                if (f.uscale2) scu = f.uscale2[ex];
+                CH_STAMP(13);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     float ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tg[i], xn));
@@ -513,6 +574,36 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                         inter[wave * 4 + i] = fx_silu(ag) * au;
                     }
                 }
+            }
+            CH_STAMP(14);
+            // the down rows of this wave's output row, for stage F: issued now, they land while the intermediates travel
+            // (four picks a step over 16 lanes each, the shared row beside the last two picks)
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                const int y = s * 4 + (lane >> 4);
+                const bool routed = y < NU;
+                const int64_t ex = routed ? ids[y] : 0;
+                load_row<W_NVFP4, 1, 16>(fd[s], f.ed_q + ex * f.d_q_stride, f.ed_s + ex * f.d_s_stride, FF, my_row, lane & 15, routed);
+            }
+            if (SF == W_Q8_0) load_row<W_Q8_0, 1, 32>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 31, lane >= 32);
+            else load_row<W_NVFP4, 1, 16>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 15, lane >= 32 && lane < 48);
+            // the picks' weights for stage F, and what the seam shows of the route (block 0)
+            if (tid < NU) {
+                const int ex = ids[tid];
+                const float w = wts[tid] / denom;
+                coef[tid] = w * my_dscale;
+                if (b == 0) {
+                    f.route_ids[tid] = ex;
+                    f.route_w[tid] = w;
+                    if (f.counts_gate) atomicAdd(f.counts_gate + ex, 1u);
+                    if (f.counts_up) atomicAdd(f.counts_up + ex, 1u);
+                    if (f.counts_down) atomicAdd(f.counts_down + ex, 1u);
+                }
+            }
+            if (b == 0 && tid == 0 && p.tally)
+                atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
+            CH_STAMP(15);
+            if (b < EB) {
                 __syncthreads();
                 if (tid < 8) {
                     // Q8_0 of the block's 32 intermediates (naive.rs:652-675), published as four quants a word
@@ -535,7 +626,9 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             }
         }
         // the next layer's in-projection rows start moving now: one stage ahead of their use
-        if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer) fetch_a(p.layer[l + 1].m, aw, b, wave, lane);
+        CH_STAMP(10);
+        const bool next_mixer = l + 1 < p.n_layers && p.layer[l + 1].has_mixer;
+        if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
 
         // -------------------------------------------------------------------- F: down, combine, residual
         {
@@ -565,6 +658,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             if (!ok) dead = 1;
             __syncthreads();
             if (dead) break;
+            CH_STAMP(11);
+            if (next_mixer && (IT_CHAIN_A_AT & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, IT_CHAIN_A_AT & 15);
             float acc = 0.0f;
             const int c = lane & 15;
 #pragma unroll
@@ -609,6 +704,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 p.x[my_row] = x_row;
             }
         }
+        CH_STAMP(12);
     }
     if (b0 == 0 && tid0 == 0) *p.epoch = e0 + 1u + (unsigned)p.n_layers;
 }
