@@ -73,6 +73,8 @@ def summarize_profile(root_dir):
 
     def family(name, grid):
         n = short(name)
+        if n.startswith("layer_chain_k"):
+            return "layer_chain (persistent kernel over a run of layers)"
         if n.startswith("fused_gemv_fast_k"):
             return "lm_head (norm + GEMV)" if grid >= 400000 else "fused_gemv (norm + quantize + dense GEMVs)"
         if n.startswith("moe_glu_fast_k"):
@@ -144,9 +146,13 @@ def summarize_profile(root_dir):
     # the last token: its third GDN layer, the attention layer after it and the output head, node by node
     last = tail[-nodes:]
     glu = [i for i, r in enumerate(last) if short(r[2]).startswith("moe_down_fast_k")]
-    cut = last[glu[1] + 1:glu[3] + 1] + last[glu[-1] + 1:] if len(glu) >= 4 else last
-    print("\nlast replayed token, layers 2 (GDN) and 3 (attention) and the output head, node by node: start offset us, "
-          "duration us, gap before us, kernel, grid threads")
+    chains = [i for i, r in enumerate(last) if short(r[2]).startswith("layer_chain_k")]
+    if len(chains) >= 2:   # with layer chains: one chain, the attention mixer behind it, the next chain, and the output head
+        cut = last[chains[0]:chains[1] + 1] + last[chains[-1] + 1:]
+    else:
+        cut = last[glu[1] + 1:glu[3] + 1] + last[glu[-1] + 1:] if len(glu) >= 4 else last
+    print("\nlast replayed token node by node (without chains: layers 2 and 3; with them: the first chain, the attention "
+          "mixer behind it and the next chain) and the output head: start offset us, duration us, gap before us, kernel, grid threads")
     t0, prev = last[0][0], None
     for s0, e0, n, g in cut:
         gap = "" if prev is None else f"{(s0 - prev) / 1e3:6.2f}"
@@ -506,8 +512,25 @@ def main():
         ids_ctl = np.asarray(eng.decode_greedy(n_g))
         be_x = ih.Hip(exact=True)
         eng_x = ih.Engine(model, be_x, args.ctx, args.max_batch)
-        lx = eng_x.prefill(prompt[:n_p])
+        eng_x.prefill(prompt[:n_p - 1], want_logits=False)
+        ckpt = eng_x.checkpoint()
+        lx = eng_x.forward(prompt[n_p - 1:n_p])
+        t_x = time.perf_counter()
         ids_exact = np.asarray(eng_x.decode_greedy(n_g))
+        be_x.sync()
+        exact_tok_s = n_g / (time.perf_counter() - t_x)
+        # a control with no fast kernel in it: exact mode against exact mode from the same checkpoint, once with the
+        # recurrent state as it was (must reproduce itself bit for bit) and once with ONE state element moved by one ulp
+        eng_x.restore(ckpt)
+        l_same = eng_x.forward(prompt[n_p - 1:n_p])
+        ids_same = np.asarray(eng_x.decode_greedy(n_g))
+        pos_c, conv_c, ssm_c = ckpt
+        ssm_u = ssm_c.copy()
+        at = int(np.argmax(np.abs(ssm_u)))
+        ssm_u[at] = np.nextafter(ssm_u[at], np.float32(np.inf))
+        eng_x.restore((pos_c, conv_c, ssm_u))
+        l_ulp = eng_x.forward(prompt[n_p - 1:n_p])
+        ids_ulp = np.asarray(eng_x.decode_greedy(n_g))
         err = be_x.take_error() or be.take_error()
         if err:
             raise SystemExit(f"device error in the mode check: {err}")
@@ -523,6 +546,15 @@ def main():
                       "exact_top1_rank_in_fast": int(np.where(np.argsort(-lf64) == top_x[0])[0][0]),
                       "top10_overlap": int(len(set(top_x.tolist()) & set(top_f.tolist()))),
                       "exact_top1_margin": float(lx64[top_x[0]] - lx64[top_x[1]]),
+                      "exact_mode_decode_tok_s": round(exact_tok_s, 1),
+                      "control_exact_vs_exact_one_ulp": {
+                          "what": "exact mode from one checkpoint after 511 prompt tokens: unchanged state, and one "
+                                  "recurrent-state element (the largest) moved by one ulp; then the 512th token and 32 greedy ids",
+                          "unchanged_state_reproduces_bits": bool(np.array_equal(np.asarray(l_same).view(np.uint32), np.asarray(lx).view(np.uint32))
+                                                                  and np.array_equal(ids_same, ids_exact)),
+                          "ids_equal": int((ids_ulp == ids_exact).sum()),
+                          "logits_max_abs_diff": float(np.abs(np.asarray(l_ulp) - np.asarray(lx)).max()),
+                          "logits_correlation": round(float(np.corrcoef(np.asarray(l_ulp, np.float64), lx64)[0, 1]), 6)},
                       "control_fast_vs_fast_other_passes": {
                           "ids_equal": int((ids_ctl == ids_fast).sum()),
                           "prefill_logits_max_abs_diff": float(np.abs(np.asarray(lc) - np.asarray(lf)).max()),

@@ -322,7 +322,10 @@ int it_hip_mfma_ceiling(it_hip*, int kind, int iters, double* ops_per_s);
  *    object, one copy per GPU, held until the process ends and shared by every call on that GPU: calls that overlap
  *    on one GPU race.  A problem whose partials (n_q * n_head * n_split * (head_dim + 2) floats; n_split =
  *    ceil(n_pos / 64) capped at 256 for head_dim 64, 128 and 256, ceil(n_pos / 128) otherwise) do not fit is refused;
- *  - it calls no hipMalloc, hipFree or allocating library routine, and needs no it_hip handle.
+ *  - it calls no hipMalloc, hipFree or allocating library routine, and needs no it_hip handle;
+ *  - the scratch's device address is looked up once per GPU (hipGetSymbolAddress, and an attribute of the tile
+ *    kernel set): at it_hip_create, else inside the first call on that GPU.  That first call is therefore not one to
+ *    make while a stream is capturing: create a backend, or make one warm-up call, before using it under capture.
  * Returns 0 = enqueued, 1 = bad argument, 2 = too large for the fixed scratch, 3 = device error; the message goes to
  * err. */
 #define IT_HIP_NOALLOC_SCRATCH_BYTES (8ull << 20)

@@ -95,6 +95,7 @@ void it_hip::drop_graph() {
 
 // what a deferred pass has recorded so far goes to the stream, fused; the pass stays deferred
 void it_hip::flush_deferred() {
+    if (chain_enabled && fuse_enabled && !exact && !expert_cold_entries && (!itk::layer_chain_fits() || !chain_acquire())) chain_enabled = false;
     for (auto& c : precopies) check(hipMemcpyAsync(c.dev, c.host, c.bytes, hipMemcpyHostToDevice, stream), "upload activation");
     precopies.clear();
     dyn_upload();
@@ -103,6 +104,8 @@ void it_hip::flush_deferred() {
     pending.clear();
     run_fused(todo);
     check(hipGetLastError(), "kernel launch");
+    mark_elided(fused_elided);
+    if (chain_launches) chain_ran = true;
 }
 
 void it_hip::need_eager(const char* why) {
@@ -257,6 +260,10 @@ it_hip::Act* it_hip::act_slot(const float* host, size_t len) {
 float* it_hip::act_in(const float* host, size_t len) {
     Act* a = act_slot(host, len);
     if (!a) return nullptr;
+    if (a->dev_current && a->elided) {
+        fail("an op reads a buffer whose producer was folded into a fused kernel that does not write it");
+        return nullptr;
+    }
     if (!a->dev_current) {
         if (mode != Mode::Eager) {
             precopies.push_back(PreCopy{a->dev, host, len * sizeof(float)});
@@ -1214,6 +1221,9 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->allow_graph = (flags & IT_HIP_NO_GRAPH) == 0;
     be->fuse_enabled = (flags & IT_HIP_NO_FUSE) == 0 && getenv("INFERRED_HIP_NO_FUSE") == nullptr;
     be->chain_enabled = (flags & IT_HIP_NO_CHAIN) == 0 && getenv("INFERRED_HIP_NO_CHAIN") == nullptr;
+    be->eager_fused = getenv("INFERRED_HIP_EAGER_FUSED") != nullptr;
+    be->count_reads_in_fused = getenv("INFERRED_HIP_NO_READ_COUNTERS") == nullptr;
+    if (getenv("INFERRED_HIP_NO_GRAPH")) be->allow_graph = false;
     if (const char* sl = getenv("INFERRED_HIP_CHAIN_SPINS")) {
         const long v = atol(sl);
         if (v > 0 && v < (1l << 30)) be->chain_spin_limit = (int)v;
@@ -1298,7 +1308,7 @@ void it_hip_rms_norm(it_hip* be, const float* x, uint64_t x_len, const float* w,
     // written by the same launch.  Single-token passes keep the two ops apart for the pass fuser.
     float* qs = nullptr;
     int8_t* qq = nullptr;
-    if (rows > 1 && be->mode == it_hip::Mode::Eager && nd % 32 == 0) {
+    if (rows > 1 && be->mode == it_hip::Mode::Eager && rms_norm_writes_q8(dx, dw, dout, nd)) {
         it_hip::Act& a = be->acts[out];
         if (be->act_q_reserve(a, out_len)) {
             qs = a.q_scales;
@@ -2079,6 +2089,9 @@ void it_hip_begin_pass(it_hip* be, uint64_t n_tokens) {
         }
     } else if (n_tokens == 1 && be->expert_cold_entries && be->fuse_enabled && !be->has_error) {
         be->mode = it_hip::Mode::Deferred;   // picks are read back inside the pass: fused launches, no graph
+    } else if (n_tokens == 1 && be->eager_fused && !be->allow_graph && be->fuse_enabled && !be->has_error && !be->prof_on) {
+        // the fused launches queued on the stream pass after pass, with no graph around them (a measurement switch)
+        be->mode = it_hip::Mode::Deferred;
     }
     for (auto& kv : be->acts) {
         kv.second.dev_current = false;

@@ -258,6 +258,8 @@ struct it_hip {
     };
     ChainRes chain;
     bool chain_enabled = true;
+    bool count_reads_in_fused = true;  // the fused decode kernels add the picks to the expert read counters (off: a measurement switch)
+    bool eager_fused = false;          // single-token passes without a graph still go through the fuser (measurement switch)
     bool chain_ran = false;            // a chain has been issued since the abort word was last looked at
     int chain_spin_limit = 1 << 21;
     uint64_t chain_launches = 0, chain_layers = 0;   // per fused pass, for the statistics

@@ -564,10 +564,12 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
     d.route_w = (const float*)rt.p[2];
     d.logit = (const float*)ml.p[5];
     d.x = (float*)rms.p[0];
-    d.counts_gate = (uint32_t*)glu.p[10];
-    d.counts_up = (uint32_t*)glu.p[11];
-    d.counts_down = (uint32_t*)ex.p[7];
-    d.tally = tally;
+    if (pl.be->count_reads_in_fused) {
+        d.counts_gate = (uint32_t*)glu.p[10];
+        d.counts_up = (uint32_t*)glu.p[11];
+        d.counts_down = (uint32_t*)ex.p[7];
+        d.tally = tally;
+    }
 
     pl.take(i, n_ops);
     const uint64_t glu_b = 2 * rows_bytes(g.fmt, (uint64_t)nu * ff, nd) + 2 * rows_bytes(g.sh_fmt, sff, nd) + (uint64_t)nd * 4 +
@@ -688,7 +690,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             cp.ll = be->chain.ll;
             cp.epoch = be->chain.epoch;
             cp.abort_flag = be->chain.abort_flag;
-            cp.tally = tally;
+            cp.tally = be->count_reads_in_fused ? tally : nullptr;
             cp.spin_limit = be->chain_spin_limit;
             const ChainP launch = cp;
             for (size_t u = 0; u < n_units; u++) {
@@ -821,6 +823,9 @@ void it_hip::finish_held() {
         }
     }
     if (done) {
+        // the conv output (first run) and the normed read-out (second run: `core` keeps the delta rule's raw values) are
+        // not what their ops would have left there
+        mark_elided({held[0].id == OP_CONV ? held[0].p[3] : held[0].p[0]});
         held.clear();
         check(hipGetLastError(), "kernel launch");
     } else {
@@ -848,7 +853,7 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
         // quantized, so there every quantization is kept
         for (size_t i = 0; i < ops.size(); i++) {
             if (!pl.consumed[i] || ops[i].id != OP_QUANT) continue;
-            if (mode == Mode::Deferred) {
+            if (mode == Mode::Deferred && expert_cold_entries) {
                 pl.consumed[i] = 0;
                 continue;
             }
@@ -862,7 +867,7 @@ void it_hip::run_fused(std::vector<OpRec>& ops) {
             }
         }
     }
-    if (fuse_enabled && mode != Mode::Deferred) build_chains(pl, expert_tally);
+    if (fuse_enabled && !expert_cold_entries) build_chains(pl, expert_tally);
     uint64_t n = 0;
     for (size_t i = 0; i < ops.size(); i++) {
         for (auto& l : pl.at[i]) {

@@ -79,11 +79,15 @@ __global__ __launch_bounds__(THREADS) void rms_norm_q8_k(const float* __restrict
     }
 }
 
+bool rms_norm_writes_q8(const float* x, const float* w, const float* out, int nd) {
+    auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    return nd % 32 == 0 && al(x) && al(w) && al(out);
+}
+
 void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
               hipStream_t s, float* q_scales, int8_t* q_quants) {
     if (n_rows <= 0) return;
-    auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    if (q_scales && q_quants && nd % 32 == 0 && al(x) && al(w) && al(out)) {
+    if (q_scales && q_quants && rms_norm_writes_q8(x, w, out, nd)) {
         hipLaunchKernelGGL(rms_norm_q8_k<256>, dim3((unsigned)n_rows), dim3(256), nd * sizeof(float), s, x, w, eps, out, nd,
                            exact, q_scales, q_quants);
         return;

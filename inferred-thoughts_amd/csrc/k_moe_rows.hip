@@ -240,6 +240,7 @@ bool launch_rows(const ExpertRowsP& p, int max_tiles, hipStream_t s) {
     const int L = U >= 64 ? 64 : U;
     const int gx = (p.n_out + p.rows_per_block - 1) / p.rows_per_block;
     const size_t lds = (size_t)RP * p.n_in + (size_t)RP * U * 4 + (size_t)(GLU ? 2 : 1) * RP * p.rows_per_block * 4;
+    if (lds > 64 * 1024) return false;   // more than a launch gets without asking: the caller takes another kernel
     const dim3 grid(gx, max_tiles), block(256);
     switch (L) {
         case 64: hipLaunchKernelGGL((expert_rows_k<FMT, GLU, 64, RP>), grid, block, lds, s, p); return true;
@@ -319,8 +320,11 @@ bool expert_rows(const ExpertsView& w, const ExpertsView* up, const int32_t* ids
     const int likely_tiles = ids ? std::min(n_picks, w.n_expert) + n_picks / RP : max_tiles;
     while (rb > 4 * step && (int64_t)likely_tiles * ((w.n_out + rb - 1) / rb) < 2048) rb = (rb / 2 + step - 1) / step * step;
     rb = std::max(step, std::min(rb, 256));
-    p.rows_per_block = rb;
     const bool glu = up != nullptr;
+    // the block's LDS (the tile's activations and scales, then its outputs) stays within what a launch gets unasked
+    auto lds_of = [&](int rows) { return (size_t)RP * w.n_in + (size_t)RP * U * 4 + (size_t)(glu ? 2 : 1) * RP * rows * 4; };
+    while (rb > step && lds_of(rb) > 64 * 1024) rb -= step;
+    p.rows_per_block = rb;
 #define IT_ROWS(F, G, R) launch_rows<F, G, R>(p, max_tiles, s)
     if (w.fmt == W_Q8_0) {
         if (RP == 16) return glu ? IT_ROWS(W_Q8_0, true, 16) : IT_ROWS(W_Q8_0, false, 16);

@@ -135,6 +135,9 @@ void moe_finish(float* out, int64_t at, int n, const float* rows, const float* w
 // quantize_q8_0 gives on it
 void rms_norm(const float* x, const float* w, float eps, float* out, int64_t n_rows, int nd, int exact,
               hipStream_t s, float* q_scales = nullptr, int8_t* q_quants = nullptr);
+// whether rms_norm writes the Q8_0 form when given the buffers for it (row length and alignments): the caller marks the
+// quantized form valid only then
+bool rms_norm_writes_q8(const float* x, const float* w, const float* out, int nd);
 void rms_norm_heads(float* x, const float* w, int head_dim, float eps, int64_t n_heads, int exact,
                     hipStream_t s);
 void l2_norm_heads(float* x, int head_dim, float eps, int64_t n_heads, int exact, hipStream_t s);

@@ -106,3 +106,37 @@ def test_gated_norm_silu_and_quantized_product(hip, orc, n, with_matmul):
         # quantization and the integer dots are the oracle's, and only the f32 additions round differently.
         orc.matmul(ob.weights(wo, ih.Q8_0, VD, 256), B[0]["z"], B[1]["out"])
         assert close(B[0]["out"], B[1]["out"], 1e-5), worst(B[0]["out"], B[1]["out"])
+
+
+def test_what_a_one_kernel_run_leaves_unwritten_is_refused_not_handed_over_stale():
+    """The one-kernel forms skip two buffers of the seam: the conv output (conv + split + l2) and the normed read-out
+    (`core` keeps the delta rule's raw values behind gated norm + silu-mul + quantize).  A host read of either after a
+    completed run raises the sticky error; a traced pass, whose read lands inside the run, still gets the op's value
+    (the run is then issued op by op: covered above)."""
+    import inferred_hip as ih
+    be = ih.Hip(exact=False)
+    try:
+        DK, n = HD, 256
+        kdim, vdim, cdim = KD, VD, NC
+        r = rng(91)
+        qkv = r.standard_normal(n * cdim).astype(np.float32)
+        conv_w = (r.standard_normal(cdim * 4) * 0.5).astype(np.float32)
+        state = np.zeros(cdim * 3, np.float32)
+        convo = np.zeros(n * cdim, np.float32)
+        q, k, v = np.zeros(n * kdim, np.float32), np.zeros(n * kdim, np.float32), np.zeros(n * vdim, np.float32)
+        for rep in range(2):       # the first pass sizes the device mirrors (which ends a held run): the second holds
+            be.begin_pass(n)
+            be.host_wrote(qkv)
+            be.ssm_conv(state, qkv, conv_w, 4, convo)
+            be.gather_chunks(convo, kdim, cdim, 0, q); be.gather_chunks(convo, kdim, cdim, kdim, k)
+            be.gather_chunks(convo, vdim, cdim, 2 * kdim, v)
+            be.l2_norm_heads(q, DK, 1e-6); be.l2_norm_heads(k, DK, 1e-6)
+            be.end_pass()
+        be.host_needs(q)
+        assert be.take_error() is None and np.abs(q).max() > 0          # what the run does write is there
+        be.host_needs(convo)
+        err = be.take_error()
+        assert err is not None and "fused kernel" in err, err
+    finally:
+        be.take_error()
+        be.close()

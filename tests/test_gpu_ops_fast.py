@@ -15,6 +15,11 @@ from util import bf16_round, f16_bits, nvfp4_weights, q8_0_weights, rng
 
 pytestmark = pytest.mark.gpu
 
+# The NVFP4 matrix-core kernels against the oracle: every entry to 2e-5 of its row's largest (the weights are exact in
+# f16, the Q8_0 activations an f16 pair of 22 bits, sums in f32 in tile order: what is left is the order of the sums,
+# which is absolute in the row's scale, not relative to an entry that cancels to nearly nothing).
+ROW_TOL = 2e-5
+
 
 @pytest.fixture(scope="module")
 def hip():
@@ -156,14 +161,14 @@ def test_moe_stage_fast_nvfp4(hip, orc, n_tok, n_expert, n_used, nd, ff):
                 ids, n_used, x, gb, sb)
     hip.host_needs(ga); hip.raise_if_error()
     scale = np.repeat(np.abs(gb.reshape(pairs, ff)).max(axis=1) + 1e-30, ff)
-    assert np.all(np.abs(ga - gb) <= 1e-3 * np.maximum(scale, np.abs(gb))), (np.abs(ga - gb) / scale).max()
+    assert np.all(np.abs(ga - gb) <= ROW_TOL * scale), (np.abs(ga - gb) / scale).max()
     oa, obuf = np.zeros(pairs * nd, np.float32), np.zeros(pairs * nd, np.float32)
     hip.matmul_experts(ih.experts(down, code, ff, nd, n_expert, scales[2]), route, gb, oa)
     orc.matmul_experts(ob.experts(down, code, ff, nd, n_expert, scales[2]), ids, n_used, gb, obuf)
     hip.host_needs(oa); hip.raise_if_error()
     assert np.isfinite(obuf).all()
     scale = np.repeat(np.abs(obuf.reshape(pairs, nd)).max(axis=1) + 1e-30, nd)
-    assert np.all(np.abs(oa - obuf) <= 1e-3 * np.maximum(scale, np.abs(obuf))), (np.abs(oa - obuf) / scale).max()
+    assert np.all(np.abs(oa - obuf) <= ROW_TOL * scale), (np.abs(oa - obuf) / scale).max()
 
 
 # A dense NVFP4 matrix over a batch (the shared expert of an NVFP4 file during prefill): from 513 tokens on it runs as
@@ -185,7 +190,7 @@ def test_matmul_nvfp4_batched_fast(hip, orc, n_in, n_out, n):
     hip.raise_if_error()
     assert np.isfinite(b).all()
     scale = np.repeat(np.abs(b.reshape(n, n_out)).max(axis=1) + 1e-30, n_out)
-    assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(scale, np.abs(b))), (np.abs(a - b) / scale).max()
+    assert np.all(np.abs(a - b) <= ROW_TOL * scale), (np.abs(a - b) / scale).max()
     # a second call in the same pass (the shared expert's up after its gate) reuses the token grouping
     a2 = np.zeros_like(a)
     hip.matmul(ih.weights(wb, ih.NVFP4, n_in, n_out), x, a2); hip.host_needs(a2)
@@ -221,7 +226,7 @@ def test_nvfp4_tiles_keep_subnormal_and_extreme_scales(hip, orc):
         hip.raise_if_error()
         assert np.isfinite(b).all() and np.abs(b).max() > 0
         scale = np.repeat(np.abs(b.reshape(n, n_out)).max(axis=1) + 1e-30, n_out)
-        assert np.all(np.abs(a - b) <= 1e-3 * np.maximum(scale, np.abs(b))), (np.abs(a - b) / scale).max()
+        assert np.all(np.abs(a - b) <= ROW_TOL * scale), (np.abs(a - b) / scale).max()
 
 
 # unquantized weights (the router and ssm alpha / beta of real files are F32): wave-split row sums for up to 16

@@ -84,6 +84,52 @@ def test_f16_decode_exhaustive_against_numpy():
     assert np.isnan(got[nan]).all()
 
 
+def test_bf16_decode_exhaustive_against_the_bit_shift():
+    """bf16 is the top half of an f32 (/root/reference src/quant/half.rs:61-63): all 65,536 codes."""
+    L = ob.lib()
+    h = np.arange(65536, dtype=np.uint32)
+    want = (h << 16).astype(np.uint32).view(np.float32)
+    got = np.array([L.orc_c_bf16_to_f32(int(v)) for v in h], np.float32)
+    nan = np.isnan(want)          # (a signalling NaN is quieted on its way back through the C float return)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.isnan(got[nan]).all()
+
+
+@pytest.mark.parametrize("ty,np_ty", [("f32", np.float32), ("f16", np.float16), ("bf16", None)])
+def test_matmul_on_unquantized_rows_is_the_serial_f32_fold_of_the_widened_weights(orc, ty, np_ty):
+    """F32 / F16 / BF16 rows (/root/reference src/ops/naive.rs:843-861): each output is the serial f32 sum of
+    widened weight times activation from zero, checked bit for bit against that fold written in numpy, and against
+    the float64 product of the widened weights (a wrong widening, a transposed operand or a dropped row would be far
+    outside it)."""
+    r = np.random.default_rng(17)
+    n_in, n_out, n_tok = 96, 7, 3
+    w32 = (r.standard_normal((n_out, n_in)) * 0.5).astype(np.float32)
+    if ty == "bf16":
+        bits = (w32.view(np.uint32) >> 16).astype(np.uint16)          # truncation picks representable values
+        wide = (bits.astype(np.uint32) << 16).view(np.float32)
+        raw, code = bits.view(np.uint8).reshape(-1).copy(), ob.BF16
+    elif ty == "f16":
+        half = w32.astype(np.float16)
+        wide = half.astype(np.float32)
+        raw, code = half.view(np.uint8).reshape(-1).copy(), ob.F16
+    else:
+        wide = w32
+        raw, code = w32.view(np.uint8).reshape(-1).copy(), ob.F32
+    x = r.standard_normal(n_tok * n_in).astype(np.float32)
+    out = np.zeros(n_tok * n_out, np.float32)
+    orc.matmul(ob.weights(raw, code, n_in, n_out), x, out)
+    want = np.zeros((n_tok, n_out), np.float32)
+    for t in range(n_tok):
+        for j in range(n_out):
+            acc = np.float32(0.0)
+            for i in range(n_in):
+                acc = np.float32(acc + np.float32(wide[j, i] * x[t * n_in + i]))
+            want[t, j] = acc
+    assert np.array_equal(out.view(np.uint32), want.reshape(-1).view(np.uint32))
+    f64 = x.reshape(n_tok, n_in).astype(np.float64) @ wide.astype(np.float64).T
+    assert np.allclose(out.reshape(n_tok, n_out), f64, rtol=0, atol=1e-4)
+
+
 def test_f32_to_f16_round_to_nearest_even_against_numpy():
     L = ob.lib()
     r = np.random.default_rng(0)

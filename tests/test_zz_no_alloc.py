@@ -71,3 +71,66 @@ def test_refuses_what_the_fixed_scratch_cannot_hold():
         assert rc == 1 and "n_pos" in msg
     finally:
         rt.free_all()
+
+
+def test_a_warm_call_leaves_free_device_memory_as_it_was():
+    """The property the entry point exists for: nothing is allocated.  After one call (the scratch address is looked
+    up, the kernels are loaded), hipMemGetInfo reads the same before and after further calls."""
+    hd, nh, nkv, n_q, n_pos, slab = 256, 16, 2, 1, 3000, 4096
+    rt = Hiprt()
+    try:
+        r = rng(77)
+        q = r.standard_normal(n_q * nh * hd).astype(np.float32)
+        k = f16_bits(r.standard_normal(slab * nkv * hd)); v = f16_bits(r.standard_normal(slab * nkv * hd))
+        dq, dk, dv, dout = rt.upload(q), rt.upload(k), rt.upload(v), rt.filled(q.nbytes, 0xff)
+        call = lambda: ih.attend_noalloc(dq, q.size, dk, dv, k.size, nkv * hd, n_pos, hd, nh, nkv, 0.0625, dout, q.size, stream=0)
+        rc, msg = call()
+        assert rc == 0, msg
+        rt.check(rt.rt.hipDeviceSynchronize(), "hipDeviceSynchronize")
+        before = rt.mem_free()
+        for _ in range(3):
+            rc, msg = call()
+            assert rc == 0, msg
+        rt.check(rt.rt.hipDeviceSynchronize(), "hipDeviceSynchronize")
+        assert rt.mem_free() == before
+    finally:
+        rt.free_all()
+
+
+_FIRST_CALL = r"""
+import sys
+sys.path.insert(0, {tests!r}); sys.path.insert(0, {pkg!r}); sys.path.insert(0, {root!r})
+import numpy as np
+import inferred_hip as ih
+from util import Hiprt, rng, f16_bits
+hd, nh, nkv, n_q, n_pos, slab = 256, 16, 2, 1, 2500, 4096
+rt = Hiprt()
+r = rng(78)
+q = r.standard_normal(n_q * nh * hd).astype(np.float32)
+k = f16_bits(r.standard_normal(slab * nkv * hd)); v = f16_bits(r.standard_normal(slab * nkv * hd))
+dq, dk, dv, dout = rt.upload(q), rt.upload(k), rt.upload(v), rt.filled(q.nbytes, 0xff)
+# no backend exists yet in this process: the call itself looks the scratch up
+rc, msg = ih.attend_noalloc(dq, q.size, dk, dv, k.size, nkv * hd, n_pos, hd, nh, nkv, 0.0625, dout, q.size, stream=0)
+assert rc == 0, msg
+got = rt.download(dout, q)
+hip = ih.Hip(exact=False)
+hip.begin_pass(1)
+want = np.zeros_like(q)
+hip.attend(q, k, v, nkv * hd, n_pos, hd, nh, nkv, 0.0625, want); hip.host_needs(want)
+hip.raise_if_error()
+assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), np.abs(got - want).max()
+hip.close(); rt.free_all()
+print("FIRST CALL OK")
+"""
+
+
+def test_the_first_call_of_a_process_needs_no_backend():
+    """In a process that has created no backend, the entry point resolves its scratch on its first call (that call is
+    not one to make under graph capture: the header says so) and gives it_hip_attend's bits."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    code = _FIRST_CALL.format(tests=str(root / "tests"), pkg=str(root / "inferred-thoughts_amd"), root=str(root))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and "FIRST CALL OK" in out.stdout, out.stdout[-2000:] + out.stderr[-2000:]

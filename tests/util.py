@@ -99,6 +99,13 @@ class Hiprt:
         self.check(self.rt.hipMemcpy(out.ctypes.data, dev, out.nbytes, 2), "hipMemcpy(device to host)")
         return out
 
+    def mem_free(self):
+        """free device memory in bytes (hipMemGetInfo)"""
+        C = self.C
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        self.check(self.rt.hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+        return int(free.value)
+
     def free_all(self):
         for p in self.held:
             self.rt.hipFree(p)
