@@ -21,7 +21,7 @@ struct Plan {
     std::vector<char> consumed;
     // which stage of a layer a fused launch is (0: none of them), with its arguments: the chain pass below rebuilds
     // runs of them as one persistent kernel
-    enum Stage { ST_NONE = 0, ST_GDN_IN, ST_GDN_CORE, ST_GDN_OUT, ST_ROUTER, ST_GLU, ST_DOWN };
+    enum Stage { ST_NONE = 0, ST_GDN_IN, ST_GDN_CORE, ST_GDN_OUT, ST_ROUTER, ST_GLU, ST_DOWN, ST_ATTN_IN, ST_ATTEND, ST_ATTN_OUT };
     struct Launch {
         int fam;         // it_hip::Family, for the per-kernel timing
         uint64_t bytes;  // algorithmic bytes of the launch (weights + state it must move once)
@@ -42,7 +42,7 @@ struct Plan {
         size_t pos;
         std::vector<const void*> bufs;
     };
-    std::vector<Skips> gdn_skips, ffn_skips;
+    std::vector<Skips> gdn_skips, ffn_skips, attn_skips;
     Plan(it_hip* b, std::vector<Op>& o) : be(b), ops(o), consumed(o.size(), 0), at(o.size()) {}
     // slot of a position scalar in the pass's device array, -1 when the pointer is not one
     int dyn_index(const void* p) const {
@@ -369,7 +369,9 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     it_hip* be = pl.be;
     // K and V rows of the live context, f16 (the position is the one this pass was recorded at)
     const uint64_t kv_bytes = (uint64_t)at.i[8] * kvd * 2 * 2;
-    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
+    Plan::Launch& l_in = pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(a), [=](hipStream_t s) { fused_gemv(a, s); });
+    const size_t in_at = pl.at[i].size() - 1;
+    (void)l_in;
     TilePrepP tp{};
     tp.qg = pp.qg;
     tp.kproj = pp.k;
@@ -381,13 +383,15 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     tp.eps = pp.eps;
     tp.k_slab = pp.k_slab;
     tp.v_slab = pp.v_slab;
+    bool three = false;
     if (at.i[6] == 0 && attend_tile_prep_ok(aa, tp)) {
         // norm + rotation of q and of the new key, and the slab writes, happen inside the tile kernel
         pl.add(i, it_hip::FAM_ATTEND, kv_bytes + (uint64_t)(2 * hd * nh + 2 * kvd) * 4,
                [=](hipStream_t s) {
                    if (!attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s))
                        be->fail("attend: the split-K kernels could not be launched");
-               });
+               }).stage = Plan::ST_ATTEND;
+        three = true;
     } else if (at.i[6] == 0) {
         pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
         pl.add(i, it_hip::FAM_ATTEND, kv_bytes, [=](hipStream_t s) {
@@ -402,7 +406,14 @@ bool match_attn(Plan& pl, size_t i, int exact) {
         pl.add(i, it_hip::FAM_ATTEND, kv_bytes, run_attend);
         pl.add(i, it_hip::FAM_OTHER, 0, run_gate);
     }
-    pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b), [=](hipStream_t s) { fused_gemv(b, s); });
+    Plan::Launch& l_out = pl.add(i, it_hip::FAM_FUSED_GEMV, gemv_bytes(b), [=](hipStream_t s) { fused_gemv(b, s); });
+    if (three) {   // the form whose in- and out-projection a layer chain may take over
+        l_out.stage = Plan::ST_ATTN_OUT;
+        l_out.gv = b;
+        pl.at[i][in_at].stage = Plan::ST_ATTN_IN;
+        pl.at[i][in_at].gv = a;
+        pl.attn_skips.push_back({i, {normed}});
+    }
     return true;
 }
 
@@ -662,14 +673,41 @@ bool chain_ffn(const FusedGemvP& r, const MoeGluP& g, const MoeDownP& d, ChainFf
     return true;
 }
 
+bool chain_attn_out(const FusedGemvP& b, ChainMixer* m) {
+    if (b.exact || b.mode != 0 || b.n_in != 4096 || b.n_mats != 1 || !q8(b.m[0], 2048, 2) || b.route_counter) return false;
+    if (!al16(b.m[0].q) || !al16(b.m[0].s) || !al16(b.x) || !al16(b.m[0].out)) return false;
+    *m = ChainMixer{};
+    m->o_q = b.m[0].q;
+    m->o_s = b.m[0].s;
+    m->attn = b.x;
+    return true;
+}
+
+bool chain_attn_in(const FusedGemvP& a, ChainTail* t) {
+    if (a.exact || a.mode != 1 || a.n_in != 2048 || a.n_mats != 3 || a.route_counter) return false;
+    if (!q8(a.m[0], 8192, 0) || !q8(a.m[1], 512, 0) || !q8(a.m[2], 512, 0)) return false;
+    for (int i = 0; i < 3; i++)
+        if (!al16(a.m[i].q) || !al16(a.m[i].s)) return false;
+    if (!al16(a.norm_w)) return false;
+    t->norm_w = a.norm_w;
+    t->q_q = a.m[0].q; t->q_s = a.m[0].s;
+    t->k_q = a.m[1].q; t->k_s = a.m[1].s;
+    t->v_q = a.m[2].q; t->v_s = a.m[2].s;
+    t->out_q = a.m[0].out; t->out_k = a.m[1].out; t->out_v = a.m[2].out;
+    t->eps = a.eps;
+    return true;
+}
+
 void build_chains(Plan& pl, unsigned long long* tally) {
     it_hip* be = pl.be;
     be->chain_launches = be->chain_layers = 0;
     if (!be->chain_enabled || be->exact || !layer_chain_fits()) return;
+    enum Kind { U_GDN, U_FFN, U_ATTN_OUT };
     struct Unit {
         size_t pos;
-        bool gdn;
+        Kind kind;
     };
+    size_t tail_pos = 0;   // position of the attention block whose in-projection is cp's tail
     ChainP cp{};
     std::vector<Unit> units;          // the blocks folded into cp so far
     bool mixer_open = false;          // the last layer of cp has its mixer and still waits for its FFN
@@ -681,9 +719,10 @@ void build_chains(Plan& pl, unsigned long long* tally) {
     auto emit = [&]() {
         int n = cp.n_layers;
         size_t n_units = units.size();
-        if (mixer_open) {   // a mixer without its FFN stays three launches
+        if (mixer_open) {   // a mixer without its FFN stays as it was
             n--;
             n_units--;
+            cp.has_tail = 0;
         }
         if (n >= 1 && be->chain_acquire()) {
             cp.n_layers = n;
@@ -693,9 +732,25 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             cp.tally = be->count_reads_in_fused ? tally : nullptr;
             cp.spin_limit = be->chain_spin_limit;
             const ChainP launch = cp;
+            auto drop_stage = [&](size_t pos, int stage) {
+                auto& v = pl.at[pos];
+                for (size_t k = 0; k < v.size(); k++)
+                    if (v[k].stage == stage) {
+                        v.erase(v.begin() + (long)k);
+                        break;
+                    }
+            };
             for (size_t u = 0; u < n_units; u++) {
-                pl.at[units[u].pos].clear();
-                skips_of(units[u].gdn ? pl.gdn_skips : pl.ffn_skips, units[u].pos, &be->fused_elided);
+                if (units[u].kind == U_ATTN_OUT) {
+                    drop_stage(units[u].pos, Plan::ST_ATTN_OUT);   // the attention kernels before it stay where they are
+                } else {
+                    pl.at[units[u].pos].clear();
+                    skips_of(units[u].kind == U_GDN ? pl.gdn_skips : pl.ffn_skips, units[u].pos, &be->fused_elided);
+                }
+            }
+            if (cp.has_tail) {
+                drop_stage(tail_pos, Plan::ST_ATTN_IN);
+                skips_of(pl.attn_skips, tail_pos, &be->fused_elided);
             }
             pl.add(units[0].pos, it_hip::FAM_CHAIN, bytes, [=](hipStream_t s) {
                 if (!layer_chain(launch, s)) be->fail("layer chain: the persistent kernel could not be launched");
@@ -712,7 +767,33 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         auto& ls = pl.at[i];
         const bool is_gdn = ls.size() == 3 && ls[0].stage == Plan::ST_GDN_IN && ls[1].stage == Plan::ST_GDN_CORE && ls[2].stage == Plan::ST_GDN_OUT;
         const bool is_ffn = ls.size() == 3 && ls[0].stage == Plan::ST_ROUTER && ls[1].stage == Plan::ST_GLU && ls[2].stage == Plan::ST_DOWN;
+        const bool is_attn = ls.size() == 3 && ls[0].stage == Plan::ST_ATTN_IN && ls[1].stage == Plan::ST_ATTEND && ls[2].stage == Plan::ST_ATTN_OUT;
         bool taken = false;
+        if (is_attn) {
+            // its in-projection closes the chain so far, its out-projection opens the next one; the attention kernels
+            // between them stay launches of their own
+            const FusedGemvP in = ls[0].gv, out = ls[2].gv;
+            const uint64_t in_bytes = ls[0].bytes, out_bytes = ls[2].bytes;
+            ChainTail t{};
+            if (cp.n_layers >= 1 && !mixer_open && cp.x == in.x && chain_attn_in(in, &t)) {
+                cp.has_tail = 1;
+                cp.tail = t;
+                tail_pos = i;
+                bytes += in_bytes;
+            }
+            emit();
+            ChainMixer m{};
+            if (chain_attn_out(out, &m)) {
+                cp.layer[0].has_mixer = 2;
+                cp.layer[0].m = m;
+                cp.x = out.m[0].out;
+                cp.n_layers = 1;
+                mixer_open = true;
+                units.push_back({i, U_ATTN_OUT});
+                bytes += out_bytes;
+            }
+            continue;
+        }
         if (is_gdn) {
             if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
             ChainMixer m{};
@@ -722,7 +803,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
                 cp.x = const_cast<float*>(ls[0].gv.x);
                 cp.n_layers++;
                 mixer_open = true;
-                units.push_back({i, true});
+                units.push_back({i, U_GDN});
                 bytes += ls[0].bytes + ls[1].bytes + ls[2].bytes;
                 taken = true;
             }
@@ -740,7 +821,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
                 cp.sh_fmt = sh_fmt;
                 cp.x = const_cast<float*>(ls[0].gv.x);
                 mixer_open = false;
-                units.push_back({i, false});
+                units.push_back({i, U_FFN});
                 bytes += ls[0].bytes + ls[1].bytes + ls[2].bytes;
                 taken = true;
             }

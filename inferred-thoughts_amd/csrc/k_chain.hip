@@ -233,6 +233,15 @@ IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int p
     }
 }
 
+// The tail stage's rows (the in-projection of the attention layer behind the chain): 36 a block, row r of the flat list
+// [wq 8192 | wk 512 | wv 512] on block r % 256; a wave takes four wq rows, waves 0..3 one more (wk: 0, 1; wv: 2, 3).
+IT_DEV void fetch_tail(const ChainTail& t, AW& a, int b, int wave, int lane) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) load_row<W_Q8_0, 2, 64>(a.t[k], t.q_q, t.q_s, D, b + NB * (wave + CW * k), lane, true);
+    const bool kk = wave < 2;
+    load_row<W_Q8_0, 2, 64>(a.t[4], kk ? t.k_q : t.v_q, kk ? t.k_s : t.v_s, D, b + NB * (wave & 1), lane, wave < 4);
+}
+
 // rms_norm (naive.rs:633-650) of the 2,048 floats the block's threads hold as quads, then Q8_0 (naive.rs:652-675)
 // into xq / xs.  Two barriers; returns false after the first when the block has to stop.
 IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
@@ -275,7 +284,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     // lane 63 of a wave owns one row of the residual stream: row 8 * block + wave
     float x_row = (tid0 & 63) == 63 ? p.x[b0 * CW + (tid0 >> 6)] : 0.0f;
     AW aw;
-    if (p.layer[0].has_mixer) fetch_a(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
+    if (p.layer[0].has_mixer == 1) fetch_a(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
     __syncthreads();
 
 #ifdef IT_CHAIN_STAMPS
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         const ChainMixer& m = L.m;
         const ChainFfn& f = L.f;
         const unsigned e = e0 + 1 + (unsigned)l;
-        const bool mixer = L.has_mixer != 0;
+        const bool mixer = L.has_mixer != 0;   // the FFN's input comes from a mixer stage of this kernel
 
         // Stage D's rows.  Waves 0, 1: router rows b and NB + b; waves 2, 3: gate and up rows 2 b and 2 b + 1 of the
         // shared expert; wave 4 of the last block: the shared expert's gate-logit row.  Issued at the head of the stage
@@ -326,7 +335,24 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         };
         if (!mixer) fetch_d();
 
-        if (mixer) {
+        if (L.has_mixer == 2) {
+            // ---------------------------------------------------------------- the attention block's out-projection + residual
+            // (quantize + matmul + add_assign, qwen35.rs:1216-1223; the input is in ordinary memory: the merge kernel wrote it)
+            WChunks<4> wo;
+            load_row<W_Q8_0, 4, 64>(wo, m.o_q, m.o_s, VDIM, my_row, lane, true);
+            fetch_d();
+#pragma unroll
+            for (int k = 0; k < 2; k++) quant_quad(((const float4*)m.attn)[tid + k * CT], true, tid + k * CT, xq, xs);
+            __syncthreads();
+            XChunks<W_Q8_0, 4> x;
+            load_x<W_Q8_0, 4, 64>(x, xq, xs, lane);
+            const float acc = reduce_lanes<64>(dot_chunks<W_Q8_0, 4>(wo, x));
+            if (lane == 63) {
+                x_row += acc;
+                ll_putf(p.ll + RC + my_row, x_row, e);
+            }
+        }
+        if (L.has_mixer == 1) {
             // ---------------------------------------------------------------- loads known from the start of the layer
             const int h = b >> 3, j0 = (b & 7) * 16, kh = h % NK;
             float* S = m.state + ((int64_t)(h * DK + j0 + (tid >> 5)) * DK + (tid & 31) * 4);
@@ -500,7 +526,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
             if (!ok) dead = 1;
             if (!norm_quant(v, nw, f.eps, xq, xs, red, &dead, tid)) break;
-            if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer && ((IT_CHAIN_A_AT >> 8) & 15))
+            if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer == 1 && ((IT_CHAIN_A_AT >> 8) & 15))
                 fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 8) & 15);
             CH_STAMP(6);
             XChunks<W_Q8_0, 2> x;
@@ -627,7 +653,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         }
         // the next layer's in-projection rows start moving now: one stage ahead of their use
         CH_STAMP(10);
-        const bool next_mixer = l + 1 < p.n_layers && p.layer[l + 1].has_mixer;
+        const bool next_mixer = l + 1 < p.n_layers && p.layer[l + 1].has_mixer == 1;
+        if (l + 1 == p.n_layers && p.has_tail) fetch_tail(p.tail, aw, b, wave, lane);
         if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
 
         // -------------------------------------------------------------------- F: down, combine, residual
@@ -706,6 +733,35 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         }
         CH_STAMP(12);
     }
+    // -------------------------------------------------------------------- tail: the next attention layer's in-projection
+    if (p.has_tail) {
+        __syncthreads();
+        if (!dead) {
+            int tid = tid0, b = b0;
+            asm volatile("" : "+v"(tid), "+s"(b));
+            const int lane = tid & 63;
+            const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+            const ChainTail& t = p.tail;
+            const unsigned e = e0 + 1u + (unsigned)p.n_layers;
+            const float4 nw = ((const float4*)t.norm_w)[tid];
+            float4 v;
+            if (!ll_wait_quad(p.ll + RX, tid, e, ctl, &v)) dead = 1;
+            if (norm_quant(v, nw, t.eps, xq, xs, red, &dead, tid)) {
+                XChunks<W_Q8_0, 2> x;
+                load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
+                float mine = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 5; k++) {
+                    const float acc = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
+                    const float r = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 63));
+                    mine = lane == k ? r : mine;
+                }
+                if (lane < 4) t.out_q[b + NB * (wave + CW * lane)] = mine;
+                else if (lane == 4 && wave < 2) t.out_k[b + NB * wave] = mine;
+                else if (lane == 4 && wave < 4) t.out_v[b + NB * (wave - 2)] = mine;
+            }
+        }
+    }
     if (b0 == 0 && tid0 == 0) *p.epoch = e0 + 1u + (unsigned)p.n_layers;
 }
 
@@ -726,6 +782,28 @@ bool layer_chain_fits() {
 bool layer_chain(const ChainP& p, hipStream_t s) {
     if (p.n_layers < 1 || p.n_layers > CHAIN_MAX_LAYERS || !p.ll || !p.epoch || !p.abort_flag || !p.x) return false;
     if (p.sh_fmt != W_Q8_0 && p.sh_fmt != W_NVFP4) return false;
+    // every pointer a stage dereferences, by the kind of the layer's mixer (an attention out-projection only as layer 0)
+    auto all = [](std::initializer_list<const void*> ptrs) {
+        for (const void* q : ptrs)
+            if (!q) return false;
+        return true;
+    };
+    for (int l = 0; l < p.n_layers; l++) {
+        const ChainMixer& m = p.layer[l].m;
+        const ChainFfn& f = p.layer[l].f;
+        const int kind = p.layer[l].has_mixer;
+        if (kind < 0 || kind > 2 || (kind == 2 && l != 0)) return false;
+        if (kind == 1 && !all({m.norm_w, m.qkv_q, m.qkv_s, m.z_q, m.z_s, m.a_q, m.a_s, m.b_q, m.b_s, m.conv_state, m.conv_w, m.ssm_a,
+                               m.dt_bias, m.state, m.head_norm_w, m.o_q, m.o_s}))
+            return false;
+        if (kind == 2 && !all({m.o_q, m.o_s, m.attn})) return false;
+        if (!all({f.norm_w, f.r_q, f.r_s, f.l_q, f.l_s, f.sg_q, f.sg_s, f.su_q, f.su_s, f.sd_q, f.sd_s, f.eg_q, f.eg_s, f.eu_q, f.eu_s,
+                  f.ed_q, f.ed_s, f.route_ids, f.route_w}))
+            return false;
+    }
+    if (p.has_tail && !all({p.tail.norm_w, p.tail.q_q, p.tail.q_s, p.tail.k_q, p.tail.k_s, p.tail.v_q, p.tail.v_s, p.tail.out_q,
+                            p.tail.out_k, p.tail.out_v}))
+        return false;
     if (!layer_chain_fits()) return false;
     if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL(layer_chain_k<W_Q8_0>, dim3(NB), dim3(CT), 0, s, p);
     else hipLaunchKernelGGL(layer_chain_k<W_NVFP4>, dim3(NB), dim3(CT), 0, s, p);

@@ -128,6 +128,7 @@ struct ChainMixer {
     const float* head_norm_w;
     const uint8_t *o_q, *o_s;
     float eps_norm, eps_l2, eps_head, q_scale;
+    const float* attn;   // has_mixer == 2 only: the attention block's gated output [4096], the out-projection's input
 };
 struct ChainFfn {
     const float* norm_w;
@@ -142,8 +143,18 @@ struct ChainFfn {
     float* route_w;
     uint32_t *counts_gate, *counts_up, *counts_down;   // expert read counters (optional)
 };
+// The in-projection of the attention layer BEHIND the chain's last layer (rms_norm + quantization + rows of wq, wk,
+// wv), run as the chain's last stage; its outputs go to ordinary memory for the attention kernels that follow.
+struct ChainTail {
+    const float* norm_w;
+    const uint8_t *q_q, *q_s, *k_q, *k_s, *v_q, *v_s;   // wq (8192 rows: query and gate of every head), wk, wv (512 rows each)
+    float *out_q, *out_k, *out_v;
+    float eps;
+};
 struct ChainLayer {
-    int has_mixer;   // 0: the layer's mixer ran before the chain (an attention layer); the chain starts at its FFN
+    // 0: the layer's mixer ran before the chain; 1: a Gated DeltaNet mixer; 2: an attention layer whose out-projection
+    // (+ residual) opens the chain (first layer only: its input is in ordinary memory when the kernel starts)
+    int has_mixer;
     ChainMixer m;
     ChainFfn f;
 };
@@ -153,6 +164,8 @@ constexpr size_t CHAIN_LL_WORDS = 24576;   // 8-byte words of hand-off space a c
 struct ChainP {
     ChainLayer layer[CHAIN_MAX_LAYERS];
     int n_layers;
+    int has_tail;
+    ChainTail tail;
     int sh_fmt;                  // the shared expert's format (W_Q8_0 or W_NVFP4)
     float* x;                    // residual stream [2048], read at the start and current after every layer
     unsigned long long* ll;      // CHAIN_LL_WORDS words of uncached device memory, zero before the first chain

@@ -125,12 +125,14 @@ def test_config5_full_size_fast_run_is_deterministic_and_clean(config5_gguf):
     assert len(set(runs[1][1].tolist())) > 1                      # not stuck on one token
     g = be.graph_stats()
     assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] >= 90, g
-    # 12 layer chains (an attention layer's routed FFN and the three Gated DeltaNet layers behind it, one persistent kernel
-    # each; the very first covers layers 0-2, the last only layer 47's FFN... see below), the attention mixers' three
-    # launches each, the output head and the arg-max + embedding step
+    # 13 layer chains, one persistent kernel each: layers 0-2 with the in-projection of layer 3's attention block as the
+    # last stage; then, per attention layer, its out-projection, its routed FFN and the three Gated DeltaNet layers
+    # behind it, closed by the next attention block's in-projection (the last chain is layer 47's out-projection and
+    # FFN alone).  Between two chains only the attention launch itself (norms, rotation, cache write, split-K attend
+    # and its gated merge) remains; then the output head and the arg-max + embedding step.
     c = be.chain_stats()
-    assert c["enabled"] and c["layers"] == 48, c
-    assert g["graph_kernels"] == c["chains"] + 12 * 3 + 2, (g, c)
+    assert c["enabled"] and c["layers"] == 48 and c["chains"] == 13, c
+    assert g["graph_kernels"] == c["chains"] + 12 + 2, (g, c)
     st = be.expert_stats()
     assert st.resident == 48 * 3 * 512 and st.oversubscribed == 0 and st.evictions == 0 and st.fetched == 0
     he.close(); hm.close(); be.close()
