@@ -512,15 +512,22 @@ def main():
         ids_ctl = np.asarray(eng.decode_greedy(n_g))
         be_x = ih.Hip(exact=True)
         eng_x = ih.Engine(model, be_x, args.ctx, args.max_batch)
-        eng_x.prefill(prompt[:n_p - 1], want_logits=False)
+        n_h = n_p // 2
+        eng_x.prefill(prompt[:n_h], want_logits=False)
+        ckpt_half = eng_x.checkpoint()
+        eng_x.forward(prompt[n_h:n_p - 1], want_logits=False) if n_p - 1 > n_h else None
         ckpt = eng_x.checkpoint()
         lx = eng_x.forward(prompt[n_p - 1:n_p])
         t_x = time.perf_counter()
         ids_exact = np.asarray(eng_x.decode_greedy(n_g))
         be_x.sync()
         exact_tok_s = n_g / (time.perf_counter() - t_x)
-        # a control with no fast kernel in it: exact mode against exact mode from the same checkpoint, once with the
-        # recurrent state as it was (must reproduce itself bit for bit) and once with ONE state element moved by one ulp
+        # Controls with no fast kernel in them, exact mode against exact mode from a checkpoint of its own state:
+        #  (a) the state as it was: must reproduce itself bit for bit;
+        #  (b) ONE recurrent-state element (the largest) moved by one ulp before the last prompt token;
+        #  (c) EVERY recurrent-state element moved by one ulp, up or down at random, half-way through the prompt, the
+        #      other half of the prompt run from there: what last-bit noise, the size of a changed summation order,
+        #      becomes over 256 tokens of this model.
         eng_x.restore(ckpt)
         l_same = eng_x.forward(prompt[n_p - 1:n_p])
         ids_same = np.asarray(eng_x.decode_greedy(n_g))
@@ -531,6 +538,12 @@ def main():
         eng_x.restore((pos_c, conv_c, ssm_u))
         l_ulp = eng_x.forward(prompt[n_p - 1:n_p])
         ids_ulp = np.asarray(eng_x.decode_greedy(n_g))
+        pos_h, conv_h, ssm_h = ckpt_half
+        up = np.random.default_rng(5).random(ssm_h.size) < 0.5
+        ssm_n = np.where(up, np.nextafter(ssm_h, np.float32(np.inf)), np.nextafter(ssm_h, np.float32(-np.inf))).astype(np.float32)
+        eng_x.restore((pos_h, conv_h, ssm_n))
+        l_all = eng_x.forward(prompt[n_h:n_p])
+        ids_all = np.asarray(eng_x.decode_greedy(n_g))
         err = be_x.take_error() or be.take_error()
         if err:
             raise SystemExit(f"device error in the mode check: {err}")
@@ -555,6 +568,12 @@ def main():
                           "ids_equal": int((ids_ulp == ids_exact).sum()),
                           "logits_max_abs_diff": float(np.abs(np.asarray(l_ulp) - np.asarray(lx)).max()),
                           "logits_correlation": round(float(np.corrcoef(np.asarray(l_ulp, np.float64), lx64)[0, 1]), 6)},
+                      "control_exact_vs_exact_every_state_element_one_ulp": {
+                          "what": f"exact mode from its own checkpoint after {n_h} prompt tokens, every recurrent-state element "
+                                  f"moved by one ulp up or down at random; then the other {n_p - n_h} prompt tokens and 32 greedy ids",
+                          "ids_equal": int((ids_all == ids_exact).sum()),
+                          "logits_max_abs_diff": float(np.abs(np.asarray(l_all) - np.asarray(lx)).max()),
+                          "logits_correlation": round(float(np.corrcoef(np.asarray(l_all, np.float64), lx64)[0, 1]), 6)},
                       "control_fast_vs_fast_other_passes": {
                           "ids_equal": int((ids_ctl == ids_fast).sum()),
                           "prefill_logits_max_abs_diff": float(np.abs(np.asarray(lc) - np.asarray(lf)).max()),

@@ -67,13 +67,29 @@ __device__ long long it_chain_stamps[16];
             tprev = now;                                     \
         }                                                    \
     } while (0)
+// per wave of block 0, inside stage E: the time since the wave's previous point (point 0 restarts the clock)
+__device__ long long it_chain_wave_stamps[8][8];
+#define CH_WSTAMP(i)                                                     \
+    do {                                                                 \
+        if (b0 == 0 && (tid0 & 63) == 0) {                               \
+            const long long now = wall_clock64();                        \
+            if (i) it_chain_wave_stamps[tid0 >> 6][i] += now - wprev;    \
+            wprev = now;                                                 \
+        }                                                                \
+    } while (0)
 #else
 #define CH_STAMP(i) \
     do {            \
     } while (0)
+#define CH_WSTAMP(i) \
+    do {             \
+    } while (0)
 #endif
 
 // Where the prefetches sit (tuning switches; the defaults are what measured best).
+#ifndef IT_CHAIN_FLOADS_EARLY
+#define IT_CHAIN_FLOADS_EARLY 0   // stage F's down rows: 1 ahead of stage E's barrier and publication, 0 behind them
+#endif
 #ifndef IT_CHAIN_WC_AT
 #define IT_CHAIN_WC_AT 0      // out-projection row: 0 at the head of stage B, 1 after stage A's input has arrived, 2 after stage A's dots
 #endif
@@ -242,6 +258,13 @@ IT_DEV void fetch_tail(const ChainTail& t, AW& a, int b, int wave, int lane) {
     load_row<W_Q8_0, 2, 64>(a.t[4], kk ? t.k_q : t.v_q, kk ? t.k_s : t.v_s, D, b + NB * (wave & 1), lane, wave < 4);
 }
 
+// a float's bits as an unsigned that orders like the value (negative below positive), and back
+IT_DEV uint32_t logit_order(float v) {
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+IT_DEV float logit_of_order(uint32_t o) { return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o); }
+
 // rms_norm (naive.rs:633-650) of the 2,048 floats the block's threads hold as quads, then Q8_0 (naive.rs:652-675)
 // into xq / xs.  Two barriers; returns false after the first when the block has to stop.
 IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
@@ -288,7 +311,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     __syncthreads();
 
 #ifdef IT_CHAIN_STAMPS
-    long long tprev = wall_clock64();
+    long long tprev = wall_clock64(), wprev = tprev;
 #endif
     for (int l = 0; l < p.n_layers; l++) {
         // The thread's coordinates pass through an empty asm statement once per layer.  Everything addressed from them
@@ -558,10 +581,15 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         WChunks<1> fd[3];
         WChunks<1> fsh;   // the shared expert's down row: lanes 32..63 (Q8_0) or 32..47 (NVFP4) beside the last two picks
         {
-            float lg4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            // The route (softmax over the 512 logits, the 10 largest, src/ops/mod.rs:1191-1216), in the order that lets
+            // the picks' rows start moving first: the picks are ranked on the logits themselves (the softmax keeps their
+            // order), and the probabilities of the ten are formed afterwards, under the rows' flight.
             uint32_t w0 = 0;
             bool ok = ll_wait1(p.ll + RD + tid, e, ctl, &w0);
-            lg4[0] = __uint_as_float(w0);
+            const float my_logit = __uint_as_float(w0);
+            const u64 my_key = ((u64)logit_order(my_logit) << 32) | (u64)(~(unsigned)tid);   // larger = earlier pick, unique
+            route_sh.keys[tid] = my_key;
+            if (tid < (CT / 64) * 16) route_sh.cand[tid] = 0ull;
             if (tid == 0) {
                 ok = ok && ll_wait1(p.ll + RD + NE, e, ctl, &w0);
                 sm[34] = __uint_as_float(w0);
@@ -570,8 +598,30 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             __syncthreads();
             if (dead) break;
             CH_STAMP(8);
-            const float denom = block_route<CT>(lg4, NE, NU, route_sh, ids, wts);
+            CH_WSTAMP(0);
+            // (a) a key's rank among the 64 of its wave: only wave ranks below 10 can be among the 10 of the block
+            wave_rank_one(route_sh.keys + (tid & ~63), my_key, NU, route_sh.cand + wave * 16);
+            __syncthreads();
+            {   // (b) the 128 candidate slots against each other: four threads a slot, a quarter of the slots each
+                const int c = tid >> 2, part = tid & 3;
+                const u64 me = route_sh.cand[c];
+                int cnt = 0;
+#pragma unroll
+                for (int c2 = 0; c2 < (CT / 64) * 2; c2++) {
+                    const ulonglong2 q = ((const ulonglong2*)route_sh.cand)[c2 * 4 + part];
+                    cnt += q.x > me ? 1 : 0;
+                    cnt += q.y > me ? 1 : 0;
+                }
+                cnt += __shfl_xor(cnt, 1, 64);
+                cnt += __shfl_xor(cnt, 2, 64);
+                if (part == 0 && me != 0ull && cnt < NU) {
+                    ids[cnt] = (int)~(unsigned)(me & 0xffffffffull);
+                    wts[cnt] = logit_of_order((uint32_t)(me >> 32));   // the pick's logit; its probability follows below
+                }
+            }
+            __syncthreads();
             CH_STAMP(9);
+            CH_WSTAMP(1);
             const float my_dscale = (tid < NU && f.dscale2) ? f.dscale2[ids[tid]] : 1.0f;   // issued ahead of the rows below
             // the picks' rows: this block's 32 gate and 32 up rows
             WChunks<1> tg[4], tu[4];
@@ -590,6 +640,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (f.gscale2) scg = f.gscale2[ex];
                 if (f.uscale2) scu = f.uscale2[ex];
                 CH_STAMP(13);
+                CH_WSTAMP(2);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     float ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tg[i], xn));
@@ -599,10 +650,13 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                         au *= scu;
                         inter[wave * 4 + i] = fx_silu(ag) * au;
                     }
+                    if (i == 0) CH_WSTAMP(3);
                 }
             }
             CH_STAMP(14);
-            // the down rows of this wave's output row, for stage F: issued now, they land while the intermediates travel
+            CH_WSTAMP(4);
+#if IT_CHAIN_FLOADS_EARLY
+            // the down rows of this wave's output row, for stage F: issued behind the publication, they land while the intermediates travel
             // (four picks a step over 16 lanes each, the shared row beside the last two picks)
 #pragma unroll
             for (int s = 0; s < 3; s++) {
@@ -613,24 +667,17 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             }
             if (SF == W_Q8_0) load_row<W_Q8_0, 1, 32>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 31, lane >= 32);
             else load_row<W_NVFP4, 1, 16>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 15, lane >= 32 && lane < 48);
-            // the picks' weights for stage F, and what the seam shows of the route (block 0)
-            if (tid < NU) {
-                const int ex = ids[tid];
-                const float w = wts[tid] / denom;
-                coef[tid] = w * my_dscale;
-                if (b == 0) {
-                    f.route_ids[tid] = ex;
-                    f.route_w[tid] = w;
-                    if (f.counts_gate) atomicAdd(f.counts_gate + ex, 1u);
-                    if (f.counts_up) atomicAdd(f.counts_up + ex, 1u);
-                    if (f.counts_down) atomicAdd(f.counts_down + ex, 1u);
-                }
+#endif
+            // the softmax's sum: exp(logit - largest logit) over the 512, by wave and then over the waves in order
+            {
+                const float part = group_sum_tail<64>(fx_expf(my_logit - wts[0]));
+                if (lane == 63) route_sh.redf[wave] = part;
             }
-            if (b == 0 && tid == 0 && p.tally)
-                atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
             CH_STAMP(15);
+            CH_WSTAMP(5);
+            __syncthreads();
+            CH_WSTAMP(6);
             if (b < EB) {
-                __syncthreads();
                 if (tid < 8) {
                     // Q8_0 of the block's 32 intermediates (naive.rs:652-675), published as four quants a word
                     const float4 v = *(const float4*)(inter + tid * 4);
@@ -649,6 +696,46 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                     ll_put(p.ll + RE + b * 8 + tid, packed, e);
                     if (tid == 0) ll_putf(p.ll + RE_SC + b, it_f16_to_f32(it_f32_to_f16(d)), e);
                 }
+            }
+#if !IT_CHAIN_FLOADS_EARLY
+            // the down rows of this wave's output row, for stage F: issued behind the publication, they land while the intermediates travel
+            // (four picks a step over 16 lanes each, the shared row beside the last two picks)
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                const int y = s * 4 + (lane >> 4);
+                const bool routed = y < NU;
+                const int64_t ex = routed ? ids[y] : 0;
+                load_row<W_NVFP4, 1, 16>(fd[s], f.ed_q + ex * f.d_q_stride, f.ed_s + ex * f.d_s_stride, FF, my_row, lane & 15, routed);
+            }
+            if (SF == W_Q8_0) load_row<W_Q8_0, 1, 32>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 31, lane >= 32);
+            else load_row<W_NVFP4, 1, 16>(fsh, f.sd_q, f.sd_s, FF, my_row, lane & 15, lane >= 32 && lane < 48);
+#endif
+            // the picks' weights for stage F (probability over the sum of the ten, naive.rs:362-376), and what the seam
+            // shows of the route (block 0): lane r of the first wave has pick r
+            if (wave == 0) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < CT / 64; i++) sum += route_sh.redf[i];
+                const float prob = lane < NU ? fx_expf(wts[lane] - wts[0]) / sum : 0.0f;
+                float denom = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    denom += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, prob), r));
+                denom = fmaxf(denom, 6.103515625e-5f);
+                if (lane < NU) {
+                    const int ex = ids[lane];
+                    const float w = prob / denom;
+                    coef[lane] = w * my_dscale;
+                    if (b == 0) {
+                        f.route_ids[lane] = ex;
+                        f.route_w[lane] = w;
+                        if (f.counts_gate) atomicAdd(f.counts_gate + ex, 1u);
+                        if (f.counts_up) atomicAdd(f.counts_up + ex, 1u);
+                        if (f.counts_down) atomicAdd(f.counts_down + ex, 1u);
+                    }
+                }
+                if (b == 0 && lane == 0 && p.tally)
+                    atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
             }
         }
         // the next layer's in-projection rows start moving now: one stage ahead of their use
