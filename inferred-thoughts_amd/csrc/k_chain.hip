@@ -87,11 +87,14 @@ __device__ long long it_chain_wave_stamps[8][8];
 #endif
 
 // Where the prefetches sit (tuning switches; the defaults are what measured best).
+#ifndef IT_CHAIN_TOUCH
+#define IT_CHAIN_TOUCH 1          // stage E's rows touched by the blocks that have none of their own
+#endif
 #ifndef IT_CHAIN_FLOADS_EARLY
 #define IT_CHAIN_FLOADS_EARLY 0   // stage F's down rows: 1 ahead of stage E's barrier and publication, 0 behind them
 #endif
 #ifndef IT_CHAIN_WC_AT
-#define IT_CHAIN_WC_AT 0      // out-projection row: 0 at the head of stage B, 1 after stage A's input has arrived, 2 after stage A's dots
+#define IT_CHAIN_WC_AT 0      // out-projection row: 0 at the head of stage B, 1 after stage A's input has arrived, 2 after stage A's dots, 3 after stage B's input has arrived
 #endif
 #ifndef IT_CHAIN_D_AT
 #define IT_CHAIN_D_AT 1       // stage D's rows: 0 at the head of stage C, 1 after stage B's input has arrived
@@ -454,6 +457,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (dead) break;
                 CH_STAMP(2);
                 if (IT_CHAIN_D_AT) fetch_d();
+                if (IT_CHAIN_WC_AT == 3) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
                 if (tid < 2 * DK) {
                     const int w2 = tid < DK ? 0 : 2;
                     const double sum = red[w2] + red[w2 + 1];
@@ -623,6 +627,31 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             CH_STAMP(9);
             CH_WSTAMP(1);
             const float my_dscale = (tid < NU && f.dscale2) ? f.dscale2[ids[tid]] : 1.0f;   // issued ahead of the rows below
+            // Rows pulled towards the caches ahead of the loads that use them.  A wave's 16-byte-a-lane load asks for eight
+            // 128-byte lines; one 4-byte load with every lane on a line of its own asks for 64, so a few such loads put a
+            // whole stage's rows in flight at once, from compute units that have nothing else to fetch.
+            // The blocks without routed rows (160..255) touch the gate / up rows of the 20 blocks that share their XCD
+            // (blocks are dealt to the eight XCDs in turn, each XCD has its own L2): 9 loads a block served.
+            uint32_t touched = 0;
+            if (IT_CHAIN_TOUCH) {
+                if (b >= EB) {
+                    const int x = b & 7;
+                    for (int wi = ((b - EB) >> 3) * CW + wave; wi < 20 * 9; wi += 12 * CW) {
+                        const int tb = x + 8 * (wi / 9), part = wi % 9;
+                        const int64_t ex = ids[tb >> 4];
+                        const int r0 = (tb & 15) * 32;
+                        const uint8_t* a;
+                        if (part < 8) {   // eight rows of 1,024 bytes: gate (parts 0..3) or up (4..7)
+                            const uint8_t* q = (part < 4 ? f.eg_q : f.eu_q) + ex * f.gu_q_stride;
+                            a = q + (int64_t)(r0 + (part & 3) * 8 + (lane >> 3)) * (D / 2) + (lane & 7) * 128;
+                        } else {          // the scales of the 32 gate rows (lanes 0..31) and of the 32 up rows
+                            const uint8_t* sc = (lane < 32 ? f.eg_s : f.eu_s) + ex * f.gu_s_stride;
+                            a = sc + (int64_t)(r0 + (lane & 31)) * (D / 16);
+                        }
+                        touched += *(const volatile uint32_t*)a;
+                    }
+                }
+            }
             // the picks' rows: this block's 32 gate and 32 up rows
             WChunks<1> tg[4], tu[4];
             float scg = 1.0f, scu = 1.0f;
@@ -737,6 +766,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (b == 0 && lane == 0 && p.tally)
                     atomicAdd(p.tally, (unsigned long long)((f.counts_gate ? 1 : 0) + (f.counts_up ? 1 : 0) + (f.counts_down ? 1 : 0)) * NU);
             }
+            asm volatile("" ::"v"(touched));
         }
         // the next layer's in-projection rows start moving now: one stage ahead of their use
         CH_STAMP(10);
