@@ -87,6 +87,12 @@ __device__ long long it_chain_wave_stamps[8][8];
 #endif
 
 // Where the prefetches sit (tuning switches; the defaults are what measured best).
+#ifndef IT_CHAIN_F_POLLERS
+#define IT_CHAIN_F_POLLERS 1     // stage F's input gathered by waves 4..7 alone (1) or by every thread (0)
+#endif
+#ifndef IT_CHAIN_B_POLLERS
+#define IT_CHAIN_B_POLLERS 1     // stage B's input gathered by waves 5..7 alone (1) or by the first 274 threads (0)
+#endif
 #ifndef IT_CHAIN_TOUCH
 #define IT_CHAIN_TOUCH 1          // stage E's rows touched by the blocks that have none of their own
 #endif
@@ -270,14 +276,7 @@ IT_DEV float logit_of_order(uint32_t o) { return __uint_as_float((o & 0x80000000
 
 // rms_norm (naive.rs:633-650) of the 2,048 floats the block's threads hold as quads, then Q8_0 (naive.rs:652-675)
 // into xq / xs.  Two barriers; returns false after the first when the block has to stop.
-IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
-    const double part = wave_sum_f64_tail(quad_sumsq(v));
-    if ((tid & 63) == 63) red[tid >> 6] = part;
-    __syncthreads();
-    if (*dead) return false;
-    double sum = 0.0;
-#pragma unroll
-    for (int i = 0; i < CW; i++) sum += red[i];
+IT_DEV void norm_quant_finish(float4 v, float4 w, float eps, double sum, int8_t* xq, float* xs, int tid) {
     const float mean = (float)(sum / (double)D);
     const float scale = 1.0f / sqrtf(mean + eps);
     v.x = v.x * scale * w.x;
@@ -286,6 +285,16 @@ IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, dou
     v.w = v.w * scale * w.w;
     quant_quad(v, true, tid, xq, xs);
     __syncthreads();
+}
+IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
+    const double part = wave_sum_f64_tail(quad_sumsq(v));
+    if ((tid & 63) == 63) red[tid >> 6] = part;
+    __syncthreads();
+    if (*dead) return false;
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < CW; i++) sum += red[i];
+    norm_quant_finish(v, w, eps, sum, xq, xs, tid);
     return true;
 }
 
@@ -433,7 +442,51 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             // ---------------------------------------------------------------- B: delta rule
             CH_STAMP(1);
             // (the out-projection's row goes out first: small loads issued at the head of a stage are back before its input is)
+#if IT_CHAIN_B_POLLERS
+            // Waves 5..7 gather the stage's 290 words and issue their out-projection row only afterwards; waves 0..4 issue
+            // theirs now and poll nothing: a poll returns behind everything its own wave has in flight.
+            if (wave < 5) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+            float k_scale, q_scale;
+            {
+                bool ok = true;
+                if (wave >= 5) {
+                    const int pt = tid - 5 * 64;
+                    if (pt < DK) {   // wave 5: the key head's k as 64 pairs, wave 6: its q
+                        const int i2 = (pt & 63) * 2;
+                        const u64* const a1[1] = {p.ll + (pt < 64 ? RA + KDIM : RA) + kh * DK + i2};
+                        uint32_t o[2];
+                        ok = ll_wait_pairs<1>(a1, e, ctl, o);
+                        const float x0 = __uint_as_float(o[0]), x1 = __uint_as_float(o[1]);
+                        *(float2*)(kq + (pt < 64 ? 0 : DK) + i2) = make_float2(x0, x1);
+                        // l2 norm: the vector's sum of squares in its own wave (f64 sums of f32 squares: exact, so the
+                        // order of the terms does not matter)
+                        const double part = wave_sum_f64_tail((double)(x0 * x0) + (double)(x1 * x1));
+                        if (lane == 63) red[wave - 5] = part;
+                    } else if (pt < DK + 16) {   // 8 pairs of v, 8 pairs of z
+                        const int i2 = ((pt - DK) & 7) * 2, j = h * DK + j0 + i2;
+                        const bool zz = pt >= DK + 8;
+                        const u64* const a1[1] = {p.ll + (zz ? RA_Z : RA + 2 * KDIM) + j};
+                        uint32_t o[2];
+                        ok = ll_wait_pairs<1>(a1, e, ctl, o);
+                        sm[(zz ? 16 : 0) + i2] = __uint_as_float(o[0]);
+                        sm[(zz ? 16 : 0) + i2 + 1] = __uint_as_float(o[1]);
+                    } else if (pt < DK + 18) {
+                        uint32_t w0 = 0;
+                        ok = ll_wait1(p.ll + (pt == DK + 16 ? RA_AL : RA_BE) + h, e, ctl, &w0);
+                        sm[32 + pt - (DK + 16)] = __uint_as_float(w0);
+                    }
+                    load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+                }
+                if (!ok) dead = 1;
+                __syncthreads();
+                if (dead) break;
+                CH_STAMP(2);
+                if (IT_CHAIN_D_AT) fetch_d();
+                k_scale = 1.0f / fmaxf(sqrtf((float)red[0]), m.eps_l2);
+                q_scale = 1.0f / fmaxf(sqrtf((float)red[1]), m.eps_l2);
+#else
             if (!IT_CHAIN_WC_AT) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
+            const float k_scale = 1.0f, q_scale = 1.0f;
             {
                 uint32_t w0 = 0, w1 = 0;
                 bool ok = true;
@@ -464,6 +517,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                     kq[tid] = kqv * (1.0f / fmaxf(sqrtf((float)sum), m.eps_l2));
                 }
                 __syncthreads();
+#endif
                 const float a = sm[32] + dt_bias;
                 const float softplus = a > 20.0f ? a : fx_logf(1.0f + fx_expf(a));
                 const float g = fx_expf(softplus * ssm_a);
@@ -471,7 +525,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 const int j = tid >> 5, seg = tid & 31;
                 const float4 kk = *(const float4*)(kq + seg * 4), qq = *(const float4*)(kq + DK + seg * 4);
                 float row[4] = {st.x, st.y, st.z, st.w};
-                const float kv[4] = {kk.x, kk.y, kk.z, kk.w}, qv[4] = {qq.x, qq.y, qq.z, qq.w};
+                const float kv[4] = {kk.x * k_scale, kk.y * k_scale, kk.z * k_scale, kk.w * k_scale};
+                const float qv[4] = {qq.x * q_scale, qq.y * q_scale, qq.z * q_scale, qq.w * q_scale};
                 float pred = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -771,24 +826,60 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         // the next layer's in-projection rows start moving now: one stage ahead of their use
         CH_STAMP(10);
         const bool next_mixer = l + 1 < p.n_layers && p.layer[l + 1].has_mixer == 1;
-        if (l + 1 == p.n_layers && p.has_tail) fetch_tail(p.tail, aw, b, wave, lane);
-        if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
+        // (the waves that gather stage F's input issue theirs behind that gather: a poll returns behind everything its
+        // own wave has in flight)
+        auto fetch_next = [&]() {
+            if (l + 1 == p.n_layers && p.has_tail) fetch_tail(p.tail, aw, b, wave, lane);
+            if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
+        };
+        if (!IT_CHAIN_F_POLLERS || wave < 4) fetch_next();
 
         // -------------------------------------------------------------------- F: down, combine, residual
         {
-            // 1,440 words of quantized routed intermediates (pairs tid and tid + 512), the shared ones as quads
-            const int pr1 = tid + CT;
-            const bool two = pr1 < (NU * FF / 4 + EB) / 2, sq = tid < FF / 4;
-            const u64* const a4[4] = {p.ll + RE + 2 * tid, two ? p.ll + RE + 2 * pr1 : p.ll + RE + 2 * tid,
-                                      sq ? p.ll + RS + 4 * tid : p.ll + RE + 2 * tid, sq ? p.ll + RS + 4 * tid + 2 : p.ll + RE + 2 * tid};
-            uint32_t o[8];
-            const bool ok = ll_wait_pairs<4>(a4, e, ctl, o);
             uint32_t* dst = (uint32_t*)xq;
             // word i < 1,280 is quad i of the routed quants; the rest are the 160 block scales
             auto place = [&](int i, uint32_t v) {
                 if (i < NU * FF / 4) dst[i] = v;
                 else xs[i - NU * FF / 4] = __uint_as_float(v);
             };
+            bool ok = true;
+#if IT_CHAIN_F_POLLERS
+            // Waves 4..7 gather: the 720 pairs of words of the routed intermediates (quants, then scales) and, waves 4 and
+            // 5, the shared ones as quads (whole waves: the quantization's lane exchange needs its eight neighbours).
+            if (wave >= 4) {
+                const int pt = tid - 4 * 64, q = pt - 128;
+                constexpr int PAIRS = (NU * FF / 4 + EB) / 2;
+                const int p2 = wave < 6 ? -1 : 512 + q, p3 = (wave >= 6 && 640 + q < PAIRS) ? 640 + q : -1;
+                const u64* const a4[4] = {p.ll + RE + 2 * pt, p.ll + RE + 2 * (pt + 256),
+                                          wave < 6 ? p.ll + RS + 4 * pt : p.ll + RE + 2 * p2,
+                                          wave < 6 ? p.ll + RS + 4 * pt + 2 : p.ll + RE + 2 * (p3 >= 0 ? p3 : pt)};
+                uint32_t o[8];
+                ok = ll_wait_pairs<4>(a4, e, ctl, o);
+                place(2 * pt, o[0]);
+                place(2 * pt + 1, o[1]);
+                place(2 * (pt + 256), o[2]);
+                place(2 * (pt + 256) + 1, o[3]);
+                if (wave < 6) {
+                    const float4 v = make_float4(__uint_as_float(o[4]), __uint_as_float(o[5]), __uint_as_float(o[6]), __uint_as_float(o[7]));
+                    quant_quad(v, true, pt, xq + NU * FF, xs + EB);
+                } else {
+                    place(2 * p2, o[4]);
+                    place(2 * p2 + 1, o[5]);
+                    if (p3 >= 0) {
+                        place(2 * p3, o[6]);
+                        place(2 * p3 + 1, o[7]);
+                    }
+                }
+                fetch_next();
+            }
+#else
+            // 1,440 words of quantized routed intermediates (pairs tid and tid + 512), the shared ones as quads
+            const int pr1 = tid + CT;
+            const bool two = pr1 < (NU * FF / 4 + EB) / 2, sq = tid < FF / 4;
+            const u64* const a4[4] = {p.ll + RE + 2 * tid, two ? p.ll + RE + 2 * pr1 : p.ll + RE + 2 * tid,
+                                      sq ? p.ll + RS + 4 * tid : p.ll + RE + 2 * tid, sq ? p.ll + RS + 4 * tid + 2 : p.ll + RE + 2 * tid};
+            uint32_t o[8];
+            ok = ll_wait_pairs<4>(a4, e, ctl, o);
             place(2 * tid, o[0]);
             place(2 * tid + 1, o[1]);
             if (two) {
@@ -799,6 +890,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 const float4 v = make_float4(__uint_as_float(o[4]), __uint_as_float(o[5]), __uint_as_float(o[6]), __uint_as_float(o[7]));
                 quant_quad(v, true, tid, xq + NU * FF, xs + EB);
             }
+#endif
             if (!ok) dead = 1;
             __syncthreads();
             if (dead) break;
