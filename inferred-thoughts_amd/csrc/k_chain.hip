@@ -106,7 +106,7 @@ __device__ long long it_chain_wave_stamps[8][8];
 #define IT_CHAIN_D_AT 1       // stage D's rows: 0 at the head of stage C, 1 after stage B's input has arrived
 #endif
 #ifndef IT_CHAIN_A_AT
-#define IT_CHAIN_A_AT 0x034   // next in-projection, a hex digit of fetch_a parts per site: after D's input | after E's publish | after F's input
+#define IT_CHAIN_A_AT 0x070   // next in-projection, a hex digit of fetch_a parts per site: after D's input | after E's publish | after F's input
 #endif
 
 struct Ctl {
