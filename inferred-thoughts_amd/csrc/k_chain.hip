@@ -86,6 +86,9 @@ __device__ long long it_chain_wave_stamps[8][8];
     } while (0)
 #endif
 
+#ifndef IT_CHAIN_FP4_HW
+#define IT_CHAIN_FP4_HW 1         // NVFP4 rows of stages D and E through the hardware's fp4 / fp8 conversions (1) or through v_perm_b32 + v_dot4 (0)
+#endif
 // Where the prefetches sit (tuning switches; the defaults are what measured best).
 #ifndef IT_CHAIN_F_POLLERS
 #define IT_CHAIN_F_POLLERS 1     // stage F's input gathered by waves 4..7 alone (1) or by every thread (0)
@@ -266,6 +269,59 @@ IT_DEV void fetch_tail(const ChainTail& t, AW& a, int b, int wave, int lane) {
     const bool kk = wave < 2;
     load_row<W_Q8_0, 2, 64>(a.t[4], kk ? t.k_q : t.v_q, kk ? t.k_s : t.v_s, D, b + NB * (wave & 1), lane, wave < 4);
 }
+
+// An NVFP4 chunk against the activation through gfx950's own conversions: v_cvt_scalef32_pk_f16_fp4 turns one byte (two
+// e2m1 nibbles) into two f16 and v_dot2_f32_f16 multiplies them with two f16 activations, 2 instructions for 2 elements
+// where nibbles -> int8 through v_perm_b32 + v_dot4 takes 7 for 4.  The activations are the Q8_0 quants as f16 (exact),
+// paired as the nibbles of a byte are (element j with element 8 + j of a 16-element sub-block); every product and sum is
+// a multiple of 0.5 below 2^24, so the f32 accumulation is exact and the result is the integer path's, bit for bit.
+// The sub-block scales come from v_cvt_pk_f32_fp8 (OCP e4m3; the format's ue4m3 is half of that, and the e2m1 values
+// here are half of the integer path's doubled ones: the two factors of 2 cancel; code 0x7f is 0 as in it_ue4m3_to_f32).
+#if IT_CHAIN_FP4_HW
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+typedef float f2v __attribute__((ext_vector_type(2)));
+struct XN {
+    uint32_t p[16];   // sub-block A: pairs (j, 8 + j) j = 0..7, then sub-block B
+    float d;
+};
+IT_DEV uint32_t pair_h(uint32_t lo, uint32_t hi, int j) {
+    const h2v v = {(_Float16)(int)(int8_t)(lo >> (8 * j)), (_Float16)(int)(int8_t)(hi >> (8 * j))};
+    return __builtin_bit_cast(uint32_t, v);
+}
+IT_DEV void load_xn(XN& x, const int8_t* xq, const float* xs, int lane) {
+    XChunks<W_NVFP4, 1> t;
+    load_x<W_NVFP4, 1, 64>(t, xq, xs, lane);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        x.p[j] = pair_h(t.a[0].x, t.a[0].z, j);
+        x.p[4 + j] = pair_h(t.a[0].y, t.a[0].w, j);
+        x.p[8 + j] = pair_h(t.b[0].x, t.b[0].z, j);
+        x.p[12 + j] = pair_h(t.b[0].y, t.b[0].w, j);
+    }
+    x.d = t.d[0];
+}
+#define IT_FP4_STEP(acc, word, sel, pi) \
+    acc = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, 1.0f, sel), __builtin_bit_cast(h2v, x.p[pi]), acc, false)
+IT_DEV float dot_xn(const WChunks<1>& t, const XN& x) {
+    const uint4 w = t.w[0];
+    float sa = 0.0f, sb = 0.0f;
+    IT_FP4_STEP(sa, w.x, 0, 0); IT_FP4_STEP(sa, w.x, 1, 1); IT_FP4_STEP(sa, w.x, 2, 2); IT_FP4_STEP(sa, w.x, 3, 3);
+    IT_FP4_STEP(sa, w.y, 0, 4); IT_FP4_STEP(sa, w.y, 1, 5); IT_FP4_STEP(sa, w.y, 2, 6); IT_FP4_STEP(sa, w.y, 3, 7);
+    IT_FP4_STEP(sb, w.z, 0, 8); IT_FP4_STEP(sb, w.z, 1, 9); IT_FP4_STEP(sb, w.z, 2, 10); IT_FP4_STEP(sb, w.z, 3, 11);
+    IT_FP4_STEP(sb, w.w, 0, 12); IT_FP4_STEP(sb, w.w, 1, 13); IT_FP4_STEP(sb, w.w, 2, 14); IT_FP4_STEP(sb, w.w, 3, 15);
+    const uint32_t sc = t.sc[0] & 0x7f7fu;
+    const f2v s2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)sc, false);
+    const float dA = (sc & 0x7fu) == 0x7fu ? 0.0f : s2.x, dB = (sc >> 8) == 0x7fu ? 0.0f : s2.y;
+    float acc = 0.0f;
+    acc += (x.d * dA) * sa;
+    acc += (x.d * dB) * sb;
+    return acc;
+}
+#else
+typedef XChunks<W_NVFP4, 1> XN;
+IT_DEV void load_xn(XN& x, const int8_t* xq, const float* xs, int lane) { load_x<W_NVFP4, 1, 64>(x, xq, xs, lane); }
+IT_DEV float dot_xn(const WChunks<1>& t, const XN& x) { return dot_chunks<W_NVFP4, 1>(t, x); }
+#endif
 
 // a float's bits as an unsigned that orders like the value (negative below positive), and back
 IT_DEV uint32_t logit_order(float v) {
@@ -598,7 +654,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
 
         // -------------------------------------------------------------------- D: router, shared gate logit, shared gate / up
         CH_STAMP(5);
-        XChunks<W_NVFP4, 1> xn;
+        XN xn;
         {
             const float4 nw = ((const float4*)f.norm_w)[tid];
             float4 v;
@@ -613,7 +669,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             CH_STAMP(6);
             XChunks<W_Q8_0, 2> x;
             load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
-            load_x<W_NVFP4, 1, 64>(xn, xq, xs, lane);
+            load_xn(xn, xq, xs, lane);
             if (wave < 2 || (wave == 4 && b == NB - 1)) {
                 const float a = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
                 if (lane == 63) ll_putf(p.ll + RD + (wave < 2 ? b + NB * wave : NE), a, e);
@@ -623,8 +679,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                     ag = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
                     au = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d1, x));
                 } else {
-                    ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(n0, xn));
-                    au = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(n1, xn));
+                    ag = reduce_lanes<64>(dot_xn(n0, xn));
+                    au = reduce_lanes<64>(dot_xn(n1, xn));
                 }
                 if (lane == 63) {
                     ag *= f.sh_gscale;
@@ -727,8 +783,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 CH_WSTAMP(2);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    float ag = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tg[i], xn));
-                    float au = reduce_lanes<64>(dot_chunks<W_NVFP4, 1>(tu[i], xn));
+                    float ag = reduce_lanes<64>(dot_xn(tg[i], xn));
+                    float au = reduce_lanes<64>(dot_xn(tu[i], xn));
                     if (lane == 63) {
                         ag *= scg;
                         au *= scu;
