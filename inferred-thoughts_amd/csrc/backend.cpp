@@ -267,10 +267,11 @@ float* it_hip::act_in(const float* host, size_t len) {
     if (!a->dev_current) {
         if (mode != Mode::Eager) {
             precopies.push_back(PreCopy{a->dev, host, len * sizeof(float)});
-        } else if ((held.empty() || (release_held(), true)) &&
-                   !check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream),
-                          "upload activation")) {
-            return nullptr;
+        } else {
+            // ops held back run later than this copy: if one of them touches the buffer, it has to run first
+            if (!held.empty() && held_touches(a->dev, a->cap * sizeof(float))) release_held();
+            if (!check(hipMemcpyAsync(a->dev, host, len * sizeof(float), hipMemcpyHostToDevice, stream), "upload activation"))
+                return nullptr;
         }
         h2d++;
         h2d_bytes += len * sizeof(float);
@@ -286,6 +287,13 @@ float* it_hip::act_out(const float* host, size_t len) {
     a->elided = false;
     a->q_valid = false;
     return a->dev;
+}
+bool it_hip::held_touches(const void* dev, size_t bytes) const {
+    const char* lo = (const char*)dev;
+    for (const OpRec& op : held)
+        for (const void* q : op.p)
+            if (q && (const char*)q >= lo && (const char*)q < lo + bytes) return true;
+    return false;
 }
 it_hip::Act* it_hip::act_by_dev(const void* dev) {
     for (auto& kv : acts) {
@@ -1223,6 +1231,7 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->chain_enabled = (flags & IT_HIP_NO_CHAIN) == 0 && getenv("INFERRED_HIP_NO_CHAIN") == nullptr;
     be->eager_fused = getenv("INFERRED_HIP_EAGER_FUSED") != nullptr;
     be->count_reads_in_fused = getenv("INFERRED_HIP_NO_READ_COUNTERS") == nullptr;
+    be->small_ffn_enabled = getenv("INFERRED_HIP_NO_SMALL_FFN") == nullptr;
     if (getenv("INFERRED_HIP_NO_GRAPH")) be->allow_graph = false;
     if (const char* sl = getenv("INFERRED_HIP_CHAIN_SPINS")) {
         const long v = atol(sl);

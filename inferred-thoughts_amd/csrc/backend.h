@@ -81,6 +81,7 @@ struct it_hip {
                        float** dev_x);
     bool act_q_reserve(Act& a, size_t len);  // room for the Q8_0 form of `len` floats
     Act* act_by_dev(const void* dev);        // the mirror whose device buffer holds `dev`, or null
+    bool held_touches(const void* dev, size_t bytes) const;   // an op held back reads or writes inside [dev, dev + bytes)
     // marks the mirrors at these device addresses as not holding their ops' values (a fused kernel skipped the writes):
     // a host read of one raises the sticky error instead of returning what the buffer happens to hold
     void mark_elided(const std::vector<const void*>& devs);
@@ -278,6 +279,8 @@ struct it_hip {
     int hold_step(const OpRec& rec) const;   // 0: not part of a run, 1: continues it, 2: completes it
     void release_held();                     // the run broke off: issue what is held op by op, in order
     void finish_held();                      // the run is complete: one kernel (or op by op when its shape is not taken)
+    bool small_ffn(const std::vector<OpRec>& run);   // the routed FFN of a short batch as two launches
+    bool small_ffn_enabled = true;           // INFERRED_HIP_NO_SMALL_FFN=1 issues it op by op (a measurement switch)
     std::vector<PreCopy> precopies;  // host -> device inputs of a graphed pass, issued before the graph
     int* dyn_dev = nullptr;    // device ints read by position-dependent kernels
     // pinned staging, double-buffered: a pass may fill one while the previous pass's async

@@ -8,6 +8,8 @@
 // scales — is simply issued op by op.  A fused launch sits at the position of its
 // block's first op; everything it replaces is dropped, except an activation
 // quantization that some unfused op still reads.
+#include <cstdio>
+#include <cstdlib>
 #include "backend.h"
 
 using namespace itk;
@@ -848,14 +850,63 @@ bool references(const Op& op, const void* a, const void* b) {
 //                                                          not written: nothing else in the loop reads them)
 //   RMS_HEADS core, EW silu_mul(z, core), QUANT z        -> gated_norm_silu_q8 (core is left unnormed)
 // The ops are held back as they arrive and checked link by link (an op's input must be the run's own buffer).
+// The routed FFN of a short batch (2..32 tokens; src/model/qwen35.rs:1630-1700) as a run:
+//   SOFTMAX, ROUTE, [QUANT x], GLU, QUANT g, EXPERTS, MATMUL shared gate, MATMUL shared up, [SCALE]*, EW silu_mul,
+//   QUANT, MATMUL shared down, [SCALE], FINISH
+// Where the run stands follows from what is held; an op is accepted by its kind here, and the links between the ops
+// (whose output feeds whom, the shapes) are checked once the run is complete: a run that fails there is issued op by op.
+namespace {
+constexpr int SMALL_FFN_MAX = 32;   // tokens (measured on the 512-expert top-10 layer: 176 against 232 us at 32, 271 against 298 at 48, behind from about 56 on)
+enum FfnAt { F_ROUTE = 1, F_QX_OR_GLU, F_GLU, F_QG, F_EXPERTS, F_SG, F_SU, F_SCALE_OR_SILU, F_QS, F_SD, F_SCALE_OR_FINISH, F_FINISH };
+int ffn_at(const std::vector<it_hip::OpRec>& held) {   // what may come next
+    int at = F_ROUTE;
+    for (size_t k = 1; k < held.size(); k++) {
+        const int id = held[k].id;
+        switch (at) {
+            case F_ROUTE: at = F_QX_OR_GLU; break;
+            case F_QX_OR_GLU: at = id == OP_QUANT ? F_GLU : F_QG; break;
+            case F_GLU: at = F_QG; break;
+            case F_QG: at = F_EXPERTS; break;
+            case F_EXPERTS: at = F_SG; break;
+            case F_SG: at = F_SU; break;
+            case F_SU: at = F_SCALE_OR_SILU; break;
+            case F_SCALE_OR_SILU: at = id == OP_SCALE ? F_SCALE_OR_SILU : F_QS; break;
+            case F_QS: at = F_SD; break;
+            case F_SD: at = F_SCALE_OR_FINISH; break;
+            case F_SCALE_OR_FINISH: at = F_FINISH; break;
+            default: break;
+        }
+    }
+    return at;
+}
+}  // namespace
+
 int it_hip::hold_step(const OpRec& r) const {
     const size_t n = held.size();
     if (n == 0) {
         if (r.id == OP_CONV && r.i[2] >= 64 && r.i[1] % 128 == 0) return 1;
         if (r.id == OP_RMS_HEADS && r.i[0] == 128 && r.i[1] >= 256) return 1;
+        if (r.id == OP_SOFTMAX && r.i[0] >= 2 && r.i[0] <= SMALL_FFN_MAX && r.i[1] >= 16 && r.i[1] <= 2048 && !expert_cold_entries && small_ffn_enabled) return 1;
         return 0;
     }
     const OpRec& h0 = held[0];
+    if (h0.id == OP_SOFTMAX) {
+        switch (ffn_at(held)) {
+            case F_ROUTE: return r.id == OP_ROUTE && r.p[0] == h0.p[0] && r.i[0] == h0.i[0] && r.i[1] == h0.i[1] && r.i[2] <= 16 ? 1 : 0;
+            case F_QX_OR_GLU: return r.id == OP_QUANT || (r.id == OP_GLU && !r.i[8]) ? 1 : 0;
+            case F_GLU: return r.id == OP_GLU && !r.i[8] ? 1 : 0;
+            case F_QG: return r.id == OP_QUANT ? 1 : 0;
+            case F_EXPERTS: return r.id == OP_EXPERTS && !r.i[8] ? 1 : 0;
+            case F_SG:
+            case F_SU:
+            case F_SD: return r.id == OP_MATMUL ? 1 : 0;
+            case F_SCALE_OR_SILU: return r.id == OP_SCALE || (r.id == OP_EW && r.i[0] == 0) ? 1 : 0;
+            case F_QS: return r.id == OP_QUANT ? 1 : 0;
+            case F_SCALE_OR_FINISH: return r.id == OP_SCALE ? 1 : r.id == OP_FINISH ? 2 : 0;
+            case F_FINISH: return r.id == OP_FINISH ? 2 : 0;
+        }
+        return 0;
+    }
     if (h0.id == OP_CONV) {
         const int64_t nc = h0.i[1], nt = h0.i[2];
         if (n <= 3) {
@@ -887,10 +938,128 @@ void it_hip::release_held() {
     check(hipGetLastError(), "kernel launch");
 }
 
+// The complete FFN run of a short batch as two launches: gate / up with the route inside (every block ranks its
+// token's logits; grid row = token), then down + combine.  False, with nothing launched, when a link or a shape is not
+// what the kernels take.
+bool it_hip::small_ffn(const std::vector<OpRec>& h) {
+    size_t k = 0;
+    auto take = [&](int id) -> const OpRec* { return k < h.size() && h[k].id == id ? &h[k++] : nullptr; };
+    const OpRec *sm = take(OP_SOFTMAX), *rt = take(OP_ROUTE), *q1 = take(OP_QUANT), *glu = take(OP_GLU), *q2 = take(OP_QUANT);
+    const OpRec *ex = take(OP_EXPERTS), *sgm = take(OP_MATMUL), *sum_ = take(OP_MATMUL);
+    if (!sm || !rt || !glu || !q2 || !ex || !sgm || !sum_) return false;
+    float sh_scale[3] = {1.0f, 1.0f, 1.0f};   // gate, up, down
+    bool has_up = false, has_gate = false;
+    while (k < h.size() && h[k].id == OP_SCALE) {   // the up product is scaled first, then the gate product
+        const OpRec& sc = h[k];
+        if (!has_up && !has_gate && sc.p[0] == sum_->p[5] && sc.i[0] == sum_->i[2] * sum_->i[3]) {
+            sh_scale[1] = sc.f[0];
+            has_up = true;
+        } else if (!has_gate && sc.p[0] == sgm->p[5] && sc.i[0] == sgm->i[2] * sgm->i[3]) {
+            sh_scale[0] = sc.f[0];
+            has_gate = true;
+        } else {
+            return false;
+        }
+        k++;
+    }
+    const OpRec *sil = take(OP_EW), *q3 = take(OP_QUANT), *sdm = take(OP_MATMUL);
+    if (!sil || !q3 || !sdm) return false;
+    if (k < h.size() && h[k].id == OP_SCALE) {
+        const OpRec& sc = h[k];
+        if (sc.p[0] != sdm->p[5] || sc.i[0] != sdm->i[2] * sdm->i[3]) return false;
+        sh_scale[2] = sc.f[0];
+        k++;
+    }
+    const OpRec* fin = take(OP_FINISH);
+    if (!fin || k != h.size()) return false;
+
+    const int64_t nt = sm->i[0], ne = sm->i[1], nu = rt->i[2];
+    const int64_t nd = glu->i[1], ff = glu->i[2], sff = sgm->i[2];
+    const void* router = sm->p[0];
+    const void* x = sgm->p[2];   // the f32 activation: the shared expert's products read the same rows as the routed ones
+    if (nt < 2 || nt > SMALL_FFN_MAX || nu < 1 || nu > 16 || ne < nu) return false;
+    if (q1 && (q1->p[0] != x || q1->i[0] != nt * nd)) return false;
+    if (glu->p[6] != rt->p[1] || glu->p[7] != sgm->p[3] || glu->p[8] != sgm->p[4] || glu->i[3] != nt * nu || glu->i[4] != nu ||
+        glu->i[5] != 1 || !quantized_fmt(glu->i[0]))
+        return false;
+    const void* g_all = glu->p[9];
+    if (q2->p[0] != g_all || q2->i[0] != nt * nu * ff) return false;
+    if (ex->p[3] != rt->p[1] || ex->p[4] != q2->p[1] || ex->p[5] != q2->p[2] || ex->i[1] != ff || ex->i[2] != nd || ex->i[3] != nt * nu ||
+        ex->i[4] != nu || ex->i[5] != 0 || !quantized_fmt(ex->i[0]))
+        return false;
+    auto reads_x = [&](const OpRec& m) {
+        return m.p[2] == x && m.p[3] == sgm->p[3] && m.p[4] == sgm->p[4] && m.i[1] == nd && m.i[3] == nt && quantized_fmt(m.i[0]);
+    };
+    if (!reads_x(*sgm) || !reads_x(*sum_) || sum_->i[2] != sff || sum_->i[0] != sgm->i[0]) return false;
+    const void* e_gate = sgm->p[5];
+    if (sil->i[0] != 0 || sil->p[0] != e_gate || sil->p[1] != sum_->p[5] || sil->i[1] != nt * sff) return false;
+    if (q3->p[0] != e_gate || q3->i[0] != nt * sff) return false;
+    if (sdm->p[2] != e_gate || sdm->p[3] != q3->p[1] || sdm->p[4] != q3->p[2] || sdm->i[1] != sff || sdm->i[2] != nd || sdm->i[3] != nt ||
+        !quantized_fmt(sdm->i[0]))
+        return false;
+    if (fin->p[1] != ex->p[6] || fin->p[2] != rt->p[2] || fin->p[3] != sdm->p[5] || fin->i[1] != nd || fin->i[2] != nt || fin->i[3] != nu)
+        return false;
+
+    MoeGluP g{};
+    g.x = (const float*)x;
+    g.gq = (const uint8_t*)glu->p[0]; g.gs = (const uint8_t*)glu->p[1]; g.uq = (const uint8_t*)glu->p[2]; g.us = (const uint8_t*)glu->p[3];
+    g.gscale2 = (const float*)glu->p[4]; g.uscale2 = (const float*)glu->p[5];
+    g.q_stride = glu->i[6]; g.s_stride = glu->i[7];
+    g.fmt = (int)glu->i[0]; g.n_in = (int)nd; g.n_out = (int)ff; g.n_expert = (int)ne; g.n_used = (int)nu;
+    g.sh_gq = (const uint8_t*)sgm->p[0]; g.sh_gs = (const uint8_t*)sgm->p[1]; g.sh_uq = (const uint8_t*)sum_->p[0]; g.sh_us = (const uint8_t*)sum_->p[1];
+    g.sh_fmt = (int)sgm->i[0]; g.sh_n_out = (int)sff;
+    g.sh_gscale = sh_scale[0]; g.sh_uscale = sh_scale[1];
+    g.out = (float*)g_all; g.sh_out = (float*)e_gate;
+    g.logits = (const float*)router;
+    g.route_ids_out = (int32_t*)rt->p[1]; g.route_w_out = (float*)rt->p[2];
+    g.n_tok = (int)nt;
+    MoeDownP d{};
+    d.g_all = (const float*)g_all; d.g_shared = (const float*)e_gate;
+    d.q = (const uint8_t*)ex->p[0]; d.s = (const uint8_t*)ex->p[1]; d.scale2 = (const float*)ex->p[2];
+    d.q_stride = ex->i[6]; d.s_stride = ex->i[7];
+    d.fmt = (int)ex->i[0]; d.n_in = (int)ff; d.n_out = (int)nd; d.n_used = (int)nu;
+    d.sh_q = (const uint8_t*)sdm->p[0]; d.sh_s = (const uint8_t*)sdm->p[1]; d.sh_fmt = (int)sdm->i[0]; d.sh_n_in = (int)sff;
+    d.sh_dscale = sh_scale[2];
+    d.route_ids = (const int32_t*)rt->p[1]; d.route_w = (const float*)rt->p[2];
+    d.logit = (const float*)fin->p[4] + fin->i[4];
+    d.y = (float*)fin->p[0] + fin->i[0];
+    d.x = d.y;
+    d.n_tok = (int)nt;
+    if (count_reads_in_fused) {
+        d.counts_gate = (uint32_t*)glu->p[10];
+        d.counts_up = (uint32_t*)glu->p[11];
+        d.counts_down = (uint32_t*)ex->p[7];
+        d.tally = expert_tally;
+    }
+    if (!moe_glu_fast(g, stream, true) || !moe_down_fast(d, stream, true)) return false;
+    moe_glu_fast(g, stream);
+    moe_down_fast(d, stream);
+    // what the two launches do not write: the probabilities (the router buffer keeps its logits), the shared expert's
+    // up product, the pairs' down products, and every quantized form of the run
+    mark_elided({router, sum_->p[5], ex->p[6], sdm->p[5]});
+    for (const OpRec* q : {q1, q2, q3})
+        if (q)
+            if (Act* a = act_by_dev(q->p[0])) a->q_valid = false;
+    return true;
+}
+
 void it_hip::finish_held() {
     bool done = false;
     uint64_t bytes = 0;
     for (auto& op : held) bytes += op.bytes;
+    if (held[0].id == OP_SOFTMAX) {
+        {
+            Span sp(this, FAM_MOE_GLU, bytes);
+            done = small_ffn(held);
+        }
+        if (done) {
+            held.clear();
+            check(hipGetLastError(), "kernel launch");
+        } else {
+            release_held();
+        }
+        return;
+    }
     {
         Span sp(this, held[0].fam, bytes);
         if (held[0].id == OP_CONV && held.size() == 6) {

@@ -17,7 +17,7 @@
 // the expert cache's device-side read counters: one token's picks on the three tensors of a routed FFN
 IT_DEV void it_count_expert_reads(const int32_t* ids, int n_used, uint32_t* cg, uint32_t* cu, uint32_t* cd,
                                   unsigned long long* tally) {
-    if (blockIdx.x != 0 || blockIdx.y != 0 || !tally) return;
+    if (blockIdx.x != 0 || !tally) return;   // a grid row is a token (or, in the order-preserving kernels, never more than one)
     const int t = threadIdx.x;
     if (t < n_used) {
         const int e = ids[t];

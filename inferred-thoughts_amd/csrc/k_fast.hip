@@ -497,6 +497,19 @@ IT_DEV void glu_job(const uint8_t* gq, const uint8_t* gs, const uint8_t* uq, con
 
 template <int EF, int ECPL, int EL, int SF, int SCPL, int SL>
 __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
+    {   // a short batch: grid row t is token t
+        const int64_t t = blockIdx.y;
+        p.x += t * p.n_in;
+        p.out += t * p.n_used * p.n_out;
+        p.sh_out += t * p.sh_n_out;
+        if (p.logits) {
+            p.logits += t * p.n_expert;
+            p.route_ids_out += t * p.n_used;
+            p.route_w_out += t * p.n_used;
+        } else {
+            p.route_ids += t * p.n_used;
+        }
+    }
     __shared__ __align__(16) int8_t xq[FT * 8];
     __shared__ float xs[FT * 8 / 32];
     __shared__ double red[FW];
@@ -561,7 +574,7 @@ __global__ __launch_bounds__(FT) void moe_glu_fast_k(MoeGluP p, GluGeo gg) {
 
 }  // namespace
 
-bool moe_glu_fast(MoeGluP p, hipStream_t s) {
+bool moe_glu_fast(MoeGluP p, hipStream_t s, bool dry_run) {
     if (p.exact) return false;
     const Geo ge = geo_of(p.fmt, p.n_in), gs = geo_of(p.sh_fmt, p.n_in);
     if (!ge.ok || !gs.ok || p.n_in > FT * 8 || p.n_used > 16 || p.n_used < 1) return false;
@@ -582,6 +595,7 @@ bool moe_glu_fast(MoeGluP p, hipStream_t s) {
     int blocks = (total + FW - 1) / FW;
     if (blocks > 1024) blocks = 1024;
     if (blocks < 1) blocks = 1;
+    const int n_tok = p.n_tok > 1 ? p.n_tok : 1;
     // a grid between one and two blocks per CU leaves some CUs with twice the jobs of others (352 blocks on 256 CUs for
     // the 35B shape): two per CU everywhere, jobs dealt round the blocks, is 1 % of the token faster
     {
@@ -589,10 +603,13 @@ bool moe_glu_fast(MoeGluP p, hipStream_t s) {
         static const int n_cu = (hipGetDevice(&dev) == hipSuccess &&
                                  hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) ? cus : 256;
         if (blocks > n_cu && blocks < 2 * n_cu) blocks = 2 * n_cu;
+        // a short batch: about four blocks per CU in all (every block repeats its token's prologue and route, so a
+        // token's jobs go to fewer blocks, which loop over them)
+        if (n_tok > 1) blocks = std::max(32, std::min(blocks, 4 * n_cu / n_tok));
     }
     // the geometry of both formats follows from n_in: (CPL, L) for Q8_0 and for NVFP4
 #define IT_LAUNCH(EF, EC, EL, SF, SC, SL) \
-    hipLaunchKernelGGL((moe_glu_fast_k<EF, EC, EL, SF, SC, SL>), dim3(blocks), dim3(FT), 0, s, p, gg)
+    hipLaunchKernelGGL((moe_glu_fast_k<EF, EC, EL, SF, SC, SL>), dim3(blocks, n_tok), dim3(FT), 0, s, p, gg)
 #define IT_BY_FMT(QC, QL, NC, NL)                                                                       \
     do {                                                                                                \
         if (p.fmt == W_Q8_0 && p.sh_fmt == W_Q8_0) IT_LAUNCH(W_Q8_0, QC, QL, W_Q8_0, QC, QL);           \
@@ -600,6 +617,8 @@ bool moe_glu_fast(MoeGluP p, hipStream_t s) {
         else if (p.fmt == W_NVFP4 && p.sh_fmt == W_NVFP4) IT_LAUNCH(W_NVFP4, NC, NL, W_NVFP4, NC, NL);  \
         else IT_LAUNCH(W_Q8_0, QC, QL, W_NVFP4, NC, NL);                                                \
     } while (0)
+    if (p.n_in != 256 && p.n_in != 512 && p.n_in != 1024 && p.n_in != 2048 && p.n_in != 4096) return false;
+    if (dry_run) return true;
     switch (p.n_in) {
         case 256: IT_BY_FMT(1, 16, 1, 8); break;
         case 512: IT_BY_FMT(1, 32, 1, 16); break;
@@ -628,6 +647,16 @@ constexpr int MAXU = 16, QUARTU = MAXU / 4;
 // thread, and two waves a SIMD cover each other's waits.
 template <int EF, int ECPL, int L, int SF, int SCPL>
 __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
+    {   // a short batch: grid row t is token t
+        const int64_t t = blockIdx.y;
+        p.g_all += t * p.n_used * p.n_in;
+        p.g_shared += t * p.sh_n_in;
+        p.route_ids += t * p.n_used;
+        p.route_w += t * p.n_used;
+        p.logit += t;
+        p.x += t * p.n_out;
+        if (p.y) p.y += t * p.n_out;
+    }
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int P = 64 / L;
     const int n_in = p.n_in, sh_in = p.sh_n_in, NU = p.n_used;
@@ -667,7 +696,7 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
         }
     }
     if (quarter == 3) load_w<SF, SCPL, L>(tsh, p.sh_q, p.sh_s, sh_in, row, sub, live);
-    const float x_old = (!quarter && sub == L - 1 && live) ? p.x[row] : 0.0f;
+    const float x_old = (!quarter && sub == L - 1 && live && !p.y) ? p.x[row] : 0.0f;
     if (tid < NU) coef[tid] = p.route_w[tid] * (p.scale2 ? p.scale2[p.route_ids[tid]] : 1.0f);
     const float gate = fx_sigmoid(p.logit[0]) * p.sh_dscale;
     IT_STAMP(1);
@@ -698,14 +727,17 @@ __global__ __launch_bounds__(DT) void moe_down_fast_k(MoeDownP p) {
     if (quarter) partial[group][quarter - 1][lane] = acc;
     __syncthreads();
     IT_STAMP(5);
-    if (!quarter && sub == L - 1 && live)
-        p.x[row] = x_old + ((acc + partial[group][0][lane]) + (partial[group][1][lane] + partial[group][2][lane]));
+    if (!quarter && sub == L - 1 && live) {
+        const float sum = (acc + partial[group][0][lane]) + (partial[group][1][lane] + partial[group][2][lane]);
+        if (p.y) p.y[row] = sum;
+        else p.x[row] = x_old + sum;
+    }
     IT_STAMP(6);
 }
 
 }  // namespace
 
-bool moe_down_fast(MoeDownP p, hipStream_t s) {
+bool moe_down_fast(MoeDownP p, hipStream_t s, bool dry_run) {
     const Geo ge = geo_of(p.fmt, p.n_in);
     if (!ge.ok || ge.cpl != 1 || p.n_used > MAXU || p.n_used < 1) return false;
     const int L = ge.l;
@@ -724,7 +756,7 @@ bool moe_down_fast(MoeDownP p, hipStream_t s) {
     if (lds > 60 * 1024 || total > 3 * DT * 4) return false;
     const int P = 64 / L;
     const int blocks = (p.n_out + (DW / 4) * P - 1) / ((DW / 4) * P);
-#define IT_LAUNCH(EF, LL, SF, SC) hipLaunchKernelGGL((moe_down_fast_k<EF, 1, LL, SF, SC>), dim3(blocks), dim3(DT), lds, s, p)
+#define IT_LAUNCH(EF, LL, SF, SC) hipLaunchKernelGGL((moe_down_fast_k<EF, 1, LL, SF, SC>), dim3(blocks, p.n_tok > 1 ? p.n_tok : 1), dim3(DT), lds, s, p)
 #define IT_BY_L(EF, SF, SC)                      \
     do {                                         \
         if (L == 64) IT_LAUNCH(EF, 64, SF, SC);  \
@@ -732,6 +764,9 @@ bool moe_down_fast(MoeDownP p, hipStream_t s) {
         else if (L == 16) IT_LAUNCH(EF, 16, SF, SC); \
         else IT_LAUNCH(EF, 8, SF, SC);           \
     } while (0)
+    const bool fmts = (p.fmt == W_NVFP4 && (p.sh_fmt == W_Q8_0 || p.sh_fmt == W_NVFP4)) || (p.fmt == W_Q8_0 && p.sh_fmt == W_Q8_0);
+    if (!fmts) return false;
+    if (dry_run) return true;
     if (p.fmt == W_NVFP4 && p.sh_fmt == W_Q8_0) {
         if (scpl == 1) IT_BY_L(W_NVFP4, W_Q8_0, 1);
         else IT_BY_L(W_NVFP4, W_Q8_0, 2);

@@ -67,6 +67,9 @@ struct MoeGluP {
     const float* logits;
     int32_t* route_ids_out;
     float* route_w_out;
+    // fast mode, a short batch: token t of n_tok is grid row t, every per-token operand above (x, logits, the picks, out,
+    // sh_out) t vectors further on.  0 or 1: one token.
+    int n_tok;
 };
 void moe_glu_fused(MoeGluP p, hipStream_t s);
 
@@ -88,6 +91,10 @@ struct MoeDownP {
     // served from device memory; block 0 adds this token's picks
     uint32_t *counts_gate, *counts_up, *counts_down;
     unsigned long long* tally;
+    // fast mode, a short batch (see MoeGluP::n_tok); `y` set: the sums are stored there instead of added to x
+    // (moe_finish without the add_assign behind it)
+    int n_tok;
+    float* y;
 };
 void moe_down_fused(MoeDownP p, hipStream_t s);
 
@@ -107,8 +114,9 @@ void attn_prep(const AttnPrepP& p, hipStream_t s);
 // the shapes, formats or alignments fall outside what it handles; the caller then uses the
 // order-preserving kernel.
 bool fused_gemv_fast(FusedGemvP p, hipStream_t s);
-bool moe_glu_fast(MoeGluP p, hipStream_t s);
-bool moe_down_fast(MoeDownP p, hipStream_t s);
+// (dry_run: only say whether the shape is taken)
+bool moe_glu_fast(MoeGluP p, hipStream_t s, bool dry_run = false);
+bool moe_down_fast(MoeDownP p, hipStream_t s, bool dry_run = false);
 
 // ------------------------------------------------------------------ layer chain (k_chain.hip, fast mode)
 // A run of decode layers as ONE persistent kernel, one block per compute unit: the six dependent launches of a
