@@ -195,7 +195,6 @@ def expert_ffn_fused_decode(ih, seed=0, n_expert=512, n_used=10, nd=2048, ff=512
                           "Q8_0 router and shared expert as in the headline model")
     finally:
         be.close()
-        be_ffn.close()
 
 
 def attention_decode(ih, be, seed=0, contexts=(1024, 8192, 32000), n_head=16, n_head_kv=2, hd=256):
@@ -288,3 +287,4 @@ def run(ih, seed=0, exact=False, ffn_tokens=None):
                 "gated_delta_net_16k_32v_128": delta_net(ih, be, seed)}
     finally:
         be.close()
+        be_ffn.close()
