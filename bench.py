@@ -74,7 +74,7 @@ def summarize_profile(root_dir):
     def family(name, grid):
         n = short(name)
         if n.startswith("layer_chain_k"):
-            return "layer_chain (persistent kernel over a run of layers)"
+            return "layer_chain (a run of layers, persistent)"
         if n.startswith("fused_gemv_fast_k"):
             return "lm_head (norm + GEMV)" if grid >= 400000 else "fused_gemv (norm + quantize + dense GEMVs)"
         if n.startswith("moe_glu_fast_k"):

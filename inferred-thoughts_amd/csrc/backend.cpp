@@ -2467,7 +2467,7 @@ int it_hip_profile_end(it_hip* be, it_profile_row* rows, int max_rows) {
                                                    "norms", "router (softmax + top-k)", "other",
                                                    "fused_gemv (norm + quantize + dense GEMVs)", "lm_head (norm + GEMV)",
                                                    "gdn_rows (l2 norm + delta rule)", "attn_prep (norm + rope + kv write)",
-                                                   "layer_chain (persistent kernel over a run of layers)"};
+                                                   "layer_chain (a run of layers, persistent)"};
     be->prof_on = false;
     be->check(hipStreamSynchronize(be->stream), "sync");
     it_profile_row acc[it_hip::FAM_COUNT];
