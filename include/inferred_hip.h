@@ -247,6 +247,10 @@ void it_hip_reserve_for_weights(it_hip*, uint64_t dense_bytes); /* placement.rs:
 void it_hip_reserve_for_kv(it_hip*, uint64_t bytes);         /* placement.rs:341 */
 void it_hip_set_prefetch(it_hip*, int on);                   /* placement.rs:164; nothing to fetch when all resident */
 void it_hip_set_model_path(it_hip*, const char* path);       /* placement.rs:357 */
+/* reads of cold experts from the model file so far: out[0] through the unbuffered (O_DIRECT) descriptor, out[1] in all
+ * (src/ops/cuda/experts.rs:310-312, 510-511: on by default on Linux, INFERRED_FETCH_DIRECT=0 / =1 overrides, a file
+ * system that refuses the flag is read buffered) */
+void it_hip_fetch_read_counts(it_hip*, uint64_t out[2]);
 void it_hip_set_map_base(it_hip*, uint64_t base);            /* placement.rs:363 */
 /* lookups / hits come from the device counters (waits for the device), placement.rs:15 */
 void it_hip_expert_stats(it_hip*, it_expert_stats* out);

@@ -63,13 +63,21 @@ class ReadPool {
         cv_.notify_all();
         for (auto& t : threads_) t.join();
         if (fd_ >= 0) close(fd_);
+        if (dfd_ >= 0) close(dfd_);
+    }
+    // reads that went through the unbuffered descriptor, and reads in all
+    void counts(uint64_t* direct, uint64_t* all) {
+        std::lock_guard<std::mutex> g(m_);
+        *direct = n_direct_;
+        *all = n_reads_;
     }
     // read from `path` at (address - base) instead of copying out of the mapping; an empty path goes back to the mapping
     void source(const std::string& path, uint64_t base) {
         std::lock_guard<std::mutex> g(m_);
         if (path == path_ && base == base_) return;
         if (fd_ >= 0) close(fd_);
-        fd_ = -1;
+        if (dfd_ >= 0) close(dfd_);
+        fd_ = dfd_ = -1;
         file_size_ = 0;
         path_ = path;
         base_ = base;
@@ -82,6 +90,13 @@ class ReadPool {
         } else if (fd >= 0) {
             close(fd);
         }
+        // Unbuffered reads (platform.rs:60-96, 200-215; fetch.rs:71-73): the fetches of a token stay out of the page
+        // cache, which the mapping of the same file would otherwise share with them.  On by default, as in the
+        // reference on Linux; INFERRED_FETCH_DIRECT=0 / =1 overrides; a file system that refuses the flag (tmpfs) or a
+        // read that fails with it falls back to the buffered descriptor.
+        const char* e = getenv("INFERRED_FETCH_DIRECT");
+        const bool want = e ? strcmp(e, "0") != 0 : true;
+        if (want && fd_ >= 0) dfd_ = open(path.c_str(), O_RDONLY | O_CLOEXEC | O_DIRECT);
     }
     void submit(const Job& j) {
         {
@@ -99,32 +114,76 @@ class ReadPool {
     }
 
   private:
+    static constexpr size_t DIRECT_ALIGN = 4096;   // platform.rs:78
     void work() {
+        uint8_t* bounce = nullptr;
+        size_t bounce_len = 0;
         for (;;) {
             Job j;
-            int fd;
+            int fd, dfd;
             uint64_t base, size;
             {
                 std::unique_lock<std::mutex> g(m_);
                 cv_.wait(g, [&] { return stop_ || !jobs_.empty(); });
-                if (jobs_.empty()) return;
+                if (jobs_.empty()) {
+                    free(bounce);
+                    return;
+                }
                 j = jobs_.front();
                 jobs_.pop_front();
                 fd = fd_;
+                dfd = dfd_;
                 base = base_;
                 size = file_size_;
             }
-            bool ok = true;
+            bool ok = true, direct = false;
             const uint64_t addr = (uint64_t)(uintptr_t)j.src;
             if (fd >= 0 && addr >= base && addr - base + j.len <= size) {
-                size_t got = 0;
-                while (got < j.len) {
-                    ssize_t r = pread(fd, j.dst + got, j.len - got, (off_t)(addr - base + got));
-                    if (r <= 0) {
-                        ok = false;
-                        break;
+                const uint64_t off = addr - base;
+                if (dfd >= 0) {
+                    // the aligned range around the expert's bytes into this thread's aligned buffer (offset, address and
+                    // length in whole DIRECT_ALIGN units; the range of the file's last expert may run past its end and
+                    // comes back short), then the bytes themselves to where the job wants them
+                    const uint64_t lo = off & ~(uint64_t)(DIRECT_ALIGN - 1);
+                    const size_t span = (size_t)(((off + j.len + DIRECT_ALIGN - 1) & ~(uint64_t)(DIRECT_ALIGN - 1)) - lo);
+                    if (span > bounce_len) {
+                        free(bounce);
+                        bounce = nullptr;
+                        bounce_len = 0;
+                        void* mem = nullptr;
+                        if (posix_memalign(&mem, DIRECT_ALIGN, span) == 0) {
+                            bounce = (uint8_t*)mem;
+                            bounce_len = span;
+                        }
                     }
-                    got += (size_t)r;
+                    if (bounce) {
+                        const size_t need = (size_t)(off - lo) + j.len;
+                        size_t got = 0;
+                        direct = true;
+                        while (got < need) {
+                            // a short read leaves an unaligned remainder: what is still missing is then read from the last
+                            // whole unit on
+                            const size_t at = got & ~(size_t)(DIRECT_ALIGN - 1);
+                            ssize_t r = pread(dfd, bounce + at, span - at, (off_t)(lo + at));
+                            if (r <= 0) {
+                                direct = false;
+                                break;
+                            }
+                            got = at + (size_t)r;
+                        }
+                        if (direct) memcpy(j.dst, bounce + (off - lo), j.len);
+                    }
+                }
+                if (!direct) {
+                    size_t got = 0;
+                    while (got < j.len) {
+                        ssize_t r = pread(fd, j.dst + got, j.len - got, (off_t)(off + got));
+                        if (r <= 0) {
+                            ok = false;
+                            break;
+                        }
+                        got += (size_t)r;
+                    }
                 }
             } else {
                 memcpy(j.dst, j.src, j.len);
@@ -132,6 +191,8 @@ class ReadPool {
             {
                 std::lock_guard<std::mutex> g(m_);
                 *j.state = ok ? 1 : 2;
+                n_reads_++;
+                if (direct) n_direct_++;
             }
             done_.notify_all();
         }
@@ -141,8 +202,8 @@ class ReadPool {
     std::condition_variable cv_, done_;
     std::deque<Job> jobs_;
     bool stop_ = false;
-    int fd_ = -1;
-    uint64_t base_ = 0, file_size_ = 0;
+    int fd_ = -1, dfd_ = -1;
+    uint64_t base_ = 0, file_size_ = 0, n_direct_ = 0, n_reads_ = 0;
     std::string path_;
 };
 
@@ -630,4 +691,9 @@ bool it_hip::cold_resolve(const uint8_t* const* keys, int n_keys, const it_route
         }
     }
     return true;
+}
+
+void it_hip_fetch_read_counts(it_hip* be, uint64_t out[2]) {
+    out[0] = out[1] = 0;
+    if (be && be->cold && be->cold->pool) be->cold->pool->counts(&out[0], &out[1]);
 }

@@ -95,7 +95,7 @@ it_hip_kv_write it_hip_host_wrote it_hip_host_needs it_hip_begin_pass it_hip_end
 it_hip_read_state it_hip_read_kv it_hip_device_report it_hip_reserve_activations it_hip_tier_counters
 it_hip_config_report it_hip_setup_cost it_hip_prefetch_hint it_hip_set_expert_budget
 it_hip_set_expert_host_budget it_hip_set_expert_slots it_hip_set_expert_pool it_hip_expert_stats
-it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_hip_chain_stats it_hip_zero_state it_hip_mfma_ceiling it_model_open
+it_hip_clock_pick it_hip_argmax it_hip_embed_argmax it_hip_read_tokens it_hip_sync it_hip_profile_begin it_hip_profile_end it_hip_release it_hip_drop_mirrors it_hip_launch_count it_hip_graph_stats it_hip_chain_stats it_hip_fetch_read_counts it_hip_zero_state it_hip_mfma_ceiling it_model_open
 it_model_close it_model_dims it_model_decode_weight_bytes it_model_token_macs it_engine_new it_engine_free it_engine_reset
 it_engine_set_trace it_engine_pos it_engine_state_sizes it_engine_checkpoint it_engine_restore it_engine_rewind it_engine_forward it_engine_prefill it_engine_generate
 it_engine_decode_greedy it_engine_last_error it_engine_ssm_state it_engine_conv_state it_engine_k_slab
@@ -206,6 +206,7 @@ def lib() -> C.CDLL:
         "it_hip_launch_count": (u64, [vp]),
         "it_hip_graph_stats": (None, [vp, vp]),
         "it_hip_chain_stats": (None, [vp, vp]),
+        "it_hip_fetch_read_counts": (None, [vp, vp]),
         "it_model_open": (vp, [C.c_char_p, C.c_char_p, C.c_size_t]),
         "it_hip_mfma_ceiling": (C.c_int, [vp, C.c_int, C.c_int, vp]),
         "it_hip_zero_state": (None, [vp]),
@@ -458,6 +459,12 @@ class Hip:
         v = (c_u64 * 4)()
         self.L.it_hip_chain_stats(self.h, v)
         return {"chains": int(v[0]), "layers": int(v[1]), "enabled": bool(v[2]), "spin_limit": int(v[3])}
+
+    def fetch_read_counts(self):
+        """Cold-tier reads from the model file: (through the unbuffered descriptor, in all)."""
+        v = (c_u64 * 2)()
+        self.L.it_hip_fetch_read_counts(self.h, v)
+        return int(v[0]), int(v[1])
 
     MFMA_KINDS = {"int8_16x16x64": 0, "int8_16x16x32": 1, "f16_32x32x16": 2, "f16_16x16x32": 3, "f32_16x16x4": 4}
 

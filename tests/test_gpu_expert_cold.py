@@ -5,6 +5,8 @@ expert the layer did not pick (GCLOCK with leases), and the placement tables are
 never change a value: every run here is compared bit for bit with the same run on a backend that holds the whole pool in
 device memory (the reference's acceptance test, the_35b_generates_identically_with_the_expert_pool_oversubscribed,
 tests/cuda_ops.rs:6475-6633)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -38,6 +40,7 @@ def run_model(gguf, exact, slots, host_experts, batches, n_new, seed, prefetch=T
     moved = be.replace_experts_by_counts()
     st, tc = be.expert_stats(), be.tier_counters()
     report, graph = be.config_report(), be.graph_stats()
+    run_model.reads = be.fetch_read_counts()
     err = be.take_error()
     he.close(); hm.close(); be.close()
     assert err is None, err
@@ -188,3 +191,32 @@ def test_a_device_tier_smaller_than_one_decision_is_refused():
     err = be.take_error() or ""
     assert "smaller than one layer's picks" in err and "2 device slots" in err
     be.close()
+
+
+def test_cold_experts_are_read_unbuffered_where_the_file_system_allows(mid_gguf, monkeypatch):
+    """The reader threads open the model file a second time with O_DIRECT and read whole 4,096-byte units around an
+    expert's bytes into an aligned buffer of their own (/root/reference src/platform.rs:60-96, 200-215;
+    src/ops/cuda/fetch.rs:71-73, experts.rs:310-312): on by default, off with INFERRED_FETCH_DIRECT=0, and buffered when
+    the file system refuses the flag.  Either way the bytes are the file's: ids and logits bit-identical to the
+    all-resident run."""
+    batches, n_new = [3, 48], 8
+    ref = run_model(mid_gguf, True, None, 0, batches, n_new, 13)
+    try:
+        fd = os.open(str(mid_gguf), os.O_RDONLY | os.O_DIRECT)
+        os.close(fd)
+        fs_allows = True
+    except OSError:
+        fs_allows = False
+    for setting in (None, "0", "1"):
+        if setting is None:
+            monkeypatch.delenv("INFERRED_FETCH_DIRECT", raising=False)
+        else:
+            monkeypatch.setenv("INFERRED_FETCH_DIRECT", setting)
+        cold = run_model(mid_gguf, True, 130, 100, batches, n_new, 13)
+        direct, reads = run_model.reads
+        print(f"INFERRED_FETCH_DIRECT={setting}: {direct} of {reads} reads unbuffered (file system allows: {fs_allows})", flush=True)
+        assert reads > 0 and cold[2].fetched > 0
+        assert direct == (reads if (setting != "0" and fs_allows) else 0), (setting, direct, reads)
+        for a, b in zip(ref[0], cold[0]):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert np.array_equal(ref[1], cold[1])
