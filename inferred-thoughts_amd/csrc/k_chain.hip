@@ -16,9 +16,19 @@
 //      weight, with the block's share of the head's sum of squares beside it
 //   C  head-norm scale, quantization, rows of ssm_out, residual
 //   D  rms_norm + quantization; router rows, the shared expert's gate logit, its gate / up rows
-//   E  softmax + top-10 of the logits in every block; 160 blocks take one 32-element block of one pick's gate / up
-//      rows each and publish it quantized; the loads of the down rows go out with them
+//   E  top-10 of the logits in every block (ranked on the logits; the softmax of the ten follows under the rows'
+//      flight); 160 blocks take one 32-element block of one pick's gate / up rows each and publish it quantized, the
+//      other 96 touch those rows' lines for the blocks of their XCD; the down rows are issued behind the publication
 //   F  down rows of the ten picks and of the shared expert, combine, residual
+// An attention layer gives the chain before it a last stage (its in-projection: rms_norm + Q8_0 + wq / wk / wv rows) and
+// the chain behind it a first one (its out-projection + residual); the attention kernels run between the two chains.
+//
+// Three things place the loads and the polls (each measured with the stage stamps below):
+//   * loads return in issue order per wave, so a poll or a publication waits for everything its wave has in flight:
+//     few-word inputs (stages B and F) are gathered by waves that issue their own rows only afterwards;
+//   * a compute unit pulls 25-30 GB/s whatever it asks for: rows are issued where the stage before leaves the pipe idle;
+//   * two waves share a SIMD's vector ALU, so instructions count double: NVFP4 rows go through the hardware's
+//     fp4 -> f16 conversion and v_dot2_f32_f16 (half the instructions of the permute + v_dot4 form, same bits).
 //
 // Every wait is bounded: a poll that runs out of tries sets the abort word, every other wait sees it and the
 // grid drains.  The grid must be resident at once (one block per compute unit), which the launcher checks.
@@ -109,7 +119,7 @@ __device__ long long it_chain_wave_stamps[8][8];
 #define IT_CHAIN_D_AT 1       // stage D's rows: 0 at the head of stage C, 1 after stage B's input has arrived
 #endif
 #ifndef IT_CHAIN_A_AT
-#define IT_CHAIN_A_AT 0x070   // next in-projection, a hex digit of fetch_a parts per site: after D's input | after E's publish | after F's input
+#define IT_CHAIN_A_AT 0x070   // next in-projection, a hex digit of fetch_a parts per site: after D's input | at the head of stage F | after F's input
 #endif
 
 struct Ctl {
@@ -234,9 +244,10 @@ IT_DEV int a_row(int k, int b, int wave) {   // row k of the wave in its own mat
     return k < 4 ? b + NB * (wave + CW * k) : k < 6 ? b + NB * (wave + CW * (k - 4)) : b < NV ? b : b - NV;
 }
 // `parts` picks what is fetched: bit 0 the first two wqkv rows and the conv windows, bit 1 the other two wqkv rows,
-// bit 2 the two wz rows and the alpha / beta row.  (A block's 105 KB are issued in pieces, each small enough to have
-// landed when the wave's next poll is due: loads return in the order they were issued, a poll behind a large
-// fetch waits for all of it.)
+// bit 2 the two wz rows and the alpha / beta row.  (A block's 105 KB can be issued in pieces at up to three sites of the
+// layer before, IT_CHAIN_A_AT: loads return in the order they were issued, and a poll behind a large fetch waits for
+// all of it.  All at the head of stage F measured best once that stage's input was gathered by waves that issue
+// theirs behind the gather.)
 IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int parts = 7) {
     if (parts & 1) {
 #pragma unroll
