@@ -618,14 +618,20 @@ bool match_ffn(Plan& pl, size_t i, int exact, unsigned* counter, unsigned long l
 bool q8(const FusedMat& m, int n_out, int epi) { return m.fmt == W_Q8_0 && m.n_out == n_out && m.epi == epi; }
 bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-bool chain_mixer(const FusedGemvP& a, const GdnCoreP& c, const FusedGemvP& b, ChainMixer* m) {
+bool f32m(const FusedMat& m, int n_out, int epi) { return m.fmt == W_F32 && m.n_out == n_out && m.epi == epi; }
+
+// rf: 1 when the small matrices (alpha / beta here, router / gate logit in the FFN) are F32, 0 when Q8_0
+bool chain_mixer(const FusedGemvP& a, const GdnCoreP& c, const FusedGemvP& b, ChainMixer* m, int* rf) {
     if (a.exact || a.n_in != 2048 || a.mode != 1 || a.n_mats != 4 || a.route_counter) return false;
-    if (!q8(a.m[0], 8192, 1) || !q8(a.m[1], 4096, 3) || !q8(a.m[2], 32, 0) || !q8(a.m[3], 32, 0)) return false;
+    if (!q8(a.m[0], 8192, 1) || !q8(a.m[1], 4096, 3)) return false;
+    if (q8(a.m[2], 32, 0) && q8(a.m[3], 32, 0)) *rf = 0;
+    else if (f32m(a.m[2], 32, 0) && f32m(a.m[3], 32, 0)) *rf = 1;
+    else return false;
     if (c.n_k_heads != 16 || c.n_v_heads != 32 || c.exact) return false;
     if (b.n_in != 4096 || b.mode != 3 || b.head_dim != 128 || b.n_mats != 1 || !q8(b.m[0], 2048, 2) || b.m[0].out != a.x) return false;
     if (c.conv != a.m[0].out || c.alpha != a.m[2].out || c.beta != a.m[3].out || b.gate != a.m[1].out || b.x != c.core) return false;
     for (int i = 0; i < 4; i++)
-        if (!al16(a.m[i].q) || !al16(a.m[i].s)) return false;
+        if (!al16(a.m[i].q) || (!(*rf && i >= 2) && !al16(a.m[i].s))) return false;
     if (!al16(b.m[0].q) || !al16(b.m[0].s) || !al16(a.norm_w) || !al16(a.conv_w) || !al16(c.state) || !al16(a.x)) return false;
     m->norm_w = a.norm_w;
     m->qkv_q = a.m[0].q; m->qkv_s = a.m[0].s;
@@ -646,15 +652,19 @@ bool chain_mixer(const FusedGemvP& a, const GdnCoreP& c, const FusedGemvP& b, Ch
     return true;
 }
 
-bool chain_ffn(const FusedGemvP& r, const MoeGluP& g, const MoeDownP& d, ChainFfn* f, int* sh_fmt) {
-    if (r.exact || r.n_in != 2048 || r.mode != 1 || r.n_mats != 2 || r.route_counter || !q8(r.m[0], 512, 0) || !q8(r.m[1], 1, 0)) return false;
+bool chain_ffn(const FusedGemvP& r, const MoeGluP& g, const MoeDownP& d, ChainFfn* f, int* sh_fmt, int* rf) {
+    if (r.exact || r.n_in != 2048 || r.mode != 1 || r.n_mats != 2 || r.route_counter) return false;
+    if (q8(r.m[0], 512, 0) && q8(r.m[1], 1, 0)) *rf = 0;
+    else if (f32m(r.m[0], 512, 0) && f32m(r.m[1], 1, 0)) *rf = 1;
+    else return false;
     if (g.exact || g.fmt != W_NVFP4 || g.n_in != 2048 || g.n_out != 512 || g.n_expert != 512 || g.n_used != 10 || g.sh_n_out != 512) return false;
     if (g.sh_fmt != W_Q8_0 && g.sh_fmt != W_NVFP4) return false;
     if (!g.logits || g.logits != r.m[0].out || !g.route_ids_out || !g.route_w_out || g.x != r.x_copy2) return false;
     if (d.exact || d.fmt != W_NVFP4 || d.n_in != 512 || d.n_out != 2048 || d.n_used != 10 || d.sh_fmt != g.sh_fmt || d.sh_n_in != 512) return false;
     if (d.g_all != g.out || d.g_shared != g.sh_out || d.logit != r.m[1].out || d.x != r.x || d.route_ids != g.route_ids_out || d.route_w != g.route_w_out)
         return false;
-    const void* ptrs[] = {r.m[0].q, r.m[0].s, r.m[1].q, r.m[1].s, g.gq, g.gs, g.uq, g.us, g.sh_gq, g.sh_gs, g.sh_uq, g.sh_us, d.q, d.s, d.sh_q, d.sh_s, r.norm_w, r.x};
+    if (!*rf && (!r.m[0].s || !r.m[1].s || !al16(r.m[0].s) || !al16(r.m[1].s))) return false;
+    const void* ptrs[] = {r.m[0].q, r.m[1].q, g.gq, g.gs, g.uq, g.us, g.sh_gq, g.sh_gs, g.sh_uq, g.sh_us, d.q, d.s, d.sh_q, d.sh_s, r.norm_w, r.x};
     for (const void* p : ptrs)
         if (!p || !al16(p)) return false;
     if (g.q_stride % 16 || g.s_stride % 16 || d.q_stride % 16 || d.s_stride % 16) return false;
@@ -713,6 +723,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
     ChainP cp{};
     std::vector<Unit> units;          // the blocks folded into cp so far
     bool mixer_open = false;          // the last layer of cp has its mixer and still waits for its FFN
+    int chain_rf = -1;                // the small matrices of cp's layers: Q8_0 (0) or F32 (1); -1 while no layer says
     uint64_t bytes = 0;
     auto skips_of = [&](const std::vector<Plan::Skips>& v, size_t pos, std::vector<const void*>* out) {
         for (auto& sk : v)
@@ -733,6 +744,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             cp.abort_flag = be->chain.abort_flag;
             cp.tally = be->count_reads_in_fused ? tally : nullptr;
             cp.spin_limit = be->chain_spin_limit;
+            cp.rf = chain_rf > 0 ? 1 : 0;
             const ChainP launch = cp;
             auto drop_stage = [&](size_t pos, int stage) {
                 auto& v = pl.at[pos];
@@ -764,6 +776,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         units.clear();
         mixer_open = false;
         bytes = 0;
+        chain_rf = -1;
     };
     for (size_t i = 0; i < pl.ops.size(); i++) {
         auto& ls = pl.at[i];
@@ -799,7 +812,9 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         if (is_gdn) {
             if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
             ChainMixer m{};
-            if (chain_mixer(ls[0].gv, ls[1].gc, ls[2].gv, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
+            int rf = 0;
+            if (chain_mixer(ls[0].gv, ls[1].gc, ls[2].gv, &m, &rf) && (cp.n_layers == 0 || cp.x == ls[0].gv.x) && (chain_rf < 0 || chain_rf == rf)) {
+                chain_rf = rf;
                 cp.layer[cp.n_layers].has_mixer = 1;
                 cp.layer[cp.n_layers].m = m;
                 cp.x = const_cast<float*>(ls[0].gv.x);
@@ -813,8 +828,11 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             ChainFfn f{};
             int sh_fmt = 0;
             if (!mixer_open && cp.n_layers == CHAIN_MAX_LAYERS) emit();
-            const bool fits = chain_ffn(ls[0].gv, ls[1].mg, ls[2].md, &f, &sh_fmt) && (cp.n_layers == 0 || (cp.x == ls[0].gv.x && (cp.sh_fmt == sh_fmt || (cp.n_layers == 1 && mixer_open))));
+            int rf = 0;
+            const bool fits = chain_ffn(ls[0].gv, ls[1].mg, ls[2].md, &f, &sh_fmt, &rf) && (chain_rf < 0 || chain_rf == rf) &&
+                              (cp.n_layers == 0 || (cp.x == ls[0].gv.x && (cp.sh_fmt == sh_fmt || (cp.n_layers == 1 && mixer_open))));
             if (fits) {
+                chain_rf = rf;
                 if (!mixer_open) {
                     cp.layer[cp.n_layers].has_mixer = 0;
                     cp.n_layers++;

@@ -239,15 +239,22 @@ struct AW {
     WChunks<2> t[7];
     float4 taps;
     float past[3];
+    float4 ab;   // unquantized alpha / beta (RF): this wave's four floats a lane of the block's row
 };
 IT_DEV int a_row(int k, int b, int wave) {   // row k of the wave in its own matrix
     return k < 4 ? b + NB * (wave + CW * k) : k < 6 ? b + NB * (wave + CW * (k - 4)) : b < NV ? b : b - NV;
 }
+// An unquantized (F32) row of 2,048 weights is summed in the order the per-stage kernels use (fused_gemv_fast_k's
+// frow_chunk / frow_tree), so that these sums come out the same, to the bit, either way: a chunk of 256 weights is one
+// multiply-add chain per lane from zero and a lane reduction, and the eight chunk sums are added as a balanced tree.
+IT_DEV float f32_chunk(const float4 w, const float4 xv) { return fmaf(w.x, xv.x, fmaf(w.y, xv.y, fmaf(w.z, xv.z, fmaf(w.w, xv.w, 0.0f)))); }
+IT_DEV float f32_tree(const float* pc) { return ((pc[0] + pc[1]) + (pc[2] + pc[3])) + ((pc[4] + pc[5]) + (pc[6] + pc[7])); }
 // `parts` picks what is fetched: bit 0 the first two wqkv rows and the conv windows, bit 1 the other two wqkv rows,
 // bit 2 the two wz rows and the alpha / beta row.  (A block's 105 KB can be issued in pieces at up to three sites of the
 // layer before, IT_CHAIN_A_AT: loads return in the order they were issued, and a poll behind a large fetch waits for
 // all of it.  All at the head of stage F measured best once that stage's input was gathered by waves that issue
 // theirs behind the gather.)
+template <int RF>
 IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int parts = 7) {
     if (parts & 1) {
 #pragma unroll
@@ -267,8 +274,15 @@ IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int p
     if (parts & 4) {
 #pragma unroll
         for (int k = 4; k < 6; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.z_q, m.z_s, D, a_row(k, b, wave), lane, true);
-        const bool extra = wave == 0 && b < 2 * NV;
-        load_row<W_Q8_0, 2, 64>(a.t[6], b < NV ? m.a_q : m.b_q, b < NV ? m.a_s : m.b_s, D, a_row(6, b, wave), lane, extra);
+        if (RF) {
+            // an F32 row of 2,048 floats is shared by the block's eight waves, 256 floats each (a row in one wave would
+            // be 32 registers a lane); the partial dots meet in LDS
+            a.ab = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (b < 2 * NV) a.ab = ((const float4*)((const float*)(b < NV ? m.a_q : m.b_q) + (int64_t)a_row(6, b, wave) * D))[wave * 64 + lane];
+        } else {
+            const bool extra = wave == 0 && b < 2 * NV;
+            load_row<W_Q8_0, 2, 64>(a.t[6], b < NV ? m.a_q : m.b_q, b < NV ? m.a_s : m.b_s, D, a_row(6, b, wave), lane, extra);
+        }
     }
 }
 
@@ -343,17 +357,18 @@ IT_DEV float logit_of_order(uint32_t o) { return __uint_as_float((o & 0x80000000
 
 // rms_norm (naive.rs:633-650) of the 2,048 floats the block's threads hold as quads, then Q8_0 (naive.rs:652-675)
 // into xq / xs.  Two barriers; returns false after the first when the block has to stop.
-IT_DEV void norm_quant_finish(float4 v, float4 w, float eps, double sum, int8_t* xq, float* xs, int tid) {
+IT_DEV void norm_quant_finish(float4 v, float4 w, float eps, double sum, int8_t* xq, float* xs, int tid, float* xf = nullptr) {
     const float mean = (float)(sum / (double)D);
     const float scale = 1.0f / sqrtf(mean + eps);
     v.x = v.x * scale * w.x;
     v.y = v.y * scale * w.y;
     v.z = v.z * scale * w.z;
     v.w = v.w * scale * w.w;
+    if (xf) ((float4*)xf)[tid] = v;   // the normed vector itself, for rows of unquantized matrices
     quant_quad(v, true, tid, xq, xs);
     __syncthreads();
 }
-IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid) {
+IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, double* red, const int* dead, int tid, float* xf = nullptr) {
     const double part = wave_sum_f64_tail(quad_sumsq(v));
     if ((tid & 63) == 63) red[tid >> 6] = part;
     __syncthreads();
@@ -361,11 +376,11 @@ IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, dou
     double sum = 0.0;
 #pragma unroll
     for (int i = 0; i < CW; i++) sum += red[i];
-    norm_quant_finish(v, w, eps, sum, xq, xs, tid);
+    norm_quant_finish(v, w, eps, sum, xq, xs, tid, xf);
     return true;
 }
 
-template <int SF>
+template <int SF, int RF>
 __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     __shared__ __align__(16) int8_t xq[NU * FF + FF];   // the stage's quantized activation (largest: the down stage's)
     __shared__ __align__(16) float xs[(NU * FF + FF) / 32];
@@ -379,6 +394,8 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     __shared__ __align__(16) float wts[16];
     __shared__ float coef[16];
     __shared__ int dead;
+    __shared__ float fpart[2 * CW];   // partial dots of rows shared by the waves (RF)
+    float* const xf = RF ? (float*)route_sh.keys : nullptr;   // the normed f32 vector of stages A and D (the route's keys come later)
     const int tid0 = threadIdx.x, b0 = blockIdx.x;
     const Ctl ctl{p.abort_flag, p.spin_limit};
     const unsigned e0 = *(const volatile unsigned*)p.epoch;
@@ -386,7 +403,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     // lane 63 of a wave owns one row of the residual stream: row 8 * block + wave
     float x_row = (tid0 & 63) == 63 ? p.x[b0 * CW + (tid0 >> 6)] : 0.0f;
     AW aw;
-    if (p.layer[0].has_mixer == 1) fetch_a(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
+    if (p.layer[0].has_mixer == 1) fetch_a<RF>(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
     __syncthreads();
 
 #ifdef IT_CHAIN_STAMPS
@@ -423,9 +440,24 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         WChunks<2> d0, d1;
         WChunks<1> n0, n1;
         const int sh_row = 2 * b + (wave - 2);
+        float4 rf0, rf1, lf;   // RF: this wave's quarter of an unquantized router row (two float4 a lane), its eighth of the gate-logit row
         auto fetch_d = [&]() {
             const bool r = wave < 2, sh = wave == 2 || wave == 3, lg = wave == 4 && b == NB - 1;
-            if (SF == W_Q8_0) {
+            if (RF) {
+                // unquantized router and gate-logit rows: row b in waves 0..3, row NB + b in waves 4..7, 512 floats a wave;
+                // the gate-logit row in the last block, 256 floats a wave; the partial dots meet in LDS
+                const float4* row = (const float4*)((const float*)f.r_q + (int64_t)(b + NB * (wave >> 2)) * D) + (wave & 3) * 128;
+                rf0 = row[lane];
+                rf1 = row[64 + lane];
+                lf = b == NB - 1 ? ((const float4*)f.l_q)[wave * 64 + lane] : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (SF == W_Q8_0) {
+                    load_row<W_Q8_0, 2, 64>(d0, f.sg_q, f.sg_s, D, sh_row, lane, sh);
+                    load_row<W_Q8_0, 2, 64>(d1, f.su_q, f.su_s, D, sh_row, lane, sh);
+                } else {
+                    load_row<W_NVFP4, 1, 64>(n0, f.sg_q, f.sg_s, D, sh_row, lane, sh);
+                    load_row<W_NVFP4, 1, 64>(n1, f.su_q, f.su_s, D, sh_row, lane, sh);
+                }
+            } else if (SF == W_Q8_0) {
                 load_row<W_Q8_0, 2, 64>(d0, r ? f.r_q : sh ? f.sg_q : f.l_q, r ? f.r_s : sh ? f.sg_s : f.l_s, D,
                                       r ? b + NB * wave : sh ? sh_row : 0, lane, r || sh || lg);
                 load_row<W_Q8_0, 2, 64>(d1, f.su_q, f.su_s, D, sh_row, lane, sh);
@@ -471,14 +503,14 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 if (l == 0) v = ((const float4*)p.x)[tid];
                 else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
                 if (!ok) dead = 1;
-                if (!norm_quant(v, nw, m.eps_norm, xq, xs, red, &dead, tid)) break;
+                if (!norm_quant(v, nw, m.eps_norm, xq, xs, red, &dead, tid, xf)) break;
                 if (IT_CHAIN_WC_AT == 1) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
                 CH_STAMP(0);
                 XChunks<W_Q8_0, 2> x;
                 load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
                 float acc[7];
 #pragma unroll
-                for (int k = 0; k < 7; k++) acc[k] = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
+                for (int k = 0; k < 7; k++) acc[k] = (RF && k == 6) ? 0.0f : reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
                 if (IT_CHAIN_WC_AT == 2) load_row<W_Q8_0, 4, 64>(wc, m.o_q, m.o_s, VDIM, my_row, lane, true);
                 // row k's dot goes from lane 63 to lane k, which finishes the row
                 float mine = 0.0f;
@@ -502,8 +534,16 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                     past[2] = mine;
                 } else if (lane < 6) {
                     ll_putf(p.ll + RA_Z + b + NB * (wave + CW * (lane - 4)), fx_silu(mine), e);
-                } else if (lane == 6 && wave == 0 && b < 2 * NV) {
+                } else if (!RF && lane == 6 && wave == 0 && b < 2 * NV) {
                     ll_putf(p.ll + RA_AL + b, mine, e);
+                }
+                if (RF) {
+                    // the unquantized alpha / beta row of blocks 0..63 against the normed f32 vector: every wave its 256 floats
+                    const float4 xa = ((const float4*)xf)[wave * 64 + lane];
+                    const float part = reduce_lanes<64>(f32_chunk(aw.ab, xa));
+                    if (lane == 63) fpart[wave] = part;
+                    __syncthreads();
+                    if (tid == 0 && b < 2 * NV) ll_putf(p.ll + RA_AL + b, f32_tree(fpart), e);
                 }
             }
             // ---------------------------------------------------------------- B: delta rule
@@ -674,17 +714,27 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             else if (l == 0) v = ((const float4*)p.x)[tid];
             else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
             if (!ok) dead = 1;
-            if (!norm_quant(v, nw, f.eps, xq, xs, red, &dead, tid)) break;
+            if (!norm_quant(v, nw, f.eps, xq, xs, red, &dead, tid, xf)) break;
             if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer == 1 && ((IT_CHAIN_A_AT >> 8) & 15))
-                fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 8) & 15);
+                fetch_a<RF>(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 8) & 15);
             CH_STAMP(6);
             XChunks<W_Q8_0, 2> x;
             load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
             load_xn(xn, xq, xs, lane);
-            if (wave < 2 || (wave == 4 && b == NB - 1)) {
+            if (RF) {
+                const float4 xa = ((const float4*)xf)[(wave & 3) * 128 + lane], xb = ((const float4*)xf)[(wave & 3) * 128 + 64 + lane];
+                const float pr = reduce_lanes<64>(f32_chunk(rf0, xa)) + reduce_lanes<64>(f32_chunk(rf1, xb));
+                const float4 xl = ((const float4*)xf)[wave * 64 + lane];
+                const float pl = reduce_lanes<64>(f32_chunk(lf, xl));
+                if (lane == 63) {
+                    fpart[wave] = pr;
+                    fpart[CW + wave] = pl;
+                }
+            } else if (wave < 2 || (wave == 4 && b == NB - 1)) {
                 const float a = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
                 if (lane == 63) ll_putf(p.ll + RD + (wave < 2 ? b + NB * wave : NE), a, e);
-            } else if (wave < 4) {
+            }
+            if (wave == 2 || wave == 3) {
                 float ag, au;
                 if (SF == W_Q8_0) {
                     ag = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(d0, x));
@@ -698,6 +748,11 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                     au *= f.sh_uscale;
                     ll_putf(p.ll + RS + sh_row, fx_silu(ag) * au, e);
                 }
+            }
+            if (RF) {
+                __syncthreads();
+                if (tid < 2) ll_putf(p.ll + RD + b + NB * tid, (fpart[4 * tid] + fpart[4 * tid + 1]) + (fpart[4 * tid + 2] + fpart[4 * tid + 3]), e);
+                if (tid == 64 && b == NB - 1) ll_putf(p.ll + RD + NE, f32_tree(fpart + CW), e);
             }
         }
 
@@ -897,7 +952,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         // own wave has in flight)
         auto fetch_next = [&]() {
             if (l + 1 == p.n_layers && p.has_tail) fetch_tail(p.tail, aw, b, wave, lane);
-            if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
+            if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a<RF>(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
         };
         if (!IT_CHAIN_F_POLLERS || wave < 4) fetch_next();
 
@@ -962,7 +1017,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             __syncthreads();
             if (dead) break;
             CH_STAMP(11);
-            if (next_mixer && (IT_CHAIN_A_AT & 15)) fetch_a(p.layer[l + 1].m, aw, b, wave, lane, IT_CHAIN_A_AT & 15);
+            if (next_mixer && (IT_CHAIN_A_AT & 15)) fetch_a<RF>(p.layer[l + 1].m, aw, b, wave, lane, IT_CHAIN_A_AT & 15);
             float acc = 0.0f;
             const int c = lane & 15;
 #pragma unroll
@@ -1048,8 +1103,10 @@ bool layer_chain_fits() {
         int dev = 0, cus = 0, occ = 0;
         if (hipGetDevice(&dev) != hipSuccess) return false;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < NB) return false;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, layer_chain_k<W_Q8_0>, CT, 0) != hipSuccess || occ < 1) return false;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, layer_chain_k<W_NVFP4>, CT, 0) != hipSuccess || occ < 1) return false;
+        const void* fns[4] = {(const void*)layer_chain_k<W_Q8_0, 0>, (const void*)layer_chain_k<W_NVFP4, 0>,
+                              (const void*)layer_chain_k<W_Q8_0, 1>, (const void*)layer_chain_k<W_NVFP4, 1>};
+        for (const void* fn : fns)
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, CT, 0) != hipSuccess || occ < 1) return false;
         return true;
     }();
     return fits;
@@ -1069,11 +1126,13 @@ bool layer_chain(const ChainP& p, hipStream_t s) {
         const ChainFfn& f = p.layer[l].f;
         const int kind = p.layer[l].has_mixer;
         if (kind < 0 || kind > 2 || (kind == 2 && l != 0)) return false;
-        if (kind == 1 && !all({m.norm_w, m.qkv_q, m.qkv_s, m.z_q, m.z_s, m.a_q, m.a_s, m.b_q, m.b_s, m.conv_state, m.conv_w, m.ssm_a,
+        if (kind == 1 && !p.rf && !all({m.a_s, m.b_s})) return false;
+        if (!p.rf && !all({f.r_s, f.l_s})) return false;
+        if (kind == 1 && !all({m.norm_w, m.qkv_q, m.qkv_s, m.z_q, m.z_s, m.a_q, m.b_q, m.conv_state, m.conv_w, m.ssm_a,
                                m.dt_bias, m.state, m.head_norm_w, m.o_q, m.o_s}))
             return false;
         if (kind == 2 && !all({m.o_q, m.o_s, m.attn})) return false;
-        if (!all({f.norm_w, f.r_q, f.r_s, f.l_q, f.l_s, f.sg_q, f.sg_s, f.su_q, f.su_s, f.sd_q, f.sd_s, f.eg_q, f.eg_s, f.eu_q, f.eu_s,
+        if (!all({f.norm_w, f.r_q, f.l_q, f.sg_q, f.sg_s, f.su_q, f.su_s, f.sd_q, f.sd_s, f.eg_q, f.eg_s, f.eu_q, f.eu_s,
                   f.ed_q, f.ed_s, f.route_ids, f.route_w}))
             return false;
     }
@@ -1081,8 +1140,10 @@ bool layer_chain(const ChainP& p, hipStream_t s) {
                             p.tail.out_k, p.tail.out_v}))
         return false;
     if (!layer_chain_fits()) return false;
-    if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL(layer_chain_k<W_Q8_0>, dim3(NB), dim3(CT), 0, s, p);
-    else hipLaunchKernelGGL(layer_chain_k<W_NVFP4>, dim3(NB), dim3(CT), 0, s, p);
+    if (p.sh_fmt == W_Q8_0 && !p.rf) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 0>), dim3(NB), dim3(CT), 0, s, p);
+    else if (!p.rf) hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 0>), dim3(NB), dim3(CT), 0, s, p);
+    else if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 1>), dim3(NB), dim3(CT), 0, s, p);
+    else hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 1>), dim3(NB), dim3(CT), 0, s, p);
     return true;
 }
 

@@ -155,17 +155,23 @@ IT_DEV int frow_locate(const FusedGemvP& p, int fr, int* j) {
 }
 // issues the loads of an F32 row's chunks (16 bytes per lane per 256 weights); false when the row is not F32
 constexpr int FC = 8;
-// (with the row shared by `split` waves, wave `part` of them takes the chunks c = part, part + split, ...)
+// (with the row shared by `split` waves, wave `part` of them takes the part-th contiguous run of its chunks)
 IT_DEV bool frow_fetch(const FusedGemvP& p, int fr, int n_in, int lane, float4 fw[FC], int split, int part) {
     int j;
     const FusedMat& m = p.m[frow_locate(p, fr, &j)];
     if (m.fmt != W_F32) return false;
     const float* row = (const float*)m.q + (int64_t)j * n_in;
+    const int per = (n_in / 256) / split;   // the row's chunks are dealt to the waves that share it in contiguous runs
 #pragma unroll
     for (int c = 0; c < FC; c++)
-        if (c * 256 < n_in && c % split == part) fw[c] = *(const float4*)(row + c * 256 + lane * 4);
+        if (c * 256 < n_in && c / per == part) fw[c] = *(const float4*)(row + c * 256 + lane * 4);
     return true;
 }
+// The order every kernel sums an F32 row of up to 2,048 weights in (the layer chain, which deals a row's chunks to
+// its waves differently, follows the same order and gets the same bits): a chunk of 256 weights is one multiply-add chain per lane from zero
+// and a lane reduction; the up to eight chunk sums are added as a balanced tree, absent chunks counting as zero.
+IT_DEV float frow_tree(const float pc[FC]) { return ((pc[0] + pc[1]) + (pc[2] + pc[3])) + ((pc[4] + pc[5]) + (pc[6] + pc[7])); }
+IT_DEV float frow_chunk(const float4 w, const float4 xv) { return fmaf(w.x, xv.x, fmaf(w.y, xv.y, fmaf(w.z, xv.z, fmaf(w.w, xv.w, 0.0f)))); }
 
 // ONE: one step per group (a matrix of few rows spreads over more blocks, i.e. more CUs pull its weights)
 // FM: the launch has unquantized matrices as well (a kernel of its own, so that the registers their rows are held in
@@ -274,6 +280,7 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
         const bool live = fr < p.total_frows;
         float* outp = nullptr;
         float acc = 0.0f;
+        bool chunked = false;
         if (live) {
             int j;
             const FusedMat& m = p.m[frow_locate(p, fr, &j)];
@@ -286,13 +293,16 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                 for (int c = 0; c < FC; c++) cur[c] = fw[c];
                 const int nxt = fr + fstride;
                 if (nxt < p.total_frows) f_loaded = frow_fetch(p, nxt, n_in, lane, fw, fsplit, fpart);
+                float pc[FC];
+                const int per = (n_in / 256) / fsplit;
 #pragma unroll
                 for (int c = 0; c < FC; c++) {
-                    if (c * 256 >= n_in) break;
-                    if (c % fsplit != fpart) continue;
-                    const float4 xv = *(const float4*)(xf + c * 256 + lane * 4);
-                    acc = fmaf(cur[c].x, xv.x, fmaf(cur[c].y, xv.y, fmaf(cur[c].z, xv.z, fmaf(cur[c].w, xv.w, acc))));
+                    pc[c] = 0.0f;
+                    if (c * 256 >= n_in || c / per != fpart) continue;
+                    pc[c] = reduce_lanes<64>(frow_chunk(cur[c], *(const float4*)(xf + c * 256 + lane * 4)));
                 }
+                acc = frow_tree(pc);
+                chunked = true;
             } else if (fpart == 0) {   // other element types and row lengths: one wave walks the row
                 const int esz = m.fmt == W_F32 ? 4 : 2;
                 const uint8_t* row = m.q + (int64_t)j * n_in * esz;
@@ -310,18 +320,15 @@ __global__ __launch_bounds__(FT) void fused_gemv_fast_k(FusedGemvP p) {
                 }
             }
         }
-        acc = reduce_lanes<64>(acc);
+        if (!chunked) acc = reduce_lanes<64>(acc);   // (the chunked form is reduced chunk by chunk: its sum is in lane 63 already)
         if (fsplit == 1) {
             if (live && lane == 63) *outp = acc;
         } else {
             float* fsum = (float*)red;   // the prologue is done with it; FW doubles hold FW floats
             if (lane == 63) fsum[wave] = acc;
             __syncthreads();
-            if (live && fpart == 0 && lane == 63) {
-                float v = fsum[wave];
-                for (int k = 1; k < fsplit; k++) v += fsum[wave + k];
-                *outp = v;
-            }
+            if (live && fpart == 0 && lane == 63)
+                *outp = fsplit == 2 ? fsum[wave] + fsum[wave + 1] : (fsum[wave] + fsum[wave + 1]) + (fsum[wave + 2] + fsum[wave + 3]);
             __syncthreads();
         }
     }

@@ -175,6 +175,8 @@ struct ChainP {
     int has_tail;
     ChainTail tail;
     int sh_fmt;                  // the shared expert's format (W_Q8_0 or W_NVFP4)
+    int rf;                      // 1: the router, the shared expert's gate-logit row and ssm alpha / beta are F32 matrices (as real
+                                 // files keep them; their *_q pointers hold floats, their *_s are null), 0: Q8_0
     float* x;                    // residual stream [2048], read at the start and current after every layer
     unsigned long long* ll;      // CHAIN_LL_WORDS words of uncached device memory, zero before the first chain
     unsigned* epoch;             // device word: the last epoch any chain has used (starts at 0)
