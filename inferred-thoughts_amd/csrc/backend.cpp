@@ -1232,6 +1232,7 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->eager_fused = getenv("INFERRED_HIP_EAGER_FUSED") != nullptr;
     be->count_reads_in_fused = getenv("INFERRED_HIP_NO_READ_COUNTERS") == nullptr;
     be->small_ffn_enabled = getenv("INFERRED_HIP_NO_SMALL_FFN") == nullptr;
+    be->chain_attn_enabled = getenv("INFERRED_HIP_NO_CHAIN_ATTN") == nullptr;
     if (getenv("INFERRED_HIP_NO_GRAPH")) be->allow_graph = false;
     if (const char* sl = getenv("INFERRED_HIP_CHAIN_SPINS")) {
         const long v = atol(sl);

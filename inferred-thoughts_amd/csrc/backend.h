@@ -259,6 +259,7 @@ struct it_hip {
     };
     ChainRes chain;
     bool chain_enabled = true;
+    bool chain_attn_enabled = true;          // attention mixers inside the chains; INFERRED_HIP_NO_CHAIN_ATTN=1 keeps their kernels between two chains (a measurement switch)
     bool count_reads_in_fused = true;  // the fused decode kernels add the picks to the expert read counters (off: a measurement switch)
     bool eager_fused = false;          // single-token passes without a graph still go through the fuser (measurement switch)
     bool chain_ran = false;            // a chain has been issued since the abort word was last looked at

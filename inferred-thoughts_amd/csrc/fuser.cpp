@@ -9,6 +9,7 @@
 // block's first op; everything it replaces is dropped, except an activation
 // quantization that some unfused op still reads.
 #include <cstdio>
+#include <memory>
 #include <cstdlib>
 #include "backend.h"
 
@@ -33,6 +34,11 @@ struct Plan {
         GdnCoreP gc{};
         MoeGluP mg{};
         MoeDownP md{};
+        AttnArgs aa{};        // ST_ATTEND
+        TilePrepP tp{};
+        const float* gate = nullptr;
+        int gate_stride = 0;
+        float* attn_out = nullptr;
     };
     std::vector<std::vector<Launch>> at;  // fused launches keyed by position
     Launch& add(size_t i, int fam, uint64_t bytes, std::function<void(hipStream_t)> fn) {
@@ -388,11 +394,16 @@ bool match_attn(Plan& pl, size_t i, int exact) {
     bool three = false;
     if (at.i[6] == 0 && attend_tile_prep_ok(aa, tp)) {
         // norm + rotation of q and of the new key, and the slab writes, happen inside the tile kernel
-        pl.add(i, it_hip::FAM_ATTEND, kv_bytes + (uint64_t)(2 * hd * nh + 2 * kvd) * 4,
-               [=](hipStream_t s) {
-                   if (!attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s))
-                       be->fail("attend: the split-K kernels could not be launched");
-               }).stage = Plan::ST_ATTEND;
+        Plan::Launch& l_at = pl.add(i, it_hip::FAM_ATTEND, kv_bytes + (uint64_t)(2 * hd * nh + 2 * kvd) * 4, [=](hipStream_t s) {
+            if (!attend_split_gated_prep(aa, tp, n_split, scratch, attn_out, gate, gate_stride, s))
+                be->fail("attend: the split-K kernels could not be launched");
+        });
+        l_at.stage = Plan::ST_ATTEND;
+        l_at.aa = aa;
+        l_at.tp = tp;
+        l_at.gate = gate;
+        l_at.gate_stride = gate_stride;
+        l_at.attn_out = attn_out;
         three = true;
     } else if (at.i[6] == 0) {
         pl.add(i, it_hip::FAM_ATTN_PREP, (uint64_t)(2 * hd * nh + 2 * kvd) * 4 + kvd * 4, [=](hipStream_t s) { attn_prep(pp, s); });
@@ -710,17 +721,48 @@ bool chain_attn_in(const FusedGemvP& a, ChainTail* t) {
     return true;
 }
 
+// a whole attention block as a chain layer: in-projection, attention launch and out-projection must be the shapes the
+// chain's stages are written for and hang together (the attention reads what the in-projection writes and writes what
+// the out-projection reads; the gate is the second half of every head's wq rows)
+bool chain_attn(const FusedGemvP& in, const Plan::Launch& at, const FusedGemvP& out, ChainAttn* a, ChainMixer* m) {
+    ChainTail t{};
+    ChainMixer mo{};
+    if (!chain_attn_in(in, &t) || !chain_attn_out(out, &mo)) return false;
+    const AttnArgs& aa = at.aa;
+    const TilePrepP& tp = at.tp;
+    if (aa.n_q != 1 || aa.n_head != 16 || aa.n_head_kv != 2 || aa.head_dim != 256 || aa.kv_dim != 512 || !aa.n_pos_dyn) return false;
+    if (tp.qg != t.out_q || tp.kproj != t.out_k || tp.vproj != t.out_v || at.gate != tp.qg + 256 || at.gate_stride != 512) return false;
+    if (at.attn_out != mo.attn || out.m[0].out != in.x) return false;
+    if (tp.k_slab != aa.k || tp.v_slab != aa.v || !tp.q_norm || !tp.k_norm || !tp.rope) return false;
+    if (tp.n_rot <= 0 || tp.n_rot > 256 || (tp.n_rot / 2) % 4 || ((tp.n_rot / 8) & (tp.n_rot / 8 - 1))) return false;
+    if (!al16(tp.q_norm) || !al16(tp.k_norm) || !al16(tp.rope) || !al16(tp.k_slab) || !al16(tp.v_slab)) return false;
+    *a = ChainAttn{};
+    a->norm_w = t.norm_w;
+    a->q_q = t.q_q; a->q_s = t.q_s; a->k_q = t.k_q; a->k_s = t.k_s; a->v_q = t.v_q; a->v_s = t.v_s;
+    a->q_norm = tp.q_norm; a->k_norm = tp.k_norm;
+    a->rope = tp.rope;
+    a->k_slab = tp.k_slab; a->v_slab = tp.v_slab;
+    a->n_pos = aa.n_pos_dyn;
+    a->eps = t.eps; a->eps_head = tp.eps; a->scale = aa.scale;
+    a->n_rot = tp.n_rot;
+    *m = ChainMixer{};
+    m->o_q = mo.o_q;
+    m->o_s = mo.o_s;
+    return true;
+}
+
 void build_chains(Plan& pl, unsigned long long* tally) {
     it_hip* be = pl.be;
     be->chain_launches = be->chain_layers = 0;
     if (!be->chain_enabled || be->exact || !layer_chain_fits()) return;
-    enum Kind { U_GDN, U_FFN, U_ATTN_OUT };
+    enum Kind { U_GDN, U_FFN, U_ATTN_OUT, U_ATTN };
     struct Unit {
         size_t pos;
         Kind kind;
     };
     size_t tail_pos = 0;   // position of the attention block whose in-projection is cp's tail
     ChainP cp{};
+    auto layer_at = [&](int k) -> ChainLayer& { return cp.layer[k]; };
     std::vector<Unit> units;          // the blocks folded into cp so far
     bool mixer_open = false;          // the last layer of cp has its mixer and still waits for its FFN
     int chain_rf = -1;                // the small matrices of cp's layers: Q8_0 (0) or F32 (1); -1 while no layer says
@@ -745,7 +787,8 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             cp.tally = be->count_reads_in_fused ? tally : nullptr;
             cp.spin_limit = be->chain_spin_limit;
             cp.rf = chain_rf > 0 ? 1 : 0;
-            const ChainP launch = cp;
+            // (30 KB: on the heap, shared by the copies a std::function makes of what it holds)
+            const auto launch = std::make_shared<const ChainP>(cp);
             auto drop_stage = [&](size_t pos, int stage) {
                 auto& v = pl.at[pos];
                 for (size_t k = 0; k < v.size(); k++)
@@ -757,6 +800,15 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             for (size_t u = 0; u < n_units; u++) {
                 if (units[u].kind == U_ATTN_OUT) {
                     drop_stage(units[u].pos, Plan::ST_ATTN_OUT);   // the attention kernels before it stay where they are
+                } else if (units[u].kind == U_ATTN) {
+                    // nothing of the block is written but the cache rows and the residual stream
+                    for (auto& l : pl.at[units[u].pos]) {
+                        if (l.stage == Plan::ST_ATTN_IN)
+                            for (int k = 0; k < 3; k++) be->fused_elided.push_back(l.gv.m[k].out);
+                        if (l.stage == Plan::ST_ATTEND) be->fused_elided.push_back(l.attn_out);
+                    }
+                    pl.at[units[u].pos].clear();
+                    skips_of(pl.attn_skips, units[u].pos, &be->fused_elided);
                 } else {
                     pl.at[units[u].pos].clear();
                     skips_of(units[u].kind == U_GDN ? pl.gdn_skips : pl.ffn_skips, units[u].pos, &be->fused_elided);
@@ -767,7 +819,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
                 skips_of(pl.attn_skips, tail_pos, &be->fused_elided);
             }
             pl.add(units[0].pos, it_hip::FAM_CHAIN, bytes, [=](hipStream_t s) {
-                if (!layer_chain(launch, s)) be->fail("layer chain: the persistent kernel could not be launched");
+                if (!layer_chain(*launch, s)) be->fail("layer chain: the persistent kernel could not be launched");
             });
             be->chain_launches++;
             be->chain_layers += (uint64_t)n;
@@ -784,6 +836,23 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         const bool is_ffn = ls.size() == 3 && ls[0].stage == Plan::ST_ROUTER && ls[1].stage == Plan::ST_GLU && ls[2].stage == Plan::ST_DOWN;
         const bool is_attn = ls.size() == 3 && ls[0].stage == Plan::ST_ATTN_IN && ls[1].stage == Plan::ST_ATTEND && ls[2].stage == Plan::ST_ATTN_OUT;
         bool taken = false;
+        if (is_attn && be->chain_attn_enabled) {
+            // the whole block as a layer of the chain (its FFN follows)
+            if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            ChainAttn a{};
+            ChainMixer m{};
+            if (chain_attn(ls[0].gv, ls[1], ls[2].gv, &a, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
+                layer_at(cp.n_layers).has_mixer = 3;
+                layer_at(cp.n_layers).a = a;
+                layer_at(cp.n_layers).m = m;
+                cp.x = const_cast<float*>(ls[0].gv.x);
+                cp.n_layers++;
+                mixer_open = true;
+                units.push_back({i, U_ATTN});
+                bytes += ls[0].bytes + ls[1].bytes + ls[2].bytes;
+                continue;
+            }
+        }
         if (is_attn) {
             // its in-projection closes the chain so far, its out-projection opens the next one; the attention kernels
             // between them stay launches of their own
@@ -799,8 +868,8 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             emit();
             ChainMixer m{};
             if (chain_attn_out(out, &m)) {
-                cp.layer[0].has_mixer = 2;
-                cp.layer[0].m = m;
+                layer_at(0).has_mixer = 2;
+                layer_at(0).m = m;
                 cp.x = out.m[0].out;
                 cp.n_layers = 1;
                 mixer_open = true;
@@ -815,8 +884,8 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             int rf = 0;
             if (chain_mixer(ls[0].gv, ls[1].gc, ls[2].gv, &m, &rf) && (cp.n_layers == 0 || cp.x == ls[0].gv.x) && (chain_rf < 0 || chain_rf == rf)) {
                 chain_rf = rf;
-                cp.layer[cp.n_layers].has_mixer = 1;
-                cp.layer[cp.n_layers].m = m;
+                layer_at(cp.n_layers).has_mixer = 1;
+                layer_at(cp.n_layers).m = m;
                 cp.x = const_cast<float*>(ls[0].gv.x);
                 cp.n_layers++;
                 mixer_open = true;
@@ -834,10 +903,10 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             if (fits) {
                 chain_rf = rf;
                 if (!mixer_open) {
-                    cp.layer[cp.n_layers].has_mixer = 0;
+                    layer_at(cp.n_layers).has_mixer = 0;
                     cp.n_layers++;
                 }
-                cp.layer[cp.n_layers - 1].f = f;
+                layer_at(cp.n_layers - 1).f = f;
                 cp.sh_fmt = sh_fmt;
                 cp.x = const_cast<float*>(ls[0].gv.x);
                 mixer_open = false;

@@ -141,4 +141,47 @@ IT_DEV float sum8_lanes(float v) {
     return v;
 }
 
+// Per-head rms_norm (weight w) and NeoX rotation at `pos` of one head's HD values, four per lane
+// (lane li of the head's HD / 4 lanes holds dims 4 li .. 4 li + 3): what rms_norm_heads + rope_neox do
+// for a single token (naive.rs:180-218, 633-650), with the sum of squares reduced across the lanes.
+template <int HD>
+IT_DEV float4 head_norm_rope(float4 v, const float* __restrict__ w, float eps, const float2* __restrict__ rope,
+                             int n_rot, int pos, int li) {
+    constexpr int LPH = HD / 4;
+    double part = (double)(v.x * v.x);
+    part += (double)(v.y * v.y);
+    part += (double)(v.z * v.z);
+    part += (double)(v.w * v.w);
+    part += dpp_f64(part, 0);
+    part += dpp_f64(part, 1);
+    part += dpp_f64(part, 2);
+    part += dpp_f64(part, 3);
+    if (LPH >= 32) part += __shfl_xor(part, 16, 64);
+    if (LPH >= 64) part += __shfl_xor(part, 32, 64);
+    const float scale = 1.0f / sqrtf((float)(part / (double)HD) + eps);
+    const float4 ww = ((const float4*)w)[li];
+    v.x = v.x * scale * ww.x;
+    v.y = v.y * scale * ww.y;
+    v.z = v.z * scale * ww.z;
+    v.w = v.w * scale * ww.w;
+    const int half = n_rot >> 1, hl = half >> 2;  // lanes per rotated half (a power of two)
+    float4 o;
+    o.x = __shfl_xor(v.x, hl, 64);
+    o.y = __shfl_xor(v.y, hl, 64);
+    o.z = __shfl_xor(v.z, hl, 64);
+    o.w = __shfl_xor(v.w, hl, 64);
+    if (li < 2 * hl) {
+        const float4* cs = (const float4*)(rope + (int64_t)pos * half + 4 * (li & (hl - 1)));
+        const float4 c01 = cs[0], c23 = cs[1];  // (cos, sin) of dims i, i+1 and i+2, i+3
+        if (li < hl) {  // x0 = mine, x1 = partner
+            v = make_float4(v.x * c01.x - o.x * c01.y, v.y * c01.z - o.y * c01.w, v.z * c23.x - o.z * c23.y,
+                            v.w * c23.z - o.w * c23.w);
+        } else {        // x0 = partner, x1 = mine
+            v = make_float4(o.x * c01.y + v.x * c01.x, o.y * c01.w + v.y * c01.z, o.z * c23.y + v.z * c23.x,
+                            o.w * c23.w + v.w * c23.z);
+        }
+    }
+    return v;
+}
+
 }  // namespace itk

@@ -32,6 +32,7 @@
 //
 // Every wait is bounded: a poll that runs out of tries sets the abort word, every other wait sees it and the
 // grid drains.  The grid must be resident at once (one block per compute unit), which the launcher checks.
+#define IT_CHAIN_DEVICE_POINTERS
 #include "it_fast.h"
 #include "kernels_fused.h"
 
@@ -62,13 +63,25 @@ constexpr int RS = RD + NE + 2;            // FF shared-expert intermediates
 constexpr int RE = RS + FF;                // NU * FF / 4 packed Q8_0 quads of the routed intermediates, then their scales
 constexpr int RE_SC = RE + NU * FF / 4;
 constexpr int R_END = RE_SC + EB;
-static_assert(R_END <= (int)CHAIN_LL_WORDS, "hand-off space");
+static_assert(R_END <= (int)CHAIN_LL_STAGE_WORDS, "hand-off space");
+// An attention mixer's hand-offs reuse the Gated DeltaNet mixer's regions (a layer has one or the other): the
+// in-projection's [query + gate of every head | key | value] where the conv output goes, the gated attention output
+// where the read-outs go.  The partial results of the key ranges have a space of their own behind the stages'.
+constexpr int NH = 16, NKV = 2, HD = 256, AG = NH / NKV, AS = CHAIN_ATTN_SPLITS;
+constexpr int RQ = RA, RK = RQ + NH * 2 * HD, RV = RK + NKV * HD, RT = RB;
+constexpr int RP = (int)CHAIN_LL_STAGE_WORDS, PW = HD + 2;   // per (query head, key range): HD sums, the maximum, the weight
+constexpr int TK = 64;            // keys of a range that are in LDS at a time
+constexpr int KSTR = HD + 8;      // f16 row stride of the K and V tiles (528 bytes)
+constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + AG * HD * 4 + AG * TK * 4 + (8 + 8 * 4 * 5) * 4;   // K tile, V tile, the eight scaled queries, their probabilities, the merge's partial sums
+static_assert(RV + NKV * HD <= RB && NH * HD <= VDIM && NB == NKV * AS && CW == AG && NB == NH * 16 && NH * 2 * HD == 32 * NB &&
+              NKV * HD == 2 * NB && NH * HD == 8 * CT && HD == 4 * 64 && (PW % 2) == 0 && (RP % 2) == 0, "attention stage shapes");
 static_assert(!(RA & 1) && !(RA_Z & 1) && !(RB & 1) && !(RB_SS & 1) && !(RC & 1) && !(RD & 1) && !(RS & 1) && !(RE & 1) && !(RE_SC & 1), "");
 
 // Stage stamps for tuning: a build with -DIT_CHAIN_STAMPS adds up, per stamp point, the 100 MHz wall clock that block
 // 0's first thread spent since its previous point; the library build compiles them away.
 #ifdef IT_CHAIN_STAMPS
-__device__ long long it_chain_stamps[16];
+__device__ long long it_chain_stamps[24];
+__device__ long long it_attn_core_stamps[8];   // inside an attention mixer's middle, the same clock
 #define CH_STAMP(i)                                          \
     do {                                                     \
         if (b0 == 0 && tid0 == 0) {                          \
@@ -128,7 +141,8 @@ struct Ctl {
 };
 
 IT_DEV void ll_put(u64* p, uint32_t bits, unsigned e) {
-    __hip_atomic_store(p, ((u64)e << 32) | (u64)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    // (the hand-off space is device memory: said so, the store is a global one wherever the pointer came from)
+    __hip_atomic_store((__attribute__((address_space(1))) u64*)p, ((u64)e << 32) | (u64)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 IT_DEV void ll_putf(u64* p, float v, unsigned e) { ll_put(p, __float_as_uint(v), e); }
 
@@ -241,6 +255,20 @@ struct AW {
     float past[3];
     float4 ab;   // unquantized alpha / beta (RF): this wave's four floats a lane of the block's row
 };
+// What the registers held is no longer wanted: without this the values of a layer before stay live, as far as the
+// compiler can tell, through every stage of a layer that loads only a part of them.
+IT_DEV void forget(AW& a) {
+#pragma unroll
+    for (int k = 0; k < 7; k++)
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            a.t[k].w[c] = make_uint4(0, 0, 0, 0);
+            a.t[k].sc[c] = 0;
+        }
+    a.taps = make_float4(0.f, 0.f, 0.f, 0.f);
+    a.past[0] = a.past[1] = a.past[2] = 0.0f;
+    a.ab = make_float4(0.f, 0.f, 0.f, 0.f);
+}
 IT_DEV int a_row(int k, int b, int wave) {   // row k of the wave in its own matrix
     return k < 4 ? b + NB * (wave + CW * k) : k < 6 ? b + NB * (wave + CW * (k - 4)) : b < NV ? b : b - NV;
 }
@@ -254,8 +282,8 @@ IT_DEV float f32_tree(const float* pc) { return ((pc[0] + pc[1]) + (pc[2] + pc[3
 // layer before, IT_CHAIN_A_AT: loads return in the order they were issued, and a poll behind a large fetch waits for
 // all of it.  All at the head of stage F measured best once that stage's input was gathered by waves that issue
 // theirs behind the gather.)
-template <int RF>
-IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int parts = 7) {
+template <int RF, class M>   // M: a ChainMixer, wherever it lives
+IT_DEV void fetch_a(const M& m, AW& a, int b, int wave, int lane, int parts = 7) {
     if (parts & 1) {
 #pragma unroll
         for (int k = 0; k < 2; k++) load_row<W_Q8_0, 2, 64>(a.t[k], m.qkv_q, m.qkv_s, D, a_row(k, b, wave), lane, true);
@@ -288,7 +316,8 @@ IT_DEV void fetch_a(const ChainMixer& m, AW& a, int b, int wave, int lane, int p
 
 // The tail stage's rows (the in-projection of the attention layer behind the chain): 36 a block, row r of the flat list
 // [wq 8192 | wk 512 | wv 512] on block r % 256; a wave takes four wq rows, waves 0..3 one more (wk: 0, 1; wv: 2, 3).
-IT_DEV void fetch_tail(const ChainTail& t, AW& a, int b, int wave, int lane) {
+template <class T>   // ChainTail or ChainAttn: the same three matrices
+IT_DEV void fetch_tail(const T& t, AW& a, int b, int wave, int lane) {
 #pragma unroll
     for (int k = 0; k < 4; k++) load_row<W_Q8_0, 2, 64>(a.t[k], t.q_q, t.q_s, D, b + NB * (wave + CW * k), lane, true);
     const bool kk = wave < 2;
@@ -380,6 +409,265 @@ IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, dou
     return true;
 }
 
+// ---- the middle of an attention mixer: this block's key range against eight query heads, then the merge of the ranges
+// with the sigmoid gate.  A function of its own (never inlined): its registers are allotted apart from the stages
+// around it, which have none to spare.  Its LDS is the launch's dynamic allocation.  Every thread runs through every
+// barrier whatever its waits return; false: one of this thread's waits gave up (the results are void).
+//
+// Key ranges.  Block b: KV head b % 2, range b / 2 of 128 equal ranges of the live context (the last range that holds
+// keys holds the new position, whose key and value rows this block forms and writes to the cache).  Wave w: query head
+// w of the KV head's eight.  The range's rows are in flight before the queries are waited for; scores with 16 lanes a
+// key, softmax bookkeeping a wave, weighted values with 4 dims a lane: all f32 on the vector ALU (a range is a few dozen
+// keys at the contexts this path is measured at; longer ones walk tiles of 64 keys).
+// Merge.  Block b: 16 dims of query head b / 16; thread t: range t / 4, four of the 16 dims.
+extern __shared__ __align__(16) uint8_t chain_dyn_lds[];   // ATTN_LDS bytes when a layer of the chain is an attention mixer
+typedef __attribute__((address_space(1))) uint16_t g_u16;
+struct AttnCoreP {   // what of a ChainAttn the function reads
+    it_gptr<const float> q_norm, k_norm;
+    it_gptr<const float2> rope;
+    it_gptr<uint16_t> k_slab, v_slab;
+    it_gptr<const int> n_pos;
+    it_gptr<const uint8_t> o_q, o_s;   // the out-projection
+    float eps_head, scale;
+    int n_rot;
+};
+struct AttnCoreR {
+    float dot;   // this wave's out-projection row against the gated attention output (in lane 63)
+    int ok;      // 0: one of this thread's waits gave up
+};
+// (the arguments one by one, so that they travel in registers: a struct by value goes through the stack)
+__attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_norm, it_gptr<const float> k_norm, it_gptr<const float2> rope,
+                                                         it_gptr<uint16_t> k_slab, it_gptr<uint16_t> v_slab, it_gptr<const int> n_pos_p,
+                                                         it_gptr<const uint8_t> o_q, it_gptr<const uint8_t> o_s, float eps_head, float scale,
+                                                         int n_rot, it_gptr<u64> ll_g, unsigned e, it_gptr<unsigned> abort_g, int spin_limit, int tid,
+                                                         int b) {
+    u64* const ll = (u64*)ll_g;   // (polled through explicit global loads, stored to as global: see ll_put)
+    unsigned* const abort_flag = (unsigned*)abort_g;
+    const AttnCoreP at{q_norm, k_norm, rope, k_slab, v_slab, n_pos_p, o_q, o_s, eps_head, scale, n_rot};
+    const Ctl ctl{abort_flag, spin_limit};
+#ifdef IT_CHAIN_STAMPS
+    long long ac_prev = wall_clock64();
+#define AC_STAMP(i)                                      \
+    do {                                                 \
+        if (b == 0 && tid == 0) {                        \
+            const long long now = wall_clock64();        \
+            it_attn_core_stamps[i] += now - ac_prev;     \
+            ac_prev = now;                               \
+        }                                                \
+    } while (0)
+#else
+#define AC_STAMP(i) \
+    do {            \
+    } while (0)
+#endif
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint16_t* const Ks = (uint16_t*)chain_dyn_lds;
+    uint16_t* const Vs = Ks + TK * KSTR;
+    float* const Qf = (float*)(Vs + TK * KSTR);
+    float* const Pf = Qf + AG * HD;
+    float* const sm = Pf + AG * TK;      // 8 wave maxima
+    float* const ws = sm + 8;            // 8 waves x 4 dim groups x (4 sums + the weight)
+    bool ok = true;
+    const int n_pos = *at.n_pos;
+    const int kpb = max(1, (n_pos + AS - 1) / AS);
+    {
+        const int kvh = b & 1, split = b >> 1;
+        const int k0 = split * kpb, k1 = min(n_pos, k0 + kpb), pos_new = n_pos - 1;
+        const int nk = k1 - k0;                                   // keys of the range (none: nothing to do, nothing published)
+        const int new_at = (pos_new >= k0 && pos_new < k1) ? pos_new - k0 : -1;   // the new position's place in the range
+        const int n_old = new_at >= 0 ? nk - 1 : nk;              // ... the others are in the cache already
+        const g_u16* kb = (const g_u16*)at.k_slab + (int64_t)k0 * (NKV * HD) + kvh * HD;
+        const g_u16* vb = (const g_u16*)at.v_slab + (int64_t)k0 * (NKV * HD) + kvh * HD;
+        typedef __attribute__((address_space(1))) v4u g_v4u;
+        auto ld16 = [](const g_u16* q) {
+            const v4u t = *(const g_v4u*)q;
+            return make_uint4(t.x, t.y, t.z, t.w);
+        };
+        uint4 rk[4], rv[4];
+        auto fetch_kv = [&](int t0) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = tid + i * CT, key = t0 + (idx >> 5), seg = idx & 31;
+                const bool live = key < n_old;
+                rk[i] = live ? ld16(kb + (int64_t)key * (NKV * HD) + seg * 8) : make_uint4(0, 0, 0, 0);
+                rv[i] = live ? ld16(vb + (int64_t)key * (NKV * HD) + seg * 8) : make_uint4(0, 0, 0, 0);
+            }
+        };
+        auto stash_kv = [&](int t0) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = tid + i * CT, key = idx >> 5, seg = idx & 31;
+                if (t0 + key == new_at) continue;   // the new position's rows come from the waves that form them
+                *(uint4*)(Ks + key * KSTR + seg * 8) = rk[i];
+                *(uint4*)(Vs + key * KSTR + seg * 8) = rv[i];
+            }
+        };
+        uint2 fresh = make_uint2(0, 0);   // wave 0: the new key row's four f16 of this lane; wave 1: the new value row's
+        if (nk > 0) {
+            fetch_kv(0);
+            float4 qv;
+            ok = ll_wait_quad(ll + RQ + (kvh * AG + wave) * 2 * HD, lane, e, ctl, &qv);
+            if (ok) {
+                qv = head_norm_rope<HD>(qv, at.q_norm, at.eps_head, at.rope, at.n_rot, pos_new, lane);
+                const float qsc = at.scale * 1.4426950408889634f;
+                ((float4*)(Qf + wave * HD))[lane] = make_float4(qv.x * qsc, qv.y * qsc, qv.z * qsc, qv.w * qsc);
+            }
+            if (ok && new_at >= 0 && wave < 2) {
+                float4 nv;
+                ok = ll_wait_quad(ll + (wave == 0 ? RK : RV) + kvh * HD, lane, e, ctl, &nv);
+                if (ok) {
+                    if (wave == 0) nv = head_norm_rope<HD>(nv, at.k_norm, at.eps_head, at.rope, at.n_rot, pos_new, lane);
+                    fresh.x = (uint32_t)it_f32_to_f16(nv.x) | ((uint32_t)it_f32_to_f16(nv.y) << 16);
+                    fresh.y = (uint32_t)it_f32_to_f16(nv.z) | ((uint32_t)it_f32_to_f16(nv.w) << 16);
+                    typedef __attribute__((address_space(1))) v2u g_v2u;
+                    *(g_v2u*)((g_u16*)(wave == 0 ? at.k_slab : at.v_slab) + (int64_t)pos_new * (NKV * HD) + kvh * HD + 4 * lane) = v2u{fresh.x, fresh.y};
+                }
+            }
+        }
+        AC_STAMP(0);   // rows issued, queries (and the new key / value) gathered and prepared
+        __syncthreads();
+        AC_STAMP(1);
+        if (nk > 0) {
+            const int j = lane >> 4, c = lane & 15;
+            float q16[16];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const float4 a0 = ((const float4*)(Qf + wave * HD + 128 * i + 8 * c))[0], a1 = ((const float4*)(Qf + wave * HD + 128 * i + 8 * c))[1];
+                q16[8 * i + 0] = a0.x; q16[8 * i + 1] = a0.y; q16[8 * i + 2] = a0.z; q16[8 * i + 3] = a0.w;
+                q16[8 * i + 4] = a1.x; q16[8 * i + 5] = a1.y; q16[8 * i + 6] = a1.z; q16[8 * i + 7] = a1.w;
+            }
+            float m_run = -INFINITY, l_run = 0.0f;
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int t0 = 0; t0 < nk; t0 += TK) {
+                if (t0) __syncthreads();   // every wave is done with the tile before
+                stash_kv(t0);
+                if (new_at >= t0 && new_at < t0 + TK && wave < 2) *(uint2*)((wave == 0 ? Ks : Vs) + (new_at - t0) * KSTR + 4 * lane) = fresh;
+                __syncthreads();
+                if (t0 + TK < nk) fetch_kv(t0 + TK);
+                const int nt = min(TK, nk - t0);
+                // scores: 16 lanes a key, four keys a step; they go to LDS, where lane k finds key k's
+#pragma unroll 2
+                for (int g = 0; g < (nt + 3) / 4; g++) {
+                    const uint16_t* kr = Ks + (4 * g + j) * KSTR + 8 * c;
+                    const uint4 ka = *(const uint4*)kr, kc = *(const uint4*)(kr + 128);
+                    const uint32_t w[8] = {ka.x, ka.y, ka.z, ka.w, kc.x, kc.y, kc.z, kc.w};
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        sum = fmaf(it_f16_to_f32(w[i] & 0xffffu), q16[2 * i], sum);
+                        sum = fmaf(it_f16_to_f32(w[i] >> 16), q16[2 * i + 1], sum);
+                    }
+                    sum = group_sum<16>(sum);
+                    if (c == 0) Pf[wave * TK + 4 * g + j] = sum;
+                }
+                const float sc = lane < nt ? Pf[wave * TK + lane] : -INFINITY;
+                const float m_new = fmaxf(m_run, group_max<64>(sc));   // finite: the tile has a key
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                const float pr = __builtin_amdgcn_exp2f(sc - m_new);
+                Pf[wave * TK + lane] = pr;
+                const float psum = group_sum<64>(pr);
+                l_run = l_run * alpha + psum;
+                o.x *= alpha; o.y *= alpha; o.z *= alpha; o.w *= alpha;
+                m_run = m_new;
+                for (int key = 0; key < nt; key++) {
+                    const float pk = Pf[wave * TK + key];
+                    const uint2 vv = *(const uint2*)(Vs + key * KSTR + 4 * lane);
+                    o.x = fmaf(pk, it_f16_to_f32(vv.x & 0xffffu), o.x);
+                    o.y = fmaf(pk, it_f16_to_f32(vv.x >> 16), o.y);
+                    o.z = fmaf(pk, it_f16_to_f32(vv.y & 0xffffu), o.z);
+                    o.w = fmaf(pk, it_f16_to_f32(vv.y >> 16), o.w);
+                }
+            }
+            AC_STAMP(2);   // the range's keys done
+            u64* part = ll + RP + (int64_t)((kvh * AG + wave) * AS + split) * PW;
+            ll_putf(part + 4 * lane, o.x, e);
+            ll_putf(part + 4 * lane + 1, o.y, e);
+            ll_putf(part + 4 * lane + 2, o.z, e);
+            ll_putf(part + 4 * lane + 3, o.w, e);
+            if (lane == 0) {
+                ll_putf(part + HD, m_run, e);
+                ll_putf(part + HD + 1, l_run, e);
+            }
+        }
+    }
+    AC_STAMP(3);   // partial results published
+    {
+        const int h = b >> 4, dc = b & 15;
+        const int n_live = (n_pos + kpb - 1) / kpb;   // ranges that hold keys
+        const int sp = tid >> 2, q4 = tid & 3;
+        float m_s = -INFINITY, l_s = 0.0f;
+        float4 o_s = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (sp < n_live) {
+            const u64* base = ll + RP + (int64_t)(h * AS + sp) * PW;
+            const u64* const a4[4] = {base + dc * 16 + q4 * 4, base + dc * 16 + q4 * 4 + 2, base + HD, base + HD};
+            uint32_t w8[8];
+            if (ll_wait_pairs<4>(a4, e, ctl, w8)) {
+                o_s = make_float4(__uint_as_float(w8[0]), __uint_as_float(w8[1]), __uint_as_float(w8[2]), __uint_as_float(w8[3]));
+                m_s = __uint_as_float(w8[4]);
+                l_s = __uint_as_float(w8[5]);
+            } else {
+                ok = false;
+            }
+        }
+        AC_STAMP(4);   // the ranges' results gathered
+        const float mx = group_max<64>(m_s);
+        if (lane == 0) sm[wave] = mx;
+        __syncthreads();
+        float big = sm[0];
+#pragma unroll
+        for (int w = 1; w < CW; w++) big = fmaxf(big, sm[w]);
+        const float wgt = m_s != -INFINITY ? __builtin_amdgcn_exp2f(m_s - big) : 0.0f;
+        float vals[5] = {wgt * o_s.x, wgt * o_s.y, wgt * o_s.z, wgt * o_s.w, wgt * l_s};
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            vals[i] += __shfl_xor(vals[i], 4, 64);
+            vals[i] += __shfl_xor(vals[i], 8, 64);
+            vals[i] += __shfl_xor(vals[i], 16, 64);
+            vals[i] += __shfl_xor(vals[i], 32, 64);
+        }
+        if (lane < 4) {
+#pragma unroll
+            for (int i = 0; i < 5; i++) ws[(wave * 4 + lane) * 5 + i] = vals[i];
+        }
+        __syncthreads();
+        if (tid < 16) {
+            const int q = tid >> 2, i = tid & 3;
+            float osum = 0.0f, lsum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < CW; w++) {
+                osum += ws[(w * 4 + q) * 5 + i];
+                lsum += ws[(w * 4 + q) * 5 + 4];
+            }
+            uint32_t gw = 0;
+            if (!ll_wait1(ll + RQ + h * 2 * HD + HD + dc * 16 + tid, e, ctl, &gw)) ok = false;
+            ll_putf(ll + RT + h * HD + dc * 16 + tid, osum / lsum * fx_sigmoid(__uint_as_float(gw)), e);
+        }
+    }
+    AC_STAMP(5);   // merged and published
+    // out-projection (quantize + matmul, qwen35.rs:1216-1223): the gated output of every head, Q8_0 (in the K tile's
+    // place: the barriers of the merge are behind every read of it), this wave's row
+    float dot;
+    {
+        const int my_row = b * CW + wave;
+        WChunks<4> wo;
+        load_row<W_Q8_0, 4, 64>(wo, at.o_q, at.o_s, VDIM, my_row, lane, true);
+        int8_t* const oq = (int8_t*)chain_dyn_lds;
+        float* const os = (float*)(chain_dyn_lds + NH * HD);
+        const u64* const a4[4] = {ll + RT + 4 * tid, ll + RT + 4 * tid + 2, ll + RT + 4 * (tid + CT), ll + RT + 4 * (tid + CT) + 2};
+        uint32_t o8[8];
+        if (!ll_wait_pairs<4>(a4, e, ctl, o8)) ok = false;
+        AC_STAMP(6);   // the gated output gathered
+        quant_quad(make_float4(__uint_as_float(o8[0]), __uint_as_float(o8[1]), __uint_as_float(o8[2]), __uint_as_float(o8[3])), true, tid, oq, os);
+        quant_quad(make_float4(__uint_as_float(o8[4]), __uint_as_float(o8[5]), __uint_as_float(o8[6]), __uint_as_float(o8[7])), true, tid + CT, oq, os);
+        __syncthreads();
+        XChunks<W_Q8_0, 4> x;
+        load_x<W_Q8_0, 4, 64>(x, oq, os, lane);
+        dot = reduce_lanes<64>(dot_chunks<W_Q8_0, 4>(wo, x));
+    }
+    AC_STAMP(7);
+    return AttnCoreR{dot, ok ? 1 : 0};
+}
+
 template <int SF, int RF>
 __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     __shared__ __align__(16) int8_t xq[NU * FF + FF];   // the stage's quantized activation (largest: the down stage's)
@@ -404,6 +692,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
     float x_row = (tid0 & 63) == 63 ? p.x[b0 * CW + (tid0 >> 6)] : 0.0f;
     AW aw;
     if (p.layer[0].has_mixer == 1) fetch_a<RF>(p.layer[0].m, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
+    if (p.layer[0].has_mixer == 3) fetch_tail(p.layer[0].a, aw, b0, __builtin_amdgcn_readfirstlane(tid0 >> 6), tid0 & 63);
     __syncthreads();
 
 #ifdef IT_CHAIN_STAMPS
@@ -428,9 +717,9 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
             wave = __builtin_amdgcn_readfirstlane(tid >> 6);   \
             my_row = b * CW + wave;                            \
         } while (0)
-        const ChainLayer& L = p.layer[l];
-        const ChainMixer& m = L.m;
-        const ChainFfn& f = L.f;
+        const auto& L = p.layer[l];
+        const auto& m = L.m;
+        const auto& f = L.f;
         const unsigned e = e0 + 1 + (unsigned)l;
         const bool mixer = L.has_mixer != 0;   // the FFN's input comes from a mixer stage of this kernel
 
@@ -485,6 +774,50 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
                 x_row += acc;
                 ll_putf(p.ll + RC + my_row, x_row, e);
             }
+        }
+        if (L.has_mixer == 3) {
+            // ---------------------------------------------------------------- a whole attention mixer
+            // (qwen35.rs:1141-1223: rms_norm, wq / wk / wv, head norms, rotation, cache rows, attention, sigmoid gate,
+            // out-projection + residual.)  Three exchanges more than a Gated DeltaNet mixer's: the in-projection's
+            // outputs, the key ranges' partial results, the gated output.
+            const auto& at = L.a;
+            {
+                const float4 nw = ((const float4*)at.norm_w)[tid];
+                float4 v;
+                bool ok = true;
+                if (l == 0) v = ((const float4*)p.x)[tid];
+                else ok = ll_wait_quad(p.ll + RX, tid, e, ctl, &v);
+                if (!ok) dead = 1;
+                CH_STAMP(16);
+                if (!norm_quant(v, nw, at.eps, xq, xs, red, &dead, tid)) break;
+                XChunks<W_Q8_0, 2> x;
+                load_x<W_Q8_0, 2, 64>(x, xq, xs, lane);
+                float mine = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 5; k++) {
+                    const float acc = reduce_lanes<64>(dot_chunks<W_Q8_0, 2>(aw.t[k], x));
+                    const float r = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc), 63));
+                    mine = lane == k ? r : mine;
+                }
+                if (lane < 4) ll_putf(p.ll + RQ + b + NB * (wave + CW * lane), mine, e);
+                else if (lane == 4 && wave < 2) ll_putf(p.ll + RK + b + NB * wave, mine, e);
+                else if (lane == 4 && wave < 4) ll_putf(p.ll + RV + b + NB * (wave - 2), mine, e);
+            }
+            CH_STAMP(17);
+            // ---------------------------------------------------------------- attention over the context, merge, sigmoid gate
+            // (a function of its own: its registers are allotted apart from the stages around it, which have none to spare)
+            forget(aw);
+            const AttnCoreR r = attn_core(at.q_norm, at.k_norm, at.rope, at.k_slab, at.v_slab, at.n_pos, m.o_q, m.o_s, at.eps_head, at.scale, at.n_rot,
+                                          (it_gptr<u64>)p.ll, e, (it_gptr<unsigned>)p.abort_flag, p.spin_limit, tid, b);
+            CH_STAMP(18);
+            fetch_d();
+            if (!r.ok) dead = 1;
+            if (lane == 63) {   // + residual
+                x_row += r.dot;
+                ll_putf(p.ll + RC + my_row, x_row, e);
+            }
+            __syncthreads();
+            if (dead) break;
         }
         if (L.has_mixer == 1) {
             // ---------------------------------------------------------------- loads known from the start of the layer
@@ -952,6 +1285,7 @@ __global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
         // own wave has in flight)
         auto fetch_next = [&]() {
             if (l + 1 == p.n_layers && p.has_tail) fetch_tail(p.tail, aw, b, wave, lane);
+            if (l + 1 < p.n_layers && p.layer[l + 1].has_mixer == 3) fetch_tail(p.layer[l + 1].a, aw, b, wave, lane);
             if (next_mixer && ((IT_CHAIN_A_AT >> 4) & 15)) fetch_a<RF>(p.layer[l + 1].m, aw, b, wave, lane, (IT_CHAIN_A_AT >> 4) & 15);
         };
         if (!IT_CHAIN_F_POLLERS || wave < 4) fetch_next();
@@ -1105,8 +1439,11 @@ bool layer_chain_fits() {
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < NB) return false;
         const void* fns[4] = {(const void*)layer_chain_k<W_Q8_0, 0>, (const void*)layer_chain_k<W_NVFP4, 0>,
                               (const void*)layer_chain_k<W_Q8_0, 1>, (const void*)layer_chain_k<W_NVFP4, 1>};
+        // (with the LDS an attention mixer's stages take: every instance is launched with it when a layer is one)
         for (const void* fn : fns)
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, CT, 0) != hipSuccess || occ < 1) return false;
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, ATTN_LDS) != hipSuccess ||
+                hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fn, CT, ATTN_LDS) != hipSuccess || occ < 1)
+                return false;
         return true;
     }();
     return fits;
@@ -1121,11 +1458,17 @@ bool layer_chain(const ChainP& p, hipStream_t s) {
             if (!q) return false;
         return true;
     };
+    bool has_attn = false;
     for (int l = 0; l < p.n_layers; l++) {
         const ChainMixer& m = p.layer[l].m;
         const ChainFfn& f = p.layer[l].f;
         const int kind = p.layer[l].has_mixer;
-        if (kind < 0 || kind > 2 || (kind == 2 && l != 0)) return false;
+        if (kind < 0 || kind > 3 || (kind == 2 && l != 0)) return false;
+        const ChainAttn& a = p.layer[l].a;
+        if (kind == 3 && (!all({a.norm_w, a.q_q, a.q_s, a.k_q, a.k_s, a.v_q, a.v_s, a.q_norm, a.k_norm, a.rope, a.k_slab, a.v_slab, a.n_pos,
+                                m.o_q, m.o_s}) || a.n_rot <= 0 || a.n_rot > HD || (a.n_rot / 2) % 4 || ((a.n_rot / 8) & (a.n_rot / 8 - 1))))
+            return false;
+        has_attn = has_attn || kind == 3;
         if (kind == 1 && !p.rf && !all({m.a_s, m.b_s})) return false;
         if (!p.rf && !all({f.r_s, f.l_s})) return false;
         if (kind == 1 && !all({m.norm_w, m.qkv_q, m.qkv_s, m.z_q, m.z_s, m.a_q, m.b_q, m.conv_state, m.conv_w, m.ssm_a,
@@ -1140,11 +1483,27 @@ bool layer_chain(const ChainP& p, hipStream_t s) {
                             p.tail.out_k, p.tail.out_v}))
         return false;
     if (!layer_chain_fits()) return false;
-    if (p.sh_fmt == W_Q8_0 && !p.rf) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 0>), dim3(NB), dim3(CT), 0, s, p);
-    else if (!p.rf) hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 0>), dim3(NB), dim3(CT), 0, s, p);
-    else if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 1>), dim3(NB), dim3(CT), 0, s, p);
-    else hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 1>), dim3(NB), dim3(CT), 0, s, p);
+    const size_t lds = has_attn ? ATTN_LDS : 0;
+    if (p.sh_fmt == W_Q8_0 && !p.rf) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 0>), dim3(NB), dim3(CT), lds, s, p);
+    else if (!p.rf) hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 0>), dim3(NB), dim3(CT), lds, s, p);
+    else if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 1>), dim3(NB), dim3(CT), lds, s, p);
+    else hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 1>), dim3(NB), dim3(CT), lds, s, p);
     return true;
 }
 
 }  // namespace itk
+
+#ifdef IT_CHAIN_STAMPS
+// tuning builds only: the stage sums (24) and the attention middle's (8), then zeroed
+namespace itk {
+bool chain_stamps_take(long long* out) {
+    long long zero[32] = {0};
+    if (hipDeviceSynchronize() != hipSuccess) return false;
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(it_chain_stamps), 24 * 8) != hipSuccess) return false;
+    if (hipMemcpyFromSymbol(out + 24, HIP_SYMBOL(it_attn_core_stamps), 8 * 8) != hipSuccess) return false;
+    return hipMemcpyToSymbol(HIP_SYMBOL(it_chain_stamps), zero, 24 * 8) == hipSuccess &&
+           hipMemcpyToSymbol(HIP_SYMBOL(it_attn_core_stamps), zero, 8 * 8) == hipSuccess;
+}
+}  // namespace itk
+extern "C" int it_hip_debug_chain_stamps(long long* out) { return itk::chain_stamps_take(out) ? 0 : -1; }
+#endif

@@ -126,49 +126,79 @@ bool moe_down_fast(MoeDownP p, hipStream_t s, bool dry_run = false);
 // weights of a stage are in the block's registers before its inputs arrive.
 // Shapes are fixed (hidden 2048; 16 key / 32 value heads of 128; 512 NVFP4 experts, top 10, 512 rows; a shared
 // expert of 512 rows in Q8_0 or NVFP4; Q8_0 dense matrices); anything else stays on the per-stage launches.
+// Pointers inside the chain's structs are device-memory pointers, and on the device they are declared as such: a
+// pointer of unknown kind that reaches a function which is not inlined is a generic one there, whose loads are FLAT
+// loads (which every wait for LDS has to drain).  Same size and layout on the host.
+#if defined(__HIP_DEVICE_COMPILE__) && defined(IT_CHAIN_DEVICE_POINTERS)   // (set by the file that holds the kernel; host code elsewhere fills plain pointers)
+template <class T> using it_gptr = T __attribute__((address_space(1)))*;
+#else
+template <class T> using it_gptr = T*;
+#endif
 struct ChainMixer {
-    const float* norm_w;
-    const uint8_t *qkv_q, *qkv_s, *z_q, *z_s, *a_q, *a_s, *b_q, *b_s;
-    float* conv_state;
-    const float* conv_w;
-    const float *ssm_a, *dt_bias;
-    float* state;
-    const float* head_norm_w;
-    const uint8_t *o_q, *o_s;
+    it_gptr<const float> norm_w;
+    it_gptr<const uint8_t> qkv_q, qkv_s, z_q, z_s, a_q, a_s, b_q, b_s;
+    it_gptr<float> conv_state;
+    it_gptr<const float> conv_w;
+    it_gptr<const float> ssm_a, dt_bias;
+    it_gptr<float> state;
+    it_gptr<const float> head_norm_w;
+    it_gptr<const uint8_t> o_q, o_s;
     float eps_norm, eps_l2, eps_head, q_scale;
-    const float* attn;   // has_mixer == 2 only: the attention block's gated output [4096], the out-projection's input
+    it_gptr<const float> attn;   // has_mixer == 2 only: the attention block's gated output [4096], the out-projection's input
 };
 struct ChainFfn {
-    const float* norm_w;
-    const uint8_t *r_q, *r_s, *l_q, *l_s;       // router rows; the shared expert's gate-logit row
-    const uint8_t *sg_q, *sg_s, *su_q, *su_s;   // shared expert gate / up
-    const uint8_t *sd_q, *sd_s;                 // shared expert down
-    const uint8_t *eg_q, *eg_s, *eu_q, *eu_s, *ed_q, *ed_s;   // routed experts
-    const float *gscale2, *uscale2, *dscale2;
+    it_gptr<const float> norm_w;
+    it_gptr<const uint8_t> r_q, r_s, l_q, l_s;   // router rows, and the shared expert's gate-logit row
+    it_gptr<const uint8_t> sg_q, sg_s, su_q, su_s;   // shared expert gate / up
+    it_gptr<const uint8_t> sd_q, sd_s;                 // shared expert down
+    it_gptr<const uint8_t> eg_q, eg_s, eu_q, eu_s, ed_q, ed_s;   // routed experts
+    it_gptr<const float> gscale2, uscale2, dscale2;
     int64_t gu_q_stride, gu_s_stride, d_q_stride, d_s_stride;
     float sh_gscale, sh_uscale, sh_dscale, eps;
-    int32_t* route_ids;     // seam outputs: this layer's picks and their weights
-    float* route_w;
-    uint32_t *counts_gate, *counts_up, *counts_down;   // expert read counters (optional)
+    it_gptr<int32_t> route_ids;     // seam outputs: this layer's picks and their weights
+    it_gptr<float> route_w;
+    it_gptr<uint32_t> counts_gate, counts_up, counts_down;   // expert read counters (optional)
 };
 // The in-projection of the attention layer BEHIND the chain's last layer (rms_norm + quantization + rows of wq, wk,
 // wv), run as the chain's last stage; its outputs go to ordinary memory for the attention kernels that follow.
 struct ChainTail {
-    const float* norm_w;
-    const uint8_t *q_q, *q_s, *k_q, *k_s, *v_q, *v_s;   // wq (8192 rows: query and gate of every head), wk, wv (512 rows each)
-    float *out_q, *out_k, *out_v;
+    it_gptr<const float> norm_w;
+    it_gptr<const uint8_t> q_q, q_s, k_q, k_s, v_q, v_s;   // wq (8192 rows: query and gate of every head), wk, wv (512 rows each)
+    it_gptr<float> out_q, out_k, out_v;
     float eps;
+};
+// A whole attention mixer inside the chain (has_mixer == 3): in-projection, norm + rotation of the query heads and of
+// the new key, the cache rows of the new position, attention over the context split over the blocks, merge + sigmoid
+// gate; the out-projection's matrix is the layer's ChainMixer o_q / o_s.  16 query heads of 256 on 2 KV heads.
+struct ChainAttn {
+    it_gptr<const float> norm_w;
+    it_gptr<const uint8_t> q_q, q_s, k_q, k_s, v_q, v_s;   // wq (8192 rows: query and gate of every head), wk, wv (512 rows each)
+    it_gptr<const float> q_norm, k_norm;
+    it_gptr<const float2> rope;      // [pos][n_rot / 2] (cos, sin)
+    it_gptr<uint16_t> k_slab, v_slab;   // f16 [pos][512]
+    it_gptr<const int> n_pos;        // device word: positions in the context, this token's included
+    float eps, eps_head, scale;
+    int n_rot;
 };
 struct ChainLayer {
     // 0: the layer's mixer ran before the chain; 1: a Gated DeltaNet mixer; 2: an attention layer whose out-projection
-    // (+ residual) opens the chain (first layer only: its input is in ordinary memory when the kernel starts)
+    // (+ residual) opens the chain (first layer only: its input is in ordinary memory when the kernel starts);
+    // 3: an attention mixer, all of it
     int has_mixer;
     ChainMixer m;
     ChainFfn f;
+    ChainAttn a;
 };
-constexpr int CHAIN_MAX_LAYERS = 4;
+// layers of one chain: a model's whole token when every block of it fits the stages.  They travel in the kernel's
+// argument block (30 KB at this limit, which the runtime takes, also for a captured launch), where the compiler knows
+// them to be readable and unchanging and loads them ahead of their uses; a table in device memory, which it must load
+// where each value is used, measured 2.7 % slower per token.
+constexpr int CHAIN_MAX_LAYERS = 56;
 constexpr int CHAIN_BLOCKS = 256;
-constexpr size_t CHAIN_LL_WORDS = 24576;   // 8-byte words of hand-off space a chain uses
+constexpr int CHAIN_ATTN_SPLITS = 128;     // key ranges of an in-chain attention (two KV heads x 128 ranges = the grid)
+constexpr size_t CHAIN_LL_STAGE_WORDS = 24576;   // 8-byte words of hand-off space of the stages
+// ... and behind them the attention partials: per (query head, key range) 256 sums, the range's maximum and its weight
+constexpr size_t CHAIN_LL_WORDS = CHAIN_LL_STAGE_WORDS + (size_t)16 * CHAIN_ATTN_SPLITS * 258;
 struct ChainP {
     ChainLayer layer[CHAIN_MAX_LAYERS];
     int n_layers;
@@ -177,11 +207,11 @@ struct ChainP {
     int sh_fmt;                  // the shared expert's format (W_Q8_0 or W_NVFP4)
     int rf;                      // 1: the router, the shared expert's gate-logit row and ssm alpha / beta are F32 matrices (as real
                                  // files keep them; their *_q pointers hold floats, their *_s are null), 0: Q8_0
-    float* x;                    // residual stream [2048], read at the start and current after every layer
-    unsigned long long* ll;      // CHAIN_LL_WORDS words of uncached device memory, zero before the first chain
-    unsigned* epoch;             // device word: the last epoch any chain has used (starts at 0)
-    unsigned* abort_flag;        // uncached device word: set when a bounded wait gave up (the results are then void)
-    unsigned long long* tally;   // expert read tally (optional)
+    it_gptr<float> x;                    // residual stream [2048], read at the start and current after every layer
+    it_gptr<unsigned long long> ll;      // CHAIN_LL_WORDS words of uncached device memory, zero before the first chain
+    it_gptr<unsigned> epoch;             // device word: the last epoch any chain has used (starts at 0)
+    it_gptr<unsigned> abort_flag;        // uncached device word: set when a bounded wait gave up (the results are then void)
+    it_gptr<unsigned long long> tally;   // expert read tally (optional)
     int spin_limit;              // polls a wait may take before it gives up
 };
 // whether this device can hold the chain's grid (one block per compute unit, all resident at once)

@@ -53,7 +53,7 @@ def far(got, want):
 class Layers:
     """Weights of `n` layers over shared expert tensors (one set of 512 experts serves every layer: 0.9 GB)."""
 
-    def __init__(self, pair, n, shared, seed=7, small_f32=False):
+    def __init__(self, pair, n, shared, seed=7, small_f32=False, mute_ffn=False):
         """small_f32: the router, the shared expert's gate-logit row and ssm alpha / beta as F32 matrices, as real files
         of this model keep them (/root/reference src/model/qwen35.rs:1626, :1273: `matmul_pair` on unquantized weights
         reads the f32 activation itself), instead of Q8_0."""
@@ -69,6 +69,8 @@ class Layers:
         g_s = (0.5 + r.random(NE)).astype(np.float32) / 54.0
         u_s = (0.5 + r.random(NE)).astype(np.float32) / 54.0
         d_s = (0.5 + r.random(NE)).astype(np.float32) / 108.0
+        if mute_ffn:   # second scales of zero on every down product: the FFN runs and adds nothing (NVFP4 shared expert)
+            d_s[:] = 0.0
         self.gate_raw = nvfp4_rows(r, NE * FF, ND)
         self.gate = pair.e(self.gate_raw, ih.NVFP4, ND, FF, NE, g_s)
         self.up = pair.e(nvfp4_rows(r, NE * FF, ND), ih.NVFP4, ND, FF, NE, u_s)
@@ -91,7 +93,7 @@ class Layers:
                 d["sg"] = pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF)
                 d["su"] = pair.w(nvfp4_rows(r, SFF, ND), ih.NVFP4, ND, SFF)
                 d["sd"] = pair.w(nvfp4_rows(r, ND, SFF), ih.NVFP4, SFF, ND)
-                d["s"] = (float(0.7 / 54.0), float(1.3 / 54.0), float(1.1 / 27.0))
+                d["s"] = (float(0.7 / 54.0), float(1.3 / 54.0), 0.0 if mute_ffn else float(1.1 / 27.0))
             d["ffn_norm"] = (0.5 + r.random(ND)).astype(np.float32)
             self.L.append(d)
 
@@ -333,10 +335,88 @@ def test_a_wait_that_gives_up_is_an_error_not_a_hang():
     assert err is None, err
 
 
-def test_an_attention_layer_between_chains():
-    """layer 0 (Gated DeltaNet + FFN), layer 1 (attention + FFN), layer 2 (Gated DeltaNet + FFN) in one pass.  The
-    attention layer's in-projection becomes the last stage of the first chain and its out-projection the first stage of
-    the second; norm + rotation + cache write + split-K attention stay the launch between them: three kernels in all.
+@pytest.mark.parametrize("pos0", [5800, 40, 12000])
+def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
+    """One attention layer whose FFN adds nothing (second scales of zero on every down product), so that the pass's
+    change of the residual stream IS the mixer's output: in-projection, head norms, rotation, the new cache rows,
+    attention over the context in 128 key ranges, merge, sigmoid gate, out-projection, all stages of the persistent
+    kernel.  Held to the oracle at 2e-3 of the vector's scale and the new K / V rows at 2e-3 of the row's, five
+    positions each: a context of 5,800 (a range is 46 keys: one tile), of 40 (fewer keys than ranges: most blocks have
+    none) and of 12,000 (a range is 94 keys: two tiles with the running maximum carried across)."""
+    NH, NKV, AHD, NROT, THETA, NCTX = 16, 2, 256, 64, 1e7, 12288
+    qd, kd = NH * AHD, NKV * AHD
+    sc = float(1.0 / np.sqrt(np.float32(AHD)))
+    pair = make_pair(True)
+    hip, orc = pair.hip, pair.orc
+    try:
+        layers = Layers(pair, 1, "nvfp4_scaled", seed=31, mute_ffn=True)
+        r = rng(32)
+        wq, wk, wv = pair.q8(r, 2 * qd, ND, 2.0), pair.q8(r, kd, ND, 2.0), pair.q8(r, kd, ND, 2.0)
+        wo = pair.q8(r, ND, qd, 2.0)
+        anorm = (0.5 + r.random(ND)).astype(np.float32)
+        qn = (0.5 + r.random(AHD)).astype(np.float32); kn = (0.5 + r.random(AHD)).astype(np.float32)
+        # keys with a spread of lengths, so that the probabilities are not flat and a few keys carry most of a head's weight
+        k0 = f16_bits(r.standard_normal(NCTX * kd) * np.repeat(np.exp(r.standard_normal(NCTX * NKV) * 0.7), AHD))
+        v0 = f16_bits(r.standard_normal(NCTX * kd))
+        k0[pos0 * kd:] = 0; v0[pos0 * kd:] = 0
+        slabs = [dict(k=k0.copy(), v=v0.copy()) for _ in range(2)]
+        A = bufs(normed=ND, qg=2 * qd, q=qd, g=qd, k=kd, v=kd, attn=qd, mixed=ND)
+        B = layers.buffers()
+
+        def run(ops, i, is_hip, pos):
+            W = lambda t: t[i]
+            b, s, x = A[i], slabs[i], B[i]["x"]
+            ops.rms_norm(x, anorm, EPS, b["normed"])
+            ops.matmul(W(wq), b["normed"], b["qg"])
+            ops.gather_chunks(b["qg"], AHD, 2 * AHD, 0, b["q"]); ops.gather_chunks(b["qg"], AHD, 2 * AHD, AHD, b["g"])
+            ops.matmul(W(wk), b["normed"], b["k"]); ops.matmul(W(wv), b["normed"], b["v"])
+            ops.rms_norm_heads(b["q"], qn, AHD, EPS); ops.rms_norm_heads(b["k"], kn, AHD, EPS)
+            ops.rope_neox(b["q"], pos, AHD, NROT, NH, THETA); ops.rope_neox(b["k"], pos, AHD, NROT, NKV, THETA)
+            ops.kv_write(s["k"], pos * kd, b["k"]); ops.kv_write(s["v"], pos * kd, b["v"])
+            ops.attend(b["q"], s["k"], s["v"], kd, pos + 1, AHD, NH, NKV, sc, b["attn"])
+            ops.sigmoid_mul(b["attn"], b["g"])
+            ops.matmul(W(wo), b["attn"], b["mixed"])
+            ops.add_assign(x, b["mixed"])
+            layers.ffn(ops, i, layers.L[0], B[i]["layers"][0], x, is_hip)
+
+        for p in range(PASSES):
+            pos = pos0 + p
+            x0 = rng(850 + p).standard_normal(ND).astype(np.float32)
+            print(f"attention mixer in the chain, pass {p} at position {pos}", flush=True)
+            B[0]["x"][:] = x0
+            hip.begin_pass(1); hip.host_wrote(B[0]["x"]); run(hip, 0, True, pos); hip.end_pass()
+            hip.host_needs(B[0]["x"]); hip.read_kv(slabs[0]["k"]); hip.read_kv(slabs[0]["v"])
+            hip.raise_if_error()
+            B[1]["x"][:] = x0
+            run(orc, 1, False, pos)
+            got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
+            assert np.abs(want).max() > 0.05
+            # (the first two passes are issued op by op, before there is a chain: their attention rounds the probabilities
+            # to f16 for the matrix cores and is held to 5e-3; the chain's is f32 throughout)
+            assert near(got, want, 5e-3 if p < 2 else 2e-3), (p, far(got, want))
+            print(f"  pass {p}: {far(got, want):.3g} of the scale", flush=True)
+            for t in "kv":
+                a = slabs[0][t].view(np.float16).astype(np.float32); b = slabs[1][t].view(np.float16).astype(np.float32)
+                assert np.array_equal(a[:pos0 * kd], b[:pos0 * kd]) and not a[(pos + 1) * kd:].any()
+                assert near(a[pos * kd:(pos + 1) * kd], b[pos * kd:(pos + 1) * kd]), (p, t)
+                slabs[1][t][pos * kd:(pos + 1) * kd] = slabs[0][t][pos * kd:(pos + 1) * kd]
+        g, c = hip.graph_stats(), hip.chain_stats()
+        assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] == PASSES - 2, g
+        assert c["chains"] == 1 and c["layers"] == 1 and g["graph_kernels"] == 1, (g, c)
+    finally:
+        err = hip.take_error()
+        hip.close()
+    assert err is None, err
+
+
+@pytest.mark.parametrize("attn_in_chain", [True, False])
+def test_an_attention_layer_between_chains(attn_in_chain, monkeypatch):
+    """layer 0 (Gated DeltaNet + FFN), layer 1 (attention + FFN), layer 2 (Gated DeltaNet + FFN) in one pass.  With the
+    attention mixer inside the chain (in-projection, head norms, rotation, cache rows, attention over 128 key ranges,
+    merge + gate, out-projection as stages of the persistent kernel) the pass is ONE kernel.  With that switched off
+    (INFERRED_HIP_NO_CHAIN_ATTN=1) the attention layer's in-projection is the last stage of the first chain and its
+    out-projection the first stage of the second; norm + rotation + cache write + split-K attention stay the launch
+    between them: three kernels in all.
 
     Held to the per-stage kernels (the same passes on a backend with the chains switched off) at the bounds of the
     module: the residual stream, both recurrent states, the new K / V rows, the picks.  Held to the oracle where a
@@ -351,6 +431,10 @@ def test_an_attention_layer_between_chains():
     qd, kd = NH * AHD, NKV * AHD
     sc = float(1.0 / np.sqrt(np.float32(AHD)))
     outs = []
+    if attn_in_chain:
+        monkeypatch.delenv("INFERRED_HIP_NO_CHAIN_ATTN", raising=False)
+    else:
+        monkeypatch.setenv("INFERRED_HIP_NO_CHAIN_ATTN", "1")
     for chain in (True, False):
         pair = make_pair(chain)
         hip, orc = pair.hip, pair.orc
@@ -421,7 +505,9 @@ def test_an_attention_layer_between_chains():
                         B[1]["layers"][li][name][:] = B[0]["layers"][li][name]
             g, c = hip.graph_stats(), hip.chain_stats()
             assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] == PASSES - 2, g
-            if chain:
+            if chain and attn_in_chain:
+                assert c["chains"] == 1 and c["layers"] == 3 and g["graph_kernels"] == 1, (g, c)
+            elif chain:
                 assert c["chains"] == 2 and c["layers"] == 3 and g["graph_kernels"] == 3, (g, c)
             else:
                 assert c["chains"] == 0, c
@@ -433,10 +519,21 @@ def test_an_attention_layer_between_chains():
             hip.close()
         assert err is None, err
     (xa, sa, ka, na), (xb, sb, kb, nb) = outs
+    for a, b in zip(ka, kb):
+        assert near(a, b), far(a, b)
+    if attn_in_chain:
+        # The chain's attention is f32 throughout, the per-stage kernel rounds the probabilities to f16 for the matrix
+        # cores: 1e-4 of the attention output, which the quantization in front of the out-projection and the two blocks
+        # behind turn into per cent (the docstring's measurement).  What is in front of the attention is held as
+        # everywhere (layer 0's state, the new K / V rows above); what is behind it grossly here, and sharply in
+        # test_the_attention_mixer_inside_a_chain_against_the_oracle.
+        for p in range(PASSES):
+            assert near(xa[p], xb[p], 0.15), (p, far(xa[p], xb[p]))
+        for a, b in zip(sa[:2], sb[:2]):
+            assert close(a, b), worst(a, b)
+        return
     for p in range(PASSES):
         assert near(xa[p], xb[p]), (p, far(xa[p], xb[p]))
     for a, b in zip(sa, sb):
         assert close(a, b), worst(a, b)
-    for a, b in zip(ka, kb):
-        assert near(a, b), far(a, b)
     assert np.array_equal(na, nb)

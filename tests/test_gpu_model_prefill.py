@@ -125,14 +125,12 @@ def test_config5_full_size_fast_run_is_deterministic_and_clean(config5_gguf):
     assert len(set(runs[1][1].tolist())) > 1                      # not stuck on one token
     g = be.graph_stats()
     assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] >= 90, g
-    # 13 layer chains, one persistent kernel each: layers 0-2 with the in-projection of layer 3's attention block as the
-    # last stage; then, per attention layer, its out-projection, its routed FFN and the three Gated DeltaNet layers
-    # behind it, closed by the next attention block's in-projection (the last chain is layer 47's out-projection and
-    # FFN alone).  Between two chains only the attention launch itself (norms, rotation, cache write, split-K attend
-    # and its gated merge) remains; then the output head and the arg-max + embedding step.
+    # ONE layer chain: all 48 layers in one persistent kernel (36 Gated DeltaNet mixers, 12 attention mixers whole:
+    # in-projection, head norms, rotation, cache rows, attention over the context, merge + gate, out-projection; every
+    # layer with its routed FFN); then the output head and the arg-max + embedding step's two kernels.
     c = be.chain_stats()
-    assert c["enabled"] and c["layers"] == 48 and c["chains"] == 13, c
-    assert g["graph_kernels"] == c["chains"] + 12 + 2, (g, c)
+    assert c["enabled"] and c["layers"] == 48 and c["chains"] == 1, c
+    assert g["graph_kernels"] == 3, (g, c)
     st = be.expert_stats()
     assert st.resident == 48 * 3 * 512 and st.oversubscribed == 0 and st.evictions == 0 and st.fetched == 0
     he.close(); hm.close(); be.close()
