@@ -70,6 +70,9 @@ static_assert(R_END <= (int)CHAIN_LL_STAGE_WORDS, "hand-off space");
 constexpr int NH = 16, NKV = 2, HD = 256, AG = NH / NKV, AS = CHAIN_ATTN_SPLITS;
 constexpr int RQ = RA, RK = RQ + NH * 2 * HD, RV = RK + NKV * HD, RT = RB;
 constexpr int RP = (int)CHAIN_LL_STAGE_WORDS, PW = HD + 2;   // per (query head, key range): HD sums, the maximum, the weight
+#ifndef ATTN_U1
+#define ATTN_U1 2   // score steps (four keys each) whose rows are read together
+#endif
 constexpr int TK = 64;            // keys of a range that are in LDS at a time
 constexpr int KSTR = HD + 8;      // f16 row stride of the K and V tiles (528 bytes)
 constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + AG * HD * 4 + AG * TK * 4 + (8 + 8 * 4 * 5) * 4;   // K tile, V tile, the eight scaled queries, their probabilities, the merge's partial sums
@@ -145,6 +148,11 @@ IT_DEV void ll_put(u64* p, uint32_t bits, unsigned e) {
     __hip_atomic_store((__attribute__((address_space(1))) u64*)p, ((u64)e << 32) | (u64)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 IT_DEV void ll_putf(u64* p, float v, unsigned e) { ll_put(p, __float_as_uint(v), e); }
+// two neighbouring words (16-byte aligned) in one store; a reader takes a pair only when both stamps are there
+IT_DEV void ll_put2f(u64* p, float v0, float v1, unsigned e) {
+    const v4u w = {__float_as_uint(v0), e, __float_as_uint(v1), e};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+}
 
 // true when the wait must stop: the tries are used up (this thread raises the abort word) or another wait gave up
 #ifndef IT_CHAIN_SLEEP
@@ -545,20 +553,28 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
                 __syncthreads();
                 if (t0 + TK < nk) fetch_kv(t0 + TK);
                 const int nt = min(TK, nk - t0);
-                // scores: 16 lanes a key, four keys a step; they go to LDS, where lane k finds key k's
-#pragma unroll 2
-                for (int g = 0; g < (nt + 3) / 4; g++) {
-                    const uint16_t* kr = Ks + (4 * g + j) * KSTR + 8 * c;
-                    const uint4 ka = *(const uint4*)kr, kc = *(const uint4*)(kr + 128);
-                    const uint32_t w[8] = {ka.x, ka.y, ka.z, ka.w, kc.x, kc.y, kc.z, kc.w};
-                    float sum = 0.0f;
+                // scores: 16 lanes a key, four keys a step, the rows of four steps read together; they go to LDS, where
+                // lane k finds key k's.  (Rows behind the tile's last key are zeros: the staging wrote all 64.)
+                for (int g0 = 0; g0 < (nt + 3) / 4; g0 += ATTN_U1) {
+                    uint4 ka[ATTN_U1], kc[ATTN_U1];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        sum = fmaf(it_f16_to_f32(w[i] & 0xffffu), q16[2 * i], sum);
-                        sum = fmaf(it_f16_to_f32(w[i] >> 16), q16[2 * i + 1], sum);
+                    for (int u = 0; u < ATTN_U1; u++) {
+                        const uint16_t* kr = Ks + (4 * (g0 + u) + j) * KSTR + 8 * c;
+                        ka[u] = *(const uint4*)kr;
+                        kc[u] = *(const uint4*)(kr + 128);
                     }
-                    sum = group_sum<16>(sum);
-                    if (c == 0) Pf[wave * TK + 4 * g + j] = sum;
+#pragma unroll
+                    for (int u = 0; u < ATTN_U1; u++) {
+                        const uint32_t w[8] = {ka[u].x, ka[u].y, ka[u].z, ka[u].w, kc[u].x, kc[u].y, kc[u].z, kc[u].w};
+                        float sum = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < 8; i++) {
+                            sum = fmaf(it_f16_to_f32(w[i] & 0xffffu), q16[2 * i], sum);
+                            sum = fmaf(it_f16_to_f32(w[i] >> 16), q16[2 * i + 1], sum);
+                        }
+                        sum = group_sum<16>(sum);
+                        if (c == 0) Pf[wave * TK + 4 * (g0 + u) + j] = sum;
+                    }
                 }
                 const float sc = lane < nt ? Pf[wave * TK + lane] : -INFINITY;
                 const float m_new = fmaxf(m_run, group_max<64>(sc));   // finite: the tile has a key
@@ -569,21 +585,26 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
                 l_run = l_run * alpha + psum;
                 o.x *= alpha; o.y *= alpha; o.z *= alpha; o.w *= alpha;
                 m_run = m_new;
-                for (int key = 0; key < nt; key++) {
-                    const float pk = Pf[wave * TK + key];
-                    const uint2 vv = *(const uint2*)(Vs + key * KSTR + 4 * lane);
-                    o.x = fmaf(pk, it_f16_to_f32(vv.x & 0xffffu), o.x);
-                    o.y = fmaf(pk, it_f16_to_f32(vv.x >> 16), o.y);
-                    o.z = fmaf(pk, it_f16_to_f32(vv.y & 0xffffu), o.z);
-                    o.w = fmaf(pk, it_f16_to_f32(vv.y >> 16), o.w);
+                // weighted values, eight keys a trip (a key behind the tile's last has probability 0 and a row of zeros)
+                for (int k8 = 0; k8 < nt; k8 += 8) {
+                    const float4 pa = *(const float4*)(Pf + wave * TK + k8), pb = *(const float4*)(Pf + wave * TK + k8 + 4);
+                    const float pk[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
+                    uint2 vv[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) vv[u] = *(const uint2*)(Vs + (k8 + u) * KSTR + 4 * lane);
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        o.x = fmaf(pk[u], it_f16_to_f32(vv[u].x & 0xffffu), o.x);
+                        o.y = fmaf(pk[u], it_f16_to_f32(vv[u].x >> 16), o.y);
+                        o.z = fmaf(pk[u], it_f16_to_f32(vv[u].y & 0xffffu), o.z);
+                        o.w = fmaf(pk[u], it_f16_to_f32(vv[u].y >> 16), o.w);
+                    }
                 }
             }
             AC_STAMP(2);   // the range's keys done
             u64* part = ll + RP + (int64_t)((kvh * AG + wave) * AS + split) * PW;
-            ll_putf(part + 4 * lane, o.x, e);
-            ll_putf(part + 4 * lane + 1, o.y, e);
-            ll_putf(part + 4 * lane + 2, o.z, e);
-            ll_putf(part + 4 * lane + 3, o.w, e);
+            ll_put2f(part + 4 * lane, o.x, o.y, e);
+            ll_put2f(part + 4 * lane + 2, o.z, o.w, e);
             if (lane == 0) {
                 ll_putf(part + HD, m_run, e);
                 ll_putf(part + HD + 1, l_run, e);
@@ -597,6 +618,10 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
         const int sp = tid >> 2, q4 = tid & 3;
         float m_s = -INFINITY, l_s = 0.0f;
         float4 o_s = make_float4(0.f, 0.f, 0.f, 0.f);
+        // (the gate of this thread's dim, the head's second half of wq's output: published a stage ago; asked for ahead of
+        // the ranges' results, whose wait hides the round trip)
+        uint32_t gw = 0;
+        if (tid < 16 && !ll_wait1(ll + RQ + h * 2 * HD + HD + dc * 16 + tid, e, ctl, &gw)) ok = false;
         if (sp < n_live) {
             const u64* base = ll + RP + (int64_t)(h * AS + sp) * PW;
             const u64* const a4[4] = {base + dc * 16 + q4 * 4, base + dc * 16 + q4 * 4 + 2, base + HD, base + HD};
@@ -638,8 +663,6 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
                 osum += ws[(w * 4 + q) * 5 + i];
                 lsum += ws[(w * 4 + q) * 5 + 4];
             }
-            uint32_t gw = 0;
-            if (!ll_wait1(ll + RQ + h * 2 * HD + HD + dc * 16 + tid, e, ctl, &gw)) ok = false;
             ll_putf(ll + RT + h * HD + dc * 16 + tid, osum / lsum * fx_sigmoid(__uint_as_float(gw)), e);
         }
     }
