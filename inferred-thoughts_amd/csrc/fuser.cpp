@@ -8,7 +8,9 @@
 // scales — is simply issued op by op.  A fused launch sits at the position of its
 // block's first op; everything it replaces is dropped, except an activation
 // quantization that some unfused op still reads.
+#include <cstddef>
 #include <cstdio>
+#include <cstring>
 #include <memory>
 #include <cstdlib>
 #include "backend.h"
@@ -761,8 +763,15 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         Kind kind;
     };
     size_t tail_pos = 0;   // position of the attention block whose in-projection is cp's tail
-    ChainP cp{};
-    auto layer_at = [&](int k) -> ChainLayer& { return cp.layer[k]; };
+    // (30 KB, nearly all of it the layer array: on the heap, and only the entries in use are cleared and copied)
+    std::unique_ptr<ChainP, void (*)(void*)> cp_box((ChainP*)calloc(1, sizeof(ChainP)), free);
+    ChainP& cp = *cp_box;
+    int cp_touched = 0;   // entries of cp.layer written since they were last cleared
+    auto layer_at = [&](int k) -> ChainLayer& {
+        if (k + 1 > cp_touched) cp_touched = k + 1;
+        return cp.layer[k];
+    };
+    const size_t cp_head = offsetof(ChainP, layer);
     std::vector<Unit> units;          // the blocks folded into cp so far
     bool mixer_open = false;          // the last layer of cp has its mixer and still waits for its FFN
     int chain_rf = -1;                // the small matrices of cp's layers: Q8_0 (0) or F32 (1); -1 while no layer says
@@ -787,8 +796,9 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             cp.tally = be->count_reads_in_fused ? tally : nullptr;
             cp.spin_limit = be->chain_spin_limit;
             cp.rf = chain_rf > 0 ? 1 : 0;
-            // (30 KB: on the heap, shared by the copies a std::function makes of what it holds)
-            const auto launch = std::make_shared<const ChainP>(cp);
+            // (on the heap, shared by the copies a std::function makes of what it holds)
+            std::shared_ptr<ChainP> launch((ChainP*)malloc(sizeof(ChainP)), free);
+            memcpy((void*)launch.get(), (const void*)&cp, cp_head + (size_t)n * sizeof(ChainLayer));
             auto drop_stage = [&](size_t pos, int stage) {
                 auto& v = pl.at[pos];
                 for (size_t k = 0; k < v.size(); k++)
@@ -824,7 +834,8 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             be->chain_launches++;
             be->chain_layers += (uint64_t)n;
         }
-        cp = ChainP{};
+        memset((void*)&cp, 0, cp_head + (size_t)cp_touched * sizeof(ChainLayer));
+        cp_touched = 0;
         units.clear();
         mixer_open = false;
         bytes = 0;

@@ -32,6 +32,8 @@
 //
 // Every wait is bounded: a poll that runs out of tries sets the abort word, every other wait sees it and the
 // grid drains.  The grid must be resident at once (one block per compute unit), which the launcher checks.
+#include <cstddef>
+#include <cstring>
 #define IT_CHAIN_DEVICE_POINTERS
 #include "it_fast.h"
 #include "kernels_fused.h"
@@ -691,8 +693,8 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
     return AttnCoreR{dot, ok ? 1 : 0};
 }
 
-template <int SF, int RF>
-__global__ __launch_bounds__(CT) void layer_chain_k(ChainP p) {
+template <int SF, int RF, int NL>
+__global__ __launch_bounds__(CT) void layer_chain_k(ChainPT<NL> p) {
     __shared__ __align__(16) int8_t xq[NU * FF + FF];   // the stage's quantized activation (largest: the down stage's)
     __shared__ __align__(16) float xs[(NU * FF + FF) / 32];
     __shared__ double red[CW];
@@ -1460,8 +1462,10 @@ bool layer_chain_fits() {
         int dev = 0, cus = 0, occ = 0;
         if (hipGetDevice(&dev) != hipSuccess) return false;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < NB) return false;
-        const void* fns[4] = {(const void*)layer_chain_k<W_Q8_0, 0>, (const void*)layer_chain_k<W_NVFP4, 0>,
-                              (const void*)layer_chain_k<W_Q8_0, 1>, (const void*)layer_chain_k<W_NVFP4, 1>};
+        const void* fns[8] = {(const void*)layer_chain_k<W_Q8_0, 0, CHAIN_MAX_LAYERS>,    (const void*)layer_chain_k<W_NVFP4, 0, CHAIN_MAX_LAYERS>,
+                              (const void*)layer_chain_k<W_Q8_0, 1, CHAIN_MAX_LAYERS>,    (const void*)layer_chain_k<W_NVFP4, 1, CHAIN_MAX_LAYERS>,
+                              (const void*)layer_chain_k<W_Q8_0, 0, CHAIN_SHORT_LAYERS>,  (const void*)layer_chain_k<W_NVFP4, 0, CHAIN_SHORT_LAYERS>,
+                              (const void*)layer_chain_k<W_Q8_0, 1, CHAIN_SHORT_LAYERS>,  (const void*)layer_chain_k<W_NVFP4, 1, CHAIN_SHORT_LAYERS>};
         // (with the LDS an attention mixer's stages take: every instance is launched with it when a layer is one)
         for (const void* fn : fns)
             if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, ATTN_LDS) != hipSuccess ||
@@ -1470,6 +1474,14 @@ bool layer_chain_fits() {
         return true;
     }();
     return fits;
+}
+
+template <int NL>
+static void launch_chain(const ChainPT<NL>& p, size_t lds, hipStream_t s) {
+    if (p.sh_fmt == W_Q8_0 && !p.rf) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 0, NL>), dim3(NB), dim3(CT), lds, s, p);
+    else if (!p.rf) hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 0, NL>), dim3(NB), dim3(CT), lds, s, p);
+    else if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 1, NL>), dim3(NB), dim3(CT), lds, s, p);
+    else hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 1, NL>), dim3(NB), dim3(CT), lds, s, p);
 }
 
 bool layer_chain(const ChainP& p, hipStream_t s) {
@@ -1507,10 +1519,13 @@ bool layer_chain(const ChainP& p, hipStream_t s) {
         return false;
     if (!layer_chain_fits()) return false;
     const size_t lds = has_attn ? ATTN_LDS : 0;
-    if (p.sh_fmt == W_Q8_0 && !p.rf) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 0>), dim3(NB), dim3(CT), lds, s, p);
-    else if (!p.rf) hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 0>), dim3(NB), dim3(CT), lds, s, p);
-    else if (p.sh_fmt == W_Q8_0) hipLaunchKernelGGL((layer_chain_k<W_Q8_0, 1>), dim3(NB), dim3(CT), lds, s, p);
-    else hipLaunchKernelGGL((layer_chain_k<W_NVFP4, 1>), dim3(NB), dim3(CT), lds, s, p);
+    if (p.n_layers <= CHAIN_SHORT_LAYERS) {   // the same kernel with room for four layers in its argument block
+        ChainPT<CHAIN_SHORT_LAYERS> q;
+        std::memcpy((void*)&q, (const void*)&p, offsetof(ChainP, layer) + (size_t)p.n_layers * sizeof(ChainLayer));
+        launch_chain(q, lds, s);
+    } else {
+        launch_chain(p, lds, s);
+    }
     return true;
 }
 

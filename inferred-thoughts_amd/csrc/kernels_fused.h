@@ -199,8 +199,7 @@ constexpr int CHAIN_ATTN_SPLITS = 128;     // key ranges of an in-chain attentio
 constexpr size_t CHAIN_LL_STAGE_WORDS = 24576;   // 8-byte words of hand-off space of the stages
 // ... and behind them the attention partials: per (query head, key range) 256 sums, the range's maximum and its weight
 constexpr size_t CHAIN_LL_WORDS = CHAIN_LL_STAGE_WORDS + (size_t)16 * CHAIN_ATTN_SPLITS * 258;
-struct ChainP {
-    ChainLayer layer[CHAIN_MAX_LAYERS];
+template <int NL> struct ChainPT {
     int n_layers;
     int has_tail;
     ChainTail tail;
@@ -213,7 +212,12 @@ struct ChainP {
     it_gptr<unsigned> abort_flag;        // uncached device word: set when a bounded wait gave up (the results are then void)
     it_gptr<unsigned long long> tally;   // expert read tally (optional)
     int spin_limit;              // polls a wait may take before it gives up
+    ChainLayer layer[NL];   // (last: host code copies and clears the n_layers entries in use, not all 30 KB)
 };
+typedef ChainPT<CHAIN_MAX_LAYERS> ChainP;
+// A chain of up to this many layers is launched with a small argument block: a launch queued outside a graph pays the
+// host's copy of its arguments (8-10 us for 30 KB against 2.5 us for 2 KB, measured; a replayed graph pays neither).
+constexpr int CHAIN_SHORT_LAYERS = 4;
 // whether this device can hold the chain's grid (one block per compute unit, all resident at once)
 bool layer_chain_fits();
 // false: not launched
