@@ -483,9 +483,19 @@ def main():
         ach = (dom["bytes"] / 1e9) / (dom["ms"] / 1e3)
         per_launch = dom["bytes"] // dom["launches"]
         prof = family_profile().get(dom["name"]) if headline else None
+        # HBM bytes per launch from the committed counter runs.  A reading below the launch's algorithmic bytes cannot
+        # be traffic (the weights alone are read once per token and fit no cache): the counters come back short for the
+        # 1.4 ms dispatch that holds a whole token, and are then left out (the same layers as thirteen short chains
+        # read 1.02 x their algorithmic bytes: profiles/decode_config5_families_attention_between_chains.txt)
+        traffic = int(prof["fetched"] + prof["written"]) if prof else None
+        traffic_note = None
+        if traffic is not None and traffic < 0.8 * per_launch:
+            traffic_note = (f"FETCH_SIZE + WRITE_SIZE read {traffic} bytes for this {round(prof['rocprof_avg_us'])} us dispatch, less than "
+                            "the weights it must read: counter reading not usable at this dispatch length")
+            traffic = None
         roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                    "traffic": int(prof["fetched"] + prof["written"]) if prof else None,
+                    "traffic": traffic, "traffic_note": traffic_note,
                     "avg_launch_us": round(1e3 * dom["ms"] / dom["launches"], 2),
                     "bytes_per_launch": per_launch,
                     # the same fraction with the launch duration rocprofv3 reports for this family inside the replayed

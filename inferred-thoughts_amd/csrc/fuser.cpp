@@ -726,7 +726,13 @@ bool chain_attn_in(const FusedGemvP& a, ChainTail* t) {
 // a whole attention block as a chain layer: in-projection, attention launch and out-projection must be the shapes the
 // chain's stages are written for and hang together (the attention reads what the in-projection writes and writes what
 // the out-projection reads; the gate is the second half of every head's wq rows)
-bool chain_attn(const FusedGemvP& in, const Plan::Launch& at, const FusedGemvP& out, ChainAttn* a, ChainMixer* m) {
+// Beyond this many positions the block stays between two chains: the chain's attention is f32 on the vector ALU (3.5 us
+// of a layer at 5,800 positions, ahead of the matrix-core kernels by 4 % of a token at 30,000; its time grows with the
+// context, theirs far less)
+constexpr int CHAIN_ATTN_MAX_POS = 65536;
+bool chain_attn(const Plan& pl, const FusedGemvP& in, const Plan::Launch& at, const FusedGemvP& out, ChainAttn* a, ChainMixer* m) {
+    const int slot = pl.dyn_index(at.aa.n_pos_dyn);
+    if (slot < 0 || pl.be->dyn_host[slot] > CHAIN_ATTN_MAX_POS) return false;
     ChainTail t{};
     ChainMixer mo{};
     if (!chain_attn_in(in, &t) || !chain_attn_out(out, &mo)) return false;
@@ -852,7 +858,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
             ChainAttn a{};
             ChainMixer m{};
-            if (chain_attn(ls[0].gv, ls[1], ls[2].gv, &a, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
+            if (chain_attn(pl, ls[0].gv, ls[1], ls[2].gv, &a, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
                 layer_at(cp.n_layers).has_mixer = 3;
                 layer_at(cp.n_layers).a = a;
                 layer_at(cp.n_layers).m = m;
