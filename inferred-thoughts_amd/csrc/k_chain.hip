@@ -20,8 +20,17 @@
 //      flight); 160 blocks take one 32-element block of one pick's gate / up rows each and publish it quantized, the
 //      other 96 touch those rows' lines for the blocks of their XCD; the down rows are issued behind the publication
 //   F  down rows of the ten picks and of the shared expert, combine, residual
-// An attention layer gives the chain before it a last stage (its in-projection: rms_norm + Q8_0 + wq / wk / wv rows) and
-// the chain behind it a first one (its out-projection + residual); the attention kernels run between the two chains.
+// An attention layer's mixer (src/model/qwen35.rs:1141-1223) is five stages of its own in front of its FFN's D, E, F:
+//   the in-projection (rms_norm + Q8_0 + wq / wk / wv rows), published like stage A's outputs;
+//   head norm + rotation of the queries and of the new key, the new cache rows, and the attention of eight query heads
+//   over one of 128 ranges of the context per block, f32 on the vector ALU, with the range's K / V rows in flight
+//   before the queries are waited for; the merge of the ranges with the sigmoid gate, 16 dims a block; the
+//   out-projection + residual.  The middle three are a function of their own (attn_core).
+// (The older form stays for contexts beyond what that attention is good for, and as a measurement switch: the
+// in-projection as the LAST stage of the chain before the layer, the out-projection as the FIRST stage of the chain
+// behind it, the matrix-core attention kernels between the two chains.)
+// A chain holds up to 56 layers, a whole token of the model this is written for; their parameters travel in the
+// kernel's argument block.
 //
 // Three things place the loads and the polls (each measured with the stage stamps below):
 //   * loads return in issue order per wave, so a poll or a publication waits for everything its wave has in flight:
