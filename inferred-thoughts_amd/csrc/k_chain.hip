@@ -82,7 +82,7 @@ constexpr int NH = 16, NKV = 2, HD = 256, AG = NH / NKV, AS = CHAIN_ATTN_SPLITS;
 constexpr int RQ = RA, RK = RQ + NH * 2 * HD, RV = RK + NKV * HD, RT = RB;
 constexpr int RP = (int)CHAIN_LL_STAGE_WORDS, PW = HD + 2;   // per (query head, key range): HD sums, the maximum, the weight
 #ifndef ATTN_U1
-#define ATTN_U1 2   // score steps (four keys each) whose rows are read together
+#define ATTN_U1 2   // score steps (four keys each) whose rows are read together (four spilled registers in the stages around the call)
 #endif
 constexpr int TK = 64;            // keys of a range that are in LDS at a time
 constexpr int KSTR = HD + 8;      // f16 row stride of the K and V tiles (528 bytes)
@@ -564,7 +564,7 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
                 __syncthreads();
                 if (t0 + TK < nk) fetch_kv(t0 + TK);
                 const int nt = min(TK, nk - t0);
-                // scores: 16 lanes a key, four keys a step, the rows of four steps read together; they go to LDS, where
+                // scores: 16 lanes a key, four keys a step, the rows of ATTN_U1 steps read together; they go to LDS, where
                 // lane k finds key k's.  (Rows behind the tile's last key are zeros: the staging wrote all 64.)
                 for (int g0 = 0; g0 < (nt + 3) / 4; g0 += ATTN_U1) {
                     uint4 ka[ATTN_U1], kc[ATTN_U1];
