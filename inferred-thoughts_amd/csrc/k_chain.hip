@@ -81,12 +81,13 @@ static_assert(R_END <= (int)CHAIN_LL_STAGE_WORDS, "hand-off space");
 constexpr int NH = 16, NKV = 2, HD = 256, AG = NH / NKV, AS = CHAIN_ATTN_SPLITS;
 constexpr int RQ = RA, RK = RQ + NH * 2 * HD, RV = RK + NKV * HD, RT = RB;
 constexpr int RP = (int)CHAIN_LL_STAGE_WORDS, PW = HD + 2;   // per (query head, key range): HD sums, the maximum, the weight
-#ifndef ATTN_U1
-#define ATTN_U1 2   // score steps (four keys each) whose rows are read together (four spilled registers in the stages around the call)
-#endif
 constexpr int TK = 64;            // keys of a range that are in LDS at a time
 constexpr int KSTR = HD + 8;      // f16 row stride of the K and V tiles (528 bytes)
-constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + AG * HD * 4 + AG * TK * 4 + (8 + 8 * 4 * 5) * 4;   // K tile, V tile, the eight scaled queries, their probabilities, the merge's partial sums
+constexpr int PSTR = TK + 8;      // f16 row stride of the probabilities (144 bytes)
+// dynamic LDS of an attention mixer's middle: K tile, V tile, the eight scaled queries as f16 pairs (16 rows), the tile's
+// scores (f32), the probabilities as f16 pairs (16 rows + 16 of zeros: the unused columns of the matrix-core product),
+// the heads' rescaling factors, the merge's partial sums
+constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + 16 * KSTR * 2 + AG * TK * 4 + 32 * PSTR * 2 + AG * 4 + (8 + 8 * 4 * 5) * 4;
 static_assert(RV + NKV * HD <= RB && NH * HD <= VDIM && NB == NKV * AS && CW == AG && NB == NH * 16 && NH * 2 * HD == 32 * NB &&
               NKV * HD == 2 * NB && NH * HD == 8 * CT && HD == 4 * 64 && (PW % 2) == 0 && (RP % 2) == 0, "attention stage shapes");
 static_assert(!(RA & 1) && !(RA_Z & 1) && !(RB & 1) && !(RB_SS & 1) && !(RC & 1) && !(RD & 1) && !(RS & 1) && !(RE & 1) && !(RE_SC & 1), "");
@@ -482,9 +483,11 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint16_t* const Ks = (uint16_t*)chain_dyn_lds;
     uint16_t* const Vs = Ks + TK * KSTR;
-    float* const Qf = (float*)(Vs + TK * KSTR);
-    float* const Pf = Qf + AG * HD;
-    float* const sm = Pf + AG * TK;      // 8 wave maxima
+    uint16_t* const Q16 = Vs + TK * KSTR;            // [16][KSTR]: rows 0..7 the high f16 halves of the scaled queries, 8..15 the low halves
+    float* const Sf = (float*)(Q16 + 16 * KSTR);     // [8][TK] the tile's scores
+    uint16_t* const P16 = (uint16_t*)(Sf + AG * TK);  // [32][PSTR]: rows 0..7 high halves of the probabilities, 8..15 low halves, 16..31 zeros
+    float* const Af = (float*)(P16 + 32 * PSTR);      // [8] what a head's sums so far are scaled by
+    float* const sm = Af + AG;           // 8 wave maxima
     float* const ws = sm + 8;            // 8 waves x 4 dim groups x (4 sums + the weight)
     bool ok = true;
     const int n_pos = *at.n_pos;
@@ -524,17 +527,39 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
         uint2 fresh = make_uint2(0, 0);   // wave 0: the new key row's four f16 of this lane; wave 1: the new value row's
         if (nk > 0) {
             fetch_kv(0);
-            float4 qv;
-            ok = ll_wait_quad(ll + RQ + (kvh * AG + wave) * 2 * HD, lane, e, ctl, &qv);
+            for (int i = tid; i < 16 * PSTR / 2; i += CT) ((uint32_t*)(P16 + 16 * PSTR))[i] = 0u;
+            // (the two waves that form the new position's key and value rows ask for them together with their query:
+            // one round trip, not two; every other block's merge waits for this block's results)
+            float4 qv, nv = make_float4(0.f, 0.f, 0.f, 0.f);
+            const u64* const qreg = ll + RQ + (kvh * AG + wave) * 2 * HD;
+            const bool forms_row = new_at >= 0 && wave < 2;
+            if (forms_row) {
+                const u64* const nreg = ll + (wave == 0 ? RK : RV) + kvh * HD;
+                const u64* const a4[4] = {qreg + 4 * lane, qreg + 4 * lane + 2, nreg + 4 * lane, nreg + 4 * lane + 2};
+                uint32_t o8[8];
+                ok = ll_wait_pairs<4>(a4, e, ctl, o8);
+                qv = make_float4(__uint_as_float(o8[0]), __uint_as_float(o8[1]), __uint_as_float(o8[2]), __uint_as_float(o8[3]));
+                nv = make_float4(__uint_as_float(o8[4]), __uint_as_float(o8[5]), __uint_as_float(o8[6]), __uint_as_float(o8[7]));
+            } else {
+                ok = ll_wait_quad(qreg, lane, e, ctl, &qv);
+            }
             if (ok) {
                 qv = head_norm_rope<HD>(qv, at.q_norm, at.eps_head, at.rope, at.n_rot, pos_new, lane);
+                // scaled for a base-2 softmax and split into an f16 pair (22 bits): the matrix cores take both halves
                 const float qsc = at.scale * 1.4426950408889634f;
-                ((float4*)(Qf + wave * HD))[lane] = make_float4(qv.x * qsc, qv.y * qsc, qv.z * qsc, qv.w * qsc);
+                const float x[4] = {qv.x * qsc, qv.y * qsc, qv.z * qsc, qv.w * qsc};
+                uint16_t hi[4], lo[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const _Float16 h = (_Float16)x[i];
+                    hi[i] = __builtin_bit_cast(uint16_t, h);
+                    lo[i] = __builtin_bit_cast(uint16_t, (_Float16)(x[i] - (float)h));
+                }
+                *(uint2*)(Q16 + wave * KSTR + 4 * lane) = make_uint2(hi[0] | ((uint32_t)hi[1] << 16), hi[2] | ((uint32_t)hi[3] << 16));
+                *(uint2*)(Q16 + (8 + wave) * KSTR + 4 * lane) = make_uint2(lo[0] | ((uint32_t)lo[1] << 16), lo[2] | ((uint32_t)lo[3] << 16));
             }
-            if (ok && new_at >= 0 && wave < 2) {
-                float4 nv;
-                ok = ll_wait_quad(ll + (wave == 0 ? RK : RV) + kvh * HD, lane, e, ctl, &nv);
-                if (ok) {
+            if (ok && forms_row) {
+                {   // the new position's key (norm + rotation) or value row: to the cache, and kept for the tile
                     if (wave == 0) nv = head_norm_rope<HD>(nv, at.k_norm, at.eps_head, at.rope, at.n_rot, pos_new, lane);
                     fresh.x = (uint32_t)it_f32_to_f16(nv.x) | ((uint32_t)it_f32_to_f16(nv.y) << 16);
                     fresh.y = (uint32_t)it_f32_to_f16(nv.z) | ((uint32_t)it_f32_to_f16(nv.w) << 16);
@@ -547,16 +572,28 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
         __syncthreads();
         AC_STAMP(1);
         if (nk > 0) {
-            const int j = lane >> 4, c = lane & 15;
-            float q16[16];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const float4 a0 = ((const float4*)(Qf + wave * HD + 128 * i + 8 * c))[0], a1 = ((const float4*)(Qf + wave * HD + 128 * i + 8 * c))[1];
-                q16[8 * i + 0] = a0.x; q16[8 * i + 1] = a0.y; q16[8 * i + 2] = a0.z; q16[8 * i + 3] = a0.w;
-                q16[8 * i + 4] = a1.x; q16[8 * i + 5] = a1.y; q16[8 * i + 6] = a1.z; q16[8 * i + 7] = a1.w;
-            }
+            // Scores and weighted values on the f16 matrix cores, exact in their operands: K and V rows are f16 as
+            // stored, queries and probabilities go in as f16 pairs (the low halves in columns of their own, added
+            // afterwards), sums in f32.
+            //   S = K Q^T   v_mfma_f32_16x16x32_f16, 16 keys x (8 heads' high halves | 8 heads' low halves), waves 0..3 one
+            //               tile of 16 keys each, eight steps of 32 dims; lane l supplies 8 dims of key / column l % 16
+            //               at dims 8 * (l / 16) and receives column l % 16, keys 4 * (l / 16) + {0..3}
+            //   O^T = V^T P^T  v_mfma_f32_32x32x16_f16, wave w the 32 dims 32 w .., columns as above (+ 16 of zeros), a step
+            //               per 16 keys; lane l supplies 8 keys of dim / column l % 32 at keys 8 * (l / 32) (the V^T
+            //               operand two bytes at a time from the [key][dim] tile) and receives column l % 32, dims
+            //               8 * (i / 4) + 4 * (l / 32) + i % 4
+            // The softmax between them runs a wave a head, a lane a key, with the scores and the probabilities in LDS.
+            typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            typedef float v16f __attribute__((ext_vector_type(16)));
+            auto ror8 = [](float v) {   // the value of the lane eight further on in its row of 16
+                return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true));
+            };
             float m_run = -INFINITY, l_run = 0.0f;
-            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            v16f o;
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[i] = 0.0f;
+            const int c16 = lane & 15, g4 = lane >> 4, c32 = lane & 31, g2 = lane >> 5;
             for (int t0 = 0; t0 < nk; t0 += TK) {
                 if (t0) __syncthreads();   // every wave is done with the tile before
                 stash_kv(t0);
@@ -564,59 +601,61 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
                 __syncthreads();
                 if (t0 + TK < nk) fetch_kv(t0 + TK);
                 const int nt = min(TK, nk - t0);
-                // scores: 16 lanes a key, four keys a step, the rows of ATTN_U1 steps read together; they go to LDS, where
-                // lane k finds key k's.  (Rows behind the tile's last key are zeros: the staging wrote all 64.)
-                for (int g0 = 0; g0 < (nt + 3) / 4; g0 += ATTN_U1) {
-                    uint4 ka[ATTN_U1], kc[ATTN_U1];
+                // (rows behind the tile's last key are zeros: the staging wrote all 64)
+                if (wave < 4 && 16 * wave < nt) {
+                    v4f sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int u = 0; u < ATTN_U1; u++) {
-                        const uint16_t* kr = Ks + (4 * (g0 + u) + j) * KSTR + 8 * c;
-                        ka[u] = *(const uint4*)kr;
-                        kc[u] = *(const uint4*)(kr + 128);
+                    for (int st = 0; st < HD / 32; st++) {
+                        const h8 ka = *(const h8*)(Ks + (16 * wave + c16) * KSTR + 32 * st + 8 * g4);
+                        const h8 qb = *(const h8*)(Q16 + c16 * KSTR + 32 * st + 8 * g4);
+                        sacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb, sacc, 0, 0, 0);
                     }
 #pragma unroll
-                    for (int u = 0; u < ATTN_U1; u++) {
-                        const uint32_t w[8] = {ka[u].x, ka[u].y, ka[u].z, ka[u].w, kc[u].x, kc[u].y, kc[u].z, kc[u].w};
-                        float sum = 0.0f;
-#pragma unroll
-                        for (int i = 0; i < 8; i++) {
-                            sum = fmaf(it_f16_to_f32(w[i] & 0xffffu), q16[2 * i], sum);
-                            sum = fmaf(it_f16_to_f32(w[i] >> 16), q16[2 * i + 1], sum);
-                        }
-                        sum = group_sum<16>(sum);
-                        if (c == 0) Pf[wave * TK + 4 * (g0 + u) + j] = sum;
-                    }
+                    for (int i = 0; i < 4; i++) sacc[i] += ror8(sacc[i]);   // high + low halves
+                    if (c16 < AG) *(float4*)(Sf + c16 * TK + 16 * wave + 4 * g4) = make_float4(sacc[0], sacc[1], sacc[2], sacc[3]);
                 }
-                const float sc = lane < nt ? Pf[wave * TK + lane] : -INFINITY;
-                const float m_new = fmaxf(m_run, group_max<64>(sc));   // finite: the tile has a key
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                const float pr = __builtin_amdgcn_exp2f(sc - m_new);
-                Pf[wave * TK + lane] = pr;
-                const float psum = group_sum<64>(pr);
-                l_run = l_run * alpha + psum;
-                o.x *= alpha; o.y *= alpha; o.z *= alpha; o.w *= alpha;
-                m_run = m_new;
-                // weighted values, eight keys a trip (a key behind the tile's last has probability 0 and a row of zeros)
-                for (int k8 = 0; k8 < nt; k8 += 8) {
-                    const float4 pa = *(const float4*)(Pf + wave * TK + k8), pb = *(const float4*)(Pf + wave * TK + k8 + 4);
-                    const float pk[8] = {pa.x, pa.y, pa.z, pa.w, pb.x, pb.y, pb.z, pb.w};
-                    uint2 vv[8];
+                __syncthreads();
+                {
+                    const float sc = lane < nt ? Sf[wave * TK + lane] : -INFINITY;
+                    const float m_new = fmaxf(m_run, group_max<64>(sc));   // finite: the tile has a key
+                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                    const float pr = __builtin_amdgcn_exp2f(sc - m_new);
+                    const _Float16 ph = (_Float16)pr;
+                    P16[wave * PSTR + lane] = __builtin_bit_cast(uint16_t, ph);
+                    P16[(8 + wave) * PSTR + lane] = __builtin_bit_cast(uint16_t, (_Float16)(pr - (float)ph));
+                    if (lane == 0) Af[wave] = alpha;
+                    l_run = l_run * alpha + group_sum<64>(pr);
+                    m_run = m_new;
+                }
+                __syncthreads();
+                {
+                    const float al = Af[c32 & 7];
 #pragma unroll
-                    for (int u = 0; u < 8; u++) vv[u] = *(const uint2*)(Vs + (k8 + u) * KSTR + 4 * lane);
+                    for (int i = 0; i < 16; i++) o[i] *= al;
+                    for (int ks = 0; ks < (nt + 15) / 16; ks++) {
+                        const uint16_t* vp = Vs + (16 * ks + 8 * g2) * KSTR + 32 * wave + c32;
+                        uint32_t a[4];
 #pragma unroll
-                    for (int u = 0; u < 8; u++) {
-                        o.x = fmaf(pk[u], it_f16_to_f32(vv[u].x & 0xffffu), o.x);
-                        o.y = fmaf(pk[u], it_f16_to_f32(vv[u].x >> 16), o.y);
-                        o.z = fmaf(pk[u], it_f16_to_f32(vv[u].y & 0xffffu), o.z);
-                        o.w = fmaf(pk[u], it_f16_to_f32(vv[u].y >> 16), o.w);
+                        for (int q = 0; q < 4; q++) a[q] = (uint32_t)vp[(2 * q) * KSTR] | ((uint32_t)vp[(2 * q + 1) * KSTR] << 16);
+                        const h8 va = __builtin_bit_cast(h8, make_uint4(a[0], a[1], a[2], a[3]));
+                        const h8 pb = *(const h8*)(P16 + c32 * PSTR + 16 * ks + 8 * g2);
+                        o = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb, o, 0, 0, 0);
                     }
                 }
             }
             AC_STAMP(2);   // the range's keys done
-            u64* part = ll + RP + (int64_t)((kvh * AG + wave) * AS + split) * PW;
-            ll_put2f(part + 4 * lane, o.x, o.y, e);
-            ll_put2f(part + 4 * lane + 2, o.z, o.w, e);
-            if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[i] += ror8(o[i]);   // high + low halves of the probabilities
+            if (c32 < AG) {   // column = head: this wave's 32 dims of it, 16 a lane
+                u64* part = ll + RP + (int64_t)((kvh * AG + c32) * AS + split) * PW + 32 * wave + 4 * g2;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    ll_put2f(part + 8 * q, o[4 * q], o[4 * q + 1], e);
+                    ll_put2f(part + 8 * q + 2, o[4 * q + 2], o[4 * q + 3], e);
+                }
+            }
+            if (lane == 0) {   // wave = head for the softmax's sums
+                u64* part = ll + RP + (int64_t)((kvh * AG + wave) * AS + split) * PW;
                 ll_putf(part + HD, m_run, e);
                 ll_putf(part + HD + 1, l_run, e);
             }
