@@ -86,8 +86,8 @@ constexpr int KSTR = HD + 8;      // f16 row stride of the K and V tiles (528 by
 constexpr int PSTR = TK + 8;      // f16 row stride of the probabilities (144 bytes)
 // dynamic LDS of an attention mixer's middle: K tile, V tile, the eight scaled queries as f16 pairs (16 rows), the tile's
 // scores (f32), the probabilities as f16 pairs (16 rows + 16 of zeros: the unused columns of the matrix-core product),
-// the heads' rescaling factors, the merge's partial sums
-constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + 16 * KSTR * 2 + AG * TK * 4 + 32 * PSTR * 2 + AG * 4 + (8 + 8 * 4 * 5) * 4;
+// the heads' rescaling factors, the merge's partial sums, a wave's results on their way to its stores
+constexpr int ATTN_LDS = 2 * TK * KSTR * 2 + 16 * KSTR * 2 + AG * TK * 4 + 32 * PSTR * 2 + AG * 4 + (8 + 8 * 4 * 5) * 4 + AG * HD * 4;
 static_assert(RV + NKV * HD <= RB && NH * HD <= VDIM && NB == NKV * AS && CW == AG && NB == NH * 16 && NH * 2 * HD == 32 * NB &&
               NKV * HD == 2 * NB && NH * HD == 8 * CT && HD == 4 * 64 && (PW % 2) == 0 && (RP % 2) == 0, "attention stage shapes");
 static_assert(!(RA & 1) && !(RA_Z & 1) && !(RB & 1) && !(RB_SS & 1) && !(RC & 1) && !(RD & 1) && !(RS & 1) && !(RE & 1) && !(RE_SC & 1), "");
@@ -160,10 +160,13 @@ IT_DEV void ll_put(u64* p, uint32_t bits, unsigned e) {
     __hip_atomic_store((__attribute__((address_space(1))) u64*)p, ((u64)e << 32) | (u64)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 IT_DEV void ll_putf(u64* p, float v, unsigned e) { ll_put(p, __float_as_uint(v), e); }
-// two neighbouring words (16-byte aligned) in one store; a reader takes a pair only when both stamps are there
+// two neighbouring words (16-byte aligned) in one store; a reader takes a pair only when both stamps are there.
+// (A store of more than 8 bytes reads its data registers up to two wait states after it issues, and the compiler does
+// not see a store inside an asm statement: without the s_nop it may refill those registers for the next store at once,
+// and the first store then carries the second one's values.)
 IT_DEV void ll_put2f(u64* p, float v0, float v1, unsigned e) {
     const v4u w = {__float_as_uint(v0), e, __float_as_uint(v1), e};
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(w) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(w) : "memory");
 }
 
 // true when the wait must stop: the tries are used up (this thread raises the abort word) or another wait gave up
@@ -489,6 +492,7 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
     float* const Af = (float*)(P16 + 32 * PSTR);      // [8] what a head's sums so far are scaled by
     float* const sm = Af + AG;           // 8 wave maxima
     float* const ws = sm + 8;            // 8 waves x 4 dim groups x (4 sums + the weight)
+    float* const Ot = ws + 8 * 4 * 5;    // [8 waves][8 heads][32 dims]: a wave's weighted sums on their way to its stores
     bool ok = true;
     const int n_pos = *at.n_pos;
     const int kpb = max(1, (n_pos + AS - 1) / AS);
@@ -646,13 +650,20 @@ __attribute__((noinline)) __device__ AttnCoreR attn_core(it_gptr<const float> q_
             AC_STAMP(2);   // the range's keys done
 #pragma unroll
             for (int i = 0; i < 16; i++) o[i] += ror8(o[i]);   // high + low halves of the probabilities
-            if (c32 < AG) {   // column = head: this wave's 32 dims of it, 16 a lane
-                u64* part = ll + RP + (int64_t)((kvh * AG + c32) * AS + split) * PW + 32 * wave + 4 * g2;
+            // The wave's 8 heads x 32 dims sit in 16 of its lanes, 16 values each; stored from there they would be eight
+            // stores of a quarter-full wave.  Through a piece of LDS of the wave's own (no barrier: a wave's LDS
+            // operations complete in order) every lane gets four dims of one head: two full stores.
+            {
+                float* const Ow = Ot + wave * (AG * 32);   // [8 heads][32 dims]
+                if (c32 < AG) {
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    ll_put2f(part + 8 * q, o[4 * q], o[4 * q + 1], e);
-                    ll_put2f(part + 8 * q + 2, o[4 * q + 2], o[4 * q + 3], e);
+                    for (int q = 0; q < 4; q++) *(float4*)(Ow + c32 * 32 + 8 * q + 4 * g2) = make_float4(o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]);
                 }
+                const int hd8 = lane >> 3, d4 = lane & 7;
+                const float4 ov = *(const float4*)(Ow + hd8 * 32 + 4 * d4);
+                u64* part = ll + RP + (int64_t)((kvh * AG + hd8) * AS + split) * PW + 32 * wave + 4 * d4;
+                ll_put2f(part, ov.x, ov.y, e);
+                ll_put2f(part + 2, ov.z, ov.w, e);
             }
             if (lane == 0) {   // wave = head for the softmax's sums
                 u64* part = ll + RP + (int64_t)((kvh * AG + wave) * AS + split) * PW;
