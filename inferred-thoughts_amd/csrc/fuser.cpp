@@ -726,9 +726,9 @@ bool chain_attn_in(const FusedGemvP& a, ChainTail* t) {
 // a whole attention block as a chain layer: in-projection, attention launch and out-projection must be the shapes the
 // chain's stages are written for and hang together (the attention reads what the in-projection writes and writes what
 // the out-projection reads; the gate is the second half of every head's wq rows)
-// Beyond this many positions the block stays between two chains: the chain's attention is f32 on the vector ALU (3.5 us
-// of a layer at 5,800 positions, ahead of the matrix-core kernels by 4 % of a token at 30,000; its time grows with the
-// context, theirs far less)
+// Beyond this many positions the block stays between two chains: the chain's attention walks a range's keys 64 at a
+// time in one block per (KV head, range) and is measured up to 30,000 positions; the split-K kernels between chains
+// size their grid to the context
 constexpr int CHAIN_ATTN_MAX_POS = 65536;
 bool chain_attn(const Plan& pl, const FusedGemvP& in, const Plan::Launch& at, const FusedGemvP& out, ChainAttn* a, ChainMixer* m) {
     const int slot = pl.dyn_index(at.aa.n_pos_dyn);

@@ -23,7 +23,8 @@
 // An attention layer's mixer (src/model/qwen35.rs:1141-1223) is five stages of its own in front of its FFN's D, E, F:
 //   the in-projection (rms_norm + Q8_0 + wq / wk / wv rows), published like stage A's outputs;
 //   head norm + rotation of the queries and of the new key, the new cache rows, and the attention of eight query heads
-//   over one of 128 ranges of the context per block, f32 on the vector ALU, with the range's K / V rows in flight
+//   over one of 128 ranges of the context per block, on the f16 matrix cores with exact operands (queries and
+//   probabilities as f16 pairs, f32 sums), with the range's K / V rows in flight
 //   before the queries are waited for; the merge of the ranges with the sigmoid gate, 16 dims a block; the
 //   out-projection + residual.  The middle three are a function of their own (attn_core).
 // (The older form stays for contexts beyond what that attention is good for, and as a measurement switch: the
@@ -439,9 +440,9 @@ IT_DEV bool norm_quant(float4 v, float4 w, float eps, int8_t* xq, float* xs, dou
 //
 // Key ranges.  Block b: KV head b % 2, range b / 2 of 128 equal ranges of the live context (the last range that holds
 // keys holds the new position, whose key and value rows this block forms and writes to the cache).  Wave w: query head
-// w of the KV head's eight.  The range's rows are in flight before the queries are waited for; scores with 16 lanes a
-// key, softmax bookkeeping a wave, weighted values with 4 dims a lane: all f32 on the vector ALU (a range is a few dozen
-// keys at the contexts this path is measured at; longer ones walk tiles of 64 keys).
+// w of the KV head's eight.  The range's rows are in flight before the queries are waited for; scores and weighted
+// values on the f16 matrix cores (layouts at the loop), softmax bookkeeping a wave per head; a range is a few dozen
+// keys at the contexts this path is measured at, longer ones walk tiles of 64 keys.
 // Merge.  Block b: 16 dims of query head b / 16; thread t: range t / 4, four of the 16 dims.
 extern __shared__ __align__(16) uint8_t chain_dyn_lds[];   // ATTN_LDS bytes when a layer of the chain is an attention mixer
 typedef __attribute__((address_space(1))) uint16_t g_u16;

@@ -392,7 +392,7 @@ def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
             got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
             assert np.abs(want).max() > 0.05
             # (the first two passes are issued op by op, before there is a chain: their attention rounds the probabilities
-            # to f16 for the matrix cores and is held to 5e-3; the chain's is f32 throughout)
+            # to f16 for the matrix cores and is held to 5e-3; the chain's takes them as exact f16 pairs)
             assert near(got, want, 5e-3 if p < 2 else 2e-3), (p, far(got, want))
             print(f"  pass {p}: {far(got, want):.3g} of the scale", flush=True)
             for t in "kv":
@@ -522,7 +522,7 @@ def test_an_attention_layer_between_chains(attn_in_chain, monkeypatch):
     for a, b in zip(ka, kb):
         assert near(a, b), far(a, b)
     if attn_in_chain:
-        # The chain's attention is f32 throughout, the per-stage kernel rounds the probabilities to f16 for the matrix
+        # The chain's attention takes the probabilities as exact f16 pairs, the per-stage kernel rounds the probabilities to f16 for the matrix
         # cores: 1e-4 of the attention output, which the quantization in front of the out-projection and the two blocks
         # behind turn into per cent (the docstring's measurement).  What is in front of the attention is held as
         # everywhere (layer 0's state, the new K / V rows above); what is behind it grossly here, and sharply in
