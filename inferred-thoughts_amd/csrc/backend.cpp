@@ -78,6 +78,9 @@ void it_hip::dyn_rotate() {
 }
 void it_hip::dyn_upload() {
     if (!dyn_count) return;
+    // a token's pass has a few dozen: they go with a small kernel's arguments (between two replayed passes a
+    // host-to-device copy is a transfer the stream waits for); a long pass's thousands are copied
+    if (itk::poke_ints(dyn_dev, dyn_host, (int)dyn_count, stream)) return;
     check(hipMemcpyAsync(dyn_dev, dyn_host, dyn_count * sizeof(int), hipMemcpyHostToDevice, stream), "upload positions");
     if (hipEventRecord(dyn_evt[dyn_cur], stream) == hipSuccess) dyn_evt_used[dyn_cur] = true;
 }

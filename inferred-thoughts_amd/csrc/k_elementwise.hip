@@ -3,6 +3,7 @@
 // Each kernel keeps the accumulation order of the reference's scalar CPU path
 // (/root/reference src/ops/naive.rs) wherever the `exact` flag is set; the fast
 // variants reorder only the long f64 sums (tree instead of serial).
+#include <cstring>
 #include "it_device.h"
 #include "kernels.h"
 #include "it_reduce.h"
@@ -328,6 +329,14 @@ __global__ void kv_write_k(uint16_t* __restrict__ slab, int64_t offset, const in
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
         slab[off + i] = it_f32_to_f16(src[i]);
 }
+// a few host values into device memory with the launch itself: they travel in the argument block, so the stream sees
+// one small kernel where a host-to-device copy would put a transfer (and its wait) between two passes
+struct PokeInts {
+    int v[POKE_MAX];
+};
+__global__ void poke_ints_k(int* __restrict__ dst, PokeInts v, int n) {
+    if ((int)threadIdx.x < n) dst[threadIdx.x] = v.v[threadIdx.x];
+}
 __global__ void fill_zero_k(uint32_t* p, int64_t n_words) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words;
          i += (int64_t)gridDim.x * blockDim.x)
@@ -429,6 +438,13 @@ void scatter_chunks(const float* src, int64_t src_len, int64_t chunk, int64_t st
 void kv_write(uint16_t* slab, int64_t offset, const int* offset_dyn, int64_t offset_mul, const float* src,
               int64_t n, hipStream_t s) {
     EW_LAUNCH(kv_write_k, n, slab, offset, offset_dyn, offset_mul, src, n);
+}
+bool poke_ints(int* dst, const int* host_values, int n, hipStream_t s) {
+    if (n < 1 || n > POKE_MAX) return false;
+    PokeInts v;
+    std::memcpy(v.v, host_values, (size_t)n * sizeof(int));
+    hipLaunchKernelGGL(poke_ints_k, dim3(1), dim3(POKE_MAX), 0, s, dst, v, n);
+    return true;
 }
 void fill_zero(void* p, int64_t bytes, hipStream_t s) {
     int64_t words = bytes / 4;

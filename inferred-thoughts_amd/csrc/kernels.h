@@ -159,6 +159,10 @@ void scatter_chunks(const float* src, int64_t src_len, int64_t chunk, int64_t st
 void kv_write(uint16_t* slab, int64_t offset, const int* offset_dyn, int64_t offset_mul, const float* src,
               int64_t n, hipStream_t s);
 void fill_zero(void* p, int64_t bytes, hipStream_t s);
+// n <= POKE_MAX host ints to device memory as one small kernel whose argument block carries them (the host array may be
+// reused as soon as the call returns); false: too many, nothing was launched
+constexpr int POKE_MAX = 256;
+bool poke_ints(int* dst, const int* host_values, int n, hipStream_t s);
 void argmax(const float* x, int64_t n, int32_t* out, int32_t* scratch_idx, float* scratch_val, hipStream_t s);
 // x = dequantized row `*token` of an embedding table (Q8_0 repacked, F16, BF16 or F32); the id goes to
 // ring[ring_dyn ? *ring_dyn : ring_idx] when ring is non-null
