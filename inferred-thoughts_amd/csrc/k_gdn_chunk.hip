@@ -41,7 +41,7 @@ namespace {
 constexpr int GC = 64;                      // tokens per chunk
 constexpr int TS = GC + 4;                  // LDS row stride of the 64 x 64 matrices
 constexpr int DVS = 16;                     // value rows per block of the scan
-constexpr int US = 20;                      // LDS row stride of U: with the token order of the state update, no bank is hit twice
+constexpr int US = 20;                      // LDS row stride of U and of R: four rows apart are 16 banks apart
 // per (chunk, head): T[64][64], P[64][64], e^{c_t}, e^{c_C - c_t}, beta_t, and e^{c_C} in one padded row
 constexpr int WS_T = 0, WS_P = GC * GC, WS_GAM = 2 * GC * GC, WS_DEC = WS_GAM + GC, WS_BET = WS_DEC + GC,
               WS_GC = WS_BET + GC, WS_FLOATS = WS_GC + GC;
@@ -192,8 +192,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_k(DeltaArgs d, const float
     float* Ps = Ts + GC * TS;        // [64][TS]
     float* Ss = Ps + GC * TS;        // [16][LS]
     float* Vs = Ss + DVS * LS;       // [64][16]
-    float* Rs = Vs + GC * DVS;       // [64][16]
-    float* Us = Rs + GC * DVS;       // [64][US]
+    float* Rs = Vs + GC * DVS;       // [64][US]
+    float* Us = Rs + GC * US;        // [64][US]
     float* gam = Us + GC * US;       // [64] e^{c_t}
     float* dec = gam + GC;           // [64] e^{c_C - c_t}
     float* bet = dec + GC;           // [64]
@@ -297,35 +297,33 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_k(DeltaArgs d, const float
         // operands of four steps are read while the four steps before them are on the matrix unit
         v4f aw = {0.f, 0.f, 0.f, 0.f}, ao = {0.f, 0.f, 0.f, 0.f};
         {
+            // (the k order inside a step of 16 is free as long as both operands agree: lane group g takes k = 4 g + j in
+            // step j, so that a lane's four values are one 16-byte read, which no two lanes of a pass take from one bank)
             constexpr int NB = DK / 16;
-            float ka[2][4], qa[2][4], sb[2][4];
-            const float* kp = Ks + (16 * w + m) * LS + g;
-            const float* qp = Qs + (16 * w + m) * LS + g;
-            const float* sp = Ss + m * LS + g;
-#pragma unroll
-            for (int u = 0; u < 4; u++) { ka[0][u] = kp[4 * u]; qa[0][u] = qp[4 * u]; sb[0][u] = sp[4 * u]; }
+            float4 ka[2], qa[2], sb[2];
+            const float* kp = Ks + (16 * w + m) * LS + 4 * g;
+            const float* qp = Qs + (16 * w + m) * LS + 4 * g;
+            const float* sp = Ss + m * LS + 4 * g;
+            ka[0] = *(const float4*)kp; qa[0] = *(const float4*)qp; sb[0] = *(const float4*)sp;
 #pragma unroll
             for (int b = 0; b < NB; b++) {
                 if (b + 1 < NB) {
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        ka[(b + 1) & 1][u] = kp[16 * (b + 1) + 4 * u];
-                        qa[(b + 1) & 1][u] = qp[16 * (b + 1) + 4 * u];
-                        sb[(b + 1) & 1][u] = sp[16 * (b + 1) + 4 * u];
-                    }
+                    ka[(b + 1) & 1] = *(const float4*)(kp + 16 * (b + 1));
+                    qa[(b + 1) & 1] = *(const float4*)(qp + 16 * (b + 1));
+                    sb[(b + 1) & 1] = *(const float4*)(sp + 16 * (b + 1));
                 }
                 __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of the products they overlap
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    aw = mfma4(ka[b & 1][u], sb[b & 1][u], aw);
-                    ao = mfma4(qa[b & 1][u], sb[b & 1][u], ao);
-                }
+                const float4 k4 = ka[b & 1], q4 = qa[b & 1], s4v = sb[b & 1];
+                aw = mfma4(k4.x, s4v.x, aw); ao = mfma4(q4.x, s4v.x, ao);
+                aw = mfma4(k4.y, s4v.y, aw); ao = mfma4(q4.y, s4v.y, ao);
+                aw = mfma4(k4.z, s4v.z, aw); ao = mfma4(q4.z, s4v.z, ao);
+                aw = mfma4(k4.w, s4v.w, aw); ao = mfma4(q4.w, s4v.w, ao);
             }
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int t = 16 * w + 4 * g + i;
-            Rs[t * DVS + m] = bet[t] * (Vs[t * DVS + m] - gam[t] * aw[i]);
+            Rs[t * US + m] = bet[t] * (Vs[t * DVS + m] - gam[t] * aw[i]);
             ao[i] *= gam[t];
         }
         GDN_STAMP(4);
@@ -336,9 +334,12 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_k(DeltaArgs d, const float
         // U = T R: rows of T at or left of the diagonal tile
         v4f au = {0.f, 0.f, 0.f, 0.f};
         for (int s4 = 0; s4 <= w; s4++) {
-#pragma unroll
-            for (int s = 4 * s4; s < 4 * s4 + 4; s++)
-                au = mfma4(Ts[(16 * w + m) * TS + 4 * s + g], Rs[(4 * s + g) * DVS + m], au);
+            const float4 t4 = *(const float4*)(Ts + (16 * w + m) * TS + 16 * s4 + 4 * g);
+            const float* rp_ = Rs + (16 * s4 + 4 * g) * US + m;
+            au = mfma4(t4.x, rp_[0], au);
+            au = mfma4(t4.y, rp_[US], au);
+            au = mfma4(t4.z, rp_[2 * US], au);
+            au = mfma4(t4.w, rp_[3 * US], au);
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) Us[(16 * w + 4 * g + i) * US + m] = au[i];
@@ -349,9 +350,12 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_k(DeltaArgs d, const float
 
         // O = e^{c} Q S0^T + P U
         for (int s4 = 0; s4 <= w; s4++) {
-#pragma unroll
-            for (int s = 4 * s4; s < 4 * s4 + 4; s++)
-                ao = mfma4(Ps[(16 * w + m) * TS + 4 * s + g], Us[(4 * s + g) * US + m], ao);
+            const float4 p4 = *(const float4*)(Ps + (16 * w + m) * TS + 16 * s4 + 4 * g);
+            const float* up_ = Us + (16 * s4 + 4 * g) * US + m;
+            ao = mfma4(p4.x, up_[0], ao);
+            ao = mfma4(p4.y, up_[US], ao);
+            ao = mfma4(p4.z, up_[2 * US], ao);
+            ao = mfma4(p4.w, up_[3 * US], ao);
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -410,7 +414,7 @@ template <int DK>
 static bool launch_chunked(const DeltaArgs& d, float* state, float* out, float* work, float q_scale, hipStream_t s) {
     constexpr int LS = DK + 4;
     const size_t prep_lds = (2 * GC * LS + 2 * GC) * sizeof(float);
-    const size_t scan_lds = (2 * GC * LS + 2 * GC * TS + DVS * LS + 2 * GC * DVS + GC * US + 4 * GC) * sizeof(float);
+    const size_t scan_lds = (2 * GC * LS + 2 * GC * TS + DVS * LS + GC * DVS + 2 * GC * US + 4 * GC) * sizeof(float);
     static bool sized = false;
     if (!sized) {
         if (hipFuncSetAttribute((const void*)gdn_chunk_prep_k<DK>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds) != hipSuccess ||
