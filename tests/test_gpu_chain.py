@@ -335,14 +335,15 @@ def test_a_wait_that_gives_up_is_an_error_not_a_hang():
     assert err is None, err
 
 
-@pytest.mark.parametrize("pos0", [5800, 40, 12000])
+@pytest.mark.parametrize("pos0", [5800, 40, 12000, 8189])
 def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
     """One attention layer whose FFN adds nothing (second scales of zero on every down product), so that the pass's
     change of the residual stream IS the mixer's output: in-projection, head norms, rotation, the new cache rows,
     attention over the context in 128 key ranges, merge, sigmoid gate, out-projection, all stages of the persistent
     kernel.  Held to the oracle at 2e-3 of the vector's scale and the new K / V rows at 2e-3 of the row's, five
     positions each: a context of 5,800 (a range is 46 keys: one tile), of 40 (fewer keys than ranges: most blocks have
-    none) and of 12,000 (a range is 94 keys: two tiles with the running maximum carried across)."""
+    none), of 12,000 (a range is 94 keys: two tiles with the running maximum carried across) and of 8,189 (a range grows
+    from 64 keys, one full tile, to 65: a second tile of one key)."""
     NH, NKV, AHD, NROT, THETA, NCTX = 16, 2, 256, 64, 1e7, 12288
     qd, kd = NH * AHD, NKV * AHD
     sc = float(1.0 / np.sqrt(np.float32(AHD)))
