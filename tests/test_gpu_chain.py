@@ -380,7 +380,13 @@ def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
             ops.add_assign(x, b["mixed"])
             layers.ffn(ops, i, layers.L[0], B[i]["layers"][0], x, is_hip)
 
-        for p in range(PASSES):
+        # Position 8,192 is where the rotation table doubles (an allocation: the recorded graph is dropped, that pass and
+        # the next run op by op, the one after is recorded again); the context that crosses it runs three passes more,
+        # so that ranges of 65 keys (a full tile and a tile of one key) go through the chain as well
+        crossing = pos0 < 8192 <= pos0 + PASSES
+        n_pass = PASSES + 3 if crossing else PASSES
+        op_by_op = {0, 1} | ({8192 - pos0, 8193 - pos0} if crossing else set())
+        for p in range(n_pass):
             pos = pos0 + p
             x0 = rng(850 + p).standard_normal(ND).astype(np.float32)
             print(f"attention mixer in the chain, pass {p} at position {pos}", flush=True)
@@ -392,9 +398,9 @@ def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
             run(orc, 1, False, pos)
             got, want = B[0]["x"] - x0, B[1]["x"].astype(np.float64) - x0
             assert np.abs(want).max() > 0.05
-            # (the first two passes are issued op by op, before there is a chain: their attention rounds the probabilities
-            # to f16 for the matrix cores and is held to 5e-3; the chain's takes them as exact f16 pairs)
-            assert near(got, want, 5e-3 if p < 2 else 2e-3), (p, far(got, want))
+            # (the passes issued op by op, before there is a chain: their attention rounds the probabilities to f16 for
+            # the matrix cores and is held to 5e-3; the chain's takes them as exact f16 pairs)
+            assert near(got, want, 5e-3 if p in op_by_op else 2e-3), (p, far(got, want))
             print(f"  pass {p}: {far(got, want):.3g} of the scale", flush=True)
             for t in "kv":
                 a = slabs[0][t].view(np.float16).astype(np.float32); b = slabs[1][t].view(np.float16).astype(np.float32)
@@ -402,7 +408,10 @@ def test_the_attention_mixer_inside_a_chain_against_the_oracle(pos0):
                 assert near(a[pos * kd:(pos + 1) * kd], b[pos * kd:(pos + 1) * kd]), (p, t)
                 slabs[1][t][pos * kd:(pos + 1) * kd] = slabs[0][t][pos * kd:(pos + 1) * kd]
         g, c = hip.graph_stats(), hip.chain_stats()
-        assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] == PASSES - 2, g
+        if crossing:
+            assert g["captures"] == 2 and g["aborts"] == 1, g
+        else:
+            assert g["captures"] == 1 and g["aborts"] == 0 and g["replays"] == PASSES - 2, g
         assert c["chains"] == 1 and c["layers"] == 1 and g["graph_kernels"] == 1, (g, c)
     finally:
         err = hip.take_error()
