@@ -1236,6 +1236,11 @@ it_hip* it_hip_create(uint32_t flags, int device, char* err, size_t err_len) {
     be->count_reads_in_fused = getenv("INFERRED_HIP_NO_READ_COUNTERS") == nullptr;
     be->small_ffn_enabled = getenv("INFERRED_HIP_NO_SMALL_FFN") == nullptr;
     be->chain_attn_enabled = getenv("INFERRED_HIP_NO_CHAIN_ATTN") == nullptr;
+    be->chain_max_layers = itk::CHAIN_MAX_LAYERS;
+    if (const char* cl = getenv("INFERRED_HIP_CHAIN_LAYERS")) {
+        const int v = atoi(cl);
+        if (v >= 1 && v <= itk::CHAIN_MAX_LAYERS) be->chain_max_layers = v;
+    }
     if (getenv("INFERRED_HIP_NO_GRAPH")) be->allow_graph = false;
     if (const char* sl = getenv("INFERRED_HIP_CHAIN_SPINS")) {
         const long v = atol(sl);

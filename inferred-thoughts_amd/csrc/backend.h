@@ -259,6 +259,7 @@ struct it_hip {
     };
     ChainRes chain;
     bool chain_enabled = true;
+    int chain_max_layers = 56;               // layers a chain may hold (CHAIN_MAX_LAYERS); INFERRED_HIP_CHAIN_LAYERS=n cuts a token into shorter chains (a measurement switch: hardware counters read short over a dispatch of a millisecond)
     bool chain_attn_enabled = true;          // attention mixers inside the chains; INFERRED_HIP_NO_CHAIN_ATTN=1 keeps their kernels between two chains (a measurement switch)
     bool count_reads_in_fused = true;  // the fused decode kernels add the picks to the expert read counters (off: a measurement switch)
     bool eager_fused = false;          // single-token passes without a graph still go through the fuser (measurement switch)

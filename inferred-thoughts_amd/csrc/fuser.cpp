@@ -855,7 +855,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         bool taken = false;
         if (is_attn && be->chain_attn_enabled) {
             // the whole block as a layer of the chain (its FFN follows)
-            if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            if (mixer_open || cp.n_layers >= be->chain_max_layers) emit();
             ChainAttn a{};
             ChainMixer m{};
             if (chain_attn(pl, ls[0].gv, ls[1], ls[2].gv, &a, &m) && (cp.n_layers == 0 || cp.x == ls[0].gv.x)) {
@@ -896,7 +896,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
             continue;
         }
         if (is_gdn) {
-            if (mixer_open || cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            if (mixer_open || cp.n_layers >= be->chain_max_layers) emit();
             ChainMixer m{};
             int rf = 0;
             if (chain_mixer(ls[0].gv, ls[1].gc, ls[2].gv, &m, &rf) && (cp.n_layers == 0 || cp.x == ls[0].gv.x) && (chain_rf < 0 || chain_rf == rf)) {
@@ -913,7 +913,7 @@ void build_chains(Plan& pl, unsigned long long* tally) {
         } else if (is_ffn) {
             ChainFfn f{};
             int sh_fmt = 0;
-            if (!mixer_open && cp.n_layers == CHAIN_MAX_LAYERS) emit();
+            if (!mixer_open && cp.n_layers >= be->chain_max_layers) emit();
             int rf = 0;
             const bool fits = chain_ffn(ls[0].gv, ls[1].mg, ls[2].md, &f, &sh_fmt, &rf) && (chain_rf < 0 || chain_rf == rf) &&
                               (cp.n_layers == 0 || (cp.x == ls[0].gv.x && (cp.sh_fmt == sh_fmt || (cp.n_layers == 1 && mixer_open))));
