@@ -29,14 +29,16 @@
 #include "kernels.h"
 
 // Phase stamps for tuning: a build with -DIT_STAMPS records the 100 MHz wall clock of one block's first
-// lane at the marked points of one k slab; the library build compiles them away.
+// lane at the marked points of five consecutive k slabs; the library build compiles them away.
 #ifdef IT_STAMPS
 __device__ long long it_gemm_stamps[32];
-__device__ int it_gemm_stamp_tile, it_gemm_stamp_slab;
-#define GEMM_STAMP(i)                                                                                        \
-    do {                                                                                                     \
-        if ((int)blockIdx.x == it_gemm_stamp_tile && blockIdx.y == 0 && s == it_gemm_stamp_slab && tid == 0) \
-            it_gemm_stamps[i] = wall_clock64();                                                              \
+__device__ int it_gemm_stamp_tile, it_gemm_stamp_slab, it_gemm_stamp_glu;
+// (five consecutive slabs of one block, six stamps each)
+#define GEMM_STAMP(i)                                                                                                  \
+    do {                                                                                                               \
+        if ((int)blockIdx.x == it_gemm_stamp_tile && (GLU ? 1 : 0) == it_gemm_stamp_glu && s >= it_gemm_stamp_slab && \
+            s < it_gemm_stamp_slab + 5 && tid == 0)                                                                    \
+            it_gemm_stamps[6 * (s - it_gemm_stamp_slab) + (i)] = wall_clock64();                                       \
     } while (0)
 #else
 #define GEMM_STAMP(i) \
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(256) void acts_split_f16_k(const int8_t* __restrict
 
 
 template <bool GLU, int T>
-__device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int4 td, uint16_t* Bh, uint16_t* Bl,
+__device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int4 td, const int row_block, uint16_t* Bh, uint16_t* Bl,
                                                  uint8_t* Wn, uint8_t* Wsc, const int* xrow_s, const int* pair_s) {
     const int64_t e = td.x;
     const int cnt = td.z;
@@ -104,7 +106,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     const int n_in = p.n_in, nslab = n_in / FK;
     // the two row sets of this wave
     const int rows_per_block = GLU ? 128 : 256;
-    const int rb0 = blockIdx.y * rows_per_block + (GLU ? 32 : 64) * wave;
+    const int rb0 = row_block * rows_per_block + (GLU ? 32 : 64) * wave;
     const int rbase[2] = {rb0, GLU ? rb0 : rb0 + 32};
     const uint8_t* wq0 = it_expert_at(p.q, p.q_tab, e, p.q_stride);
     const uint8_t* ws0 = it_expert_at(p.s, p.s_tab, e, p.s_stride);
@@ -120,7 +122,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     for (int i = 0; i < 4; i++) {
         const int seg = (tid >> 3) + 64 * i;
         const int z = GLU ? seg >> 7 : 0;
-        const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? seg & 127 : seg), p.n_out - 1);
+        const int64_t row = min(row_block * rows_per_block + (GLU ? seg & 127 : seg), p.n_out - 1);
         // (picked by a conditional, not by an index into the array: a pointer that went through an indexed array is a
         // generic pointer to the compiler, and loads through it are flat loads that every LDS wait has to drain)
         wload[i] = (z ? wq[1] : wq[0]) + row * (n_in >> 1) + piece * 16;
@@ -129,7 +131,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     {
         const int st = tid & 255;
         const int z = GLU ? st >> 7 : 0;
-        const int64_t row = min((int)blockIdx.y * rows_per_block + (GLU ? st & 127 : st), p.n_out - 1);
+        const int64_t row = min(row_block * rows_per_block + (GLU ? st & 127 : st), p.n_out - 1);
         sload = (z ? ws[1] : ws[0]) + row * (n_in >> 4);
     }
 
@@ -138,7 +140,10 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     // then reads its own 16 nibble bytes and 2 scale bytes of the NEXT 64-wide slab and expands them to
     // f16 fragments one at a time between the MFMA groups of the current slab.  Tokens run one slab
     // ahead through registers into the other LDS token buffer.  Inside a slab the token fragments of the
-    // next MFMA group are read from LDS while the current group is on the matrix unit.
+    // next MFMA group are read from LDS while the current group is on the matrix unit.  Loads and LDS
+    // stores are dealt out between the MFMA groups one or two at a time (loads over the first groups,
+    // the stores of what they brought over the later ones), and the slab's one barrier stands in front
+    // of its last group.
     const int n_super = n_in / FSUPER;
     uint4 rw[4], rsw;
     uint4 rbh[T], rbl[T];   // 64 * T tokens x 8 segments of 16 bytes = 512 * T segments per array
@@ -200,6 +205,31 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
             *(uint2*)(dl + 4) = make_uint2(rbl[u].z, rbl[u].w);
         }
     };
+    // The same stores one at a time, to go between the MFMA groups of the slab's second half: issued together at the
+    // slab's end, the stores of all eight waves are a burst that the LDS works off while no wave has a product to issue,
+    // and every wave's first read of the next slab queues behind it (measured with the stores, or the barrier behind
+    // them, taken out: a third of the kernel's time).
+    // (one address register per staged row: buffer, hi / lo half and part are constant offsets from it; Bl lies
+    // 2 * FPAIRS * FBS behind Bh)
+    uint16_t* xdst[T];
+#pragma unroll
+    for (int u = 0; u < T; u++) {
+        const int idx = tid + u * 512;
+        xdst[u] = Bh + (idx >> 3) * FBS + (idx & 7) * 8;
+    }
+    auto stash_x_part = [&](int buf, int i) __attribute__((always_inline)) {   // i < 4 T
+        const int u = i >> 2, part = i & 3;
+        uint16_t* d = xdst[u] + buf * FPAIRS * FBS + (part < 2 ? 0 : 2 * FPAIRS * FBS) + 4 * (part & 1);
+        const uint4 v = part < 2 ? rbh[u] : rbl[u];
+        *(uint2*)d = (part & 1) ? make_uint2(v.z, v.w) : make_uint2(v.x, v.y);
+    };
+    auto stash_w_part = [&](int b, int i) __attribute__((always_inline)) {   // i < 5
+        // (the register set picked by conditionals: indexed by a value the compiler does not fold early enough, the
+        // array would live in scratch memory)
+        const uint4 v = i == 0 ? rw[0] : i == 1 ? rw[1] : i == 2 ? rw[2] : rw[3];
+        if (i < 4) *(uint4*)(Wn + (b * 256 + (tid >> 3) + 64 * i) * FWS + piece * 16) = v;
+        else if (tid < 256) *(uint4*)(Wsc + (b * 256 + tid) * 16) = rsw;
+    };
     // this lane's nibbles and scales of slab j of the super-slab in weight buffer b
     uint4 ra[2];
     uint32_t rs[2];
@@ -258,7 +288,14 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
     for (int z = 0; z < 2; z++)
 #pragma unroll
         for (int n = 0; n < 4; n++) af[0][z][n] = expand(z, n);
-    // one super-slab (four slabs) per trip so that every register array is indexed by a constant
+    if (live_half) read_nib(0, 1);   // (a row has at least one super-slab: slab 1 is there)
+    Tok first = read_tok(0, 0, 0);
+    // One super-slab (four slabs) per trip so that every register array is indexed by a constant.
+    // The slab's barrier stands IN FRONT of its last MFMA group, whose operands are in registers by then: behind it every
+    // wave asks for the first token fragment and the nibbles of what comes next and then still has that group to issue,
+    // so the wait for the slowest wave and the LDS round trip of the first read run under products instead of between
+    // two slabs.  Everything that the barrier orders is ahead of it: the last read of this slab's token buffer, the
+    // stores of the next slab's tokens and of the next super-slab's weights.
     for (int S = 0; S < n_super; S++) {
         const int wb = S & 1;
         const bool more_w = S + 1 < n_super;
@@ -267,10 +304,10 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
             const int par = j & 1;
             const int s = 4 * S + j;
             const bool more = j < 3 || more_w;
+            const bool more2 = j < 2 || more_w;
             GEMM_STAMP(0);
             GEMM_STAMP(1);
-            if (more && live_half) read_nib(j < 3 ? wb : wb ^ 1, j < 3 ? j + 1 : 0);
-            Tok cur = read_tok(par, 0, 0);
+            Tok cur = first;
 #pragma unroll
             for (int n = 0; n < 4; n++) {
                 // one fragment pair of the next slab between the MFMA groups of this one
@@ -285,6 +322,28 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
                     if (g1 < 4 * T) nxt = read_tok(par, g1 / T, g1 % T);
 #pragma unroll
                     for (int q = (g1 - 1) * LPG; q < g1 * LPG; q++) fetch_one(q, s + 1, S + 1, more, j == 0 && more_w);
+                    // the next super-slab's weights (loaded a slab ago) over this slab's first groups, the next slab's
+                    // tokens (asked for in this slab's first groups) over the groups of its second half but the last
+                    if (j == 1 && more_w) {
+                        constexpr int WPG = T == 1 ? 2 : 1;
+#pragma unroll
+                        for (int i = (g1 - 1) * WPG; i < g1 * WPG; i++)
+                            if (i < 5) stash_w_part(wb ^ 1, i);
+                    }
+                    if (more && g1 > 2 * T && g1 < 4 * T) {
+                        constexpr int PPG = (4 * T + 2 * T - 2) / (2 * T - 1);
+#pragma unroll
+                        for (int i = (g1 - 2 * T - 1) * PPG; i < (g1 - 2 * T) * PPG; i++)
+                            if (i < 4 * T) stash_x_part(par ^ 1, i);
+                    }
+                    if (g1 == 4 * T) {
+                        GEMM_STAMP(2);
+                        __syncthreads();
+                        GEMM_STAMP(3);
+                        if (more) first = read_tok(par ^ 1, 0, 0);
+                        // (the nibbles of the slab after next: this slab's expansions are done)
+                        if (more2 && live_half) read_nib(j < 2 ? wb : wb ^ 1, (j + 2) & 3);
+                    }
                     __builtin_amdgcn_sched_barrier(0);   // the reads stay ahead of the products they overlap
                     if (live_half) {   // a wave set whose token groups lie past the tile's pairs only helps with the staging
 #pragma unroll
@@ -296,12 +355,7 @@ __device__ __forceinline__ void experts_f16_body(const ExpertsF16P& p, const int
                     cur = nxt;
                 }
             }
-            GEMM_STAMP(2);
-            if (j == 1 && more_w) stash_w(wb ^ 1);
-            GEMM_STAMP(3);
-            if (more) stash_x(par ^ 1);
             GEMM_STAMP(4);
-            __syncthreads();
             GEMM_STAMP(5);
         }
     }
@@ -348,7 +402,12 @@ __global__ __launch_bounds__(512) void experts_f16_k(ExpertsF16P p) {
     uint8_t* Wn = (uint8_t*)(flds + 4 * FPAIRS * FBS);   // [2][256][FWS]: nibble bytes of 256 row segments x 256 k
     uint8_t* Wsc = Wn + 2 * 256 * FWS;             // [2][256][16]: their scale bytes
     __shared__ int xrow_s[FPAIRS], pair_s[FPAIRS];
-    const int tile = blockIdx.x;
+    // Blocks go to the 8 XCDs in turn.  The row blocks of one tile read the same token rows (k slab by k slab, each
+    // row block once: far more bytes than the weights): they take consecutive places on ONE XCD, so that they run
+    // side by side and all but the first find the rows in that XCD's L2.
+    const int n_rb = (p.n_out + (GLU ? 128 : 256) - 1) / (GLU ? 128 : 256);
+    const int lin = blockIdx.x;
+    const int tile = 8 * (lin / (8 * n_rb)) + (lin & 7), row_block = (lin >> 3) % n_rb;
     if (tile >= *p.n_tiles) return;
     const int4 td = p.tiles[tile];
     const int cnt = td.z;
@@ -359,8 +418,8 @@ __global__ __launch_bounds__(512) void experts_f16_k(ExpertsF16P p) {
     }
     __syncthreads();
     // waves 0..3 take the first T token groups of the tile, waves 4..7 the next T
-    if (cnt <= 64) experts_f16_body<GLU, 1>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
-    else experts_f16_body<GLU, 2>(p, td, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
+    if (cnt <= 64) experts_f16_body<GLU, 1>(p, td, row_block, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
+    else experts_f16_body<GLU, 2>(p, td, row_block, Bh, Bl, Wn, Wsc, xrow_s, pair_s);
 }
 
 }  // namespace
@@ -432,9 +491,23 @@ bool experts_gemm_f16(const ExpertsView& w, const ExpertsView* up, const int32_t
     p.n_tiles = n_tiles;
     p.tiles = tiles;
     p.order = order;
-    if (up) hipLaunchKernelGGL(experts_f16_k<true>, dim3(max_tiles, (w.n_out + 127) / 128), dim3(512), lds, s, p);
-    else hipLaunchKernelGGL(experts_f16_k<false>, dim3(max_tiles, (w.n_out + 255) / 256), dim3(512), lds, s, p);
+    const int tiles8 = (max_tiles + 7) / 8 * 8;   // (the kernel deals tiles to the XCDs in groups of eight)
+    if (up) hipLaunchKernelGGL(experts_f16_k<true>, dim3(tiles8 * ((w.n_out + 127) / 128)), dim3(512), lds, s, p);
+    else hipLaunchKernelGGL(experts_f16_k<false>, dim3(tiles8 * ((w.n_out + 255) / 256)), dim3(512), lds, s, p);
     return true;
 }
 
 }  // namespace itk
+
+#ifdef IT_STAMPS
+// tuning builds only: the stamps of the selected block, then the next selection
+extern "C" int it_hip_debug_gemm_stamps(long long* out, int block, int slab, int glu) {
+    if (hipDeviceSynchronize() != hipSuccess) return -1;
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(it_gemm_stamps), 32 * 8) != hipSuccess) return -1;
+    if (hipMemcpyToSymbol(HIP_SYMBOL(it_gemm_stamp_tile), &block, 4) != hipSuccess ||
+        hipMemcpyToSymbol(HIP_SYMBOL(it_gemm_stamp_slab), &slab, 4) != hipSuccess ||
+        hipMemcpyToSymbol(HIP_SYMBOL(it_gemm_stamp_glu), &glu, 4) != hipSuccess)
+        return -1;
+    return 0;
+}
+#endif
