@@ -671,7 +671,7 @@ class Engine:
             self.h = None
 
 
-# ---- the BASELINE configs as synthetic-model recipes ----
+# ---- the benchmark configurations as synthetic-model recipes ----
 def tiny_config(seed: int = 0, **over) -> SynthConfig:
     """Config 1: 4 layers (3 GDN + 1 attention), hidden 512, vocab 4096, 16 experts top-4, all Q8_0."""
     c = SynthConfig(n_layer=4, n_embd=512, n_vocab=4096, n_head=8, n_head_kv=2, head_dim=64, n_rot=16,

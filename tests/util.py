@@ -13,7 +13,7 @@ def q8_0_weights(oracle, r, n_out, n_in, std=0.02):
 
 
 def nvfp4_weights(r, n_out, n_in):
-    """NVFP4 rows as BASELINE config 2 draws them: nibbles uniform over the 16 codes, UE4M3
+    """NVFP4 rows as benchmark configuration 2 draws them: nibbles uniform over the 16 codes, UE4M3
     scale bytes from |N(0,1)| (nearest code, never 0x00/0x7f)."""
     n_blocks = n_out * n_in // 64
     out = np.zeros((n_blocks, 36), np.uint8)
